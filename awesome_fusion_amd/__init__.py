@@ -1,0 +1,24 @@
+"""MI355X-native bfAintBGemm: bf16 activations x int8/int4 weights, fp32 accumulate, bf16 out.
+
+The product is ``libbfaintb_gemm.so`` (hand-written HIP for gfx950 behind the C ABI declared in
+``include/bfaintb_gemm.h``) and the C++ host driver under ``host/``.  This Python package is the
+thin ctypes binding tests and the benchmark call through; it holds no arithmetic of its own and
+has no CPU fallback: without the built library every call raises.
+"""
+from .gemm import (  # noqa: F401
+    BfaintbError,
+    DECODE,
+    PREFILL,
+    AUTO,
+    build_library,
+    dequant,
+    error_string,
+    gemm,
+    kernel_name,
+    lib,
+    library_path,
+    split_k,
+    variant,
+    workspace_bytes,
+    workspace_init,
+)

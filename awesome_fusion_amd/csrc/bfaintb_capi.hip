@@ -1,0 +1,220 @@
+// C ABI of the library: argument validation, kernel-family choice, split-K sizing, launches.
+// Stands where the reference driver packs its kernarg block and calls hipModuleLaunchKernel
+// (/root/reference/bfAintBGemm/bfAintBGemm.cc:107-152); unlike GPU_CHECK_ERROR
+// (gpu_utils.hpp:5-11, print and exit(0)) every failure is returned to the caller.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "bfaintb_device.hpp"
+#include "../../include/bfaintb_gemm.h"
+
+namespace bfaintb {
+hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_dequant(uint16_t* w, const uint8_t* b, const uint16_t* scale, uint32_t n, uint32_t k, uint32_t ldb_bytes,
+                          uint32_t ldw, int bits, uint32_t group_size, hipStream_t stream);
+hipError_t launch_fill_u32(uint32_t* dst, uint32_t count, uint32_t value, hipStream_t stream);
+}  // namespace bfaintb
+
+namespace {
+
+using bfaintb::GemmParams;
+using bfaintb::kCounterSlots;
+
+constexpr uint32_t kDecodeMaxM = 32;
+constexpr uint32_t kDecodeColsPerWg = 256;
+constexpr uint32_t kDecodeRowsPerWgUnit = 128;  // 4 waves x 32 rows
+constexpr uint32_t kDecodeTargetWgs = 512;      // two workgroups per CU on a 256-CU part
+constexpr uint32_t kMaxSplits = 64;
+constexpr size_t kCounterBytes = (size_t)kCounterSlots * sizeof(uint32_t);
+
+int check_format(uint32_t k, int bits, uint32_t group_size)
+{
+    if (bits != 8 && bits != 4) return BFAINTB_ERR_UNSUPPORTED;
+    if (group_size != 0 && (group_size % 32u != 0 || k % group_size != 0)) return BFAINTB_ERR_UNSUPPORTED;
+    return BFAINTB_OK;
+}
+
+int check_shape(uint32_t m, uint32_t n, uint32_t k)
+{
+    if (k == 0 || n % 16u != 0 || k % 64u != 0) return BFAINTB_ERR_BAD_SHAPE;
+    if (m >= (1u << 31) || n >= (1u << 31) || k >= (1u << 31)) return BFAINTB_ERR_BAD_SHAPE;
+    if ((n + kDecodeColsPerWg - 1) / kDecodeColsPerWg > (uint32_t)kCounterSlots) return BFAINTB_ERR_BAD_SHAPE;
+    return BFAINTB_OK;
+}
+
+int resolve_variant(uint32_t m, int variant)
+{
+    if (variant == BFAINTB_VARIANT_AUTO) return m <= kDecodeMaxM ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
+    if (variant == BFAINTB_VARIANT_PREFILL) return variant;
+    return BFAINTB_ERR_BAD_VARIANT;
+}
+
+// Rows of k per workgroup and number of workgroups along k for the decode variant.
+void decode_split(uint32_t n, uint32_t k, uint32_t forced, uint32_t* k_per_wg, uint32_t* splits)
+{
+    const uint32_t col_blocks = (n + kDecodeColsPerWg - 1) / kDecodeColsPerWg;
+    const uint32_t max_splits = k / kDecodeRowsPerWgUnit ? k / kDecodeRowsPerWgUnit : 1;
+    uint32_t s = forced ? forced : (kDecodeTargetWgs + col_blocks - 1) / col_blocks;
+    if (s > max_splits) s = max_splits;
+    if (s > kMaxSplits) s = kMaxSplits;
+    if (s < 1) s = 1;
+    uint32_t per = (k + s - 1) / s;
+    per = (per + kDecodeRowsPerWgUnit - 1) / kDecodeRowsPerWgUnit * kDecodeRowsPerWgUnit;
+    *k_per_wg = per;
+    *splits = (k + per - 1) / per;
+}
+
+size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int variant, uint32_t forced_split)
+{
+    if (variant != BFAINTB_VARIANT_DECODE || m == 0 || n == 0) return 0;
+    uint32_t per, splits;
+    decode_split(n, k, forced_split, &per, &splits);
+    if (splits <= 1) return 0;
+    return kCounterBytes + (size_t)splits * m * n * sizeof(float);
+}
+
+inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+}  // namespace
+
+extern "C" {
+
+int bfaintb_version(void) { return BFAINTB_VERSION; }
+
+const char* bfaintb_error_string(int code)
+{
+    switch (code) {
+        case BFAINTB_OK: return "success";
+        case BFAINTB_ERR_NULL_POINTER: return "null device pointer";
+        case BFAINTB_ERR_BAD_SHAPE: return "unsupported shape: need n % 16 == 0, k % 64 == 0, k > 0, sizes below 2^31";
+        case BFAINTB_ERR_BAD_LD: return "bad leading dimension: need lda >= k, ldb >= n, ldc >= n, lda % 8 == 0, ldb % 16 == 0, ldc % 8 == 0";
+        case BFAINTB_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
+        case BFAINTB_ERR_UNSUPPORTED: return "unsupported format: weight_bits must be 8 or 4; group_size 0 or a multiple of 32 that divides k";
+        case BFAINTB_ERR_WORKSPACE: return "workspace missing or smaller than bfaintb_gemm_workspace_bytes reports";
+        case BFAINTB_ERR_BAD_VARIANT: return "unknown kernel variant, or variant cannot run this shape";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "unknown bfaintb error code";
+}
+
+int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
+{
+    int e = check_format(k, weight_bits, group_size);
+    if (e) return e;
+    e = check_shape(m, n, k);
+    if (e) return e;
+    return resolve_variant(m, BFAINTB_VARIANT_AUTO);
+}
+
+uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
+{
+    if (bfaintb_gemm_variant(m, n, k, weight_bits, group_size) != BFAINTB_VARIANT_DECODE) return 1;
+    uint32_t per, splits;
+    decode_split(n, k, 0, &per, &splits);
+    return splits;
+}
+
+size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant,
+                                       uint32_t split_k)
+{
+    if (check_format(k, weight_bits, group_size) || check_shape(m, n, k)) return 0;
+    const int v = resolve_variant(m, variant);
+    if (v < 0) return 0;
+    return workspace_need(m, n, k, v, split_k);
+}
+
+size_t bfaintb_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
+{
+    return bfaintb_gemm_workspace_bytes_ex(m, n, k, weight_bits, group_size, BFAINTB_VARIANT_AUTO, 0);
+}
+
+int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (workspace == nullptr || workspace_bytes == 0) return BFAINTB_OK;
+    if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
+    if (workspace_bytes < kCounterBytes) return BFAINTB_ERR_WORKSPACE;
+    // a fill kernel rather than hipMemsetAsync, so the call may be recorded into a HIP graph
+    return (int)bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)kCounterSlots, 0u,
+                                         static_cast<hipStream_t>(stream));
+}
+
+int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
+                    uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                    size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
+{
+    int e = check_format(k, weight_bits, group_size);
+    if (e) return e;
+    e = check_shape(m, n, k);
+    if (e) return e;
+    if (lda < k || ldb < n || ldc < n || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
+    const int v = resolve_variant(m, variant);
+    if (v < 0) return v;
+    if (m == 0 || n == 0) return BFAINTB_OK;
+    if (c == nullptr || a == nullptr || b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    if (misaligned16(c) || misaligned16(a) || misaligned16(b) || misaligned16(scale)) return BFAINTB_ERR_ALIGNMENT;
+
+    GemmParams p{};
+    p.c = static_cast<uint16_t*>(c);
+    p.a = static_cast<const uint16_t*>(a);
+    p.b = static_cast<const uint8_t*>(b);
+    p.scale = static_cast<const uint16_t*>(scale);
+    p.m = m; p.n = n; p.k = k;
+    p.lda = lda;
+    p.ldb_bytes = weight_bits == 8 ? ldb : ldb / 2u;
+    p.ldc = ldc;
+    p.lds = n;
+    p.group_size = group_size;
+    p.k_per_wg = k;
+    p.splits = 1;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    if (v == BFAINTB_VARIANT_PREFILL) return (int)bfaintb::launch_prefill(p, weight_bits, st);
+
+    decode_split(n, k, split_k, &p.k_per_wg, &p.splits);
+    if (p.splits > 1) {
+        const size_t need = kCounterBytes + (size_t)p.splits * m * n * sizeof(float);
+        if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
+        if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
+        p.counters = static_cast<uint32_t*>(workspace);
+        p.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kCounterBytes);
+    }
+    return (int)bfaintb::launch_decode(p, weight_bits, st);
+}
+
+int bfaintb_gemm(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
+                 uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                 size_t workspace_bytes, void* stream)
+{
+    return bfaintb_gemm_ex(c, a, b, scale, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes,
+                           stream, BFAINTB_VARIANT_AUTO, 0);
+}
+
+int bfaintb_dequant(void* w, const void* b, const void* scale, uint32_t n, uint32_t k, uint32_t ldb, uint32_t ldw,
+                    int weight_bits, uint32_t group_size, void* stream)
+{
+    int e = check_format(k, weight_bits, group_size);
+    if (e) return e;
+    if (k == 0 || n % 16u != 0 || k % 2u != 0) return BFAINTB_ERR_BAD_SHAPE;
+    if (ldb < n || ldw < n || ldb % 16u != 0 || ldw % 8u != 0) return BFAINTB_ERR_BAD_LD;
+    if (n == 0) return BFAINTB_OK;
+    if (w == nullptr || b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    if (misaligned16(w) || misaligned16(b) || misaligned16(scale)) return BFAINTB_ERR_ALIGNMENT;
+    return (int)bfaintb::launch_dequant(static_cast<uint16_t*>(w), static_cast<const uint8_t*>(b),
+                                        static_cast<const uint16_t*>(scale), n, k, weight_bits == 8 ? ldb : ldb / 2u, ldw,
+                                        weight_bits, group_size, static_cast<hipStream_t>(stream));
+}
+
+const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m)
+{
+    const int v = resolve_variant(m, variant);
+    if (v == BFAINTB_VARIANT_DECODE) return "bfaintb_decode_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL) return "bfaintb_prefill_kernel";
+    (void)weight_bits;
+    (void)group_size;
+    return "";
+}
+
+}  // extern "C"

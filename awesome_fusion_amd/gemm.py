@@ -1,0 +1,147 @@
+"""ctypes binding of the C ABI in include/bfaintb_gemm.h.
+
+Arguments mirror the reference's launch block {c, a, b, scale, m, n, k, lda, ldb, ldc}
+(/root/reference/bfAintBGemm/bfAintBGemm.cc:119-133).  Tensors are only carriers of device
+pointers (``data_ptr()``); torch supplies device memory and streams, nothing else.
+"""
+import ctypes as C
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libbfaintb_gemm.so")
+
+AUTO, DECODE, PREFILL = 0, 1, 2
+
+
+class BfaintbError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__(f"{what} failed: [{code}] {error_string(code)}")
+
+
+def library_path():
+    return _LIB
+
+
+def build_library(verbose=False):
+    """Compile every HIP source for gfx950 into libbfaintb_gemm.so (hipcc cross-compiles without a GPU)."""
+    global _lib
+    r = subprocess.run(["make", "-C", os.path.join(_HERE, "csrc"), "-B", "-j8"], capture_output=True, text=True)
+    if verbose or r.returncode != 0:
+        print(r.stdout[-4000:])
+        print(r.stderr[-4000:])
+    if r.returncode != 0:
+        raise RuntimeError("building libbfaintb_gemm.so failed")
+    _lib = None
+
+
+_lib = None
+_u32 = C.c_uint32
+_vp = C.c_void_p
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise RuntimeError(
+                f"{_LIB} is missing: build it with `make -C awesome_fusion_amd/csrc` "
+                "(or __graft_entry__.build()); this package has no CPU fallback")
+        L = C.CDLL(_LIB)
+        L.bfaintb_gemm.restype = C.c_int
+        L.bfaintb_gemm.argtypes = [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
+                                   C.c_size_t, _vp]
+        L.bfaintb_gemm_ex.restype = C.c_int
+        L.bfaintb_gemm_ex.argtypes = L.bfaintb_gemm.argtypes + [C.c_int, _u32]
+        L.bfaintb_gemm_workspace_bytes.restype = C.c_size_t
+        L.bfaintb_gemm_workspace_bytes.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
+        L.bfaintb_gemm_workspace_bytes_ex.restype = C.c_size_t
+        L.bfaintb_gemm_workspace_bytes_ex.argtypes = [_u32, _u32, _u32, C.c_int, _u32, C.c_int, _u32]
+        L.bfaintb_workspace_init.restype = C.c_int
+        L.bfaintb_workspace_init.argtypes = [_vp, C.c_size_t, _vp]
+        L.bfaintb_gemm_variant.restype = C.c_int
+        L.bfaintb_gemm_variant.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
+        L.bfaintb_gemm_split_k.restype = _u32
+        L.bfaintb_gemm_split_k.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
+        L.bfaintb_dequant.restype = C.c_int
+        L.bfaintb_dequant.argtypes = [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
+        L.bfaintb_kernel_name.restype = C.c_char_p
+        L.bfaintb_kernel_name.argtypes = [C.c_int, C.c_int, _u32, _u32]
+        L.bfaintb_error_string.restype = C.c_char_p
+        L.bfaintb_error_string.argtypes = [C.c_int]
+        L.bfaintb_version.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def error_string(code):
+    return lib().bfaintb_error_string(int(code)).decode()
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()
+
+
+def _stream_handle(stream):
+    if stream is None:
+        import torch
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream
+
+
+def variant(m, n, k, weight_bits=8, group_size=0):
+    return lib().bfaintb_gemm_variant(m, n, k, weight_bits, group_size)
+
+
+def split_k(m, n, k, weight_bits=8, group_size=0):
+    return lib().bfaintb_gemm_split_k(m, n, k, weight_bits, group_size)
+
+
+def kernel_name(m, weight_bits=8, group_size=0, which=AUTO):
+    return lib().bfaintb_kernel_name(which, weight_bits, group_size, m).decode()
+
+
+def workspace_bytes(m, n, k, weight_bits=8, group_size=0, which=AUTO, force_split_k=0):
+    return lib().bfaintb_gemm_workspace_bytes_ex(m, n, k, weight_bits, group_size, which, force_split_k)
+
+
+def workspace_init(workspace, nbytes=None, stream=None):
+    if nbytes is None:
+        nbytes = workspace.numel() * workspace.element_size()
+    rc = lib().bfaintb_workspace_init(_ptr(workspace), nbytes, _stream_handle(stream))
+    if rc:
+        raise BfaintbError(rc, "bfaintb_workspace_init")
+
+
+def gemm(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, group_size=0, workspace=None,
+         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True):
+    """C = A x dequant(B, scale) through bfaintb_gemm_ex.  Returns the library's return code
+    (raises on non-zero when ``check``)."""
+    lda = k if lda is None else lda
+    ldb = n if ldb is None else ldb
+    ldc = n if ldc is None else ldc
+    if workspace_nbytes is None:
+        workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
+    rc = lib().bfaintb_gemm_ex(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), m, n, k, lda, ldb, ldc, weight_bits, group_size,
+                               _ptr(workspace), workspace_nbytes, _stream_handle(stream), which, force_split_k)
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_gemm")
+    return rc
+
+
+def dequant(w, b, scale, n, k, ldb=None, ldw=None, weight_bits=8, group_size=0, stream=None, check=True):
+    ldb = n if ldb is None else ldb
+    ldw = n if ldw is None else ldw
+    rc = lib().bfaintb_dequant(_ptr(w), _ptr(b), _ptr(scale), n, k, ldb, ldw, weight_bits, group_size,
+                               _stream_handle(stream))
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_dequant")
+    return rc

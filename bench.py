@@ -1,0 +1,289 @@
+#!/usr/bin/env python3
+"""Benchmark of the bfAintBGemm hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+
+A step is one GEMM launch through the C ABI on synthetic, seeded inputs already resident in HBM.
+The headline workload is the decode shape the metric is quoted on (bf16 A [1,4096] x int8 B
+[4096,4096], per-channel bf16 scales); the prefill shape (M = 4096) is measured in the same run and
+reported under "extra".  The metric definitions follow the reference driver's printout
+(/root/reference/bfAintBGemm/bfAintBGemm.cc:186-195: flops = 2mnk, bytes = 2(mk+mn) + nk) with two
+corrections stated in the output: decimal units, and the scale bytes are counted.
+
+Timing: W untimed warm-up launches, then exactly K launches recorded into one HIP graph and replayed
+once between a pair of events on the launch stream (and a host clock, after/before a device
+synchronize).  The graph keeps host launch overhead out of a microsecond-scale kernel's
+measurement; the reference's own protocol is the same minus the graph (10 launches in one event pair,
+bfAintBGemm.cc:171-186).  For the decode shape consecutive launches read DIFFERENT copies of B
+(enough copies to exceed the 256 MB last-level cache), so the figure is an HBM figure; the
+same-buffer ("hot") figure is reported beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+LLC_BYTES = 256 << 20
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
+# scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(m, n, k, bits, group):
+    groups = k // group if group else 1
+    return 2 * m * k + k * n * bits // 8 + 2 * groups * n + 2 * m * n
+
+
+class Workload:
+    def __init__(self, name, m, n, k, bits=8, group=0, seed=0, copies=None):
+        import torch
+        self.name, self.m, self.n, self.k, self.bits, self.group = name, m, n, k, bits, group
+        rng = np.random.Generator(np.random.PCG64(seed))
+        self.a_f32 = rng.standard_normal((m, k), dtype=np.float32)
+        lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+        self.q = rng.integers(lo, hi, size=(k, n), dtype=np.int8)
+        groups = k // group if group else 1
+        self.s_f32 = rng.uniform(0.001, 0.01 if bits == 8 else 0.02, size=(groups, n)).astype(np.float32)
+        if bits == 8:
+            b_host = (self.q.astype(np.int16) + 128).astype(np.uint8)          # excess-128 (mem_transfer.hpp:30)
+        else:
+            u = (self.q.astype(np.int16) + 8).astype(np.uint8)
+            b_host = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)         # excess-8, even column in the low nibble
+        self.a = torch.from_numpy(self.a_f32).cuda().to(torch.bfloat16)
+        self.s = torch.from_numpy(self.s_f32).cuda().to(torch.bfloat16)
+        b0 = torch.from_numpy(b_host).cuda()
+        if copies is None:
+            copies = 1
+        self.b = [b0] + [b0.clone() for _ in range(copies - 1)]
+        self.c = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        self.bytes = algorithmic_bytes(m, n, k, bits, group)
+        self.flops = 2 * m * n * k
+
+    def workspace(self, af):
+        import torch
+        need = af.workspace_bytes(self.m, self.n, self.k, self.bits, self.group)
+        if not need:
+            return None
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        af.workspace_init(ws)
+        return ws
+
+
+def time_graph(af, w, steps, warmup, rotate):
+    """Returns (event_ms_per_step, wall_ms_per_step)."""
+    import torch
+    ws = w.workspace(af)
+    nb = len(w.b) if rotate else 1
+
+    def launch(i):
+        af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
+
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(steps):
+            launch(i)
+    g.replay()  # untimed: first replay pays graph upload
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return e0.elapsed_time(e1) / steps, (t1 - t0) * 1e3 / steps
+
+
+def time_eager(af, w, steps, warmup):
+    """The reference protocol: launches in a loop inside one event pair, no graph."""
+    import torch
+    ws = w.workspace(af)
+    for i in range(warmup):
+        af.gemm(w.c, w.a, w.b[0], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(steps):
+        af.gemm(w.c, w.a, w.b[0], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def roofline_entry(w, ms, bound):
+    if bound == "hbm":
+        achieved = w.bytes / (ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = w.flops / (ms * 1e-3) / 1e12
+        peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name), "kernel_us": round(ms * 1e3, 3),
+            "algorithmic_bytes": w.bytes, "flops": w.flops}
+
+
+def cpu_baseline(w, c_gpu_f32, budget_s=12.0):
+    """host_ref.hpp's gemm_rrr timed on this machine's cores on the same inputs the GPU consumed:
+    the reference's own compiled routine when the wrapper library is present, else the C port."""
+    import ctypes as C
+    from concurrent.futures import ThreadPoolExecutor
+    import oracle
+    import torch
+    fp = C.POINTER(C.c_float)
+    a = w.a.float().cpu().numpy()                       # the bf16 activations, widened
+    s = w.s.float().cpu().numpy()[0].copy()             # the bf16 scales, widened (per-channel workloads)
+    b = w.q.astype(np.float32)
+    m, n, k = w.m, w.n, w.k
+    if oracle.have_ref():
+        fn, kind = oracle.ref().ref_gemm_rrr, "reference"
+    else:
+        fn, kind = oracle.lib.orc_gemm_rrr, "port"
+    c = np.zeros((m, n), np.float32)
+
+    def call(n0, nb):
+        fn(C.cast(c.ctypes.data + 4 * n0, fp), a.ctypes.data_as(fp), C.cast(b.ctypes.data + 4 * n0, fp),
+           C.cast(s.ctypes.data + 4 * n0, fp), m, nb, k, k, n, n)
+
+    # 1 thread, the way the reference runs it
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        call(0, n)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s * 0.6 or reps >= 50:
+            break
+    t1 = el / reps
+    c_single = c.copy()
+    # all cores: columns split over threads, each output still one sequential-K fp32 sum
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    blk = max(16, (n // (cores * 4)) // 16 * 16)
+    jobs = [(n0, min(blk, n - n0)) for n0 in range(0, n, blk)]
+    with ThreadPoolExecutor(max_workers=cores) as ex:
+        reps2, t0 = 0, time.perf_counter()
+        while True:
+            list(ex.map(lambda j: call(*j), jobs))
+            reps2 += 1
+            el = time.perf_counter() - t0
+            if el > budget_s * 0.4 or reps2 >= 200:
+                break
+    tn = el / reps2
+    assert np.array_equal(c.view(np.uint32), c_single.view(np.uint32)), "threaded CPU baseline changed the result"
+    d = c_gpu_f32 - c
+    nrms = float(np.sqrt((d.astype(np.float64) ** 2).sum() / (2.0 * (c.astype(np.float64) ** 2).sum())))
+    unit_val = lambda t: w.bytes / t / 1e9
+    return ({"value": round(unit_val(t1), 4), "unit": "GB/s", "cores": 1, "kind": kind,
+             "sample": f"full {w.name} problem x{reps} repetitions ({el and t1 * reps:.1f} s), gemm_rrr on float inputs",
+             "gflops": round(w.flops / t1 / 1e9, 3), "ms_per_step": round(t1 * 1e3, 3)},
+            {"value": round(unit_val(tn), 4), "unit": "GB/s", "cores": cores, "kind": kind,
+             "sample": f"full {w.name} problem x{reps2} repetitions, columns split over {cores} threads",
+             "gflops": round(w.flops / tn / 1e9, 3), "ms_per_step": round(tn * 1e3, 3)},
+            nrms)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (decode sweep, int4 group-128)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="time only this workload family: decode | prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM shards over n with no "
+              "exchange; see DESIGN.md).  Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    import awesome_fusion_amd as af
+    af.lib()
+
+    K, W = args.steps, args.warmup
+    out_extra = {}
+
+    # ---- headline: decode M=1, N=K=4096, int8 per-channel; cold B (rotating copies > last-level cache)
+    res = None
+    if args.only in ("", "decode"):
+        copies = LLC_BYTES * 2 // (4096 * 4096) + 8  # 40 copies = 640 MiB
+        w = Workload("decode_m1_n4096_k4096_int8_perchannel", 1, 4096, 4096, copies=copies)
+        ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True)
+        hot_ms, _ = time_graph(af, w, K, W, rotate=False)
+        eager_ms = time_eager(af, w, K, W)
+        c_gpu = w.c.float().cpu().numpy()
+        res = {
+            "metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=1: effective HBM bandwidth (algorithmic bytes / time per launch, B cold)",
+            "value": round(w.bytes / (wall_ms * 1e-3) / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+            "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": w.name, "m": 1, "n": 4096, "k": 4096, "weight_bits": 8, "group_size": 0,
+                       "b_copies_rotated": copies, "split_k": af.split_k(1, 4096, 4096), "launch": "hip graph of K launches",
+                       "units": "decimal; scale bytes counted"},
+            "roofline": roofline_entry(w, ev_ms, "hbm"),
+        }
+        res["tflops"] = round(w.flops / (wall_ms * 1e-3) / 1e12, 4)
+        out_extra["decode_m1_hot_same_buffer"] = {"kernel_us": round(hot_ms * 1e3, 3), "GB/s": round(w.bytes / hot_ms / 1e6, 1),
+                                                  "note": "B re-read from cache: not an HBM figure"}
+        out_extra["decode_m1_eager_launch_loop"] = {"us_per_launch": round(eager_ms * 1e3, 3),
+                                                    "note": "reference protocol (no graph): host launch rate included"}
+        if not args.no_cpu:
+            one, allc, nrms = cpu_baseline(w, c_gpu)
+            res["cpu_baseline"] = one
+            out_extra["cpu_baseline_all_cores"] = allc
+            out_extra["gpu_vs_cpu_nrms"] = round(nrms, 6)
+        del w
+        torch.cuda.empty_cache()
+
+    # ---- prefill M=4096, N=K=4096
+    if args.only in ("", "prefill"):
+        w = Workload("prefill_m4096_n4096_k4096_int8_perchannel", 4096, 4096, 4096, copies=2)
+        pk = max(20, min(K, 100))
+        ev_ms, wall_ms = time_graph(af, w, pk, max(5, W // 4), rotate=True)
+        entry = {"value": round(w.flops / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "steps": pk,
+                 "ms_per_step": round(wall_ms, 6), "GB/s": round(w.bytes / (wall_ms * 1e-3) / 1e9, 1),
+                 "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma")}
+        out_extra["prefill_m4096"] = entry
+        if res is None:
+            res = {"metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=4096: TFLOP/s", "value": entry["value"], "unit": "TFLOP/s",
+                   "n_gpus": 1, "steps": pk, "warmup": W, "ms_per_step": entry["ms_per_step"], "higher_is_better": True,
+                   "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                   "config": entry["config"], "roofline": entry["roofline"]}
+        del w
+        torch.cuda.empty_cache()
+
+    if args.sweep:
+        sweep = []
+        for m in (1, 4, 8, 16, 32):
+            w = Workload(f"decode_m{m}_n11008_k4096_int8_perchannel", m, 11008, 4096, copies=14)
+            ev_ms, _ = time_graph(af, w, min(K, 200), W, rotate=True)
+            sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "hbm")})
+            del w
+            torch.cuda.empty_cache()
+        for m in (1, 16, 2048):
+            w = Workload(f"m{m}_n28672_k8192_int4_group128", m, 28672, 8192, bits=4, group=128, copies=6 if m <= 32 else 1)
+            ev_ms, _ = time_graph(af, w, min(K, 100) if m <= 32 else 10, min(W, 10), rotate=True)
+            sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "hbm" if m <= 32 else "mfma")})
+            del w
+            torch.cuda.empty_cache()
+        out_extra["sweep"] = sweep
+
+    res["extra"] = out_extra
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

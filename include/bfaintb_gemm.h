@@ -1,0 +1,129 @@
+/*
+ * bfaintb_gemm.h — C ABI of the MI355X (gfx950) bf16-activation x integer-weight GEMM.
+ *
+ *     C[m,n] = sum_k A[m,k] * W[k,n],      W[k,n] = bf16( float(q[k,n]) * float(scale[g(k),n]) )
+ *
+ * A, C: bf16, row-major.  B: packed integer codes q, row-major K x N.  fp32 accumulation, one
+ * rounding (to nearest even) when W is formed and one when C is stored.
+ *
+ * The entry points replace the raw module launch of the reference driver
+ * (/root/reference/bfAintBGemm/bfAintBGemm.cc:65-66 hipModuleLoad/hipModuleGetFunction and
+ * :119-152 packed kernarg + hipModuleLaunchKernel).  The argument order of bfaintb_gemm is that
+ * kernarg block — {c, a, b, scale, m, n, k, lda, ldb, ldc} (bfAintBGemm.cc:119-133, kernel side
+ * bf16gemm_kernel_gfx90a.s:97-108) — followed by what the reference did not have.
+ *
+ * All pointers are DEVICE pointers owned by the caller.  Calls are asynchronous and ordered on
+ * `stream` (a hipStream_t passed as void*; NULL is the default stream, which is what the reference
+ * launches on).  No call allocates, frees or synchronises.  Return value: 0 on success, a negative
+ * BFAINTB_ERR_* for a rejected argument (nothing was launched), or a positive hipError_t.
+ */
+#ifndef BFAINTB_GEMM_H
+#define BFAINTB_GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define BFAINTB_API __attribute__((visibility("default")))
+#else
+#define BFAINTB_API
+#endif
+
+#define BFAINTB_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum {
+    BFAINTB_OK = 0,
+    BFAINTB_ERR_NULL_POINTER = -1,  /* c, a, b or scale is NULL (with m,n,k all non-zero) */
+    BFAINTB_ERR_BAD_SHAPE = -2,     /* n not a multiple of 16, k not a multiple of 64, or sizes overflow 2^31 */
+    BFAINTB_ERR_BAD_LD = -3,        /* lda < k, ldb < n, ldc < n, or a leading dimension that breaks 16-byte rows */
+    BFAINTB_ERR_ALIGNMENT = -4,     /* a pointer is not 16-byte aligned */
+    BFAINTB_ERR_UNSUPPORTED = -5,   /* weight_bits not 8 or 4; group_size not 0 or a multiple of 32 dividing k */
+    BFAINTB_ERR_WORKSPACE = -6,     /* workspace NULL/too small for this shape (see bfaintb_gemm_workspace_bytes) */
+    BFAINTB_ERR_BAD_VARIANT = -7    /* unknown variant, or a variant that cannot run this shape */
+};
+
+/* Which kernel family runs a shape. */
+enum {
+    BFAINTB_VARIANT_AUTO = 0,
+    BFAINTB_VARIANT_DECODE = 1, /* split-K weight-streaming kernel, m <= 32 (HBM-bound) */
+    BFAINTB_VARIANT_PREFILL = 2 /* 256x256 LDS-tiled MFMA kernel (MFMA-bound) */
+};
+
+/*
+ * Data formats.
+ *   a      bf16 [m, lda], lda in elements (bfAintBGemm.cc:47,119-133; the kernel doubles it, asm:216).
+ *   b      weight_bits == 8: one byte per weight, [k, ldb] bytes, excess-128 code u = q + 128 — the
+ *          byte format the reference's host writes (mem_transfer.hpp:30) and its kernel decodes
+ *          (bf16gemm_kernel_gfx90a.s:19-27).
+ *          weight_bits == 4: two weights per byte along n, row stride ldb/2 bytes; byte j of a row
+ *          holds column 2j in its low nibble and column 2j+1 in its high nibble, each excess-8
+ *          (q + 8).  ldb is in ELEMENTS in both cases, like the reference's ldb.
+ *   scale  bf16 [groups, n] with row stride n, groups = group_size ? k / group_size : 1.
+ *          (The reference stores fp32 scales, bfAintBGemm.cc:27; this build's contract is bf16,
+ *          which makes q*scale exact in fp32 and the dequantised weight a single rounding.)
+ *   c      bf16 [m, ldc].
+ * Requirements: n % 16 == 0, k % 64 == 0, lda % 8 == 0, ldb % 16 == 0, ldc % 8 == 0, all four
+ * pointers 16-byte aligned, |scale| finite and below 2^120.
+ */
+
+/*
+ * The GEMM.  Replaces hipModuleLaunchKernel(kernel_func, ...) at bfAintBGemm.cc:152 and :176.
+ *   weight_bits   8 or 4
+ *   group_size    0: one scale per output channel (the reference's only mode);
+ *                 otherwise rows per scale group along k (multiple of 32, divides k)
+ *   workspace     device scratch of at least bfaintb_gemm_workspace_bytes(...) bytes that has been
+ *                 passed through bfaintb_workspace_init once (or is all zero bytes).  The call
+ *                 leaves it ready for the next call.  Two calls that may run concurrently must not
+ *                 share a workspace.  May be NULL when the required size is 0.
+ */
+BFAINTB_API int bfaintb_gemm(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
+                 uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
+/* Same, with the kernel family and the split-K factor forced (0 = choose).  For benchmarks and
+ * tests; split_k is ignored by the prefill variant. */
+BFAINTB_API int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
+                    uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                    size_t workspace_bytes, void* stream, int variant, uint32_t split_k);
+
+/* Scratch the GEMM needs for a shape: split-K partial sums and arrival counters.  Depends only on
+ * its arguments.  The reference kernel has no scratch (no split-K, bfAintBGemm.cc:107-109). */
+BFAINTB_API size_t bfaintb_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
+BFAINTB_API size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
+                                       int variant, uint32_t split_k);
+
+/* Clears the arrival counters at the head of a freshly allocated workspace (stream-ordered). */
+BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */
+BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
+
+/* The split-K factor the decode variant would use for a shape (1 for the prefill variant). */
+BFAINTB_API uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
+
+/*
+ * Writes the dequantised weights W[k,n] as bf16 to w (row stride ldw elements), using the same
+ * device dequantisation routine as the GEMM kernels.  Successor of the reference's ASM_PRINT debug
+ * channel (bfAintBGemm.cc:113-118,156-169; bf16gemm_kernel_gfx90a.s:2-16), which was its only way
+ * to look at in-kernel values.
+ */
+BFAINTB_API int bfaintb_dequant(void* w, const void* b, const void* scale, uint32_t n, uint32_t k, uint32_t ldb, uint32_t ldw,
+                    int weight_bits, uint32_t group_size, void* stream);
+
+/* Name of the __global__ function a variant launches for (weight_bits, group_size, m), as it
+ * appears in a kernel trace. */
+BFAINTB_API const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m);
+
+/* Text for a return code of this library (negative codes; positive ones are hipError_t values). */
+BFAINTB_API const char* bfaintb_error_string(int code);
+
+BFAINTB_API int bfaintb_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BFAINTB_GEMM_H */

@@ -1,0 +1,108 @@
+"""Shared test plumbing: seeded inputs in the wire formats, device round trips, comparisons.
+
+Inputs are made with numpy's PCG64 and converted with the oracle's restatements of the reference's
+host converters; the GPU side is reached only through the C ABI (awesome_fusion_amd.gemm is a
+ctypes shim over it).
+"""
+import numpy as np
+
+import oracle
+
+
+def widen(bits):
+    return (np.asarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class Problem:
+    """One GEMM instance in device wire formats plus what the oracle needs."""
+
+    def __init__(self, m, n, k, bits=8, group_size=0, seed=0, scale_lo=0.001, scale_hi=0.01, regime="normal"):
+        rng = np.random.Generator(np.random.PCG64(seed))
+        self.m, self.n, self.k, self.bits, self.group_size = m, n, k, bits, group_size
+        groups = k // group_size if group_size else 1
+        lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+        if regime == "normal":
+            a = rng.standard_normal((m, k), dtype=np.float32)
+            q = rng.integers(lo, hi, size=(k, n), dtype=np.int64).astype(np.int8)
+            s = rng.uniform(scale_lo, scale_hi, size=(groups, n)).astype(np.float32)
+        elif regime == "small_int":  # the reference's own test data: everything in {-2,-1,0,1}
+            a = rng.integers(-2, 2, size=(m, k)).astype(np.float32)
+            q = rng.integers(-2, 2, size=(k, n)).astype(np.int8)
+            s = rng.integers(-2, 2, size=(groups, n)).astype(np.float32)
+        else:
+            raise ValueError(regime)
+        self.a_bf = oracle.f32_to_bf16_rne(a)
+        self.q = q
+        self.s_bf = oracle.f32_to_bf16_rne(s)
+        if bits == 8:
+            self.b_bytes = oracle.mem_transfer_int8(q.astype(np.float32))
+        else:
+            self.b_bytes = oracle.pack_int4(q)
+        self._w = None
+
+    @property
+    def w_bf(self):
+        if self._w is None:
+            self._w = oracle.dequant(self.b_bytes, self.s_bf, self.k, self.n, self.bits, self.group_size)
+        return self._w
+
+    def c_ref(self, rows=None, threads=8):
+        a = self.a_bf if rows is None else self.a_bf[rows]
+        return oracle.gemm_bf16_rows(a, self.w_bf, threads=threads)
+
+
+def to_dev(x):
+    import torch
+    x = np.ascontiguousarray(x)
+    if x.dtype == np.uint16:
+        return torch.from_numpy(x.view(np.int16)).cuda()
+    return torch.from_numpy(x).cuda()
+
+
+def from_dev_u16(t):
+    return t.cpu().numpy().view(np.uint16)
+
+
+class Workspace:
+    """A zero-initialised device scratch, grown on demand."""
+
+    def __init__(self):
+        self.t = None
+
+    def get(self, nbytes):
+        import torch
+        import awesome_fusion_amd as af
+        if nbytes == 0:
+            return None
+        if self.t is None or self.t.numel() < nbytes:
+            self.t = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device="cuda")
+            af.workspace_init(self.t)
+        return self.t
+
+
+_ws = Workspace()
+
+
+def run_gemm(p, which=0, force_split_k=0, lda=None, ldb=None, ldc=None, a_dev=None, b_dev=None, s_dev=None, c_fill=None):
+    """Runs the library on Problem p; returns C as uint16 bits [m, ldc or n]."""
+    import torch
+    import awesome_fusion_amd as af
+    m, n, k = p.m, p.n, p.k
+    a_dev = to_dev(p.a_bf) if a_dev is None else a_dev
+    b_dev = to_dev(p.b_bytes) if b_dev is None else b_dev
+    s_dev = to_dev(p.s_bf) if s_dev is None else s_dev
+    ldc_ = n if ldc is None else ldc
+    c_dev = torch.full((m, ldc_), 0x7FC0 if c_fill is None else c_fill, dtype=torch.int16, device="cuda")
+    ws = _ws.get(af.workspace_bytes(m, n, k, p.bits, p.group_size, which, force_split_k))
+    af.gemm(c_dev, a_dev, b_dev, s_dev, m, n, k, lda, ldb, ldc, p.bits, p.group_size, ws, None, None, which, force_split_k)
+    torch.cuda.synchronize()
+    return from_dev_u16(c_dev)
+
+
+def assert_close_ulp(c_ref, c_bits, what, max_ulp=2.0, allow=0):
+    """The acceptance bound: <= 2 bf16 ULP of the fp32-accumulated oracle, or relative error
+    <= 1e-2 where |ref| < 1e-3."""
+    bad, worst, idx = oracle.check_ulp(c_ref, c_bits, max_ulp, 1e-3, 1e-2)
+    assert bad <= allow, f"{what}: {bad} of {c_ref.size} outside tolerance; worst {worst:.3f} ULP at flat index {idx} " \
+                         f"(ref {c_ref.ravel()[idx]!r}, got {widen(c_bits.ravel()[idx:idx+1])[0]!r})"
+    return worst

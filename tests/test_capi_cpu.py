@@ -1,0 +1,91 @@
+"""The C-ABI library on a machine without a GPU: it loads, exports what the header declares, and
+rejects bad arguments before touching the device (so none of this launches anything)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import awesome_fusion_amd as af
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+P = 0x10000  # a fake, non-null, 16-byte aligned "device pointer": validation never dereferences
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "bfaintb_gemm.h")).read()
+    return re.findall(r"BFAINTB_API\s+[\w\s\*]+?\b(bfaintb_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) >= 11 and "bfaintb_gemm" in names and "bfaintb_dequant" in names
+    lib = C.CDLL(af.library_path())
+    for name in names:
+        assert hasattr(lib, name), name
+    assert af.lib().bfaintb_version() == 100
+
+
+def test_variant_choice_and_split():
+    assert af.variant(1, 4096, 4096) == af.DECODE
+    assert af.variant(32, 4096, 4096) == af.DECODE
+    assert af.variant(33, 4096, 4096) == af.PREFILL
+    assert af.variant(4096, 4096, 4096) == af.PREFILL
+    assert af.variant(1, 28672, 8192, 4, 128) == af.DECODE
+    assert af.split_k(4096, 4096, 4096) == 1
+    s = af.split_k(1, 4096, 4096)
+    assert 1 < s <= 64 and 4096 % s == 0
+    # workspace = counters + splits * m * n fp32; none for the prefill variant
+    assert af.workspace_bytes(1, 4096, 4096) == 4096 * 4 + s * 1 * 4096 * 4
+    assert af.workspace_bytes(4096, 4096, 4096) == 0
+    assert af.workspace_bytes(8, 4096, 4096, force_split_k=1) == 0
+    assert af.kernel_name(1) == "bfaintb_decode_kernel" and af.kernel_name(4096) == "bfaintb_prefill_kernel"
+
+
+def rc(**kw):
+    d = dict(c=P, a=P, b=P, scale=P, m=64, n=128, k=256, weight_bits=8, group_size=0, workspace=None, stream=0, check=False)
+    d.update(kw)
+    return af.gemm(d.pop("c"), d.pop("a"), d.pop("b"), d.pop("scale"), d.pop("m"), d.pop("n"), d.pop("k"), **d)
+
+
+def test_rejects_bad_arguments_without_launching():
+    L = af.lib()
+    assert rc(weight_bits=5) == -5
+    assert rc(group_size=48) == -5            # not a multiple of 32
+    assert rc(group_size=96) == -5            # does not divide k = 256
+    assert rc(n=100) == -2                    # n % 16
+    assert rc(k=100) == -2                    # k % 64 (the reference kernel has the same limit, asm main loop)
+    assert rc(k=0) == -2
+    assert rc(lda=128) == -3                  # lda < k
+    assert rc(ldb=64) == -3
+    assert rc(ldc=64) == -3
+    assert rc(lda=260) == -3                  # rows of A would lose 16-byte alignment
+    assert rc(a=None) == -1
+    assert rc(c=0) == -1
+    assert rc(b=P + 4) == -4
+    assert rc(which=9) == -7
+    assert rc(which=af.DECODE) == -7          # m = 64 cannot run the decode variant
+    assert rc(m=8, which=af.DECODE, force_split_k=2) == -6   # split-K needs a workspace
+    assert rc(m=8, which=af.DECODE, force_split_k=2, workspace=P, workspace_nbytes=64) == -6
+    assert rc(m=0) == 0                       # nothing to do
+    for code in (-1, -2, -3, -4, -5, -6, -7):
+        assert len(af.error_string(code)) > 10
+    with pytest.raises(af.BfaintbError) as e:
+        rc(n=100, check=True)
+    assert e.value.code == -2
+    # dequant entry point
+    assert af.dequant(P, P, P, 128, 256, stream=0, weight_bits=3, check=False) == -5
+    assert af.dequant(P, P, P, 100, 256, stream=0, check=False) == -2
+    assert af.dequant(P, P, None, 128, 256, stream=0, check=False) == -1
+    assert L.bfaintb_workspace_init(P, 64, None) == -6
+    assert L.bfaintb_workspace_init(None, 0, None) == 0
+
+
+def test_product_does_not_reach_for_the_oracle():
+    # the shipped package and the C/HIP sources must not import, include or link anything under oracle/
+    pkg = os.path.join(ROOT, "awesome_fusion_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cc", ".cpp", "Makefile")):
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)

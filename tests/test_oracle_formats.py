@@ -1,0 +1,143 @@
+"""Pins the oracle's number-format and wire-format functions (CPU only).
+
+Each check is chosen so that a plausible slip — wrong shift, missing tie rule, sign of the +128 —
+fails it: reference-produced fixtures, the reference's own compiled routines where built,
+exhaustive identities, and torch.bfloat16 as an independent RNE implementation.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import widen
+
+L = oracle.lib
+
+
+def test_bf16_round_trip_exhaustive(golden_dir):
+    g = np.load(f"{golden_dir}/converters.npz")
+    all16 = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    f = oracle.bf16_to_f32(all16)
+    # widening is a 16-bit shift: compare bit patterns with what the reference's converter produced
+    assert np.array_equal(f.view(np.uint32), g["bf16_to_f32_bits"])
+    assert np.array_equal(f.view(np.uint32), all16.astype(np.uint32) << 16)
+    # truncation inverts widening for every bf16 value, NaNs included (bit-level)
+    assert np.array_equal(oracle.f32_to_bf16_rtz(f), all16)
+    # RNE leaves exactly representable values alone (NaN payloads aside)
+    notnan = ~np.isnan(f)
+    assert np.array_equal(oracle.f32_to_bf16_rne(f)[notnan], all16[notnan])
+
+
+def test_known_answers():
+    ka_rtz = {0x3F800000: 0x3F80, 0x3F7FFFFF: 0x3F7F, 0xBF7FFFFF: 0xBF7F}
+    ka_rne = {0x3F808000: 0x3F80,  # tie, kept mantissa even -> stays
+              0x3F818000: 0x3F82,  # tie, kept mantissa odd -> up
+              0x3F808001: 0x3F81,  # just above the tie
+              0x3F807FFF: 0x3F80,  # just below
+              0x3F7FFFFF: 0x3F80,  # carry into the exponent
+              0x7F7FFFFF: 0x7F80,  # rounds up to Inf
+              0x7F800000: 0x7F80, 0xFF800000: 0xFF80,
+              0x7F800001: 0x7F81,  # signalling NaN keeps a payload bit
+              0x00008000: 0x0000, 0x00018000: 0x0002}
+    for bits, want in ka_rtz.items():
+        assert L.orc_f32_to_bf16_rtz(C.c_float(np.uint32(bits).view(np.float32))) == want
+    for bits, want in ka_rne.items():
+        assert oracle.f32_to_bf16_rne(np.array([bits], np.uint32).view(np.float32))[0] == want, hex(bits)
+
+
+def test_converters_match_reference_fixture(golden_dir):
+    g = np.load(f"{golden_dir}/converters.npz")
+    f = g["f32_bits"].view(np.float32)
+    assert np.array_equal(oracle.f32_to_bf16_rne(f), g["rne"])
+    assert np.array_equal(oracle.f32_to_bf16_rtz(f), g["rtz"])
+    assert np.array_equal(oracle.mem_transfer_int8(g["int8_values"]), g["int8_bytes"])
+
+
+def test_rne_matches_torch_bfloat16():
+    import torch
+    rng = np.random.Generator(np.random.PCG64(7))
+    bits = rng.integers(0, 2**32, size=1 << 20, dtype=np.uint64).astype(np.uint32)
+    f = bits.view(np.float32)
+    keep = ~np.isnan(f)
+    f = f[keep]
+    t = torch.from_numpy(f.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(oracle.f32_to_bf16_rne(f), t)
+
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="reference wrapper not built (needs /root/reference)")
+def test_converters_match_compiled_reference():
+    r = oracle.ref()
+    rng = np.random.Generator(np.random.PCG64(11))
+    bits = rng.integers(0, 2**32, size=20000, dtype=np.uint64).astype(np.uint32)
+    f = bits.view(np.float32)
+    u16p, fp = C.POINTER(C.c_uint16), C.POINTER(C.c_float)
+    for mine, theirs in ((oracle.f32_to_bf16_rne, r.ref_f32_to_bf16_rne_n), (oracle.f32_to_bf16_rtz, r.ref_f32_to_bf16_rtz_n)):
+        out = np.zeros(f.size, np.uint16)
+        theirs(out.ctypes.data_as(u16p), f.ctypes.data_as(fp), f.size)
+        assert np.array_equal(mine(f), out)
+    x = rng.standard_normal(4096).astype(np.float32) * 100
+    out = np.zeros(4096, np.uint16)
+    r.ref_mem_transfer_bf16(out.ctypes.data_as(C.POINTER(C.c_uint16)), x.ctypes.data_as(C.POINTER(C.c_float)), x.size)
+    assert np.array_equal(out, oracle.f32_to_bf16_rtz(x))
+    assert r.ref_row_major_name() == b"RowMajor" and r.ref_column_major_name() == b"ColumnMajor"
+
+
+def test_excess128_closed_form():
+    q = np.arange(-128, 128)
+    got = oracle.mem_transfer_int8(q.astype(np.float32))
+    assert np.array_equal(got, ((q + 128) & 0xFF).astype(np.uint8))
+    assert got[0] == 0x00 and got[128] == 0x80 and got[255] == 0xFF
+    # fractional inputs truncate toward zero before the offset (static_cast<int8_t>)
+    assert oracle.mem_transfer_int8(np.array([1.9, -1.9, 0.5], np.float32)).tolist() == [129, 127, 128]
+
+
+def test_magic_number_decode_is_exact():
+    for u in range(256):
+        assert L.orc_magic_dequant_int8(u) == float(u - 128)
+
+
+def test_int4_packing_brute_force():
+    rng = np.random.Generator(np.random.PCG64(3))
+    q = rng.integers(-8, 8, size=(6, 32)).astype(np.int8)
+    packed = oracle.pack_int4(q)
+    assert packed.shape == (6, 16)
+    for i in range(6):
+        for j in range(32):
+            byte = int(packed[i, j // 2])
+            code = (byte >> 4) if j % 2 else (byte & 0xF)
+            assert code - 8 == q[i, j]
+    # the extremes land where the format says
+    assert oracle.pack_int4(np.array([[-8, 7]], np.int8))[0, 0] == 0xF0
+
+
+@pytest.mark.parametrize("bits,group", [(8, 0), (8, 32), (4, 0), (4, 128)])
+def test_dequant_against_numpy(bits, group):
+    rng = np.random.Generator(np.random.PCG64(5))
+    k, n = 256, 64
+    lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+    q = rng.integers(lo, hi, size=(k, n)).astype(np.int8)
+    groups = k // group if group else 1
+    s_bf = oracle.f32_to_bf16_rne(rng.uniform(0.001, 0.02, size=(groups, n)).astype(np.float32))
+    b = oracle.mem_transfer_int8(q.astype(np.float32)) if bits == 8 else oracle.pack_int4(q)
+    w = oracle.dequant(b, s_bf, k, n, bits, group)
+    # independent statement: float64 product (exact), rounded once to bf16 by torch
+    import torch
+    srow = widen(s_bf).astype(np.float64)
+    gidx = (np.arange(k) // group) if group else np.zeros(k, int)
+    prod = q.astype(np.float64) * srow[gidx]
+    assert np.array_equal(prod.astype(np.float32).astype(np.float64), prod), "int x bf16 must be exact in fp32"
+    want = torch.from_numpy(prod.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(w, want)
+    # truncating variant differs from RNE somewhere and never exceeds it in magnitude
+    w_rtz = oracle.dequant(b, s_bf, k, n, bits, group, rtz=True)
+    assert np.array_equal(w_rtz, (prod.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    assert (w_rtz != w).any()
+
+
+def test_int_times_bf16_scale_is_exact_exhaustive():
+    # every 8-bit integer times every positive normal bf16 significand pattern: the fp32 product equals the exact one
+    q = np.arange(-128, 128, dtype=np.float64)[:, None]
+    sig = widen(np.arange(0x3F80, 0x4000, dtype=np.uint32).astype(np.uint16)).astype(np.float64)[None, :]
+    exact = q * sig
+    assert np.array_equal(exact.astype(np.float32).astype(np.float64), exact)
