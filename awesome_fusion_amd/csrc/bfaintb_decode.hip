@@ -32,17 +32,16 @@ struct RawStep {
     uint32_t d[8][kDwords];  // 8 rows x 16 codes
 };
 
-// Code of column C (0..15) in one row's dwords, as fp32.
+// Signed value of column C (0..15) of one prepared row, as fp32 (x16 for 4-bit codes).
 template <int BITS, int C>
-__device__ __forceinline__ float code_f32(const uint32_t (&row)[RawStep<BITS>::kDwords])
+__device__ __forceinline__ float value_f32(const uint32_t (&row)[4])
 {
     if constexpr (BITS == 8) {
-        return ubyte_to_f32<C % 4>(row[C / 4]);
+        return sbyte_to_f32<C % 4>(row[C / 4]);
     } else {
-        // byte (C%8)/2 of dword C/8; even columns in the low nibble
-        const uint32_t x = row[C / 8];
-        const uint32_t nib = (C % 2) ? ((x >> 4) & 0x0f0f0f0fu) : (x & 0x0f0f0f0fu);
-        return ubyte_to_f32<(C % 8) / 2>(nib);
+        // prepared 4-bit row: dwords {even columns of raw dword 0, odd of 0, even of 1, odd of 1};
+        // column C sits in raw dword C/8, byte (C%8)/2
+        return sbyte_to_f32<(C % 8) / 2>(row[2 * (C / 8) + (C % 2)]);
     }
 }
 
@@ -63,15 +62,30 @@ __device__ __forceinline__ void load_raw(RawStep<BITS>& raw, const uint8_t* rowp
     }
 }
 
+// Stored codes of one row -> four dwords of two's-complement bytes.
+template <int BITS>
+__device__ __forceinline__ void prepare_row(uint32_t (&out)[4], const uint32_t (&in)[RawStep<BITS>::kDwords])
+{
+    if constexpr (BITS == 8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = codes8_to_s8(in[i]);
+    } else {
+        out[0] = codes4_even_to_s8x16(in[0]);
+        out[1] = codes4_odd_to_s8x16(in[0]);
+        out[2] = codes4_even_to_s8x16(in[1]);
+        out[3] = codes4_odd_to_s8x16(in[1]);
+    }
+}
+
 template <int BITS, int MB, int C>
-__device__ __forceinline__ void mac_column(const RawStep<BITS>& raw, const ColScale (&cs)[16], const uint4 (&afrag)[MB],
+__device__ __forceinline__ void mac_column(const uint32_t (&rows)[8][4], const float (&cs)[16], const uint4 (&afrag)[MB],
                                            f32x4_t (&acc)[MB][16])
 {
     uint4 w;
-    w.x = pack_bf16_rne(dequant_code(code_f32<BITS, C>(raw.d[0]), cs[C]), dequant_code(code_f32<BITS, C>(raw.d[1]), cs[C]));
-    w.y = pack_bf16_rne(dequant_code(code_f32<BITS, C>(raw.d[2]), cs[C]), dequant_code(code_f32<BITS, C>(raw.d[3]), cs[C]));
-    w.z = pack_bf16_rne(dequant_code(code_f32<BITS, C>(raw.d[4]), cs[C]), dequant_code(code_f32<BITS, C>(raw.d[5]), cs[C]));
-    w.w = pack_bf16_rne(dequant_code(code_f32<BITS, C>(raw.d[6]), cs[C]), dequant_code(code_f32<BITS, C>(raw.d[7]), cs[C]));
+    w.x = pack_bf16_rne(value_f32<BITS, C>(rows[0]) * cs[C], value_f32<BITS, C>(rows[1]) * cs[C]);
+    w.y = pack_bf16_rne(value_f32<BITS, C>(rows[2]) * cs[C], value_f32<BITS, C>(rows[3]) * cs[C]);
+    w.z = pack_bf16_rne(value_f32<BITS, C>(rows[4]) * cs[C], value_f32<BITS, C>(rows[5]) * cs[C]);
+    w.w = pack_bf16_rne(value_f32<BITS, C>(rows[6]) * cs[C], value_f32<BITS, C>(rows[7]) * cs[C]);
     const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, w);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -80,10 +94,13 @@ __device__ __forceinline__ void mac_column(const RawStep<BITS>& raw, const ColSc
 }
 
 template <int BITS, int MB, int... Cs>
-__device__ __forceinline__ void mac_step(const RawStep<BITS>& raw, const ColScale (&cs)[16], const uint4 (&afrag)[MB],
+__device__ __forceinline__ void mac_step(const RawStep<BITS>& raw, const float (&cs)[16], const uint4 (&afrag)[MB],
                                          f32x4_t (&acc)[MB][16], std::integer_sequence<int, Cs...>)
 {
-    (mac_column<BITS, MB, Cs>(raw, cs, afrag, acc), ...);
+    uint32_t rows[8][4];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) prepare_row<BITS>(rows[r], raw.d[r]);
+    (mac_column<BITS, MB, Cs>(rows, cs, afrag, acc), ...);
 }
 
 template <int BITS>
@@ -98,7 +115,7 @@ __device__ __forceinline__ void load_scales(uint4 (&sraw)[2], const uint16_t* sp
 }
 
 template <int BITS>
-__device__ __forceinline__ void apply_scales(ColScale (&cs)[16], const uint4 (&sraw)[2])
+__device__ __forceinline__ void apply_scales(float (&cs)[16], const uint4 (&sraw)[2])
 {
     const uint32_t d[8] = {sraw[0].x, sraw[0].y, sraw[0].z, sraw[0].w, sraw[1].x, sraw[1].y, sraw[1].z, sraw[1].w};
 #pragma unroll
@@ -153,7 +170,7 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
 #pragma unroll
         for (int c = 0; c < 16; ++c) acc[mb][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    ColScale cs[16];
+    float cs[16];
     uint4 sraw[2];
     uint32_t cur_group = 0;
     {
@@ -330,8 +347,7 @@ template <int BITS, int MB, bool GROUPED>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
     const dim3 grid((p.n + 255u) / 256u, p.splits, 1);
-    hipLaunchKernelGGL((bfaintb_decode_kernel<BITS, MB, GROUPED>), grid, dim3(256, 1, 1), 0, stream, p);
-    return hipGetLastError();
+    return launch_kernel(bfaintb_decode_kernel<BITS, MB, GROUPED>, grid, dim3(256, 1, 1), 0, stream, p);
 }
 
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)

@@ -1,5 +1,5 @@
 // Dequantised-weight dump: W[k,n] = bf16(float(q) * float(scale)) written to memory, through the
-// same device routines (make_col_scale, dequant_code, pack_bf16_rne) the GEMM kernels use.
+// same device routines (codes*_to_s8*, sbyte_to_f32, make_col_scale, pack_bf16_rne) the GEMM kernels use.
 // Successor of the reference's ASM_PRINT channel (/root/reference/bfAintBGemm/bfAintBGemm.cc:113-118,
 // 156-169; bf16gemm_kernel_gfx90a.s:2-16): the way to look at in-kernel dequantised values.
 #include "bfaintb_device.hpp"
@@ -28,25 +28,24 @@ __global__ void __launch_bounds__(256) bfaintb_dequant_kernel(const DequantParam
         if constexpr (BITS == 8) x[r] = *reinterpret_cast<const uint32_t*>(src);
         else x[r] = *reinterpret_cast<const uint16_t*>(src);
     }
-    float code[2][4];
+    uint32_t y[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
         if constexpr (BITS == 8) {
-            code[r][0] = ubyte_to_f32<0>(x[r]); code[r][1] = ubyte_to_f32<1>(x[r]);
-            code[r][2] = ubyte_to_f32<2>(x[r]); code[r][3] = ubyte_to_f32<3>(x[r]);
+            y[r] = codes8_to_s8(x[r]);
         } else {
-            const uint32_t lo = x[r] & 0x0f0fu, hi = (x[r] >> 4) & 0x0f0fu;
-            code[r][0] = ubyte_to_f32<0>(lo); code[r][1] = ubyte_to_f32<0>(hi);
-            code[r][2] = ubyte_to_f32<1>(lo); code[r][3] = ubyte_to_f32<1>(hi);
+            y[r] = codes4_quad_to_s8x16(x[r]);
         }
     }
     const uint32_t g = p.group_size ? row / p.group_size : 0u;  // group_size is even: both rows share a group
     const uint2 sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + col);
-    ColScale cs[4] = {make_col_scale<BITS>(sr.x & 0xffffu), make_col_scale<BITS>(sr.x >> 16),
-                      make_col_scale<BITS>(sr.y & 0xffffu), make_col_scale<BITS>(sr.y >> 16)};
+    const float cs[4] = {make_col_scale<BITS>(sr.x & 0xffffu), make_col_scale<BITS>(sr.x >> 16),
+                         make_col_scale<BITS>(sr.y & 0xffffu), make_col_scale<BITS>(sr.y >> 16)};
     uint32_t pk[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) pk[j] = pack_bf16_rne(dequant_code(code[0][j], cs[j]), dequant_code(code[1][j], cs[j]));
+    pk[0] = pack_bf16_rne(sbyte_to_f32<0>(y[0]) * cs[0], sbyte_to_f32<0>(y[1]) * cs[0]);
+    pk[1] = pack_bf16_rne(sbyte_to_f32<1>(y[0]) * cs[1], sbyte_to_f32<1>(y[1]) * cs[1]);
+    pk[2] = pack_bf16_rne(sbyte_to_f32<2>(y[0]) * cs[2], sbyte_to_f32<2>(y[1]) * cs[2]);
+    pk[3] = pack_bf16_rne(sbyte_to_f32<3>(y[0]) * cs[3], sbyte_to_f32<3>(y[1]) * cs[3]);
     // row `row`: low halves; row+1: high halves
     uint2 o0, o1;
     o0.x = (pk[0] & 0xffffu) | (pk[1] << 16);
@@ -62,9 +61,8 @@ hipError_t launch_dequant(uint16_t* w, const uint8_t* b, const uint16_t* scale, 
 {
     DequantParams p{w, b, scale, n, k, ldb_bytes, ldw, n, group_size};
     const dim3 grid((n / 4u + 255u) / 256u, k / 2u, 1);
-    if (bits == 8) hipLaunchKernelGGL(bfaintb_dequant_kernel<8>, grid, dim3(256, 1, 1), 0, stream, p);
-    else hipLaunchKernelGGL(bfaintb_dequant_kernel<4>, grid, dim3(256, 1, 1), 0, stream, p);
-    return hipGetLastError();
+    if (bits == 8) return launch_kernel(bfaintb_dequant_kernel<8>, grid, dim3(256, 1, 1), 0, stream, p);
+    return launch_kernel(bfaintb_dequant_kernel<4>, grid, dim3(256, 1, 1), 0, stream, p);
 }
 
 __global__ void __launch_bounds__(256) bfaintb_fill_u32_kernel(uint32_t* dst, uint32_t count, uint32_t value)
@@ -75,8 +73,7 @@ __global__ void __launch_bounds__(256) bfaintb_fill_u32_kernel(uint32_t* dst, ui
 
 hipError_t launch_fill_u32(uint32_t* dst, uint32_t count, uint32_t value, hipStream_t stream)
 {
-    hipLaunchKernelGGL(bfaintb_fill_u32_kernel, dim3((count + 255u) / 256u, 1, 1), dim3(256, 1, 1), 0, stream, dst, count, value);
-    return hipGetLastError();
+    return launch_kernel(bfaintb_fill_u32_kernel, dim3((count + 255u) / 256u, 1, 1), dim3(256, 1, 1), 0, stream, dst, count, value);
 }
 
 }  // namespace bfaintb

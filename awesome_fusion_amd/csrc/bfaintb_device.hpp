@@ -8,6 +8,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <tuple>
+#include <utility>
 
 namespace bfaintb {
 
@@ -17,6 +19,12 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 constexpr int kCounterSlots = 4096;  // arrival counters at the head of a workspace (uint32 each)
+
+template <typename Tuple, size_t... I>
+inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
+{
+    ((argv[I] = const_cast<void*>(static_cast<const void*>(&std::get<I>(t)))), ...);
+}
 
 struct GemmParams {
     uint16_t* c;
@@ -36,6 +44,18 @@ struct GemmParams {
     uint32_t* counters;  // [column blocks]
 };
 
+// Launch through hipLaunchKernel so that the error returned belongs to THIS launch:
+// hipGetLastError() would also hand back whatever an earlier, unrelated runtime call left behind.
+template <typename... Params, typename... Args>
+inline hipError_t launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t dyn_lds, hipStream_t stream, Args... args)
+{
+    static_assert(sizeof...(Params) == sizeof...(Args), "argument count");
+    std::tuple<Params...> pack{static_cast<Params>(args)...};
+    void* argv[sizeof...(Params)];
+    fill_argv(argv, pack, std::index_sequence_for<Params...>{});
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, dyn_lds, stream);
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
 // Two fp32 -> one dword of two bf16 (lo in bits 15:0), round to nearest even.
@@ -47,30 +67,39 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi)
     return __builtin_bit_cast(uint32_t, v);
 }
 
-// Byte `I` of a dword as fp32 (v_cvt_f32_ubyteI).
+// Signed byte `I` of a dword as fp32: one v_cvt_f32_i32 with an SDWA sign-extending byte select.
 template <int I>
-__device__ __forceinline__ float ubyte_to_f32(uint32_t x)
+__device__ __forceinline__ float sbyte_to_f32(uint32_t x)
 {
-    return (float)((x >> (8 * I)) & 0xffu);
+    if constexpr (I == 3) return (float)((int32_t)x >> 24);
+    return (float)(int32_t)(int8_t)((x >> (8 * I)) & 0xffu);
 }
 
-// A column's scale prepared for dequantisation: w = fma(code, s, o) with o = -bias*s.
-// code*s is exact inside the fma (<= 8 significant bits each), o is exact (bias is a power of
-// two) and the sum (code-bias)*s has at most 16 significant bits, so the fma returns exactly
-// float(q)*float(s), which is then rounded once to bf16.
-struct ColScale {
-    float s, o;
-};
+// Stored codes -> two's complement bytes the conversion above can read.
+//   8-bit: excess-128 byte u = q + 128; u ^ 0x80 is q as int8.
+//   4-bit: excess-8 nibble c = q + 8; c ^ 8 is q as int4; moved to the HIGH nibble of a byte it reads
+//          as the int8 value 16*q, and the column's scale is pre-divided by 16 (exact: a power of two).
+__device__ __forceinline__ uint32_t codes8_to_s8(uint32_t x) { return x ^ 0x80808080u; }
+__device__ __forceinline__ uint32_t codes4_even_to_s8x16(uint32_t x) { return ((x ^ 0x88888888u) << 4) & 0xf0f0f0f0u; }
+__device__ __forceinline__ uint32_t codes4_odd_to_s8x16(uint32_t x) { return (x ^ 0x88888888u) & 0xf0f0f0f0u; }
 
+// 16 bits holding four consecutive 4-bit codes (column j in nibble j) -> dword whose byte j reads as int8(16*q_j).
+__device__ __forceinline__ uint32_t codes4_quad_to_s8x16(uint32_t x)
+{
+    const uint32_t y = (x & 0xffu) | ((x & 0xff00u) << 8);  // bytes {c1c0, 0, c3c2, 0}
+    const uint32_t t = y ^ 0x00880088u;
+    return ((t << 4) & 0x00f000f0u) | ((t & 0x00f000f0u) << 8);
+}
+
+// A column's multiplier: the bf16 scale widened to fp32 (times 1/16 for 4-bit codes, see above).
+// w = value * multiplier is one IEEE fp32 multiply of float(q) (or float(16 q)) by it — exact for a
+// bf16 scale (8 x 8 significant bits), with the sign of zero of a true product — and is then
+// rounded once to bf16.
 template <int BITS>
-__device__ __forceinline__ ColScale make_col_scale(uint32_t scale_bf16_bits)
+__device__ __forceinline__ float make_col_scale(uint32_t scale_bf16_bits)
 {
-    ColScale cs;
-    cs.s = bf16_bits_to_f32(scale_bf16_bits);
-    cs.o = (BITS == 8 ? -128.0f : -8.0f) * cs.s;
-    return cs;
+    const float s = bf16_bits_to_f32(scale_bf16_bits);
+    return BITS == 8 ? s : s * 0.0625f;
 }
-
-__device__ __forceinline__ float dequant_code(float code, const ColScale& cs) { return __builtin_fmaf(code, cs.s, cs.o); }
 
 }  // namespace bfaintb

@@ -80,7 +80,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         w_dst[j] = kTileBytes + tile_off(rho, wave);
     }
 
-    ColScale cs[4];
+    float cs[4];
     uint32_t cur_group = 0xffffffffu;
     auto fetch_scales = [&](uint32_t g) {
         uint2 sr = make_uint2(0, 0);
@@ -114,14 +114,17 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         }
     };
 
-    // code of column J (0..3) of row register x
-    auto code = [&](uint32_t x, auto jc) -> float {
+    // signed value of column J (0..3) of a prepared row register (x16 for 4-bit codes)
+    auto value = [&](uint32_t x, auto jc) -> float {
         constexpr int J = decltype(jc)::value;
+        return sbyte_to_f32<J>(x);
+    };
+    // stored codes of one row (4 columns) -> 4 two's-complement bytes, byte J = column J
+    auto prepare = [&](uint32_t x) -> uint32_t {
         if constexpr (BITS == 8) {
-            return ubyte_to_f32<J>(x);
+            return codes8_to_s8(x);
         } else {
-            const uint32_t nib = (J % 2) ? ((x >> 4) & 0x0f0fu) : (x & 0x0f0fu);
-            return ubyte_to_f32<J / 2>(nib);
+            return codes4_quad_to_s8x16(x);
         }
     };
 
@@ -136,13 +139,16 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                 fetch_scales(g);
             }
         }
+        uint32_t b_s8[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) b_s8[r] = prepare(b_reg[r]);
         auto put = [&](auto jc) {
             constexpr int J = decltype(jc)::value;
             uint4 w;
-            w.x = pack_bf16_rne(dequant_code(code(b_reg[0], jc), cs[J]), dequant_code(code(b_reg[1], jc), cs[J]));
-            w.y = pack_bf16_rne(dequant_code(code(b_reg[2], jc), cs[J]), dequant_code(code(b_reg[3], jc), cs[J]));
-            w.z = pack_bf16_rne(dequant_code(code(b_reg[4], jc), cs[J]), dequant_code(code(b_reg[5], jc), cs[J]));
-            w.w = pack_bf16_rne(dequant_code(code(b_reg[6], jc), cs[J]), dequant_code(code(b_reg[7], jc), cs[J]));
+            w.x = pack_bf16_rne(value(b_s8[0], jc) * cs[J], value(b_s8[1], jc) * cs[J]);
+            w.y = pack_bf16_rne(value(b_s8[2], jc) * cs[J], value(b_s8[3], jc) * cs[J]);
+            w.z = pack_bf16_rne(value(b_s8[4], jc) * cs[J], value(b_s8[5], jc) * cs[J]);
+            w.w = pack_bf16_rne(value(b_s8[6], jc) * cs[J], value(b_s8[7], jc) * cs[J]);
             *reinterpret_cast<uint4*>(base + w_dst[J]) = w;
         };
         put(std::integral_constant<int, 0>{});
@@ -232,8 +238,7 @@ static hipError_t launch_prefill_t(const GemmParams& p, hipStream_t stream)
         attr_set = true;
     }
     const uint32_t tiles = ((p.m + kBM - 1) / kBM) * ((p.n + kBN - 1) / kBN);
-    hipLaunchKernelGGL((bfaintb_prefill_kernel<BITS, GROUPED>), dim3(tiles, 1, 1), dim3(512, 1, 1), kLdsBytes, stream, p);
-    return hipGetLastError();
+    return launch_kernel(bfaintb_prefill_kernel<BITS, GROUPED>, dim3(tiles, 1, 1), dim3(512, 1, 1), kLdsBytes, stream, p);
 }
 
 hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream)

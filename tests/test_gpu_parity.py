@@ -70,9 +70,11 @@ def test_reference_regime_bit_for_bit(af, m, n, k):
     p = Problem(m, n, k, regime="small_int", seed=m + n)
     c_ref = oracle.gemm_rrr(widen(p.a_bf), p.q.astype(np.float32), widen(p.s_bf)[0])  # host_ref as main() calls it
     c = run_gemm(p)
-    assert np.array_equal(widen(c), c_ref)
-    ok, pp, _ = oracle.valid_vector(c_ref, c)
-    assert pp == 0 and (ok or not c_ref.any())
+    # the fp32 sums are exact; the only rounding is the store to bf16 (odd integers above 256 are not bf16 numbers)
+    assert np.array_equal(widen(c), widen(oracle.f32_to_bf16_rne(c_ref)))
+    if np.abs(c_ref).max() <= 256 and c_ref.any():
+        ok, pp, _ = oracle.valid_vector(c_ref, c)  # the reference's own acceptance test (validation.hpp:7-46)
+        assert ok and pp == 0
 
 
 def test_golden_int_regime_fixture(af, golden_dir):
@@ -98,7 +100,10 @@ def test_config1_golden(af, golden_dir):
     p = Problem(64, 128, 256)
     p.a_bf, p.b_bytes, p.s_bf = g["a_bf"], g["b_bytes"], g["s_bf"].reshape(1, -1)
     c = run_gemm(p)
-    assert_close_ulp(g["c_oracle"], c, "C1 vs reference-produced fixture")
+    # fixture output = the reference's gemm_rrr on (bf16 A, bf16 W, unit scales); no near-zero escape here
+    bad, worst, _ = oracle.check_ulp(g["c_oracle"], c)
+    assert bad == 0, (bad, worst)
+    assert np.array_equal(p.w_bf, g["w_bf"])
 
 
 @pytest.mark.parametrize("m", [1, 4, 8, 16, 32])
@@ -107,30 +112,21 @@ def test_config2_and_3_decode(af, m):
         p = Problem(m, n, 4096, seed=m)
         c = run_gemm(p)
         assert af.variant(m, n, 4096) == af.DECODE
-        assert_close_ulp(p.c_ref(), c, f"decode m={m} n={n}")
+        assert_close_ulp(p, c, f"decode m={m} n={n}")
 
 
 def test_config4_prefill_full_size(af):
     p = Problem(4096, 4096, 4096, seed=4)
     c = run_gemm(p)
-    c_ref = p.c_ref(threads=16)
-    bad, worst, idx = oracle.check_ulp(c_ref, c)
-    # 16.7 M outputs; sums of 4096 terms with sigma ~ 20 leave a few outputs near zero whose ULP is
-    # below the fp32 summation-order noise of EITHER side: report them, allow a handful, and require
-    # that each is explained by that noise (absolute error tiny against the row's magnitude)
-    err = np.abs(widen(c).astype(np.float64) - c_ref)
-    assert err.max() < 0.2, err.max()
-    assert bad <= 64, f"{bad} outputs outside 2 ULP (worst {worst:.2f} at {idx})"
-    if bad:
-        ulp_ok = oracle.check_ulp(c_ref, c, 2.0, 0.05, 1.0)[0]  # everything failing sits below |ref| = 0.05
-        assert ulp_ok == 0
+    worst, near_zero = assert_close_ulp(p, c, "prefill 4096^3", threads=16, max_frac=1e-4)
+    print(f"prefill 4096^3: worst {worst:.3f} ULP, {near_zero} near-zero outputs beyond 2 ULP (within fp32 summation noise)")
 
 
 @pytest.mark.parametrize("m", [1, 16])
 def test_config5_int4_group128_decode(af, m):
     p = Problem(m, 28672, 8192, 4, 128, seed=50 + m, scale_lo=0.001, scale_hi=0.02)
     c = run_gemm(p)
-    assert_close_ulp(p.c_ref(threads=16), c, f"int4 g128 m={m}")
+    assert_close_ulp(p, c, f"int4 g128 m={m}", threads=16)
 
 
 def test_config5_int4_group128_prefill_rows(af):
@@ -138,7 +134,7 @@ def test_config5_int4_group128_prefill_rows(af):
     p = Problem(m, 28672, 8192, 4, 128, seed=52, scale_lo=0.001, scale_hi=0.02)
     c = run_gemm(p)
     rows = np.arange(5, m, 16)  # 128 rows touching every 32-row MFMA block of every tile
-    assert_close_ulp(p.c_ref(rows, threads=16), c[rows], "int4 g128 m=2048 (row sample)", allow=8)
+    assert_close_ulp(p, np.ascontiguousarray(c[rows]), "int4 g128 m=2048 (row sample)", rows=rows, threads=16)
 
 
 # ---------------------------------------------------------------------------- shapes, strides, split-K
@@ -148,7 +144,7 @@ def test_config5_int4_group128_prefill_rows(af):
 def test_ragged_shapes(af, m, n, k, bits, group):
     p = Problem(m, n, k, bits, group, seed=m * 7 + n)
     c = run_gemm(p)
-    assert_close_ulp(p.c_ref(), c, f"ragged {m}x{n}x{k} bits={bits}")
+    assert_close_ulp(p, c, f"ragged {m}x{n}x{k} bits={bits}")
 
 
 @pytest.mark.parametrize("m", [5, 80])
@@ -159,17 +155,16 @@ def test_leading_dimensions_and_untouched_padding(af, m):
     a_pad = np.full((m, lda), 0x7FC0, np.uint16); a_pad[:, :k] = p.a_bf
     b_pad = np.full((k, ldb), 0xAB, np.uint8); b_pad[:, :n] = p.b_bytes
     c = run_gemm(p, lda=lda, ldb=ldb, ldc=ldc, a_dev=to_dev(a_pad), b_dev=to_dev(b_pad), c_fill=0x1234)
-    assert_close_ulp(p.c_ref(), np.ascontiguousarray(c[:, :n]), "strided")
+    assert_close_ulp(p, np.ascontiguousarray(c[:, :n]), "strided")
     assert (c[:, n:] == 0x1234).all(), "columns beyond n were written"
 
 
 def test_split_k_is_deterministic_and_consistent(af):
     p = Problem(7, 768, 4096, seed=12)
-    ref = p.c_ref()
     outs = {}
     for split in (1, 2, 5, 32):
         c = run_gemm(p, which=af.DECODE, force_split_k=split)
-        assert_close_ulp(ref, c, f"split_k={split}")
+        assert_close_ulp(p, c, f"split_k={split}")
         for _ in range(3):  # same split: same bits, whatever order the workgroups arrived in
             assert np.array_equal(run_gemm(p, which=af.DECODE, force_split_k=split), c)
         outs[split] = c
@@ -180,14 +175,13 @@ def test_workspace_is_left_ready_for_the_next_call(af):
     shapes = [(1, 4096, 4096), (16, 1024, 8192), (32, 272, 512), (1, 4096, 4096)]
     for i, (m, n, k) in enumerate(shapes):
         p = Problem(m, n, k, seed=i)
-        assert_close_ulp(p.c_ref(), run_gemm(p), f"call {i}")
+        assert_close_ulp(p, run_gemm(p), f"call {i}")
 
 
 def test_prefill_variant_on_small_m_matches_decode(af):
     p = Problem(24, 512, 1024, seed=77)
-    ref = p.c_ref()
-    assert_close_ulp(ref, run_gemm(p, which=af.PREFILL), "prefill kernel at m=24")
-    assert_close_ulp(ref, run_gemm(p, which=af.DECODE), "decode kernel at m=24")
+    assert_close_ulp(p, run_gemm(p, which=af.PREFILL), "prefill kernel at m=24")
+    assert_close_ulp(p, run_gemm(p, which=af.DECODE), "decode kernel at m=24")
 
 
 def test_row_permutation_permutes_output(af):

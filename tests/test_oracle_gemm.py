@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Problem, widen
+from helpers import Problem, ulp_violations, widen
 
 fp = C.POINTER(C.c_float)
 
@@ -145,3 +145,13 @@ def test_check_ulp():
         assert bad == want_bad, (i, worst)
     bad, worst, idx = oracle.check_ulp(ref, bits)
     assert bad == 2
+
+
+def test_numpy_and_c_acceptance_checks_agree():
+    rng = np.random.Generator(np.random.PCG64(8))
+    ref = (rng.standard_normal(20000) * np.exp(rng.uniform(-12, 4, 20000))).astype(np.float32)
+    noisy = ref * (1 + rng.standard_normal(20000).astype(np.float32) * 0.006)
+    bits = oracle.f32_to_bf16_rne(noisy)
+    bad_np, _ = ulp_violations(ref, bits)
+    bad_c, _, _ = oracle.check_ulp(ref, bits)
+    assert 100 < bad_c < 19000 and bad_c == len(bad_np)
