@@ -181,6 +181,9 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
         p.counters = static_cast<uint32_t*>(workspace);
         p.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kCounterBytes);
     }
+#ifdef BFAINTB_TRACE
+    if (workspace != nullptr) p.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kCounterBytes);  // timestamp sink
+#endif
     return (int)bfaintb::launch_decode(p, weight_bits, st);
 }
 

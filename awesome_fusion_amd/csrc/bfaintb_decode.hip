@@ -46,17 +46,15 @@ __device__ __forceinline__ float value_f32(const uint32_t (&row)[4])
 }
 
 template <int BITS>
-__device__ __forceinline__ void load_raw(RawStep<BITS>& raw, const uint8_t* rowptr, uint32_t ldb_bytes, bool ok)
+__device__ __forceinline__ void load_raw(RawStep<BITS>& raw, const uint8_t* rowptr, uint32_t ldb_bytes)
 {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
         if constexpr (BITS == 8) {
-            uint4 v = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);
-            if (ok) v = *reinterpret_cast<const uint4*>(rowptr + (size_t)r * ldb_bytes);
+            const uint4 v = *reinterpret_cast<const uint4*>(rowptr + (size_t)r * ldb_bytes);
             raw.d[r][0] = v.x; raw.d[r][1] = v.y; raw.d[r][2] = v.z; raw.d[r][3] = v.w;
         } else {
-            uint2 v = make_uint2(0x88888888u, 0x88888888u);
-            if (ok) v = *reinterpret_cast<const uint2*>(rowptr + (size_t)r * ldb_bytes);
+            const uint2 v = *reinterpret_cast<const uint2*>(rowptr + (size_t)r * ldb_bytes);
             raw.d[r][0] = v.x; raw.d[r][1] = v.y;
         }
     }
@@ -104,14 +102,10 @@ __device__ __forceinline__ void mac_step(const RawStep<BITS>& raw, const float (
 }
 
 template <int BITS>
-__device__ __forceinline__ void load_scales(uint4 (&sraw)[2], const uint16_t* sptr, bool ok)
+__device__ __forceinline__ void load_scales(uint4 (&sraw)[2], const uint16_t* sptr)
 {
-    sraw[0] = make_uint4(0, 0, 0, 0);
-    sraw[1] = make_uint4(0, 0, 0, 0);
-    if (ok) {
-        sraw[0] = *reinterpret_cast<const uint4*>(sptr);
-        sraw[1] = *reinterpret_cast<const uint4*>(sptr + 8);
-    }
+    sraw[0] = *reinterpret_cast<const uint4*>(sptr);
+    sraw[1] = *reinterpret_cast<const uint4*>(sptr + 8);
 }
 
 template <int BITS>
@@ -125,14 +119,21 @@ __device__ __forceinline__ void apply_scales(float (&cs)[16], const uint4 (&sraw
     }
 }
 
+#ifdef BFAINTB_TRACE
+#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) reinterpret_cast<unsigned long long*>(p.partials)[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define TRACE_MARK(i) do { } while (0)
+#endif
+
 constexpr int kRedStride = 260;  // floats per row of the LDS reduction buffer (256 + 4: spreads rows over banks)
 
 template <int BITS, int MB, bool GROUPED>
 __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
 {
-    __shared__ float red[2][MB * 16][kRedStride];
+    extern __shared__ __attribute__((aligned(16))) float red[];  // [4 waves][m rows][kRedStride], at least 4096 floats
     __shared__ uint32_t s_is_last;
 
+    TRACE_MARK(0);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int nl = lane & 15;
@@ -140,9 +141,10 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
     const uint32_t cb = blockIdx.x;
     const uint32_t ks = blockIdx.y;
 
-    // ---- this lane's 16 weight columns
-    const uint32_t n_ld = cb * 256u + (uint32_t)nl * 16u;
-    const bool col_ok = n_ld < p.n;
+    // ---- this lane's 16 weight columns.  A lane past the last column reads the last 16 columns
+    //      instead (no predicated loads in the hot loop); what it computes is never stored.
+    uint32_t n_ld = cb * 256u + (uint32_t)nl * 16u;
+    if (n_ld >= p.n) n_ld = p.n - 16u;
 
     // ---- this wave's rows of k
     const uint32_t k_per_wave = p.k_per_wg >> 2;
@@ -154,14 +156,15 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
     const uint8_t* bptr = p.b + (size_t)(kb + 8u * kg) * p.ldb_bytes + (BITS == 8 ? n_ld : n_ld / 2);
     const size_t bstep = (size_t)32 * p.ldb_bytes;
 
-    // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg
+    // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg.
+    // Lanes whose row is past m re-read row m-1; their accumulator columns are never stored.
     const uint16_t* aptr[MB];
-    bool a_ok[MB];
+    bool row_ok[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const uint32_t mi = 16u * mb + (uint32_t)nl;
-        a_ok[mb] = mi < p.m;
-        aptr[mb] = p.a + (size_t)(a_ok[mb] ? mi : 0) * p.lda + kb + 8u * kg;
+        row_ok[mb] = mi < p.m;
+        aptr[mb] = p.a + (size_t)(row_ok[mb] ? mi : p.m - 1u) * p.lda + kb + 8u * kg;
     }
 
     f32x4_t acc[MB][16];
@@ -170,184 +173,159 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
 #pragma unroll
         for (int c = 0; c < 16; ++c) acc[mb][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    float cs[16];
-    uint4 sraw[2];
-    uint32_t cur_group = 0;
-    {
-        if constexpr (GROUPED) cur_group = (kb < p.k ? kb : 0) / p.group_size;
-        load_scales<BITS>(sraw, p.scale + (size_t)cur_group * p.lds + n_ld, col_ok);
-        apply_scales<BITS>(cs, sraw);
-    }
-
-    RawStep<BITS> raw0, raw1;
-    uint4 af0[MB], af1[MB];
-    auto load_a = [&](uint4(&af)[MB], int step) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            af[mb] = make_uint4(0, 0, 0, 0);
-            if (a_ok[mb]) af[mb] = *reinterpret_cast<const uint4*>(aptr[mb] + (size_t)step * 32);
-        }
-    };
-    // Scales for the group a step belongs to are fetched one step ahead, when the group changes.
-    auto prefetch_scales = [&](int step) -> bool {
-        if constexpr (GROUPED) {
-            const uint32_t g = (kb + 32u * step) / p.group_size;
-            if (g != cur_group) {
-                cur_group = g;
-                load_scales<BITS>(sraw, p.scale + (size_t)g * p.lds + n_ld, col_ok);
-                return true;
-            }
-        }
-        return false;
-    };
-
     if (nsteps > 0) {
-        load_raw<BITS>(raw0, bptr, p.ldb_bytes, col_ok);
-        load_a(af0, 0);
+        // Software pipeline of depth one: the loads of step s+1 are issued before step s is
+        // computed.  Every load inside the loop is unconditional, so the wait counts the compiler
+        // derives are exact (a load behind a branch would make it wait for the prefetch as well);
+        // the last step, which has nothing to prefetch, is peeled off behind the loop.
+        RawStep<BITS> cur, nxt;
+        uint4 af_cur[MB], af_nxt[MB];
+        float cs[16];
+        uint4 sraw[2], sraw_nxt[2];
+        const uint16_t* sptr = p.scale + n_ld;
+        auto group_of = [&](int step) -> uint32_t {
+            if constexpr (GROUPED) return (kb + 32u * (uint32_t)step) / p.group_size;
+            return 0u;
+        };
+
+        load_scales<BITS>(sraw, sptr + (size_t)group_of(0) * p.lds);
+        load_raw<BITS>(cur, bptr, p.ldb_bytes);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) af_cur[mb] = *reinterpret_cast<const uint4*>(aptr[mb]);
+        apply_scales<BITS>(cs, sraw);
+
+        for (int s = 0; s + 1 < nsteps; ++s) {
+            load_raw<BITS>(nxt, bptr + (size_t)(s + 1) * bstep, p.ldb_bytes);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) af_nxt[mb] = *reinterpret_cast<const uint4*>(aptr[mb] + (size_t)(s + 1) * 32);
+            if constexpr (GROUPED) load_scales<BITS>(sraw_nxt, sptr + (size_t)group_of(s + 1) * p.lds);
+            mac_step<BITS, MB>(cur, cs, af_cur, acc, std::make_integer_sequence<int, 16>{});
+            TRACE_MARK(1);
+            cur = nxt;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) af_cur[mb] = af_nxt[mb];
+            if constexpr (GROUPED) apply_scales<BITS>(cs, sraw_nxt);
+        }
+        mac_step<BITS, MB>(cur, cs, af_cur, acc, std::make_integer_sequence<int, 16>{});
     }
-    int s = 0;
-    bool new_scales = false;
-    while (s < nsteps) {
-        bool ns_next = false;
-        if (s + 1 < nsteps) {
-            load_raw<BITS>(raw1, bptr + (size_t)(s + 1) * bstep, p.ldb_bytes, col_ok);
-            load_a(af1, s + 1);
-        }
-        if (new_scales) apply_scales<BITS>(cs, sraw);
-        if (s + 1 < nsteps) ns_next = prefetch_scales(s + 1);
-        mac_step<BITS, MB>(raw0, cs, af0, acc, std::make_integer_sequence<int, 16>{});
-        new_scales = ns_next;
-        if (++s >= nsteps) break;
+    TRACE_MARK(2);
 
-        ns_next = false;
-        if (s + 1 < nsteps) {
-            load_raw<BITS>(raw0, bptr + (size_t)(s + 1) * bstep, p.ldb_bytes, col_ok);
-            load_a(af0, s + 1);
-        }
-        if (new_scales) apply_scales<BITS>(cs, sraw);
-        if (s + 1 < nsteps) ns_next = prefetch_scales(s + 1);
-        mac_step<BITS, MB>(raw1, cs, af1, acc, std::make_integer_sequence<int, 16>{});
-        new_scales = ns_next;
-        ++s;
+    // ---- add the 4 waves' partial sums through LDS: one barrier, then thread t finishes two
+    //      neighbouring columns.  acc[mb][c][r] of lane (nl, kg) is row mi = 16*mb + nl,
+    //      local column (4*kg + r)*16 + c.
+    const uint32_t rows_out = p.m;  // <= 16*MB
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        if (!row_ok[mb]) continue;
+        float* row = red + ((size_t)wave * rows_out + (mb * 16 + nl)) * kRedStride;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
+                                       acc[mb][4 * c4 + 3][r]);
+                *reinterpret_cast<float4*>(row + (4 * kg + r) * 16 + 4 * c4) = v;
+            }
     }
-
-    // ---- add the 4 waves' partial sums.  acc[mb][c][r] of lane (nl, kg) is
-    //      row mi = 16*mb + nl, local column (4*kg + r)*16 + c.
-    auto lds_store = [&](int slot) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            if (!a_ok[mb]) continue;
-            float* row = &red[slot][mb * 16 + nl][0];
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-#pragma unroll
-                for (int c4 = 0; c4 < 4; ++c4) {
-                    float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
-                                           acc[mb][4 * c4 + 3][r]);
-                    *reinterpret_cast<float4*>(row + (4 * kg + r) * 16 + 4 * c4) = v;
-                }
-        }
-    };
-    auto lds_add = [&](int slot) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            if (!a_ok[mb]) continue;
-            const float* row = &red[slot][mb * 16 + nl][0];
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-#pragma unroll
-                for (int c4 = 0; c4 < 4; ++c4) {
-                    const float4 v = *reinterpret_cast<const float4*>(row + (4 * kg + r) * 16 + 4 * c4);
-                    acc[mb][4 * c4 + 0][r] += v.x;
-                    acc[mb][4 * c4 + 1][r] += v.y;
-                    acc[mb][4 * c4 + 2][r] += v.z;
-                    acc[mb][4 * c4 + 3][r] += v.w;
-                }
-        }
-    };
-    if (wave >= 2) lds_store(wave - 2);
     __syncthreads();
-    if (wave < 2) lds_add(wave);
-    __syncthreads();
-    if (wave == 1) lds_store(0);
-    __syncthreads();
-    if (wave == 0) lds_add(0);
-
-    // ---- output
-    if (p.splits == 1) {
-        if (wave == 0) {
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                if (!a_ok[mb]) continue;
-                const uint32_t mi = 16u * mb + (uint32_t)nl;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t n_out = cb * 256u + (uint32_t)(4 * kg + r) * 16u;
-                    if (n_out >= p.n) continue;
-                    uint4 lo, hi;
-                    lo.x = pack_bf16_rne(acc[mb][0][r], acc[mb][1][r]);
-                    lo.y = pack_bf16_rne(acc[mb][2][r], acc[mb][3][r]);
-                    lo.z = pack_bf16_rne(acc[mb][4][r], acc[mb][5][r]);
-                    lo.w = pack_bf16_rne(acc[mb][6][r], acc[mb][7][r]);
-                    hi.x = pack_bf16_rne(acc[mb][8][r], acc[mb][9][r]);
-                    hi.y = pack_bf16_rne(acc[mb][10][r], acc[mb][11][r]);
-                    hi.z = pack_bf16_rne(acc[mb][12][r], acc[mb][13][r]);
-                    hi.w = pack_bf16_rne(acc[mb][14][r], acc[mb][15][r]);
-                    uint16_t* dst = p.c + (size_t)mi * p.ldc + n_out;
-                    *reinterpret_cast<uint4*>(dst) = lo;
-                    *reinterpret_cast<uint4*>(dst + 8) = hi;
+    TRACE_MARK(3);
+    {
+        const uint32_t cp = threadIdx.x & 127u, rsel = threadIdx.x >> 7;
+        const uint32_t col = cb * 256u + 2u * cp;
+        if (col < p.n) {
+            for (uint32_t row = rsel; row < rows_out; row += 2u) {
+                const float* src = red + (size_t)row * kRedStride + 2u * cp;
+                const float2 w0 = *reinterpret_cast<const float2*>(src);
+                const float2 w1 = *reinterpret_cast<const float2*>(src + (size_t)rows_out * kRedStride);
+                const float2 w2 = *reinterpret_cast<const float2*>(src + (size_t)2 * rows_out * kRedStride);
+                const float2 w3 = *reinterpret_cast<const float2*>(src + (size_t)3 * rows_out * kRedStride);
+                const float sx = (w0.x + w1.x) + (w2.x + w3.x);
+                const float sy = (w0.y + w1.y) + (w2.y + w3.y);
+                if (p.splits == 1) {
+                    *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col) = pack_bf16_rne(sx, sy);
+                } else {
+                    // split-K partial tile, written with a device-scope (write-through) store: no L2
+                    // write-back is needed before announcing arrival, only the store's acknowledgement
+                    const unsigned long long bits = (unsigned long long)__float_as_uint(sx) | ((unsigned long long)__float_as_uint(sy) << 32);
+                    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p.partials + ((size_t)ks * p.m + row) * p.n + col), bits,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
         }
-        return;
     }
+    if (p.splits == 1) return;
 
-    // ---- split-K: publish this workgroup's partial tile, last arrival reduces
-    if (wave == 0) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            if (!a_ok[mb]) continue;
-            const uint32_t mi = 16u * mb + (uint32_t)nl;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const uint32_t n_out = cb * 256u + (uint32_t)(4 * kg + r) * 16u;
-                if (n_out >= p.n) continue;
-                float* dst = p.partials + ((size_t)ks * p.m + mi) * p.n + n_out;
-#pragma unroll
-                for (int c4 = 0; c4 < 4; ++c4) {
-                    *reinterpret_cast<float4*>(dst + 4 * c4) =
-                        make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r], acc[mb][4 * c4 + 3][r]);
-                }
-            }
-        }
-        __threadfence();  // release the partial tile at device scope before announcing arrival
-    }
+    // ---- split-K: the last workgroup to arrive at this column block adds all partial tiles in a
+    // fixed order and writes C.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt vmcnt(0): this wave's stores are acknowledged
     __syncthreads();
     if (threadIdx.x == 0) {
-        const uint32_t arrived = atomicAdd(p.counters + cb, 1u);
+        const uint32_t arrived = __hip_atomic_fetch_add(p.counters + cb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_is_last = (arrived == p.splits - 1u) ? 1u : 0u;
     }
     __syncthreads();
     if (s_is_last == 0u) return;
-    __threadfence();  // acquire: the other workgroups' tiles are visible from here on
+    // acquire at device scope: drops lines of the partial tiles this XCD's L2 may still hold from an
+    // earlier launch, so the plain (vectorisable, pipelined) loads below see the other workgroups' stores
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
-    const uint32_t col = cb * 256u + threadIdx.x;
-    if (col < p.n) {
-        for (uint32_t mi = 0; mi < p.m; ++mi) {
-            const float* src = p.partials + (size_t)mi * p.n + col;
-            float sum = 0.f;
-            for (uint32_t sp = 0; sp < p.splits; ++sp) sum += src[(size_t)sp * p.m * p.n];
-            p.c[(size_t)mi * p.ldc + col] = (uint16_t)(pack_bf16_rne(sum, 0.f) & 0xffffu);
+    // thread t: 4 consecutive columns (cg = t%64), splits sp = sub, sub+4, ... (sub = t/64), rows in
+    // chunks of 4; the four sub-sums are combined through LDS in a fixed order
+    {
+        const uint32_t cg = threadIdx.x & 63u, sub = threadIdx.x >> 6;
+        const uint32_t col = cb * 256u + 4u * cg;
+        const bool col_ok = col < p.n;
+        __syncthreads();               // every wave is done reading its sums out of red
+        float* stage = red;            // [4 subs][4 rows][256 cols] = 4096 floats
+        for (uint32_t m0 = 0; m0 < p.m; m0 += 4u) {
+            const uint32_t rows = p.m - m0 < 4u ? p.m - m0 : 4u;
+            for (uint32_t ri = 0; ri < rows; ++ri) {
+                float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (col_ok) {
+                    const float* src = p.partials + (size_t)(m0 + ri) * p.n + col;
+                    for (uint32_t sp = sub; sp < p.splits; sp += 4u) {
+                        const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sp * p.m * p.n);
+                        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+                    }
+                }
+                *reinterpret_cast<float4*>(stage + (sub * 4u + ri) * 256u + 4u * cg) = sum;
+            }
+            __syncthreads();
+            {
+                const uint32_t ri = sub;  // thread t finishes row t/64 of the chunk
+                if (ri < rows && col_ok) {
+                    const float4 s0 = *reinterpret_cast<const float4*>(stage + (0u * 4u + ri) * 256u + 4u * cg);
+                    const float4 s1 = *reinterpret_cast<const float4*>(stage + (1u * 4u + ri) * 256u + 4u * cg);
+                    const float4 s2 = *reinterpret_cast<const float4*>(stage + (2u * 4u + ri) * 256u + 4u * cg);
+                    const float4 s3 = *reinterpret_cast<const float4*>(stage + (3u * 4u + ri) * 256u + 4u * cg);
+                    uint2 o;
+                    o.x = pack_bf16_rne((s0.x + s1.x) + (s2.x + s3.x), (s0.y + s1.y) + (s2.y + s3.y));
+                    o.y = pack_bf16_rne((s0.z + s1.z) + (s2.z + s3.z), (s0.w + s1.w) + (s2.w + s3.w));
+                    *reinterpret_cast<uint2*>(p.c + (size_t)(m0 + ri) * p.ldc + col) = o;
+                }
+            }
+            __syncthreads();
         }
     }
-    if (threadIdx.x == 0) p.counters[cb] = 0u;  // ready for the next launch on this workspace
+    if (threadIdx.x == 0) __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
 }
 
 template <int BITS, int MB, bool GROUPED>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
     const dim3 grid((p.n + 255u) / 256u, p.splits, 1);
-    return launch_kernel(bfaintb_decode_kernel<BITS, MB, GROUPED>, grid, dim3(256, 1, 1), 0, stream, p);
+    size_t lds = (size_t)4 * p.m * kRedStride * sizeof(float);
+    if (lds < 4096 * sizeof(float)) lds = 4096 * sizeof(float);
+    if (lds > 64 * 1024) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, MB, GROUPED>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 4 * 32 * kRedStride * (int)sizeof(float));
+            if (e != hipSuccess) return e;
+            attr_set = true;
+        }
+    }
+    return launch_kernel(bfaintb_decode_kernel<BITS, MB, GROUPED>, grid, dim3(256, 1, 1), lds, stream, p);
 }
 
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)
