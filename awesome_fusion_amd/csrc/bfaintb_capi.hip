@@ -171,7 +171,11 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     p.splits = 1;
     hipStream_t st = static_cast<hipStream_t>(stream);
 
-    if (v == BFAINTB_VARIANT_PREFILL) return (int)bfaintb::launch_prefill(p, weight_bits, st);
+    if (v == BFAINTB_VARIANT_PREFILL) {
+        // the prefill kernel addresses B and a 256-row panel of A through 32-bit buffer extents
+        if ((uint64_t)k * p.ldb_bytes >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
+        return (int)bfaintb::launch_prefill(p, weight_bits, st);
+    }
 
     decode_split(n, k, split_k, &p.k_per_wg, &p.splits);
     if (p.splits > 1) {

@@ -6,35 +6,47 @@
 // LDS layouts :346-393, epilogue :594-630).
 //
 // Shape of the computation
-//   grid = ceil(m/256) * ceil(n/256) workgroups of 512 threads (8 waves, 2 along m x 4 along n);
-//   each wave owns a 128 x 64 block of the tile = 4 x 2 accumulators of v_mfma_f32_32x32x16_bf16.
-//   K advances 64 per step.  LDS holds two stages of {A tile, dequantised W tile}, each tile
-//   256 rows x 64 k of bf16 (row = 128 bytes = 8 chunks of 16 bytes), so a step needs one barrier.
-//   Chunk c of row r lives at chunk position c ^ ((r >> 1) & 7): with 64 LDS banks, 16 lanes that
-//   read or write the same chunk of 16 consecutive rows then touch 16 different 16-byte bank
-//   groups (no conflicts).
-// A path: 16-byte global loads (8 lanes per row) -> registers -> ds_write_b128.
-// W path: wave w loads rows 8w..8w+7 of the step, one dword (4 codes) per lane per row, so that a
-//   lane ends up with 8 consecutive k of 4 columns; it dequantises them (cvt_ubyte, fma, cvt_pk)
-//   and writes one 16-byte chunk per column: column (4*lane + j) goes to LDS row
-//   rho = (j>>1)*128 + (j&1)*32 + (lane&31) + (lane>>5)*64, which makes consecutive lanes write
-//   consecutive rows.  The MFMA "column" index is the LDS row, so wave wn / accumulator t / lane
+//   One workgroup of 512 threads (8 waves, 2 along m x 4 along n) per 256x256 tile of C; each wave
+//   owns a 128 x 64 block = 4 x 2 accumulators of v_mfma_f32_32x32x16_bf16.  K advances 64 per step.
+//   LDS holds two stages of {A tile, dequantised W tile}; a tile is 256 rows x 64 k of bf16 (a row is
+//   128 bytes = 8 chunks of 16 bytes), so one barrier per step suffices.  Chunk c of row r lives at
+//   chunk position c ^ ((r >> 1) & 7): 16 lanes that read, or 8 lanes that write, the same chunk of
+//   consecutive rows land in different 16-byte bank groups.
+//   Workgroup ids are remapped so that the workgroups an XCD receives (id mod 8) form a compact
+//   4 x 8 block of tiles: each XCD's L2 then fetches 4 row-panels of A and 8 column-panels of B
+//   instead of every row-panel of A.
+// Global loads are raw buffer loads: a lane's byte offset sits in one VGPR, the K advance (and for B
+// the row) in an SGPR offset, so the loop carries no vector address arithmetic and no predication.
+// The buffers' extents end with the tile's last valid row of A and the last row of B (gfx9-family
+// range checks add the SGPR offset to the lane offset): rows of A past m read as zero; columns of B
+// past n read whatever lies there, or zero past the end of B, and feed only columns that are never stored.
+// A path: 16-byte loads (8 lanes per row) -> registers -> ds_write_b128.
+// W path: wave w loads rows 8w..8w+7 of the step, one dword (4 codes) per lane per row, so a lane
+//   ends up with 8 consecutive k of 4 columns; it dequantises them (xor, cvt with sign-extending
+//   byte select, multiply, cvt_pk) and writes one 16-byte chunk per column.  Column (4*lane + j)
+//   goes to LDS row rho = (j>>1)*128 + (j&1)*32 + (lane&31) + (lane>>5)*64, so consecutive lanes
+//   write consecutive rows.  The MFMA "column" index is the LDS row: wave wn, accumulator t, lane
 //   column jl hold tile column 4*(32*(wn&1) + jl) + 2*(wn>>1) + t.
-// Epilogue: accumulators are rounded to bf16 (v_cvt_pk_bf16_f32; t = 0,1 are neighbouring
-//   columns and share a dword), staged in LDS in true [m][n] order and stored with 16-byte
-//   row-contiguous writes.
+// Pipeline per step (registers hold the raw tile of step+1, loaded one step earlier): MFMAs of the
+//   current stage; the raw tile is converted and written to the other stage in the second half of
+//   the step, between MFMAs; then the loads for step+2 are issued; barrier.
+// Epilogue: accumulators are rounded to bf16 (v_cvt_pk_bf16_f32; t = 0,1 are neighbouring columns
+//   and share a dword), staged in LDS in true [m][n] order and stored with 16-byte row-contiguous writes.
 #include <utility>
 #include "bfaintb_device.hpp"
 
 namespace bfaintb {
 
 constexpr int kBM = 256, kBN = 256, kBK = 64;
-constexpr int kTileBytes = 256 * 128;             // one A or W tile in LDS
-constexpr int kStageBytes = 2 * kTileBytes;       // A + W
-constexpr int kCRowBytes = 256 * 2 + 16;          // epilogue staging row (padded)
-constexpr int kLdsBytes = 256 * kCRowBytes;       // 135168 >= 2 stages (131072)
+constexpr uint32_t kTileBytes = 256 * 128;              // one A or W tile in LDS
+constexpr uint32_t kAOff = 0, kWOff = 2 * kTileBytes;   // LDS: A stage 0, A stage 1, W stage 0, W stage 1
+constexpr int kCRowBytes = 256 * 2 + 16;                // epilogue staging row (padded)
+constexpr int kLdsBytes = 256 * kCRowBytes;             // 135168 >= 4 tiles (131072)
+constexpr int kBufferFlags = 0x00027000;                // raw buffer, 32-bit data format
 
-__device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t swizzled_off(uint32_t row, uint32_t chunk)
 {
     return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
@@ -46,40 +58,54 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
     const uint32_t wm = wave >> 2;   // 0..1
     const uint32_t wn = wave & 3u;   // 0..3
 
-    const uint32_t tiles_n = (p.n + kBN - 1) / kBN;
-    const uint32_t tm = blockIdx.x / tiles_n;
-    const uint32_t tn = blockIdx.x % tiles_n;
-    const uint32_t m0 = tm * kBM;
-    const uint32_t n0 = tn * kBN;
+    // ---- tile of this workgroup: ids that share an XCD (id mod 8) cover consecutive logical ids;
+    //      logical ids walk groups of 4 tile-rows column by column
+    const uint32_t tiles_m = (p.m + kBM - 1) / kBM, tiles_n = (p.n + kBN - 1) / kBN;
+    const uint32_t total = tiles_m * tiles_n;
+    const uint32_t per_xcd = (total + 7u) / 8u;
+    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    const uint32_t group = logical / (4u * tiles_n);
+    const uint32_t first_m = group * 4u;
+    const uint32_t group_rows = tiles_m - first_m < 4u ? tiles_m - first_m : 4u;
+    const uint32_t in_group = logical - group * 4u * tiles_n;
+    const uint32_t tm = first_m + in_group % group_rows;
+    const uint32_t tn = in_group / group_rows;
+    const uint32_t m0 = tm * kBM, n0 = tn * kBN;
 
-    // ---- A global -> LDS mapping: 4 chunks per thread, chunk id q = tid + 512*i
-    const uint16_t* a_src[4];
-    bool a_ok[4];
-    uint32_t a_dst[4];
+    // ---- buffer resources over this tile's rows of A and columns of B
+    const uint32_t rows_valid = p.m - m0 < (uint32_t)kBM ? p.m - m0 : (uint32_t)kBM;
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)(((rows_valid - 1u) * p.lda + p.k) * 2u), kBufferFlags);
+    const uint32_t cols_valid = p.n - n0 < (uint32_t)kBN ? p.n - n0 : (uint32_t)kBN;
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
+        kBufferFlags);
+
+    // A: chunk id q = tid + 512*i -> row (tid>>3) + 64*i, chunk tid&7
+    uint32_t a_voff[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t q = tid + 512u * i;
-        const uint32_t row = q >> 3, ch = q & 7u;
-        a_ok[i] = (m0 + row) < p.m;
-        a_src[i] = p.a + (size_t)(a_ok[i] ? (m0 + row) : 0) * p.lda + ch * 8u;
-        a_dst[i] = tile_off(row, ch);
+    for (uint32_t i = 0; i < 4; ++i) a_voff[i] = (((tid >> 3) + 64u * i) * p.lda + (tid & 7u) * 8u) * 2u;
+    const uint32_t a_dst = kAOff + swizzled_off(tid >> 3, tid & 7u);  // + 8192*i + stage*kTileBytes
+    // W: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
+    const uint32_t b_voff = BITS == 8 ? 4u * lane : 2u * lane;
+    const uint32_t w_dst = kWOff + swizzled_off((lane & 31u) + (lane >> 5) * 64u, wave);  // + (j&1)*4096 + (j>>1)*16384 + stage*kTileBytes
+    // fragment reads: row (lane&31) of a 32-row block, chunk 2*kk + lane/32
+    uint32_t a_rd[4], w_rd[4];
+#pragma unroll
+    for (uint32_t kk = 0; kk < 4; ++kk) {
+        const uint32_t x = swizzled_off(lane & 31u, 2u * kk + (lane >> 5));
+        a_rd[kk] = kAOff + wm * 16384u + x;  // + mt*4096 + stage*kTileBytes
+        w_rd[kk] = kWOff + wn * 8192u + x;   // + t*4096 + stage*kTileBytes
     }
 
-    // ---- W mapping: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
+    // ---- scales of this lane's 4 columns
     const uint32_t ncol = n0 + 4u * lane;
     const bool w_ok = ncol < p.n;
-    const uint8_t* b_src = p.b + (size_t)(8u * wave) * p.ldb_bytes + (BITS == 8 ? ncol : ncol / 2);
-    uint32_t w_dst[4];
-#pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) {
-        const uint32_t rho = (j >> 1) * 128u + (j & 1u) * 32u + (lane & 31u) + (lane >> 5) * 64u;
-        w_dst[j] = kTileBytes + tile_off(rho, wave);
-    }
-
     float cs[4];
     uint32_t cur_group = 0xffffffffu;
     auto fetch_scales = [&](uint32_t g) {
@@ -92,69 +118,50 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     };
     if constexpr (!GROUPED) fetch_scales(0);
 
-    uint4 a_reg[4];
+    u32x4_t a_reg[4];
     uint32_t b_reg[8];
+    const uint32_t ksteps = p.k / kBK;
 
-    auto gload = [&](uint32_t k0) {
+    // raw tile of K-step `kt` -> registers (kt is clamped by the callers, so every load is in range)
+    auto gload = [&](uint32_t kt) {
+        const uint32_t k0 = kt * (uint32_t)kBK;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            a_reg[i] = make_uint4(0, 0, 0, 0);
-            if (a_ok[i]) a_reg[i] = *reinterpret_cast<const uint4*>(a_src[i] + k0);
-        }
-        const uint8_t* bp = b_src + (size_t)k0 * p.ldb_bytes;
+        for (int i = 0; i < 4; ++i) a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, a_voff[i], k0 * 2u, 0);
+        const uint32_t row0 = (k0 + 8u * wave) * p.ldb_bytes;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            if constexpr (BITS == 8) {
-                b_reg[r] = 0x80808080u;
-                if (w_ok) b_reg[r] = *reinterpret_cast<const uint32_t*>(bp + (size_t)r * p.ldb_bytes);
-            } else {
-                b_reg[r] = 0x8888u;
-                if (w_ok) b_reg[r] = *reinterpret_cast<const uint16_t*>(bp + (size_t)r * p.ldb_bytes);
-            }
+        for (uint32_t r = 0; r < 8; ++r) {
+            if constexpr (BITS == 8) b_reg[r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
+            else b_reg[r] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
         }
     };
-
-    // signed value of column J (0..3) of a prepared row register (x16 for 4-bit codes)
-    auto value = [&](uint32_t x, auto jc) -> float {
-        constexpr int J = decltype(jc)::value;
-        return sbyte_to_f32<J>(x);
-    };
-    // stored codes of one row (4 columns) -> 4 two's-complement bytes, byte J = column J
-    auto prepare = [&](uint32_t x) -> uint32_t {
-        if constexpr (BITS == 8) {
-            return codes8_to_s8(x);
-        } else {
-            return codes4_quad_to_s8x16(x);
-        }
-    };
-
-    auto lds_store = [&](uint32_t stage, uint32_t k0) {
-        uint8_t* base = lds + stage * kStageBytes;
+    auto store_a = [&](auto stage_c) {
+        constexpr uint32_t S = decltype(stage_c)::value;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(base + a_dst[i]) = a_reg[i];
+        for (uint32_t i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(lds + a_dst + 8192u * i + S * kTileBytes) = a_reg[i];
+    };
+    // column J of the raw W registers -> bf16 -> LDS
+    auto store_w_col = [&](auto stage_c, auto j_c, const uint32_t (&b_s8)[8]) {
+        constexpr uint32_t S = decltype(stage_c)::value;
+        constexpr int J = decltype(j_c)::value;
+        uint4 w;
+        w.x = pack_bf16_rne(sbyte_to_f32<J>(b_s8[0]) * cs[J], sbyte_to_f32<J>(b_s8[1]) * cs[J]);
+        w.y = pack_bf16_rne(sbyte_to_f32<J>(b_s8[2]) * cs[J], sbyte_to_f32<J>(b_s8[3]) * cs[J]);
+        w.z = pack_bf16_rne(sbyte_to_f32<J>(b_s8[4]) * cs[J], sbyte_to_f32<J>(b_s8[5]) * cs[J]);
+        w.w = pack_bf16_rne(sbyte_to_f32<J>(b_s8[6]) * cs[J], sbyte_to_f32<J>(b_s8[7]) * cs[J]);
+        *reinterpret_cast<uint4*>(lds + w_dst + (J & 1) * 4096u + (J >> 1) * 16384u + S * kTileBytes) = w;
+    };
+    auto prepare = [&](uint32_t (&b_s8)[8]) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) b_s8[r] = BITS == 8 ? codes8_to_s8(b_reg[r]) : codes4_quad_to_s8x16(b_reg[r]);
+    };
+    auto update_scales = [&](uint32_t kt) {
         if constexpr (GROUPED) {
-            const uint32_t g = (k0 + 8u * wave) / p.group_size;
+            const uint32_t g = (kt * (uint32_t)kBK + 8u * wave) / p.group_size;
             if (g != cur_group) {
                 cur_group = g;
                 fetch_scales(g);
             }
         }
-        uint32_t b_s8[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r) b_s8[r] = prepare(b_reg[r]);
-        auto put = [&](auto jc) {
-            constexpr int J = decltype(jc)::value;
-            uint4 w;
-            w.x = pack_bf16_rne(value(b_s8[0], jc) * cs[J], value(b_s8[1], jc) * cs[J]);
-            w.y = pack_bf16_rne(value(b_s8[2], jc) * cs[J], value(b_s8[3], jc) * cs[J]);
-            w.z = pack_bf16_rne(value(b_s8[4], jc) * cs[J], value(b_s8[5], jc) * cs[J]);
-            w.w = pack_bf16_rne(value(b_s8[6], jc) * cs[J], value(b_s8[7], jc) * cs[J]);
-            *reinterpret_cast<uint4*>(base + w_dst[J]) = w;
-        };
-        put(std::integral_constant<int, 0>{});
-        put(std::integral_constant<int, 1>{});
-        put(std::integral_constant<int, 2>{});
-        put(std::integral_constant<int, 3>{});
     };
 
     f32x16_t acc[4][2];
@@ -165,52 +172,91 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
 
-    // fragment read offsets (chunk part added per kk)
-    const uint32_t frag_row_a = wm * 128u + (lane & 31u);
-    const uint32_t frag_row_w = wn * 64u + (lane & 31u);
-    const uint32_t frag_half = lane >> 5;
-
-    auto compute = [&](uint32_t stage) {
-        const uint8_t* base = lds + stage * kStageBytes;
+    auto read_frags = [&](auto stage_c, auto kk_c, bf16x8_t (&af)[4], bf16x8_t (&wf)[2]) {
+        constexpr uint32_t S = decltype(stage_c)::value;
+        constexpr uint32_t KK = decltype(kk_c)::value;
 #pragma unroll
-        for (uint32_t kk = 0; kk < 4; ++kk) {
-            bf16x8_t af[4], wf[2];
+        for (uint32_t mt = 0; mt < 4; ++mt) af[mt] = *reinterpret_cast<const bf16x8_t*>(lds + a_rd[KK] + mt * 4096u + S * kTileBytes);
 #pragma unroll
-            for (uint32_t mt = 0; mt < 4; ++mt)
-                af[mt] = *reinterpret_cast<const bf16x8_t*>(base + tile_off(frag_row_a + 32u * mt, 2u * kk + frag_half));
+        for (uint32_t t = 0; t < 2; ++t) wf[t] = *reinterpret_cast<const bf16x8_t*>(lds + w_rd[KK] + t * 4096u + S * kTileBytes);
+    };
+    auto mma = [&](const bf16x8_t (&af)[4], const bf16x8_t (&wf)[2]) {
 #pragma unroll
-            for (uint32_t t = 0; t < 2; ++t)
-                wf[t] = *reinterpret_cast<const bf16x8_t*>(base + kTileBytes + tile_off(frag_row_w + 32u * t, 2u * kk + frag_half));
+        for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mt], wf[t], acc[mt][t], 0, 0, 0);
-        }
+            for (int t = 0; t < 2; ++t) acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mt], wf[t], acc[mt][t], 0, 0, 0);
     };
 
-    const uint32_t ksteps = p.k / kBK;
-    gload(0);
-    lds_store(0, 0);
-    __syncthreads();
-    for (uint32_t kt = 0; kt < ksteps; ++kt) {
-        const uint32_t stage = kt & 1u;
-        const bool more = kt + 1 < ksteps;
-        if (more) gload((kt + 1) * kBK);
-        compute(stage);
-        if (more) lds_store(stage ^ 1u, (kt + 1) * kBK);
+    using C0 = std::integral_constant<uint32_t, 0>;
+    using C1 = std::integral_constant<uint32_t, 1>;
+    using C2 = std::integral_constant<uint32_t, 2>;
+    using C3 = std::integral_constant<uint32_t, 3>;
+    using J0 = std::integral_constant<int, 0>;
+    using J1 = std::integral_constant<int, 1>;
+    using J2 = std::integral_constant<int, 2>;
+    using J3 = std::integral_constant<int, 3>;
+
+    // One K-step: MFMAs on stage S; the raw tile in registers (step kt+1) goes to stage S^1;
+    // then the registers are refilled with step kt+2.
+    auto step = [&](auto stage_c, uint32_t kt) {
+        constexpr uint32_t S = decltype(stage_c)::value;
+        using Other = std::integral_constant<uint32_t, S ^ 1u>;
+        bf16x8_t af0[4], wf0[2], af1[4], wf1[2];
+        uint32_t b_s8[8];
+        read_frags(stage_c, C0{}, af0, wf0);
+        read_frags(stage_c, C1{}, af1, wf1);
+        mma(af0, wf0);
+        read_frags(stage_c, C2{}, af0, wf0);
+        mma(af1, wf1);
+        read_frags(stage_c, C3{}, af1, wf1);
+        // second half: convert and store the next tile between the MFMAs.  Nothing may be hoisted
+        // above this point: the raw tile's loads were issued at the end of the previous step and
+        // are still in flight during the first half.
+        __builtin_amdgcn_sched_barrier(0);
+        update_scales(kt + 1 < ksteps ? kt + 1 : kt);
+        store_a(Other{});
+        prepare(b_s8);
+        store_w_col(Other{}, J0{}, b_s8);
+        store_w_col(Other{}, J1{}, b_s8);
+        mma(af0, wf0);
+        store_w_col(Other{}, J2{}, b_s8);
+        store_w_col(Other{}, J3{}, b_s8);
+        mma(af1, wf1);
+        gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
         __syncthreads();
+    };
+
+    // ---- prologue: tile 0 -> stage 0, tile 1 -> registers
+    gload(0);
+    {
+        uint32_t b_s8[8];
+        update_scales(0);
+        store_a(C0{});
+        prepare(b_s8);
+        store_w_col(C0{}, J0{}, b_s8);
+        store_w_col(C0{}, J1{}, b_s8);
+        store_w_col(C0{}, J2{}, b_s8);
+        store_w_col(C0{}, J3{}, b_s8);
     }
+    gload(ksteps > 1 ? 1 : 0);
+    __syncthreads();
+
+    uint32_t kt = 0;
+    for (; kt + 1 < ksteps; kt += 2) {
+        step(C0{}, kt);
+        step(C1{}, kt + 1);
+    }
+    if (kt < ksteps) step(C0{}, kt);
 
     // ---- epilogue: bf16 tile through LDS, then 16-byte row-contiguous stores
     {
-        const uint32_t jl = lane & 31u;
+        const uint32_t jl = lane & 31u, half = lane >> 5;
         const uint32_t colbyte = 8u * (32u * (wn & 1u) + jl) + 4u * (wn >> 1);
 #pragma unroll
         for (uint32_t mt = 0; mt < 4; ++mt)
 #pragma unroll
             for (uint32_t i = 0; i < 16; ++i) {
-                const uint32_t row = wm * 128u + 32u * mt + 8u * (i >> 2) + 4u * frag_half + (i & 3u);
+                const uint32_t row = wm * 128u + 32u * mt + 8u * (i >> 2) + 4u * half + (i & 3u);
                 *reinterpret_cast<uint32_t*>(lds + row * kCRowBytes + colbyte) = pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
             }
     }
@@ -238,7 +284,8 @@ static hipError_t launch_prefill_t(const GemmParams& p, hipStream_t stream)
         attr_set = true;
     }
     const uint32_t tiles = ((p.m + kBM - 1) / kBM) * ((p.n + kBN - 1) / kBN);
-    return launch_kernel(bfaintb_prefill_kernel<BITS, GROUPED>, dim3(tiles, 1, 1), dim3(512, 1, 1), kLdsBytes, stream, p);
+    const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
+    return launch_kernel(bfaintb_prefill_kernel<BITS, GROUPED>, dim3(grid, 1, 1), dim3(512, 1, 1), kLdsBytes, stream, p);
 }
 
 hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream)
