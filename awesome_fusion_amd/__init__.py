@@ -17,6 +17,7 @@ from .gemm import (  # noqa: F401
     kernel_name,
     lib,
     library_path,
+    probe_read,
     split_k,
     variant,
     workspace_bytes,

@@ -14,6 +14,7 @@ hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_dequant(uint16_t* w, const uint8_t* b, const uint16_t* scale, uint32_t n, uint32_t k, uint32_t ldb_bytes,
                           uint32_t ldw, int bits, uint32_t group_size, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* dst, uint32_t count, uint32_t value, hipStream_t stream);
+hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, hipStream_t stream);
 }  // namespace bfaintb
 
 namespace {
@@ -23,8 +24,7 @@ using bfaintb::kCounterSlots;
 
 constexpr uint32_t kDecodeMaxM = 32;
 constexpr uint32_t kDecodeColsPerWg = 256;
-constexpr uint32_t kDecodeRowsPerWgUnit = 128;  // 4 waves x 32 rows
-constexpr uint32_t kDecodeTargetWgs = 512;      // two workgroups per CU on a 256-CU part
+constexpr uint32_t kDecodeTargetWgs = 480;      // a little under two workgroups per CU on a 256-CU part
 constexpr uint32_t kMaxSplits = 64;
 constexpr size_t kCounterBytes = (size_t)kCounterSlots * sizeof(uint32_t);
 
@@ -51,28 +51,42 @@ int resolve_variant(uint32_t m, int variant)
     return BFAINTB_ERR_BAD_VARIANT;
 }
 
-// Rows of k per workgroup and number of workgroups along k for the decode variant.
-void decode_split(uint32_t n, uint32_t k, uint32_t forced, uint32_t* k_per_wg, uint32_t* splits)
+// Launch shape of the decode variant: waves per workgroup, rows of k per workgroup, workgroups along k.
+struct DecodePlan {
+    uint32_t waves, k_per_wg, splits;
+};
+
+DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
 {
+    DecodePlan pl;
+    pl.waves = 4u;
+    const uint32_t unit = 32u * pl.waves;  // rows one workgroup covers per step of its waves
     const uint32_t col_blocks = (n + kDecodeColsPerWg - 1) / kDecodeColsPerWg;
-    const uint32_t max_splits = k / kDecodeRowsPerWgUnit ? k / kDecodeRowsPerWgUnit : 1;
-    uint32_t s = forced ? forced : (kDecodeTargetWgs + col_blocks - 1) / col_blocks;
-    if (s > max_splits) s = max_splits;
-    if (s > kMaxSplits) s = kMaxSplits;
-    if (s < 1) s = 1;
-    uint32_t per = (k + s - 1) / s;
-    per = (per + kDecodeRowsPerWgUnit - 1) / kDecodeRowsPerWgUnit * kDecodeRowsPerWgUnit;
-    *k_per_wg = per;
-    *splits = (k + per - 1) / per;
+    uint32_t splits = forced_splits;
+    if (splits == 0) {
+        // about kDecodeTargetWgs workgroups: close to two resident workgroups per CU, so that one
+        // workgroup's reduction and output overlap another's streaming ...
+        splits = (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
+        // ... while the split-K partial sums (written and read back as fp32) stay below a quarter of the weight bytes
+        uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (256u * (m ? m : 1u)));
+        if (cap < 1) cap = 1;
+        if (splits > cap) splits = cap;
+    }
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits < 1) splits = 1;
+    uint32_t per = (k + splits - 1) / splits;
+    per = (per + unit - 1) / unit * unit;
+    pl.k_per_wg = per;
+    pl.splits = (k + per - 1) / per;
+    return pl;
 }
 
-size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int variant, uint32_t forced_split)
+size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant, uint32_t forced_split)
 {
     if (variant != BFAINTB_VARIANT_DECODE || m == 0 || n == 0) return 0;
-    uint32_t per, splits;
-    decode_split(n, k, forced_split, &per, &splits);
-    if (splits <= 1) return 0;
-    return kCounterBytes + (size_t)splits * m * n * sizeof(float);
+    const DecodePlan pl = decode_plan(m, n, k, bits, forced_split);
+    if (pl.splits <= 1) return 0;
+    return kCounterBytes + (size_t)pl.splits * m * n * sizeof(float);
 }
 
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
@@ -112,9 +126,7 @@ int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, ui
 uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
 {
     if (bfaintb_gemm_variant(m, n, k, weight_bits, group_size) != BFAINTB_VARIANT_DECODE) return 1;
-    uint32_t per, splits;
-    decode_split(n, k, 0, &per, &splits);
-    return splits;
+    return decode_plan(m, n, k, weight_bits, 0).splits;
 }
 
 size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant,
@@ -123,7 +135,7 @@ size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int w
     if (check_format(k, weight_bits, group_size) || check_shape(m, n, k)) return 0;
     const int v = resolve_variant(m, variant);
     if (v < 0) return 0;
-    return workspace_need(m, n, k, v, split_k);
+    return workspace_need(m, n, k, weight_bits, v, split_k);
 }
 
 size_t bfaintb_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
@@ -177,7 +189,10 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
         return (int)bfaintb::launch_prefill(p, weight_bits, st);
     }
 
-    decode_split(n, k, split_k, &p.k_per_wg, &p.splits);
+    const DecodePlan pl = decode_plan(m, n, k, weight_bits, split_k);
+    p.k_per_wg = pl.k_per_wg;
+    p.splits = pl.splits;
+    p.decode_waves = pl.waves;
     if (p.splits > 1) {
         const size_t need = kCounterBytes + (size_t)p.splits * m * n * sizeof(float);
         if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
@@ -212,6 +227,15 @@ int bfaintb_dequant(void* w, const void* b, const void* scale, uint32_t n, uint3
     return (int)bfaintb::launch_dequant(static_cast<uint16_t*>(w), static_cast<const uint8_t*>(b),
                                         static_cast<const uint16_t*>(scale), n, k, weight_bits == 8 ? ldb : ldb / 2u, ldw,
                                         weight_bits, group_size, static_cast<hipStream_t>(stream));
+}
+
+int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream)
+{
+    if (bytes == 0) return BFAINTB_OK;
+    if (src == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    if (misaligned16(src)) return BFAINTB_ERR_ALIGNMENT;
+    if (bytes / 16 / 512 / 4 >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
+    return (int)bfaintb::launch_probe_read(src, bytes, sink, static_cast<hipStream_t>(stream));
 }
 
 const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m)

@@ -5,8 +5,8 @@
 // each MFMA at m = 1 and launches only n/64 workgroups with no split along k.
 //
 // Work decomposition
-//   grid  = (ceil(n/256), splits); block = 256 threads = 4 waves.
-//   A workgroup owns 256 consecutive columns and k_per_wg rows of B; each wave owns a quarter of
+//   grid  = (ceil(n/256), splits); block = 4 waves (the kernel itself accepts 4 or 8).
+//   A workgroup owns 256 consecutive columns and k_per_wg rows of B; each wave owns an equal share of
 //   those rows and walks them in steps of 32 rows.
 //   Within a wave, lane = (kg, nl) with nl = lane%16, kg = lane/16.  Per step the lane loads, from
 //   each of the 8 rows k0 + 8*kg + r, the 16 consecutive weights of columns n0 + 16*nl .. +15
@@ -17,7 +17,7 @@
 //   8-element operand of lane (nl, kg); the activations A[mi][k0 + 8*kg .. +7] of row mi = lane%16
 //   are the other operand, so one instruction multiplies 16 columns x 32 rows by up to 16 rows of A.
 //   Rows of A beyond m are zero operands.
-//   The 4 waves' partial sums are added through LDS; with splits > 1 each workgroup stores its
+//   The waves' partial sums are added through LDS; with splits > 1 each workgroup stores its
 //   fp32 partial tile to the workspace and the LAST workgroup to arrive at a column block (an
 //   arrival counter, no spinning) adds the partials in split order and writes bf16 C — the
 //   summation order is fixed, so results are reproducible run to run.
@@ -98,7 +98,15 @@ __device__ __forceinline__ void mac_step(const RawStep<BITS>& raw, const float (
     uint32_t rows[8][4];
 #pragma unroll
     for (int r = 0; r < 8; ++r) prepare_row<BITS>(rows[r], raw.d[r]);
+#if defined(BFAINTB_EXPERIMENT) && (BFAINTB_EXPERIMENT == 1 || BFAINTB_EXPERIMENT == 2)
+    // timing experiment: consume the loaded data without the dequantisation and MFMA work
+    uint32_t x = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) x ^= rows[r][0] ^ rows[r][1] ^ rows[r][2] ^ rows[r][3];
+    acc[0][0][0] += __uint_as_float(x & 0x3fffffffu) * cs[0] + __uint_as_float(afrag[0].x);
+#else
     (mac_column<BITS, MB, Cs>(rows, cs, afrag, acc), ...);
+#endif
 }
 
 template <int BITS>
@@ -128,9 +136,9 @@ __device__ __forceinline__ void apply_scales(float (&cs)[16], const uint4 (&sraw
 constexpr int kRedStride = 260;  // floats per row of the LDS reduction buffer (256 + 4: spreads rows over banks)
 
 template <int BITS, int MB, bool GROUPED>
-__global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
+__global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
 {
-    extern __shared__ __attribute__((aligned(16))) float red[];  // [4 waves][m rows][kRedStride], at least 4096 floats
+    extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][m rows][kRedStride], at least waves*1024 floats
     __shared__ uint32_t s_is_last;
 
     TRACE_MARK(0);
@@ -147,7 +155,8 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
     if (n_ld >= p.n) n_ld = p.n - 16u;
 
     // ---- this wave's rows of k
-    const uint32_t k_per_wave = p.k_per_wg >> 2;
+    const uint32_t nwaves = blockDim.x >> 6;  // 4 or 8
+    const uint32_t k_per_wave = p.k_per_wg / nwaves;
     const uint32_t kb = ks * p.k_per_wg + (uint32_t)wave * k_per_wave;
     uint32_t ke = kb + k_per_wave;
     if (ke > p.k) ke = p.k;
@@ -174,41 +183,56 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
         for (int c = 0; c < 16; ++c) acc[mb][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     if (nsteps > 0) {
-        // Software pipeline of depth one: the loads of step s+1 are issued before step s is
-        // computed.  Every load inside the loop is unconditional, so the wait counts the compiler
-        // derives are exact (a load behind a branch would make it wait for the prefetch as well);
-        // the last step, which has nothing to prefetch, is peeled off behind the loop.
-        RawStep<BITS> cur, nxt;
-        uint4 af_cur[MB], af_nxt[MB];
-        float cs[16];
-        uint4 sraw[2], sraw_nxt[2];
-        const uint16_t* sptr = p.scale + n_ld;
-        auto group_of = [&](int step) -> uint32_t {
-            if constexpr (GROUPED) return (kb + 32u * (uint32_t)step) / p.group_size;
-            return 0u;
+        // Two register stages, used alternately: the loads of step s+1 are issued before step s is
+        // computed.  Every load is unconditional and sits in straight-line code (the tail of one
+        // or two steps is peeled off behind the loop), so the wait counts the compiler derives are
+        // exact; a load behind a branch, or a stage copied into another, makes it wait for the
+        // prefetch as well.
+        struct Stage {
+            RawStep<BITS> raw;
+            uint4 af[MB];
+            uint4 sraw[2];
         };
-
-        load_scales<BITS>(sraw, sptr + (size_t)group_of(0) * p.lds);
-        load_raw<BITS>(cur, bptr, p.ldb_bytes);
+        float cs[16];
+        const uint16_t* sptr = p.scale + n_ld;
+        auto load_stage = [&](Stage& st, int step) {
+            load_raw<BITS>(st.raw, bptr + (size_t)step * bstep, p.ldb_bytes);
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) af_cur[mb] = *reinterpret_cast<const uint4*>(aptr[mb]);
-        apply_scales<BITS>(cs, sraw);
-
-        for (int s = 0; s + 1 < nsteps; ++s) {
-            load_raw<BITS>(nxt, bptr + (size_t)(s + 1) * bstep, p.ldb_bytes);
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) af_nxt[mb] = *reinterpret_cast<const uint4*>(aptr[mb] + (size_t)(s + 1) * 32);
-            if constexpr (GROUPED) load_scales<BITS>(sraw_nxt, sptr + (size_t)group_of(s + 1) * p.lds);
-            mac_step<BITS, MB>(cur, cs, af_cur, acc, std::make_integer_sequence<int, 16>{});
-            TRACE_MARK(1);
-            cur = nxt;
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) af_cur[mb] = af_nxt[mb];
-            if constexpr (GROUPED) apply_scales<BITS>(cs, sraw_nxt);
+            for (int mb = 0; mb < MB; ++mb) st.af[mb] = *reinterpret_cast<const uint4*>(aptr[mb] + (size_t)step * 32);
+            if constexpr (GROUPED) load_scales<BITS>(st.sraw, sptr + (size_t)((kb + 32u * (uint32_t)step) / p.group_size) * p.lds);
+            __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic that follows
+        };
+        auto compute_stage = [&](Stage& st) {
+            if constexpr (GROUPED) apply_scales<BITS>(cs, st.sraw);
+            mac_step<BITS, MB>(st.raw, cs, st.af, acc, std::make_integer_sequence<int, 16>{});
+        };
+        Stage s0, s1;
+        if constexpr (!GROUPED) {
+            load_scales<BITS>(s0.sraw, sptr);
         }
-        mac_step<BITS, MB>(cur, cs, af_cur, acc, std::make_integer_sequence<int, 16>{});
+        load_stage(s0, 0);
+        if constexpr (!GROUPED) apply_scales<BITS>(cs, s0.sraw);
+        int s = 0;
+        for (; s + 2 < nsteps; s += 2) {
+            load_stage(s1, s + 1);
+            compute_stage(s0);
+            load_stage(s0, s + 2);
+            compute_stage(s1);
+        }
+        if (nsteps - s == 2) {
+            load_stage(s1, s + 1);
+            compute_stage(s0);
+            compute_stage(s1);
+        } else {
+            compute_stage(s0);
+        }
     }
     TRACE_MARK(2);
+#if defined(BFAINTB_EXPERIMENT) && BFAINTB_EXPERIMENT == 2
+    // timing experiment: streaming phase only
+    if (acc[0][0][0] == 123.456f) p.c[threadIdx.x] = 1;
+    return;
+#endif
 
     // ---- add the 4 waves' partial sums through LDS: one barrier, then thread t finishes two
     //      neighbouring columns.  acc[mb][c][r] of lane (nl, kg) is row mi = 16*mb + nl,
@@ -233,14 +257,14 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
         const uint32_t cp = threadIdx.x & 127u, rsel = threadIdx.x >> 7;
         const uint32_t col = cb * 256u + 2u * cp;
         if (col < p.n) {
-            for (uint32_t row = rsel; row < rows_out; row += 2u) {
+            for (uint32_t row = rsel; row < rows_out; row += (blockDim.x >> 7)) {
                 const float* src = red + (size_t)row * kRedStride + 2u * cp;
-                const float2 w0 = *reinterpret_cast<const float2*>(src);
-                const float2 w1 = *reinterpret_cast<const float2*>(src + (size_t)rows_out * kRedStride);
-                const float2 w2 = *reinterpret_cast<const float2*>(src + (size_t)2 * rows_out * kRedStride);
-                const float2 w3 = *reinterpret_cast<const float2*>(src + (size_t)3 * rows_out * kRedStride);
-                const float sx = (w0.x + w1.x) + (w2.x + w3.x);
-                const float sy = (w0.y + w1.y) + (w2.y + w3.y);
+                float sx = 0.f, sy = 0.f;
+                for (uint32_t w = 0; w < nwaves; ++w) {  // fixed order: wave 0 first
+                    const float2 v = *reinterpret_cast<const float2*>(src + (size_t)w * rows_out * kRedStride);
+                    sx += v.x;
+                    sy += v.y;
+                }
                 if (p.splits == 1) {
                     *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col) = pack_bf16_rne(sx, sy);
                 } else {
@@ -254,6 +278,9 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
         }
     }
     if (p.splits == 1) return;
+#if defined(BFAINTB_EXPERIMENT) && BFAINTB_EXPERIMENT == 4
+    return;  // timing experiment: partial stores only
+#endif
 
     // ---- split-K: the last workgroup to arrive at this column block adds all partial tiles in a
     // fixed order and writes C.
@@ -265,25 +292,29 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
     }
     __syncthreads();
     if (s_is_last == 0u) return;
+#if defined(BFAINTB_EXPERIMENT) && BFAINTB_EXPERIMENT == 3
+    if (threadIdx.x == 0) __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;  // timing experiment: no final reduction
+#endif
     // acquire at device scope: drops lines of the partial tiles this XCD's L2 may still hold from an
     // earlier launch, so the plain (vectorisable, pipelined) loads below see the other workgroups' stores
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
-    // thread t: 4 consecutive columns (cg = t%64), splits sp = sub, sub+4, ... (sub = t/64), rows in
-    // chunks of 4; the four sub-sums are combined through LDS in a fixed order
+    // thread t: 4 consecutive columns (cg = t%64), splits sp = sub, sub+waves, ... (sub = t/64), rows
+    // in chunks of 4; the per-wave sub-sums are combined through LDS in a fixed order
     {
         const uint32_t cg = threadIdx.x & 63u, sub = threadIdx.x >> 6;
         const uint32_t col = cb * 256u + 4u * cg;
         const bool col_ok = col < p.n;
         __syncthreads();               // every wave is done reading its sums out of red
-        float* stage = red;            // [4 subs][4 rows][256 cols] = 4096 floats
+        float* stage = red;            // [waves][4 rows][256 cols]
         for (uint32_t m0 = 0; m0 < p.m; m0 += 4u) {
             const uint32_t rows = p.m - m0 < 4u ? p.m - m0 : 4u;
             for (uint32_t ri = 0; ri < rows; ++ri) {
                 float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (col_ok) {
                     const float* src = p.partials + (size_t)(m0 + ri) * p.n + col;
-                    for (uint32_t sp = sub; sp < p.splits; sp += 4u) {
+                    for (uint32_t sp = sub; sp < p.splits; sp += nwaves) {
                         const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sp * p.m * p.n);
                         sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
                     }
@@ -294,13 +325,14 @@ __global__ void __launch_bounds__(256) bfaintb_decode_kernel(const GemmParams p)
             {
                 const uint32_t ri = sub;  // thread t finishes row t/64 of the chunk
                 if (ri < rows && col_ok) {
-                    const float4 s0 = *reinterpret_cast<const float4*>(stage + (0u * 4u + ri) * 256u + 4u * cg);
-                    const float4 s1 = *reinterpret_cast<const float4*>(stage + (1u * 4u + ri) * 256u + 4u * cg);
-                    const float4 s2 = *reinterpret_cast<const float4*>(stage + (2u * 4u + ri) * 256u + 4u * cg);
-                    const float4 s3 = *reinterpret_cast<const float4*>(stage + (3u * 4u + ri) * 256u + 4u * cg);
+                    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                    for (uint32_t w = 0; w < nwaves; ++w) {
+                        const float4 v = *reinterpret_cast<const float4*>(stage + (w * 4u + ri) * 256u + 4u * cg);
+                        t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+                    }
                     uint2 o;
-                    o.x = pack_bf16_rne((s0.x + s1.x) + (s2.x + s3.x), (s0.y + s1.y) + (s2.y + s3.y));
-                    o.y = pack_bf16_rne((s0.z + s1.z) + (s2.z + s3.z), (s0.w + s1.w) + (s2.w + s3.w));
+                    o.x = pack_bf16_rne(t.x, t.y);
+                    o.y = pack_bf16_rne(t.z, t.w);
                     *reinterpret_cast<uint2*>(p.c + (size_t)(m0 + ri) * p.ldc + col) = o;
                 }
             }
@@ -314,8 +346,9 @@ template <int BITS, int MB, bool GROUPED>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
     const dim3 grid((p.n + 255u) / 256u, p.splits, 1);
-    size_t lds = (size_t)4 * p.m * kRedStride * sizeof(float);
-    if (lds < 4096 * sizeof(float)) lds = 4096 * sizeof(float);
+    const uint32_t waves = p.decode_waves;
+    size_t lds = (size_t)waves * p.m * kRedStride * sizeof(float);
+    if (lds < (size_t)waves * 1024 * sizeof(float)) lds = (size_t)waves * 1024 * sizeof(float);
     if (lds > 64 * 1024) {
         static bool attr_set = false;
         if (!attr_set) {
@@ -325,7 +358,7 @@ static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
             attr_set = true;
         }
     }
-    return launch_kernel(bfaintb_decode_kernel<BITS, MB, GROUPED>, grid, dim3(256, 1, 1), lds, stream, p);
+    return launch_kernel(bfaintb_decode_kernel<BITS, MB, GROUPED>, grid, dim3(64 * waves, 1, 1), lds, stream, p);
 }
 
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)

@@ -71,6 +71,34 @@ __global__ void __launch_bounds__(256) bfaintb_fill_u32_kernel(uint32_t* dst, ui
     if (i < count) dst[i] = value;
 }
 
+// Measurement aid: reads `n16` 16-byte words with the widest coalesced loads (a wave reads 8 KiB in
+// 8 loads issued back to back) and throws them away.  Its time is what this GPU needs merely to
+// fetch that many bytes in one kernel launch: the practical ceiling for a weight-streaming GEMV.
+__global__ void __launch_bounds__(256) bfaintb_probe_read_kernel(const uint4* __restrict__ src, uint32_t* sink, size_t n16)
+{
+    const size_t wave = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const size_t base = wave * 512 + (threadIdx.x & 63);
+    uint4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const size_t idx = base + (size_t)i * 64;
+        v[i] = idx < n16 ? src[idx] : make_uint4(0, 0, 0, 0);
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (x == 0x9e3779b9u && sink != nullptr) sink[threadIdx.x & 63] = x;  // practically never: keeps the loads alive
+}
+
+hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, hipStream_t stream)
+{
+    const size_t n16 = bytes / 16;
+    const size_t waves = (n16 + 511) / 512;
+    const uint32_t grid = (uint32_t)((waves + 3) / 4);
+    return launch_kernel(bfaintb_probe_read_kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, static_cast<const uint4*>(src),
+                         static_cast<uint32_t*>(sink), n16);
+}
+
 hipError_t launch_fill_u32(uint32_t* dst, uint32_t count, uint32_t value, hipStream_t stream)
 {
     return launch_kernel(bfaintb_fill_u32_kernel, dim3((count + 255u) / 256u, 1, 1), dim3(256, 1, 1), 0, stream, dst, count, value);

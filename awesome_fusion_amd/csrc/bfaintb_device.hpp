@@ -38,7 +38,8 @@ struct GemmParams {
     uint32_t lds;        // elements per scale row (= n)
     uint32_t group_size; // rows of k per scale group; 0 = one group
     // split-K (decode variant only)
-    uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 128)
+    uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_waves)
+    uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)
     uint32_t splits;     // workgroups along k
     float* partials;     // [splits][m][n] fp32
     uint32_t* counters;  // [column blocks]

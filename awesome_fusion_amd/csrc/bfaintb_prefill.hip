@@ -27,9 +27,11 @@
 //   goes to LDS row rho = (j>>1)*128 + (j&1)*32 + (lane&31) + (lane>>5)*64, so consecutive lanes
 //   write consecutive rows.  The MFMA "column" index is the LDS row: wave wn, accumulator t, lane
 //   column jl hold tile column 4*(32*(wn&1) + jl) + 2*(wn>>1) + t.
-// Pipeline per step (registers hold the raw tile of step+1, loaded one step earlier): MFMAs of the
-//   current stage; the raw tile is converted and written to the other stage in the second half of
-//   the step, between MFMAs; then the loads for step+2 are issued; barrier.
+// Pipeline per step (registers hold the raw tile of step+1, loaded one step earlier): the 32 MFMAs
+//   of the current stage run in four quarters; the raw tile is converted and written to the other
+//   stage between the MFMAs of the second and third quarter, the registers it frees are refilled
+//   with step+2 at once, and the barrier sits before the last quarter so that the first fragments
+//   of the next stage are fetched behind those MFMAs.
 // Epilogue: accumulators are rounded to bf16 (v_cvt_pk_bf16_f32; t = 0,1 are neighbouring columns
 //   and share a dword), staged in LDS in true [m][n] order and stored with 16-byte row-contiguous writes.
 #include <utility>
@@ -196,34 +198,77 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     using J2 = std::integral_constant<int, 2>;
     using J3 = std::integral_constant<int, 3>;
 
-    // One K-step: MFMAs on stage S; the raw tile in registers (step kt+1) goes to stage S^1;
-    // then the registers are refilled with step kt+2.
+    // One K-step in four quarters of 8 MFMAs (stage S is current, O = S^1 receives step kt+1, whose
+    // raw tile sits in a_reg/b_reg; fragments are double-buffered in f0/f1; on entry f0 holds kk=0):
+    //   Q1  MFMA kk=0 (f0)          | LDS reads kk=1 -> f1
+    //   Q2  MFMA kk=1 (f1)          | LDS reads kk=2 -> f0; A registers -> LDS(O); raw W -> signed bytes;
+    //                                 buffer loads of step kt+2 into the freed registers; W columns 0,1 -> LDS(O)
+    //   Q3  MFMA kk=2 (f0)          | LDS reads kk=3 -> f1; W columns 2,3 -> LDS(O)
+    //   barrier                       (every wave has filled O)
+    //   Q4  MFMA kk=3 (f1)          | LDS reads kk=0 of O -> f0 for the next step
+    // The raw tile is loaded a full step before it is used, and the first fragments of the next
+    // stage are fetched behind the last 8 MFMAs of this one.
+    bf16x8_t af0[4], wf0[2], af1[4], wf1[2];
     auto step = [&](auto stage_c, uint32_t kt) {
         constexpr uint32_t S = decltype(stage_c)::value;
         using Other = std::integral_constant<uint32_t, S ^ 1u>;
-        bf16x8_t af0[4], wf0[2], af1[4], wf1[2];
         uint32_t b_s8[8];
-        read_frags(stage_c, C0{}, af0, wf0);
+        // Q1
         read_frags(stage_c, C1{}, af1, wf1);
         mma(af0, wf0);
-        read_frags(stage_c, C2{}, af0, wf0);
-        mma(af1, wf1);
-        read_frags(stage_c, C3{}, af1, wf1);
-        // second half: convert and store the next tile between the MFMAs.  Nothing may be hoisted
-        // above this point: the raw tile's loads were issued at the end of the previous step and
-        // are still in flight during the first half.
         __builtin_amdgcn_sched_barrier(0);
+        // Q2
+        read_frags(stage_c, C2{}, af0, wf0);
         update_scales(kt + 1 < ksteps ? kt + 1 : kt);
         store_a(Other{});
         prepare(b_s8);
+        gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
         store_w_col(Other{}, J0{}, b_s8);
         store_w_col(Other{}, J1{}, b_s8);
-        mma(af0, wf0);
+        mma(af1, wf1);
+        // interleave: 4 x {MFMA, A write, 2 xor}, the 12 buffer loads, then per W column 2 x {MFMA, 10 VALU} and its write
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x020, 12, 0);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // Q3
+        read_frags(stage_c, C3{}, af1, wf1);
         store_w_col(Other{}, J2{}, b_s8);
         store_w_col(Other{}, J3{}, b_s8);
-        mma(af1, wf1);
-        gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
+        mma(af0, wf0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
         __syncthreads();
+        // Q4
+        read_frags(Other{}, C0{}, af0, wf0);
+        mma(af1, wf1);
     };
 
     // ---- prologue: tile 0 -> stage 0, tile 1 -> registers
@@ -240,6 +285,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     }
     gload(ksteps > 1 ? 1 : 0);
     __syncthreads();
+    read_frags(C0{}, C0{}, af0, wf0);
 
     uint32_t kt = 0;
     for (; kt + 1 < ksteps; kt += 2) {
@@ -247,6 +293,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         step(C1{}, kt + 1);
     }
     if (kt < ksteps) step(C0{}, kt);
+    __syncthreads();  // the last step's fragment prefetch has read LDS: done before the epilogue overwrites it
 
     // ---- epilogue: bf16 tile through LDS, then 16-byte row-contiguous stores
     {

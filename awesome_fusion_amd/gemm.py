@@ -67,6 +67,8 @@ def lib():
         L.bfaintb_gemm_split_k.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
         L.bfaintb_dequant.restype = C.c_int
         L.bfaintb_dequant.argtypes = [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
+        L.bfaintb_probe_read.restype = C.c_int
+        L.bfaintb_probe_read.argtypes = [_vp, C.c_size_t, _vp, _vp]
         L.bfaintb_kernel_name.restype = C.c_char_p
         L.bfaintb_kernel_name.argtypes = [C.c_int, C.c_int, _u32, _u32]
         L.bfaintb_error_string.restype = C.c_char_p
@@ -145,3 +147,12 @@ def dequant(w, b, scale, n, k, ldb=None, ldw=None, weight_bits=8, group_size=0, 
     if rc and check:
         raise BfaintbError(rc, "bfaintb_dequant")
     return rc
+
+
+def probe_read(src, nbytes=None, stream=None):
+    """Streams a buffer through the GPU and discards it (measurement aid: the fetch-only ceiling)."""
+    if nbytes is None:
+        nbytes = src.numel() * src.element_size()
+    rc = lib().bfaintb_probe_read(_ptr(src), nbytes, None, _stream_handle(stream))
+    if rc:
+        raise BfaintbError(rc, "bfaintb_probe_read")

@@ -107,6 +107,27 @@ def time_graph(af, w, steps, warmup, rotate):
     return e0.elapsed_time(e1) / steps, (t1 - t0) * 1e3 / steps
 
 
+def time_read_ceiling(af, w, steps, warmup):
+    """The same rotation of B copies through a kernel that only fetches the bytes."""
+    import torch
+    nb = len(w.b)
+    for i in range(warmup):
+        af.probe_read(w.b[i % nb])
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(steps):
+            af.probe_read(w.b[i % nb])
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
 def time_eager(af, w, steps, warmup):
     """The reference protocol: launches in a loop inside one event pair, no graph."""
     import torch
@@ -224,6 +245,7 @@ def main():
         ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True)
         hot_ms, _ = time_graph(af, w, K, W, rotate=False)
         eager_ms = time_eager(af, w, K, W)
+        read_ms = time_read_ceiling(af, w, K, W)
         c_gpu = w.c.float().cpu().numpy()
         res = {
             "metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=1: effective HBM bandwidth (algorithmic bytes / time per launch, B cold)",
@@ -236,6 +258,10 @@ def main():
             "roofline": roofline_entry(w, ev_ms, "hbm"),
         }
         res["tflops"] = round(w.flops / (wall_ms * 1e-3) / 1e12, 4)
+        b_bytes = w.b[0].numel()
+        res["roofline"]["fetch_only_kernel_us"] = round(read_ms * 1e3, 3)
+        res["roofline"]["fetch_only_GBps"] = round(b_bytes / read_ms / 1e6, 1)
+        res["roofline"]["frac_of_fetch_only"] = round(read_ms / ev_ms, 4)
         out_extra["decode_m1_hot_same_buffer"] = {"kernel_us": round(hot_ms * 1e3, 3), "GB/s": round(w.bytes / hot_ms / 1e6, 1),
                                                   "note": "B re-read from cache: not an HBM figure"}
         out_extra["decode_m1_eager_launch_loop"] = {"us_per_launch": round(eager_ms * 1e3, 3),

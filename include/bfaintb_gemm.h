@@ -114,6 +114,13 @@ BFAINTB_API uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, in
 BFAINTB_API int bfaintb_dequant(void* w, const void* b, const void* scale, uint32_t n, uint32_t k, uint32_t ldb, uint32_t ldw,
                     int weight_bits, uint32_t group_size, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: reads `bytes` bytes from src with fully
+ * coalesced 16-byte loads and discards them (sink may be NULL).  Timing it on the same buffers as the
+ * decode GEMM gives the time this GPU needs just to fetch the weights in one launch.
+ */
+BFAINTB_API int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream);
+
 /* Name of the __global__ function a variant launches for (weight_bits, group_size, m), as it
  * appears in a kernel trace. */
 BFAINTB_API const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m);
