@@ -35,7 +35,12 @@ LLC_BYTES = 256 << 20
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # fetch 8449.2 KiB x 1.997 + write 272.5 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
+    "decode_m1_n4096_k4096_int8_perchannel": 17557045,
+    # fetch 66957.3 KiB x 1.997 + write 35328.0 KiB
+    "prefill_m4096_n4096_k4096_int8_perchannel": 173098729,
+}
 
 
 def algorithmic_bytes(m, n, k, bits, group):
