@@ -27,6 +27,8 @@ constexpr uint32_t kDecodeColsPerWg = 256;
 constexpr uint32_t kDecodeTargetWgs = 480;      // a little under two workgroups per CU on a 256-CU part
 constexpr uint32_t kMaxSplits = 64;
 constexpr size_t kCounterBytes = (size_t)kCounterSlots * sizeof(uint32_t);
+constexpr size_t kHeaderBytes = 2 * kCounterBytes;  // arrival counters, then epochs
+constexpr size_t kSlotBytes = 8;                    // {fp32 partial sum, uint32 tag}
 
 int check_format(uint32_t k, int bits, uint32_t group_size)
 {
@@ -86,7 +88,7 @@ size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant,
     if (variant != BFAINTB_VARIANT_DECODE || m == 0 || n == 0) return 0;
     const DecodePlan pl = decode_plan(m, n, k, bits, forced_split);
     if (pl.splits <= 1) return 0;
-    return kCounterBytes + (size_t)pl.splits * m * n * sizeof(float);
+    return kHeaderBytes + (size_t)pl.splits * m * n * kSlotBytes;
 }
 
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
@@ -147,9 +149,10 @@ int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream
 {
     if (workspace == nullptr || workspace_bytes == 0) return BFAINTB_OK;
     if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
-    if (workspace_bytes < kCounterBytes) return BFAINTB_ERR_WORKSPACE;
+    if (workspace_bytes < kHeaderBytes || workspace_bytes / 4 >= (1ull << 32)) return BFAINTB_ERR_WORKSPACE;
+    // the whole workspace is cleared (counters, epochs and the tagged slots: tag 0 is never used by a launch);
     // a fill kernel rather than hipMemsetAsync, so the call may be recorded into a HIP graph
-    return (int)bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)kCounterSlots, 0u,
+    return (int)bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)(workspace_bytes / 4), 0u,
                                          static_cast<hipStream_t>(stream));
 }
 
@@ -194,14 +197,15 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     p.splits = pl.splits;
     p.decode_waves = pl.waves;
     if (p.splits > 1) {
-        const size_t need = kCounterBytes + (size_t)p.splits * m * n * sizeof(float);
+        const size_t need = kHeaderBytes + (size_t)p.splits * m * n * kSlotBytes;
         if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
         if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
         p.counters = static_cast<uint32_t*>(workspace);
-        p.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kCounterBytes);
+        p.epochs = p.counters + kCounterSlots;
+        p.partials = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + kHeaderBytes);
     }
 #ifdef BFAINTB_TRACE
-    if (workspace != nullptr) p.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kCounterBytes);  // timestamp sink
+    if (workspace != nullptr) p.partials = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + kHeaderBytes);  // timestamp sink
 #endif
     return (int)bfaintb::launch_decode(p, weight_bits, st);
 }

@@ -19,8 +19,8 @@
 //   Rows of A beyond m are zero operands.
 //   The waves' partial sums are added through LDS; with splits > 1 each workgroup stores its
 //   fp32 partial tile to the workspace and the LAST workgroup to arrive at a column block (an
-//   arrival counter, no spinning) adds the partials in split order and writes bf16 C — the
-//   summation order is fixed, so results are reproducible run to run.
+//   arrival counter; nobody waits for another workgroup) adds the partials in split order and writes
+//   bf16 C — the summation order is fixed, so results are reproducible run to run.
 #include <utility>
 #include "bfaintb_device.hpp"
 
@@ -128,11 +128,13 @@ __device__ __forceinline__ void apply_scales(float (&cs)[16], const uint4 (&sraw
 }
 
 #ifdef BFAINTB_TRACE
-#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) reinterpret_cast<unsigned long long*>(p.partials)[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
+#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) p.partials[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
 #else
 #define TRACE_MARK(i) do { } while (0)
 #endif
 
+constexpr uint32_t kTaggedMaxM = 4;         // up to this m split-K partial sums travel in tagged slots
+constexpr uint32_t kMaxSlotRetries = 1u << 16;  // re-reads of a split-K slot before giving up (each is a memory round trip)
 constexpr int kRedStride = 260;  // floats per row of the LDS reduction buffer (256 + 4: spreads rows over banks)
 
 template <int BITS, int MB, bool GROUPED>
@@ -148,6 +150,17 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
     const int kg = lane >> 4;
     const uint32_t cb = blockIdx.x;
     const uint32_t ks = blockIdx.y;
+
+    // tag of this launch's split-K slots: one more than the column block's stored epoch, which the
+    // last workgroup of the previous launch on this workspace left behind (read early, used late)
+    const bool tagged = p.m <= kTaggedMaxM;
+    // The tag carries the column block too, so that no two (column block, launch) pairs on one
+    // workspace share a tag, whatever shapes the launches had.
+    uint32_t epoch = 0, tag = 0;
+    if (p.splits > 1) {
+        epoch = __hip_atomic_load(p.epochs + cb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        tag = ((epoch & 0xfffffu) << 12) | cb;  // cb < 4096
+    }
 
     // ---- this lane's 16 weight columns.  A lane past the last column reads the last 16 columns
     //      instead (no predicated loads in the hot loop); what it computes is never stored.
@@ -268,23 +281,34 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
                 if (p.splits == 1) {
                     *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col) = pack_bf16_rne(sx, sy);
                 } else {
-                    // split-K partial tile, written with a device-scope (write-through) store: no L2
-                    // write-back is needed before announcing arrival, only the store's acknowledgement
-                    const unsigned long long bits = (unsigned long long)__float_as_uint(sx) | ((unsigned long long)__float_as_uint(sy) << 32);
-                    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p.partials + ((size_t)ks * p.m + row) * p.n + col), bits,
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    // split-K partial sums go to 8-byte slots {value, tag}, written whole with device-scope
+                    // (write-through) stores that nobody waits for: the reader recognises a slot of this
+                    // launch by its tag
+                    if (tagged) {
+                        unsigned long long* slot = p.partials + ((size_t)ks * p.m + row) * p.n + col;
+                        __hip_atomic_store(slot, (unsigned long long)__float_as_uint(sx) | ((unsigned long long)tag << 32), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(slot + 1, (unsigned long long)__float_as_uint(sy) | ((unsigned long long)tag << 32), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    } else {
+                        // larger m: plain fp32 partials (half the bytes, 16-byte loads for the reader); the
+                        // arrival count then has to wait for the stores' acknowledgement
+                        __hip_atomic_store(reinterpret_cast<unsigned long long*>(reinterpret_cast<float*>(p.partials) + ((size_t)ks * p.m + row) * p.n + col),
+                                           (unsigned long long)__float_as_uint(sx) | ((unsigned long long)__float_as_uint(sy) << 32), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
             }
         }
     }
     if (p.splits == 1) return;
-#if defined(BFAINTB_EXPERIMENT) && BFAINTB_EXPERIMENT == 4
-    return;  // timing experiment: partial stores only
-#endif
-
     // ---- split-K: the last workgroup to arrive at this column block adds all partial tiles in a
-    // fixed order and writes C.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt vmcnt(0): this wave's stores are acknowledged
+    // fixed order and writes C.  The arrival count is bumped as soon as this workgroup's stores have
+    // been ISSUED (the barrier), not acknowledged: a slot whose store is still in flight shows an old
+    // tag and is simply read again.  That wait is on memory operations already under way, never on
+    // another workgroup being scheduled, so it cannot deadlock.  (For m > kTaggedMaxM the partials are
+    // untagged and the count waits for the acknowledgements instead.)
+    if (!tagged) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt vmcnt(0)
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t arrived = __hip_atomic_fetch_add(p.counters + cb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -296,6 +320,8 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
     if (threadIdx.x == 0) __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;  // timing experiment: no final reduction
 #endif
+
+    if (!tagged) {
     // acquire at device scope: drops lines of the partial tiles this XCD's L2 may still hold from an
     // earlier launch, so the plain (vectorisable, pipelined) loads below see the other workgroups' stores
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -313,7 +339,7 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
             for (uint32_t ri = 0; ri < rows; ++ri) {
                 float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (col_ok) {
-                    const float* src = p.partials + (size_t)(m0 + ri) * p.n + col;
+                    const float* src = reinterpret_cast<const float*>(p.partials) + (size_t)(m0 + ri) * p.n + col;
                     for (uint32_t sp = sub; sp < p.splits; sp += nwaves) {
                         const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sp * p.m * p.n);
                         sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
@@ -339,7 +365,42 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
             __syncthreads();
         }
     }
-    if (threadIdx.x == 0) __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    } else {
+    // thread t owns column cb*256 + t: all splits of a row are fetched together (device-scope loads,
+    // which bypass whatever this XCD's L2 holds from an earlier launch), then added in split order
+        const uint32_t col = cb * 256u + threadIdx.x;
+        constexpr uint32_t kBatch = 16;
+        if (threadIdx.x < 256u && col < p.n) {
+            for (uint32_t mi = 0; mi < p.m; ++mi) {
+                const unsigned long long* src = p.partials + (size_t)mi * p.n + col;
+                const size_t stride = (size_t)p.m * p.n;
+                float sum = 0.f;
+                for (uint32_t sp0 = 0; sp0 < p.splits; sp0 += kBatch) {
+                    unsigned long long v[kBatch];
+#pragma unroll
+                    for (uint32_t i = 0; i < kBatch; ++i) {
+                        const uint32_t sp = sp0 + i < p.splits ? sp0 + i : p.splits - 1u;
+                        v[i] = __hip_atomic_load(src + (size_t)sp * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (uint32_t i = 0; i < kBatch; ++i) {
+                        if (sp0 + i < p.splits) {
+                            // store still in flight: read the slot again (bounded, so the kernel ends whatever happens;
+                            // a slot that never shows its tag poisons the output with a NaN instead of hanging)
+                            for (uint32_t tries = 0; (uint32_t)(v[i] >> 32) != tag && tries < kMaxSlotRetries; ++tries)
+                                v[i] = __hip_atomic_load(src + (size_t)(sp0 + i) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            sum += (uint32_t)(v[i] >> 32) == tag ? __uint_as_float((uint32_t)v[i]) : __uint_as_float(0x7fc00000u);
+                        }
+                    }
+                }
+                p.c[(size_t)mi * p.ldc + col] = (uint16_t)(pack_bf16_rne(sum, 0.f) & 0xffffu);
+            }
+        }
+    }
+    if (threadIdx.x == 0) {  // ready for the next launch: new tag, counter back to zero
+        __hip_atomic_store(p.epochs + cb, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 template <int BITS, int MB, bool GROUPED>

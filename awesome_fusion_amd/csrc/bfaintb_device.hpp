@@ -41,8 +41,9 @@ struct GemmParams {
     uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_waves)
     uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)
     uint32_t splits;     // workgroups along k
-    float* partials;     // [splits][m][n] fp32
-    uint32_t* counters;  // [column blocks]
+    unsigned long long* partials;  // [splits][m][n] slots of {fp32 value, uint32 tag}
+    uint32_t* counters;  // [column blocks] arrivals of the running launch (zero at rest)
+    uint32_t* epochs;    // [column blocks] tag of the last finished launch
 };
 
 // Launch through hipLaunchKernel so that the error returned belongs to THIS launch:

@@ -90,13 +90,13 @@ BFAINTB_API int bfaintb_gemm_ex(void* c, const void* a, const void* b, const voi
                     uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k);
 
-/* Scratch the GEMM needs for a shape: split-K partial sums and arrival counters.  Depends only on
+/* Scratch the GEMM needs for a shape: tagged split-K partial sums, arrival counters and epochs.  Depends only on
  * its arguments.  The reference kernel has no scratch (no split-K, bfAintBGemm.cc:107-109). */
 BFAINTB_API size_t bfaintb_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 BFAINTB_API size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
                                        int variant, uint32_t split_k);
 
-/* Clears the arrival counters at the head of a freshly allocated workspace (stream-ordered). */
+/* Clears a freshly allocated workspace: arrival counters, epochs and partial-sum slots (stream-ordered). */
 BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */

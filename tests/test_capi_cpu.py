@@ -35,8 +35,8 @@ def test_variant_choice_and_split():
     assert af.split_k(4096, 4096, 4096) == 1
     s = af.split_k(1, 4096, 4096)
     assert 1 < s <= 64 and 4096 % s == 0
-    # workspace = counters + splits * m * n fp32; none for the prefill variant
-    assert af.workspace_bytes(1, 4096, 4096) == 4096 * 4 + s * 1 * 4096 * 4
+    # workspace = counters + epochs + splits * m * n tagged 8-byte slots; none for the prefill variant
+    assert af.workspace_bytes(1, 4096, 4096) == 2 * 4096 * 4 + s * 1 * 4096 * 8
     assert af.workspace_bytes(4096, 4096, 4096) == 0
     assert af.workspace_bytes(8, 4096, 4096, force_split_k=1) == 0
     assert af.kernel_name(1) == "bfaintb_decode_kernel" and af.kernel_name(4096) == "bfaintb_prefill_kernel"
