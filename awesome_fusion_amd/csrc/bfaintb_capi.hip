@@ -189,6 +189,9 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     if (v == BFAINTB_VARIANT_PREFILL) {
         // the prefill kernel addresses B and a 256-row panel of A through 32-bit buffer extents
         if ((uint64_t)k * p.ldb_bytes >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
+#ifdef BFAINTB_TRACE
+        p.partials = static_cast<unsigned long long*>(workspace);  // per-quarter cycle totals, 8 words per wave
+#endif
         return (int)bfaintb::launch_prefill(p, weight_bits, st);
     }
 

@@ -41,9 +41,7 @@ namespace bfaintb {
 
 constexpr int kBM = 256, kBN = 256, kBK = 64;
 constexpr uint32_t kTileBytes = 256 * 128;              // one A or W tile in LDS
-constexpr uint32_t kAOff = 0, kWOff = 2 * kTileBytes;   // LDS: A stage 0, A stage 1, W stage 0, W stage 1
-constexpr int kCRowBytes = 256 * 2 + 16;                // epilogue staging row (padded)
-constexpr int kLdsBytes = 256 * kCRowBytes;             // 135168 >= 4 tiles (131072)
+constexpr int kCRowBytes = 256 * 2;                     // epilogue staging row: 64 rows fill one 32 KiB tile array
 constexpr int kBufferFlags = 0x00027000;                // raw buffer, 32-bit data format
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -56,7 +54,15 @@ __device__ __forceinline__ uint32_t swizzled_off(uint32_t row, uint32_t chunk)
 template <int BITS, bool GROUPED>
 __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // Four separate LDS arrays (A and W tiles, two stages each) rather than one block: the compiler
+    // then knows that fragment reads of one stage cannot alias the asynchronous global->LDS writes
+    // into the other, and does not make them wait for those writes.
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_w0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_w1[kTileBytes];
+    auto a_tile = [&](auto stage_c) -> uint8_t* { return decltype(stage_c)::value == 0 ? lds_a0 : lds_a1; };
+    auto w_tile = [&](auto stage_c) -> uint8_t* { return decltype(stage_c)::value == 0 ? lds_w0 : lds_w1; };
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -88,21 +94,25 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
         kBufferFlags);
 
-    // A: chunk id q = tid + 512*i -> row (tid>>3) + 64*i, chunk tid&7
+    // A goes global -> LDS directly (buffer_load_dwordx4 ... lds): instruction j of wave w fills the 1 KiB
+    // of rows 32w + 8j .. +7; lane l lands at byte 16*l of it, i.e. row 32w + 8j + l/8, chunk POSITION l%8,
+    // so the lane fetches the chunk that the swizzle puts there: chunk (l%8) ^ ((row >> 1) & 7).
     uint32_t a_voff[4];
 #pragma unroll
-    for (uint32_t i = 0; i < 4; ++i) a_voff[i] = (((tid >> 3) + 64u * i) * p.lda + (tid & 7u) * 8u) * 2u;
-    const uint32_t a_dst = kAOff + swizzled_off(tid >> 3, tid & 7u);  // + 8192*i + stage*kTileBytes
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t row = 32u * wave + 8u * j + (lane >> 3);
+        a_voff[j] = (row * p.lda + (((lane & 7u) ^ ((row >> 1) & 7u)) * 8u)) * 2u;
+    }
     // W: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
     const uint32_t b_voff = BITS == 8 ? 4u * lane : 2u * lane;
-    const uint32_t w_dst = kWOff + swizzled_off((lane & 31u) + (lane >> 5) * 64u, wave);  // + (j&1)*4096 + (j>>1)*16384 + stage*kTileBytes
+    const uint32_t w_dst = swizzled_off((lane & 31u) + (lane >> 5) * 64u, wave);  // + (j&1)*4096 + (j>>1)*16384
     // fragment reads: row (lane&31) of a 32-row block, chunk 2*kk + lane/32
     uint32_t a_rd[4], w_rd[4];
 #pragma unroll
     for (uint32_t kk = 0; kk < 4; ++kk) {
         const uint32_t x = swizzled_off(lane & 31u, 2u * kk + (lane >> 5));
-        a_rd[kk] = kAOff + wm * 16384u + x;  // + mt*4096 + stage*kTileBytes
-        w_rd[kk] = kWOff + wn * 8192u + x;   // + t*4096 + stage*kTileBytes
+        a_rd[kk] = wm * 16384u + x;  // + mt*4096
+        w_rd[kk] = wn * 8192u + x;   // + t*4096
     }
 
     // ---- scales of this lane's 4 columns
@@ -120,37 +130,35 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     };
     if constexpr (!GROUPED) fetch_scales(0);
 
-    u32x4_t a_reg[4];
     uint32_t b_reg[8];
     const uint32_t ksteps = p.k / kBK;
 
-    // raw tile of K-step `kt` -> registers (kt is clamped by the callers, so every load is in range)
-    auto gload = [&](uint32_t kt) {
-        const uint32_t k0 = kt * (uint32_t)kBK;
+    // A tile of K-step `kt` -> LDS stage (asynchronous; counted by vmcnt like any other load)
+    auto dma_a = [&](auto stage_c, uint32_t kt) {
+        uint8_t* base = a_tile(stage_c) + wave * 4096u;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, a_voff[i], k0 * 2u, 0);
-        const uint32_t row0 = (k0 + 8u * wave) * p.ldb_bytes;
+        for (uint32_t j = 0; j < 4; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
+                                                     a_voff[j], kt * (uint32_t)kBK * 2u, 0, 0);
+    };
+    // raw W codes of K-step `kt` -> registers (kt is clamped by the callers, so every load is in range)
+    auto gload = [&](uint32_t kt) {
+        const uint32_t row0 = (kt * (uint32_t)kBK + 8u * wave) * p.ldb_bytes;
 #pragma unroll
         for (uint32_t r = 0; r < 8; ++r) {
             if constexpr (BITS == 8) b_reg[r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
             else b_reg[r] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
         }
     };
-    auto store_a = [&](auto stage_c) {
-        constexpr uint32_t S = decltype(stage_c)::value;
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) *reinterpret_cast<u32x4_t*>(lds + a_dst + 8192u * i + S * kTileBytes) = a_reg[i];
-    };
     // column J of the raw W registers -> bf16 -> LDS
     auto store_w_col = [&](auto stage_c, auto j_c, const uint32_t (&b_s8)[8]) {
-        constexpr uint32_t S = decltype(stage_c)::value;
         constexpr int J = decltype(j_c)::value;
         uint4 w;
         w.x = pack_bf16_rne(sbyte_to_f32<J>(b_s8[0]) * cs[J], sbyte_to_f32<J>(b_s8[1]) * cs[J]);
         w.y = pack_bf16_rne(sbyte_to_f32<J>(b_s8[2]) * cs[J], sbyte_to_f32<J>(b_s8[3]) * cs[J]);
         w.z = pack_bf16_rne(sbyte_to_f32<J>(b_s8[4]) * cs[J], sbyte_to_f32<J>(b_s8[5]) * cs[J]);
         w.w = pack_bf16_rne(sbyte_to_f32<J>(b_s8[6]) * cs[J], sbyte_to_f32<J>(b_s8[7]) * cs[J]);
-        *reinterpret_cast<uint4*>(lds + w_dst + (J & 1) * 4096u + (J >> 1) * 16384u + S * kTileBytes) = w;
+        *reinterpret_cast<uint4*>(w_tile(stage_c) + w_dst + (J & 1) * 4096u + (J >> 1) * 16384u) = w;
     };
     auto prepare = [&](uint32_t (&b_s8)[8]) {
 #pragma unroll
@@ -175,12 +183,11 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
 
     auto read_frags = [&](auto stage_c, auto kk_c, bf16x8_t (&af)[4], bf16x8_t (&wf)[2]) {
-        constexpr uint32_t S = decltype(stage_c)::value;
         constexpr uint32_t KK = decltype(kk_c)::value;
 #pragma unroll
-        for (uint32_t mt = 0; mt < 4; ++mt) af[mt] = *reinterpret_cast<const bf16x8_t*>(lds + a_rd[KK] + mt * 4096u + S * kTileBytes);
+        for (uint32_t mt = 0; mt < 4; ++mt) af[mt] = *reinterpret_cast<const bf16x8_t*>(a_tile(stage_c) + a_rd[KK] + mt * 4096u);
 #pragma unroll
-        for (uint32_t t = 0; t < 2; ++t) wf[t] = *reinterpret_cast<const bf16x8_t*>(lds + w_rd[KK] + t * 4096u + S * kTileBytes);
+        for (uint32_t t = 0; t < 2; ++t) wf[t] = *reinterpret_cast<const bf16x8_t*>(w_tile(stage_c) + w_rd[KK] + t * 4096u);
     };
     auto mma = [&](const bf16x8_t (&af)[4], const bf16x8_t (&wf)[2]) {
 #pragma unroll
@@ -209,47 +216,51 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     // The raw tile is loaded a full step before it is used, and the first fragments of the next
     // stage are fetched behind the last 8 MFMAs of this one.
     bf16x8_t af0[4], wf0[2], af1[4], wf1[2];
+#ifdef BFAINTB_TRACE
+    long long tq[5] = {0, 0, 0, 0, 0};
+#define PF_MARK(i) do { const long long now_ = clock64(); tq[i] += now_ - tlast; tlast = now_; } while (0)
+    long long tlast = clock64();
+#else
+#define PF_MARK(i) do { } while (0)
+#endif
     auto step = [&](auto stage_c, uint32_t kt) {
         constexpr uint32_t S = decltype(stage_c)::value;
         using Other = std::integral_constant<uint32_t, S ^ 1u>;
         uint32_t b_s8[8];
         // Q1
+        dma_a(Other{}, kt + 1 < ksteps ? kt + 1 : kt);
         read_frags(stage_c, C1{}, af1, wf1);
         mma(af0, wf0);
         __builtin_amdgcn_sched_barrier(0);
+        PF_MARK(0);
         // Q2
         read_frags(stage_c, C2{}, af0, wf0);
         update_scales(kt + 1 < ksteps ? kt + 1 : kt);
-        store_a(Other{});
         prepare(b_s8);
         gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
         store_w_col(Other{}, J0{}, b_s8);
         store_w_col(Other{}, J1{}, b_s8);
         mma(af1, wf1);
-        // interleave: 4 x {MFMA, A write, 2 xor}, the 12 buffer loads, then per W column 2 x {MFMA, 10 VALU} and its write
+        // interleave: 2 x {MFMA, 4 xor, 3 LDS reads}, the 8 buffer loads, then per W column 3 x {MFMA, 7 VALU} and its write
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
         }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x020, 12, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
+        PF_MARK(1);
         // Q3
         read_frags(stage_c, C3{}, af1, wf1);
         store_w_col(Other{}, J2{}, b_s8);
@@ -265,18 +276,23 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             }
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
+        PF_MARK(2);
+        // this wave's part of the next A tile has landed in LDS (the 8 W loads issued after it may still fly)
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         __syncthreads();
+        PF_MARK(3);
         // Q4
         read_frags(Other{}, C0{}, af0, wf0);
         mma(af1, wf1);
+        PF_MARK(4);
     };
 
-    // ---- prologue: tile 0 -> stage 0, tile 1 -> registers
+    // ---- prologue: tile 0 -> stage 0, raw W of tile 1 -> registers
+    dma_a(C0{}, 0);
     gload(0);
     {
         uint32_t b_s8[8];
         update_scales(0);
-        store_a(C0{});
         prepare(b_s8);
         store_w_col(C0{}, J0{}, b_s8);
         store_w_col(C0{}, J1{}, b_s8);
@@ -284,6 +300,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         store_w_col(C0{}, J3{}, b_s8);
     }
     gload(ksteps > 1 ? 1 : 0);
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     __syncthreads();
     read_frags(C0{}, C0{}, af0, wf0);
 
@@ -293,28 +310,37 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         step(C1{}, kt + 1);
     }
     if (kt < ksteps) step(C0{}, kt);
-    __syncthreads();  // the last step's fragment prefetch has read LDS: done before the epilogue overwrites it
 
-    // ---- epilogue: bf16 tile through LDS, then 16-byte row-contiguous stores
+#ifdef BFAINTB_TRACE
+    if (lane == 0 && p.partials != nullptr)
+        for (int i = 0; i < 5; ++i) p.partials[(size_t)(blockIdx.x * 8 + wave) * 8 + i] = (unsigned long long)tq[i];
+#endif
+    // ---- epilogue: bf16 tile through LDS (rows 64q..64q+63 in the q-th of the four arrays), then
+    //      16-byte row-contiguous stores
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
+    __syncthreads();
+    auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_w0 : lds_w1; };
     {
         const uint32_t jl = lane & 31u, half = lane >> 5;
         const uint32_t colbyte = 8u * (32u * (wn & 1u) + jl) + 4u * (wn >> 1);
 #pragma unroll
-        for (uint32_t mt = 0; mt < 4; ++mt)
+        for (uint32_t mt = 0; mt < 4; ++mt) {
+            uint8_t* base = c_rows(wm * 2u + (mt >> 1));
 #pragma unroll
             for (uint32_t i = 0; i < 16; ++i) {
-                const uint32_t row = wm * 128u + 32u * mt + 8u * (i >> 2) + 4u * half + (i & 3u);
-                *reinterpret_cast<uint32_t*>(lds + row * kCRowBytes + colbyte) = pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                const uint32_t row = 32u * (mt & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) = pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
             }
+        }
     }
     __syncthreads();
-#pragma unroll 4
+#pragma unroll
     for (uint32_t pass = 0; pass < 16; ++pass) {
         const uint32_t row = pass * 16u + (tid >> 5);
         const uint32_t ch = tid & 31u;
         const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
         if (gm < p.m && gn < p.n) {
-            const uint4 v = *reinterpret_cast<const uint4*>(lds + row * kCRowBytes + ch * 16u);
+            const uint4 v = *reinterpret_cast<const uint4*>(c_rows(pass >> 2) + (row & 63u) * kCRowBytes + ch * 16u);
             *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) = v;
         }
     }
@@ -323,16 +349,9 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 template <int BITS, bool GROUPED>
 static hipError_t launch_prefill_t(const GemmParams& p, hipStream_t stream)
 {
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_prefill_kernel<BITS, GROUPED>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
     const uint32_t tiles = ((p.m + kBM - 1) / kBM) * ((p.n + kBN - 1) / kBN);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    return launch_kernel(bfaintb_prefill_kernel<BITS, GROUPED>, dim3(grid, 1, 1), dim3(512, 1, 1), kLdsBytes, stream, p);
+    return launch_kernel(bfaintb_prefill_kernel<BITS, GROUPED>, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
 }
 
 hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream)
