@@ -4,6 +4,7 @@
 // (gpu_utils.hpp:5-11, print and exit(0)) every failure is returned to the caller.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "bfaintb_device.hpp"
 #include "../../include/bfaintb_gemm.h"
@@ -20,15 +21,12 @@ hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, hipStrea
 namespace {
 
 using bfaintb::GemmParams;
-using bfaintb::kCounterSlots;
+using bfaintb::kEmptyWord;
 
 constexpr uint32_t kDecodeMaxM = 32;
-constexpr uint32_t kDecodeColsPerWg = 256;
-constexpr uint32_t kDecodeTargetWgs = 480;      // a little under two workgroups per CU on a 256-CU part
+constexpr uint32_t kDecodeTargetWgs = 480;        // 4-wave workgroups: a little under two per CU on a 256-CU part
+constexpr uint32_t kDecodeTargetWgsNarrow = 256;  // 8-wave workgroups: one per CU
 constexpr uint32_t kMaxSplits = 64;
-constexpr size_t kCounterBytes = (size_t)kCounterSlots * sizeof(uint32_t);
-constexpr size_t kHeaderBytes = 2 * kCounterBytes;  // arrival counters, then epochs
-constexpr size_t kSlotBytes = 8;                    // {fp32 partial sum, uint32 tag}
 
 int check_format(uint32_t k, int bits, uint32_t group_size)
 {
@@ -41,7 +39,6 @@ int check_shape(uint32_t m, uint32_t n, uint32_t k)
 {
     if (k == 0 || n % 16u != 0 || k % 64u != 0) return BFAINTB_ERR_BAD_SHAPE;
     if (m >= (1u << 31) || n >= (1u << 31) || k >= (1u << 31)) return BFAINTB_ERR_BAD_SHAPE;
-    if ((n + kDecodeColsPerWg - 1) / kDecodeColsPerWg > (uint32_t)kCounterSlots) return BFAINTB_ERR_BAD_SHAPE;
     return BFAINTB_OK;
 }
 
@@ -53,22 +50,39 @@ int resolve_variant(uint32_t m, int variant)
     return BFAINTB_ERR_BAD_VARIANT;
 }
 
-// Launch shape of the decode variant: waves per workgroup, rows of k per workgroup, workgroups along k.
+// Launch shape of the decode variant: columns and waves per workgroup, rows of k per workgroup, workgroups along k.
 struct DecodePlan {
-    uint32_t waves, k_per_wg, splits;
+    uint32_t cols, waves, k_per_wg, splits;
 };
 
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
 {
     DecodePlan pl;
-    pl.waves = 4u;
-    const uint32_t unit = 32u * pl.waves;  // rows one workgroup covers per step of its waves
-    const uint32_t col_blocks = (n + kDecodeColsPerWg - 1) / kDecodeColsPerWg;
+    // 8-bit codes, 128 columns x 8 waves (a lane loads 8 bytes of a row, 16 lanes one 128-byte line): half
+    // the splits, so half the partial-sum traffic, for the same number of waves.  Measured faster than the
+    // wide block while the weights are few (the launch is latency-bound) and for the m where the partial
+    // sums weigh most; large weight matrices stream better in 256-byte row segments.
+    // Otherwise, and for 4-bit codes: 256 columns x 4 waves.
+    const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
+    const bool few = weight_bytes <= (32ull << 20);
+    const bool narrow = bits == 8 && (few || (m >= 8 && m <= 16));
+    pl.cols = narrow ? 128u : 256u;
+    pl.waves = narrow ? 8u : 4u;
+    uint32_t target = narrow ? (few ? kDecodeTargetWgsNarrow : kDecodeTargetWgsNarrow * 3u / 2u) : kDecodeTargetWgs;
+#ifdef BFAINTB_TUNE
+    if (const char* e = getenv("BFAINTB_DECODE_COLS")) {
+        if (atoi(e) == 256) { pl.cols = 256u; pl.waves = 4u; target = kDecodeTargetWgs; }
+    }
+    if (const char* e = getenv("BFAINTB_DECODE_WAVES")) pl.waves = (uint32_t)atoi(e);
+    if (const char* e = getenv("BFAINTB_DECODE_TARGET")) target = (uint32_t)atoi(e);
+#endif
+    // rows one workgroup covers per pipeline step of its waves
+    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16) * pl.waves;
+    const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
     uint32_t splits = forced_splits;
     if (splits == 0) {
-        // about kDecodeTargetWgs workgroups: close to two resident workgroups per CU, so that one
-        // workgroup's reduction and output overlap another's streaming ...
-        splits = (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
+        // about `target` workgroups: enough waves on every CU to keep the memory system busy ...
+        splits = (target + col_blocks / 2) / col_blocks;
         // ... while the split-K partial sums (written and read back as fp32) stay below a quarter of the weight bytes
         uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (256u * (m ? m : 1u)));
         if (cap < 1) cap = 1;
@@ -88,7 +102,8 @@ size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant,
     if (variant != BFAINTB_VARIANT_DECODE || m == 0 || n == 0) return 0;
     const DecodePlan pl = decode_plan(m, n, k, bits, forced_split);
     if (pl.splits <= 1) return 0;
-    return kHeaderBytes + (size_t)pl.splits * m * n * kSlotBytes;
+    // one fp32 word per (split but the last, row, column), rounded up to 256 bytes
+    return (((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u;
 }
 
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
@@ -149,10 +164,10 @@ int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream
 {
     if (workspace == nullptr || workspace_bytes == 0) return BFAINTB_OK;
     if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
-    if (workspace_bytes < kHeaderBytes || workspace_bytes / 4 >= (1ull << 32)) return BFAINTB_ERR_WORKSPACE;
-    // the whole workspace is cleared (counters, epochs and the tagged slots: tag 0 is never used by a launch);
-    // a fill kernel rather than hipMemsetAsync, so the call may be recorded into a HIP graph
-    return (int)bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)(workspace_bytes / 4), 0u,
+    if (workspace_bytes % 4 != 0 || workspace_bytes / 4 >= (1ull << 32)) return BFAINTB_ERR_WORKSPACE;
+    // every word becomes "no partial sum here"; a fill kernel rather than hipMemsetAsync, so that the
+    // call may be recorded into a HIP graph
+    return (int)bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)(workspace_bytes / 4), kEmptyWord,
                                          static_cast<hipStream_t>(stream));
 }
 
@@ -190,7 +205,7 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
         // the prefill kernel addresses B and a 256-row panel of A through 32-bit buffer extents
         if ((uint64_t)k * p.ldb_bytes >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
 #ifdef BFAINTB_TRACE
-        p.partials = static_cast<unsigned long long*>(workspace);  // per-quarter cycle totals, 8 words per wave
+        p.trace = static_cast<unsigned long long*>(workspace);  // per-quarter cycle totals, 8 words per wave
 #endif
         return (int)bfaintb::launch_prefill(p, weight_bits, st);
     }
@@ -199,16 +214,16 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     p.k_per_wg = pl.k_per_wg;
     p.splits = pl.splits;
     p.decode_waves = pl.waves;
+    p.decode_cols = pl.cols;
     if (p.splits > 1) {
-        const size_t need = kHeaderBytes + (size_t)p.splits * m * n * kSlotBytes;
+        const size_t need = workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k);
         if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
         if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
-        p.counters = static_cast<uint32_t*>(workspace);
-        p.epochs = p.counters + kCounterSlots;
-        p.partials = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + kHeaderBytes);
+        p.partials = static_cast<unsigned long long*>(workspace);
     }
 #ifdef BFAINTB_TRACE
-    if (workspace != nullptr) p.partials = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + kHeaderBytes);  // timestamp sink
+    // timestamp sink: behind the split-K area (instrumented callers pass a larger workspace)
+    p.trace = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + ((workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) + 255) & ~(size_t)255));
 #endif
     return (int)bfaintb::launch_decode(p, weight_bits, st);
 }

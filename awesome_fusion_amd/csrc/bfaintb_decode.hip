@@ -5,36 +5,37 @@
 // each MFMA at m = 1 and launches only n/64 workgroups with no split along k.
 //
 // Work decomposition
-//   grid  = (ceil(n/256), splits); block = 4 waves (the kernel itself accepts 4 or 8).
-//   A workgroup owns 256 consecutive columns and k_per_wg rows of B; each wave owns an equal share of
+//   grid  = (ceil(n/COLS), splits); block = 4 or 8 waves.  CPL = weights per lane and row (16 or 8),
+//   COLS = 16*CPL columns per workgroup (256 or 128).
+//   A workgroup owns COLS consecutive columns and k_per_wg rows of B; each wave owns an equal share of
 //   those rows and walks them in steps of 32 rows.
 //   Within a wave, lane = (kg, nl) with nl = lane%16, kg = lane/16.  Per step the lane loads, from
-//   each of the 8 rows k0 + 8*kg + r, the 16 consecutive weights of columns n0 + 16*nl .. +15
-//   (one 128-bit load per row for 8-bit codes, one 64-bit load for 4-bit codes): a wave request
-//   covers 4 rows x 256 contiguous bytes (8-bit).  Nothing of B goes through LDS.
+//   each of the 8 rows k0 + 8*kg + r, the CPL consecutive weights of columns n0 + CPL*nl .. +CPL-1
+//   (128-bit or 64-bit loads): a wave request covers 4 rows x 16 lanes of contiguous bytes, whole
+//   128-byte lines or more.  Nothing of B goes through LDS.
 //   The products run on v_mfma_f32_16x16x32_bf16 with the operands swapped (C^T = W^T A^T): for
-//   c = 0..15 the dequantised weights of column 16*nl + c, rows 8*kg..8*kg+7, are exactly the
+//   c = 0..CPL-1 the dequantised weights of column CPL*nl + c, rows 8*kg..8*kg+7, are exactly the
 //   8-element operand of lane (nl, kg); the activations A[mi][k0 + 8*kg .. +7] of row mi = lane%16
 //   are the other operand, so one instruction multiplies 16 columns x 32 rows by up to 16 rows of A.
-//   Rows of A beyond m are zero operands.
-//   The waves' partial sums are added through LDS; with splits > 1 each workgroup stores its
-//   fp32 partial tile to the workspace and the LAST workgroup to arrive at a column block (an
-//   arrival counter; nobody waits for another workgroup) adds the partials in split order and writes
-//   bf16 C — the summation order is fixed, so results are reproducible run to run.
+//   Rows of A beyond m re-read row m-1; their results are never stored.
+//   The waves' partial sums are added through LDS; with splits > 1 the partial tiles of a column
+//   block meet in the workspace and the workgroup of the last split adds them in split order and
+//   writes bf16 C — the summation order is fixed, so results are reproducible run to run.  The narrower block (CPL = 8)
+//   needs half the splits for the same number of workgroups, i.e. half the partial-sum traffic.
 #include <utility>
 #include "bfaintb_device.hpp"
 
 namespace bfaintb {
 
-template <int BITS>
+template <int BITS, int CPL>
 struct RawStep {
-    static constexpr int kDwords = BITS == 8 ? 4 : 2;
-    uint32_t d[8][kDwords];  // 8 rows x 16 codes
+    static constexpr int kDwords = CPL * BITS / 32;  // 4 or 2
+    uint32_t d[8][kDwords];  // 8 rows x CPL codes
 };
 
-// Signed value of column C (0..15) of one prepared row, as fp32 (x16 for 4-bit codes).
-template <int BITS, int C>
-__device__ __forceinline__ float value_f32(const uint32_t (&row)[4])
+// Signed value of column C (0..CPL-1) of one prepared row, as fp32 (x16 for 4-bit codes).
+template <int BITS, int C, int PD>
+__device__ __forceinline__ float value_f32(const uint32_t (&row)[PD])
 {
     if constexpr (BITS == 8) {
         return sbyte_to_f32<C % 4>(row[C / 4]);
@@ -45,12 +46,12 @@ __device__ __forceinline__ float value_f32(const uint32_t (&row)[4])
     }
 }
 
-template <int BITS>
-__device__ __forceinline__ void load_raw(RawStep<BITS>& raw, const uint8_t* rowptr, uint32_t ldb_bytes)
+template <int BITS, int CPL>
+__device__ __forceinline__ void load_raw(RawStep<BITS, CPL>& raw, const uint8_t* rowptr, uint32_t ldb_bytes)
 {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-        if constexpr (BITS == 8) {
+        if constexpr (RawStep<BITS, CPL>::kDwords == 4) {
             const uint4 v = *reinterpret_cast<const uint4*>(rowptr + (size_t)r * ldb_bytes);
             raw.d[r][0] = v.x; raw.d[r][1] = v.y; raw.d[r][2] = v.z; raw.d[r][3] = v.w;
         } else {
@@ -60,14 +61,15 @@ __device__ __forceinline__ void load_raw(RawStep<BITS>& raw, const uint8_t* rowp
     }
 }
 
-// Stored codes of one row -> four dwords of two's-complement bytes.
-template <int BITS>
-__device__ __forceinline__ void prepare_row(uint32_t (&out)[4], const uint32_t (&in)[RawStep<BITS>::kDwords])
+// Stored codes of one row -> CPL/4 dwords of two's-complement bytes.
+template <int BITS, int CPL>
+__device__ __forceinline__ void prepare_row(uint32_t (&out)[CPL / 4], const uint32_t (&in)[RawStep<BITS, CPL>::kDwords])
 {
     if constexpr (BITS == 8) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = codes8_to_s8(in[i]);
+        for (int i = 0; i < CPL / 4; ++i) out[i] = codes8_to_s8(in[i]);
     } else {
+        static_assert(BITS == 8 || CPL == 16, "4-bit codes: 16 columns per lane");
         out[0] = codes4_even_to_s8x16(in[0]);
         out[1] = codes4_odd_to_s8x16(in[0]);
         out[2] = codes4_even_to_s8x16(in[1]);
@@ -75,15 +77,16 @@ __device__ __forceinline__ void prepare_row(uint32_t (&out)[4], const uint32_t (
     }
 }
 
-template <int BITS, int MB, int C>
-__device__ __forceinline__ void mac_column(const uint32_t (&rows)[8][4], const float (&cs)[16], const uint4 (&afrag)[MB],
-                                           f32x4_t (&acc)[MB][16])
+template <int BITS, int CPL, int MB, int C>
+__device__ __forceinline__ void mac_column(const uint32_t (&rows)[8][CPL / 4], const float (&cs)[CPL], const uint4 (&afrag)[MB],
+                                           f32x4_t (&acc)[MB][CPL])
 {
+    constexpr int PD = CPL / 4;
     uint4 w;
-    w.x = pack_bf16_rne(value_f32<BITS, C>(rows[0]) * cs[C], value_f32<BITS, C>(rows[1]) * cs[C]);
-    w.y = pack_bf16_rne(value_f32<BITS, C>(rows[2]) * cs[C], value_f32<BITS, C>(rows[3]) * cs[C]);
-    w.z = pack_bf16_rne(value_f32<BITS, C>(rows[4]) * cs[C], value_f32<BITS, C>(rows[5]) * cs[C]);
-    w.w = pack_bf16_rne(value_f32<BITS, C>(rows[6]) * cs[C], value_f32<BITS, C>(rows[7]) * cs[C]);
+    w.x = pack_bf16_rne(value_f32<BITS, C, PD>(rows[0]) * cs[C], value_f32<BITS, C, PD>(rows[1]) * cs[C]);
+    w.y = pack_bf16_rne(value_f32<BITS, C, PD>(rows[2]) * cs[C], value_f32<BITS, C, PD>(rows[3]) * cs[C]);
+    w.z = pack_bf16_rne(value_f32<BITS, C, PD>(rows[4]) * cs[C], value_f32<BITS, C, PD>(rows[5]) * cs[C]);
+    w.w = pack_bf16_rne(value_f32<BITS, C, PD>(rows[6]) * cs[C], value_f32<BITS, C, PD>(rows[7]) * cs[C]);
     const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, w);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -91,57 +94,138 @@ __device__ __forceinline__ void mac_column(const uint32_t (&rows)[8][4], const f
     }
 }
 
-template <int BITS, int MB, int... Cs>
-__device__ __forceinline__ void mac_step(const RawStep<BITS>& raw, const float (&cs)[16], const uint4 (&afrag)[MB],
-                                         f32x4_t (&acc)[MB][16], std::integer_sequence<int, Cs...>)
+template <int BITS, int CPL, int MB, int... Cs>
+__device__ __forceinline__ void mac_step(const RawStep<BITS, CPL>& raw, const float (&cs)[CPL], const uint4 (&afrag)[MB],
+                                         f32x4_t (&acc)[MB][CPL], std::integer_sequence<int, Cs...>)
 {
-    uint32_t rows[8][4];
+    uint32_t rows[8][CPL / 4];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) prepare_row<BITS>(rows[r], raw.d[r]);
-#if defined(BFAINTB_EXPERIMENT) && (BFAINTB_EXPERIMENT == 1 || BFAINTB_EXPERIMENT == 2)
-    // timing experiment: consume the loaded data without the dequantisation and MFMA work
-    uint32_t x = 0;
-#pragma unroll
-    for (int r = 0; r < 8; ++r) x ^= rows[r][0] ^ rows[r][1] ^ rows[r][2] ^ rows[r][3];
-    acc[0][0][0] += __uint_as_float(x & 0x3fffffffu) * cs[0] + __uint_as_float(afrag[0].x);
-#else
-    (mac_column<BITS, MB, Cs>(rows, cs, afrag, acc), ...);
-#endif
+    for (int r = 0; r < 8; ++r) prepare_row<BITS, CPL>(rows[r], raw.d[r]);
+    (mac_column<BITS, CPL, MB, Cs>(rows, cs, afrag, acc), ...);
 }
 
-template <int BITS>
-__device__ __forceinline__ void load_scales(uint4 (&sraw)[2], const uint16_t* sptr)
+template <int CPL>
+__device__ __forceinline__ void load_scales(uint4 (&sraw)[CPL / 8], const uint16_t* sptr)
 {
-    sraw[0] = *reinterpret_cast<const uint4*>(sptr);
-    sraw[1] = *reinterpret_cast<const uint4*>(sptr + 8);
+#pragma unroll
+    for (int i = 0; i < CPL / 8; ++i) sraw[i] = *reinterpret_cast<const uint4*>(sptr + 8 * i);
 }
 
-template <int BITS>
-__device__ __forceinline__ void apply_scales(float (&cs)[16], const uint4 (&sraw)[2])
+template <int BITS, int CPL>
+__device__ __forceinline__ void apply_scales(float (&cs)[CPL], const uint4 (&sraw)[CPL / 8])
 {
-    const uint32_t d[8] = {sraw[0].x, sraw[0].y, sraw[0].z, sraw[0].w, sraw[1].x, sraw[1].y, sraw[1].z, sraw[1].w};
+    uint32_t d[CPL / 2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < CPL / 8; ++i) {
+        d[4 * i] = sraw[i].x; d[4 * i + 1] = sraw[i].y; d[4 * i + 2] = sraw[i].z; d[4 * i + 3] = sraw[i].w;
+    }
+#pragma unroll
+    for (int i = 0; i < CPL / 2; ++i) {
         cs[2 * i] = make_col_scale<BITS>(d[i] & 0xffffu);
         cs[2 * i + 1] = make_col_scale<BITS>(d[i] >> 16);
     }
 }
 
 #ifdef BFAINTB_TRACE
-#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) p.partials[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
+#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) p.trace[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
 #else
 #define TRACE_MARK(i) do { } while (0)
 #endif
 
-constexpr uint32_t kTaggedMaxM = 4;         // up to this m split-K partial sums travel in tagged slots
-constexpr uint32_t kMaxSlotRetries = 1u << 16;  // re-reads of a split-K slot before giving up (each is a memory round trip)
-constexpr int kRedStride = 260;  // floats per row of the LDS reduction buffer (256 + 4: spreads rows over banks)
+constexpr uint32_t kMaxSlotRetries = 1u << 18;  // re-reads of a split-K word before giving up (each is a memory round trip)
 
-template <int BITS, int MB, bool GROUPED>
-__global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
+// Dynamic LDS of one workgroup, in floats: the waves' tiles [waves][m][COLS + 4].
+__host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t m, uint32_t cols)
 {
-    extern __shared__ __attribute__((aligned(16))) float red[];  // [waves][m rows][kRedStride], at least waves*1024 floats
-    __shared__ uint32_t s_is_last;
+    return waves * m * (cols + 4u);
+}
+
+// Split-K, the reducing workgroup's part for one thread: R rows (rs, rs + nrs, ...) of 4 columns.
+// Fetches the other splits' partial sums, adds them in split order with the thread's own sums last,
+// writes bf16 C and leaves the workspace words empty again.  sum[] may hold more than R rows; the
+// rest is not this launch's.
+template <uint32_t R, uint32_t NSUM>
+__device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 (&sum)[NSUM], uint32_t rs, uint32_t nrs, uint32_t col, bool col_ok)
+{
+    static_assert(R <= NSUM, "rows per thread");
+    constexpr uint32_t kSplitBatch = 16u / R;  // splits whose partial sums a thread fetches together
+    constexpr unsigned long long kEmptyPair = ((unsigned long long)kEmptyWord << 32) | kEmptyWord;
+    const uint32_t rows_out = p.m;
+    const uint32_t others = p.splits - 1u;
+    const size_t split_words = (size_t)p.m * p.n;
+    float* const words = reinterpret_cast<float*>(p.partials);
+    float4 total[R];
+#pragma unroll
+    for (uint32_t i = 0; i < R; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t sp0 = 0; sp0 < others; sp0 += kSplitBatch) {
+        unsigned long long v[kSplitBatch][R][2];
+        // All words of the batch are fetched together, and fetched again together while any of them is
+        // still empty: one memory round trip per attempt, however many words were late.
+        // Rows past m and splits past the last one re-read a word that exists; what they fetch is not used.
+        bool complete = false;
+        for (uint32_t tries = 0; !complete && tries < kMaxSlotRetries; ++tries) {
+            if (tries) __builtin_amdgcn_s_sleep(2);
+#pragma unroll
+            for (uint32_t j = 0; j < kSplitBatch; ++j) {
+                const uint32_t sp = sp0 + j < others ? sp0 + j : others - 1u;
+#pragma unroll
+                for (uint32_t i = 0; i < R; ++i) {
+                    uint32_t row = rs + i * nrs;
+                    if (row >= rows_out) row = rows_out - 1u;
+                    const unsigned long long* src =
+                        reinterpret_cast<const unsigned long long*>(words + (size_t)sp * split_words + (size_t)row * p.n + (col_ok ? col : 0u));
+                    v[j][i][0] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    v[j][i][1] = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            complete = true;
+#pragma unroll
+            for (uint32_t j = 0; j < kSplitBatch; ++j)
+#pragma unroll
+                for (uint32_t i = 0; i < R; ++i)
+                    if (sp0 + j < others && rs + i * nrs < rows_out && col_ok)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            if ((uint32_t)v[j][i][h] == kEmptyWord || (uint32_t)(v[j][i][h] >> 32) == kEmptyWord) complete = false;
+        }
+        // a word that never arrived is still the empty pattern, a NaN, and turns its sum into one
+#pragma unroll
+        for (uint32_t j = 0; j < kSplitBatch; ++j) {
+#pragma unroll
+            for (uint32_t i = 0; i < R; ++i) {
+                const uint32_t row = rs + i * nrs;
+                if (sp0 + j < others && row < rows_out && col_ok) {
+                    unsigned long long* src = reinterpret_cast<unsigned long long*>(words + (size_t)(sp0 + j) * split_words + (size_t)row * p.n + col);
+                    __hip_atomic_store(src, kEmptyPair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(src + 1, kEmptyPair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    total[i].x += __uint_as_float((uint32_t)v[j][i][0]);
+                    total[i].y += __uint_as_float((uint32_t)(v[j][i][0] >> 32));
+                    total[i].z += __uint_as_float((uint32_t)v[j][i][1]);
+                    total[i].w += __uint_as_float((uint32_t)(v[j][i][1] >> 32));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < R; ++i) {
+        const uint32_t row = rs + i * nrs;
+        if (row < rows_out && col_ok) {
+            uint2 o;
+            o.x = pack_bf16_rne(total[i].x + sum[i].x, total[i].y + sum[i].y);
+            o.y = pack_bf16_rne(total[i].z + sum[i].z, total[i].w + sum[i].w);
+            *reinterpret_cast<uint2*>(p.c + (size_t)row * p.ldc + col) = o;
+        }
+    }
+}
+
+template <int BITS, int CPL, int MB, bool GROUPED>
+__global__ void __launch_bounds__((CPL == 8 || MB == 1) ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
+{
+    constexpr int KB = decode_blocks_per_step(BITS, CPL);  // blocks of 32 rows per pipeline step
+    constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
+    constexpr uint32_t kRedStride = kCols + 4u;       // floats per row of a wave's tile in LDS (+4: spreads rows over banks)
+    constexpr uint32_t kLaneBytes = CPL * BITS / 8;   // bytes of one row a lane loads
+    extern __shared__ __attribute__((aligned(16))) float red[];
 
     TRACE_MARK(0);
     const int lane = threadIdx.x & 63;
@@ -151,21 +235,10 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
     const uint32_t cb = blockIdx.x;
     const uint32_t ks = blockIdx.y;
 
-    // tag of this launch's split-K slots: one more than the column block's stored epoch, which the
-    // last workgroup of the previous launch on this workspace left behind (read early, used late)
-    const bool tagged = p.m <= kTaggedMaxM;
-    // The tag carries the column block too, so that no two (column block, launch) pairs on one
-    // workspace share a tag, whatever shapes the launches had.
-    uint32_t epoch = 0, tag = 0;
-    if (p.splits > 1) {
-        epoch = __hip_atomic_load(p.epochs + cb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-        tag = ((epoch & 0xfffffu) << 12) | cb;  // cb < 4096
-    }
-
-    // ---- this lane's 16 weight columns.  A lane past the last column reads the last 16 columns
+    // ---- this lane's CPL weight columns.  A lane past the last column reads the last CPL columns
     //      instead (no predicated loads in the hot loop); what it computes is never stored.
-    uint32_t n_ld = cb * 256u + (uint32_t)nl * 16u;
-    if (n_ld >= p.n) n_ld = p.n - 16u;
+    uint32_t n_ld = cb * kCols + (uint32_t)nl * CPL;
+    if (n_ld >= p.n) n_ld = p.n - CPL;
 
     // ---- this wave's rows of k
     const uint32_t nwaves = blockDim.x >> 6;  // 4 or 8
@@ -173,10 +246,11 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
     const uint32_t kb = ks * p.k_per_wg + (uint32_t)wave * k_per_wave;
     uint32_t ke = kb + k_per_wave;
     if (ke > p.k) ke = p.k;
-    const int nsteps = kb < ke ? (int)((ke - kb) >> 5) : 0;
+    const int nsteps = kb < ke ? (int)((ke - kb) / (32u * KB)) : 0;  // k_per_wave and k are multiples of 32*KB
 
-    const uint8_t* bptr = p.b + (size_t)(kb + 8u * kg) * p.ldb_bytes + (BITS == 8 ? n_ld : n_ld / 2);
+    const uint8_t* bptr = p.b + (size_t)(kb + 8u * kg) * p.ldb_bytes + (size_t)n_ld * BITS / 8;
     const size_t bstep = (size_t)32 * p.ldb_bytes;
+    static_assert(kLaneBytes == 16 || kLaneBytes == 8, "lane loads 16 or 8 bytes of a row");
 
     // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg.
     // Lanes whose row is past m re-read row m-1; their accumulator columns are never stored.
@@ -189,42 +263,50 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
         aptr[mb] = p.a + (size_t)(row_ok[mb] ? mi : p.m - 1u) * p.lda + kb + 8u * kg;
     }
 
-    f32x4_t acc[MB][16];
+    f32x4_t acc[MB][CPL];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int c = 0; c < 16; ++c) acc[mb][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < CPL; ++c) acc[mb][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     if (nsteps > 0) {
         // Two register stages, used alternately: the loads of step s+1 are issued before step s is
-        // computed.  Every load is unconditional and sits in straight-line code (the tail of one
-        // or two steps is peeled off behind the loop), so the wait counts the compiler derives are
-        // exact; a load behind a branch, or a stage copied into another, makes it wait for the
-        // prefetch as well.
+        // computed.  A step is KB blocks of 32 rows, so that a lane has 128 bytes of B in flight per
+        // stage whatever CPL is.  Every load is unconditional and sits in straight-line code (the
+        // tail of one or two steps is peeled off behind the loop), so the wait counts the compiler
+        // derives are exact; a load behind a branch, or a stage copied into another, makes it wait
+        // for the prefetch as well.
         struct Stage {
-            RawStep<BITS> raw;
-            uint4 af[MB];
-            uint4 sraw[2];
+            RawStep<BITS, CPL> raw[KB];
+            uint4 af[KB][MB];
+            uint4 sraw[KB][CPL / 8];
         };
-        float cs[16];
+        float cs[CPL];
         const uint16_t* sptr = p.scale + n_ld;
         auto load_stage = [&](Stage& st, int step) {
-            load_raw<BITS>(st.raw, bptr + (size_t)step * bstep, p.ldb_bytes);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) st.af[mb] = *reinterpret_cast<const uint4*>(aptr[mb] + (size_t)step * 32);
-            if constexpr (GROUPED) load_scales<BITS>(st.sraw, sptr + (size_t)((kb + 32u * (uint32_t)step) / p.group_size) * p.lds);
+            for (int q = 0; q < KB; ++q) {
+                const size_t blk = (size_t)step * KB + q;
+                load_raw<BITS, CPL>(st.raw[q], bptr + blk * bstep, p.ldb_bytes);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) st.af[q][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + blk * 32);
+                if constexpr (GROUPED) load_scales<CPL>(st.sraw[q], sptr + (size_t)((kb + 32u * (uint32_t)blk) / p.group_size) * p.lds);
+            }
             __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic that follows
         };
         auto compute_stage = [&](Stage& st) {
-            if constexpr (GROUPED) apply_scales<BITS>(cs, st.sraw);
-            mac_step<BITS, MB>(st.raw, cs, st.af, acc, std::make_integer_sequence<int, 16>{});
+#pragma unroll
+            for (int q = 0; q < KB; ++q) {
+                if constexpr (GROUPED) apply_scales<BITS, CPL>(cs, st.sraw[q]);
+                mac_step<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
+            }
         };
         Stage s0, s1;
         if constexpr (!GROUPED) {
-            load_scales<BITS>(s0.sraw, sptr);
+            load_scales<CPL>(s0.sraw[0], sptr);
         }
         load_stage(s0, 0);
-        if constexpr (!GROUPED) apply_scales<BITS>(cs, s0.sraw);
+        if constexpr (!GROUPED) apply_scales<BITS, CPL>(cs, s0.sraw[0]);
         int s = 0;
         for (; s + 2 < nsteps; s += 2) {
             load_stage(s1, s + 1);
@@ -241,15 +323,10 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
         }
     }
     TRACE_MARK(2);
-#if defined(BFAINTB_EXPERIMENT) && BFAINTB_EXPERIMENT == 2
-    // timing experiment: streaming phase only
-    if (acc[0][0][0] == 123.456f) p.c[threadIdx.x] = 1;
-    return;
-#endif
 
-    // ---- add the 4 waves' partial sums through LDS: one barrier, then thread t finishes two
-    //      neighbouring columns.  acc[mb][c][r] of lane (nl, kg) is row mi = 16*mb + nl,
-    //      local column (4*kg + r)*16 + c.
+    // ---- add the waves' partial sums through LDS: one barrier, then each thread finishes a few
+    //      neighbouring columns of some rows.  acc[mb][c][r] of lane (nl, kg) is row mi = 16*mb + nl,
+    //      local column (4*kg + r)*CPL + c.
     const uint32_t rows_out = p.m;  // <= 16*MB
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -258,180 +335,117 @@ __global__ void __launch_bounds__(MB == 1 ? 512 : 256) bfaintb_decode_kernel(con
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
+            for (int c4 = 0; c4 < CPL / 4; ++c4) {
                 float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
                                        acc[mb][4 * c4 + 3][r]);
-                *reinterpret_cast<float4*>(row + (4 * kg + r) * 16 + 4 * c4) = v;
+                *reinterpret_cast<float4*>(row + (4 * kg + r) * CPL + 4 * c4) = v;
             }
     }
     __syncthreads();
     TRACE_MARK(3);
-    {
-        const uint32_t cp = threadIdx.x & 127u, rsel = threadIdx.x >> 7;
-        const uint32_t col = cb * 256u + 2u * cp;
-        if (col < p.n) {
-            for (uint32_t row = rsel; row < rows_out; row += (blockDim.x >> 7)) {
-                const float* src = red + (size_t)row * kRedStride + 2u * cp;
-                float sx = 0.f, sy = 0.f;
-                for (uint32_t w = 0; w < nwaves; ++w) {  // fixed order: wave 0 first
-                    const float2 v = *reinterpret_cast<const float2*>(src + (size_t)w * rows_out * kRedStride);
-                    sx += v.x;
-                    sy += v.y;
-                }
-                if (p.splits == 1) {
-                    *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col) = pack_bf16_rne(sx, sy);
-                } else {
-                    // split-K partial sums go to 8-byte slots {value, tag}, written whole with device-scope
-                    // (write-through) stores that nobody waits for: the reader recognises a slot of this
-                    // launch by its tag
-                    if (tagged) {
-                        unsigned long long* slot = p.partials + ((size_t)ks * p.m + row) * p.n + col;
-                        __hip_atomic_store(slot, (unsigned long long)__float_as_uint(sx) | ((unsigned long long)tag << 32), __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-                        __hip_atomic_store(slot + 1, (unsigned long long)__float_as_uint(sy) | ((unsigned long long)tag << 32), __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-                    } else {
-                        // larger m: plain fp32 partials (half the bytes, 16-byte loads for the reader); the
-                        // arrival count then has to wait for the stores' acknowledgement
-                        __hip_atomic_store(reinterpret_cast<unsigned long long*>(reinterpret_cast<float*>(p.partials) + ((size_t)ks * p.m + row) * p.n + col),
-                                           (unsigned long long)__float_as_uint(sx) | ((unsigned long long)__float_as_uint(sy) << 32), __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                }
-            }
-        }
-    }
-    if (p.splits == 1) return;
-    // ---- split-K: the last workgroup to arrive at this column block adds all partial tiles in a
-    // fixed order and writes C.  The arrival count is bumped as soon as this workgroup's stores have
-    // been ISSUED (the barrier), not acknowledged: a slot whose store is still in flight shows an old
-    // tag and is simply read again.  That wait is on memory operations already under way, never on
-    // another workgroup being scheduled, so it cannot deadlock.  (For m > kTaggedMaxM the partials are
-    // untagged and the count waits for the acknowledgements instead.)
-    if (!tagged) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // s_waitcnt vmcnt(0)
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const uint32_t arrived = __hip_atomic_fetch_add(p.counters + cb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_is_last = (arrived == p.splits - 1u) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (s_is_last == 0u) return;
-#if defined(BFAINTB_EXPERIMENT) && BFAINTB_EXPERIMENT == 3
-    if (threadIdx.x == 0) __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return;  // timing experiment: no final reduction
-#endif
 
-    if (!tagged) {
-    // acquire at device scope: drops lines of the partial tiles this XCD's L2 may still hold from an
-    // earlier launch, so the plain (vectorisable, pipelined) loads below see the other workgroups' stores
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    // thread t: 4 consecutive columns (cg = t % (kCols/4)) of rows t / (kCols/4), + threads/(kCols/4), ...
+    constexpr uint32_t kQuads = kCols / 4u;
+    constexpr uint32_t kMaxR = 16u * MB * kQuads / 256u;      // rows per thread with 4 waves (half that with 8)
+    const uint32_t cg = threadIdx.x % kQuads, rs = threadIdx.x / kQuads, nrs = blockDim.x / kQuads;
+    const uint32_t col = cb * kCols + 4u * cg;
+    const bool col_ok = col < p.n;
+    float4 sum[kMaxR];
+#pragma unroll
+    for (uint32_t i = 0; i < kMaxR; ++i) {
+        const uint32_t row = rs + i * nrs;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row < rows_out) {
+            const float* src = red + (size_t)row * kRedStride + 4u * cg;
+            for (uint32_t w = 0; w < nwaves; ++w) {  // fixed order: wave 0 first
+                const float4 v = *reinterpret_cast<const float4*>(src + (size_t)w * rows_out * kRedStride);
+                t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+            }
+        }
+        sum[i] = t;
+    }
+    auto store_c = [&](uint32_t row, const float4& t) {
+        uint2 o;
+        o.x = pack_bf16_rne(t.x, t.y);
+        o.y = pack_bf16_rne(t.z, t.w);
+        *reinterpret_cast<uint2*>(p.c + (size_t)row * p.ldc + col) = o;
+    };
+    if (p.splits == 1) {
+#pragma unroll
+        for (uint32_t i = 0; i < kMaxR; ++i) {
+            const uint32_t row = rs + i * nrs;
+            if (row < rows_out && col_ok) store_c(row, sum[i]);
+        }
+        return;
+    }
 
-    // thread t: 4 consecutive columns (cg = t%64), splits sp = sub, sub+waves, ... (sub = t/64), rows
-    // in chunks of 4; the per-wave sub-sums are combined through LDS in a fixed order
-    {
-        const uint32_t cg = threadIdx.x & 63u, sub = threadIdx.x >> 6;
-        const uint32_t col = cb * 256u + 4u * cg;
-        const bool col_ok = col < p.n;
-        __syncthreads();               // every wave is done reading its sums out of red
-        float* stage = red;            // [waves][4 rows][256 cols]
-        for (uint32_t m0 = 0; m0 < p.m; m0 += 4u) {
-            const uint32_t rows = p.m - m0 < 4u ? p.m - m0 : 4u;
-            for (uint32_t ri = 0; ri < rows; ++ri) {
-                float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (col_ok) {
-                    const float* src = reinterpret_cast<const float*>(p.partials) + (size_t)(m0 + ri) * p.n + col;
-                    for (uint32_t sp = sub; sp < p.splits; sp += nwaves) {
-                        const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sp * p.m * p.n);
-                        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
-                    }
-                }
-                *reinterpret_cast<float4*>(stage + (sub * 4u + ri) * 256u + 4u * cg) = sum;
-            }
-            __syncthreads();
-            {
-                const uint32_t ri = sub;  // thread t finishes row t/64 of the chunk
-                if (ri < rows && col_ok) {
-                    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-                    for (uint32_t w = 0; w < nwaves; ++w) {
-                        const float4 v = *reinterpret_cast<const float4*>(stage + (w * 4u + ri) * 256u + 4u * cg);
-                        t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
-                    }
-                    uint2 o;
-                    o.x = pack_bf16_rne(t.x, t.y);
-                    o.y = pack_bf16_rne(t.z, t.w);
-                    *reinterpret_cast<uint2*>(p.c + (size_t)(m0 + ri) * p.ldc + col) = o;
-                }
-            }
-            __syncthreads();
-        }
-    }
-    } else {
-    // thread t owns column cb*256 + t: all splits of a row are fetched together (device-scope loads,
-    // which bypass whatever this XCD's L2 holds from an earlier launch), then added in split order
-        const uint32_t col = cb * 256u + threadIdx.x;
-        constexpr uint32_t kBatch = 16;
-        if (threadIdx.x < 256u && col < p.n) {
-            for (uint32_t mi = 0; mi < p.m; ++mi) {
-                const unsigned long long* src = p.partials + (size_t)mi * p.n + col;
-                const size_t stride = (size_t)p.m * p.n;
-                float sum = 0.f;
-                for (uint32_t sp0 = 0; sp0 < p.splits; sp0 += kBatch) {
-                    unsigned long long v[kBatch];
+    // ---- split-K.  The workspace holds one fp32 word per (split, row, column); at rest every word is
+    // kEmptyWord, a NaN pattern no sum of products of bf16 numbers takes.  The workgroups of all splits
+    // but the last write their sums there with device-scope (write-through) stores and are done: they
+    // wait for nothing, not even the stores' acknowledgement.  The workgroup of the LAST split
+    // (dispatched after the others) fetches the words with device-scope loads, reads again whichever
+    // still shows kEmptyWord (a store in flight), adds them in split order with its own sums last,
+    // writes C and puts kEmptyWord back for the next launch.  No counter, no flag, no read-modify-write;
+    // only this workgroup ever waits, and only on workgroups that wait for nothing, so the wait ends
+    // whatever order they run in.  It is bounded all the same: a word that never arrives leaves a NaN
+    // in the output instead of hanging the kernel.
+    const size_t split_words = (size_t)p.m * p.n;
+    float* const words = reinterpret_cast<float*>(p.partials);
+    auto pair_of = [](float lo, float hi) { return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32); };
+    if (ks != p.splits - 1u) {
 #pragma unroll
-                    for (uint32_t i = 0; i < kBatch; ++i) {
-                        const uint32_t sp = sp0 + i < p.splits ? sp0 + i : p.splits - 1u;
-                        v[i] = __hip_atomic_load(src + (size_t)sp * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-#pragma unroll
-                    for (uint32_t i = 0; i < kBatch; ++i) {
-                        if (sp0 + i < p.splits) {
-                            // store still in flight: read the slot again (bounded, so the kernel ends whatever happens;
-                            // a slot that never shows its tag poisons the output with a NaN instead of hanging)
-                            for (uint32_t tries = 0; (uint32_t)(v[i] >> 32) != tag && tries < kMaxSlotRetries; ++tries)
-                                v[i] = __hip_atomic_load(src + (size_t)(sp0 + i) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            sum += (uint32_t)(v[i] >> 32) == tag ? __uint_as_float((uint32_t)v[i]) : __uint_as_float(0x7fc00000u);
-                        }
-                    }
-                }
-                p.c[(size_t)mi * p.ldc + col] = (uint16_t)(pack_bf16_rne(sum, 0.f) & 0xffffu);
+        for (uint32_t i = 0; i < kMaxR; ++i) {
+            const uint32_t row = rs + i * nrs;
+            if (row < rows_out && col_ok) {
+                unsigned long long* dst = reinterpret_cast<unsigned long long*>(words + (size_t)ks * split_words + (size_t)row * p.n + col);
+                __hip_atomic_store(dst, pair_of(sum[i].x, sum[i].y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + 1, pair_of(sum[i].z, sum[i].w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+        TRACE_MARK(4);
+        return;
     }
-    if (threadIdx.x == 0) {  // ready for the next launch: new tag, counter back to zero
-        __hip_atomic_store(p.epochs + cb, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(p.counters + cb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    // rows this launch gives a thread: a power of two up to kMaxR; the fewer, the more splits are fetched at once
+    const uint32_t rows_per_thread = (rows_out + nrs - 1u) / nrs;
+    if (rows_per_thread <= 1u) reduce_splits<1>(p, sum, rs, nrs, col, col_ok);
+    else if (rows_per_thread <= 2u) reduce_splits<(kMaxR < 2u ? kMaxR : 2u)>(p, sum, rs, nrs, col, col_ok);
+    else if (rows_per_thread <= 4u) reduce_splits<(kMaxR < 4u ? kMaxR : 4u)>(p, sum, rs, nrs, col, col_ok);
+    else reduce_splits<kMaxR>(p, sum, rs, nrs, col, col_ok);
+    TRACE_MARK(5);
 }
 
-template <int BITS, int MB, bool GROUPED>
+template <int BITS, int CPL, int MB, bool GROUPED>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
-    const dim3 grid((p.n + 255u) / 256u, p.splits, 1);
+    constexpr uint32_t kCols = 16u * CPL;
+    const dim3 grid((p.n + kCols - 1u) / kCols, p.splits, 1);
     const uint32_t waves = p.decode_waves;
-    size_t lds = (size_t)waves * p.m * kRedStride * sizeof(float);
-    if (lds < (size_t)waves * 1024 * sizeof(float)) lds = (size_t)waves * 1024 * sizeof(float);
+    const size_t lds = (size_t)decode_red_floats(waves, p.m, kCols) * sizeof(float);
     if (lds > 64 * 1024) {
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, MB, GROUPED>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 4 * 32 * kRedStride * (int)sizeof(float));
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, CPL, MB, GROUPED>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
             if (e != hipSuccess) return e;
             attr_set = true;
         }
     }
-    return launch_kernel(bfaintb_decode_kernel<BITS, MB, GROUPED>, grid, dim3(64 * waves, 1, 1), lds, stream, p);
+    if (lds > 160 * 1024 - 64) return hipErrorInvalidValue;
+    return launch_kernel(bfaintb_decode_kernel<BITS, CPL, MB, GROUPED>, grid, dim3(64 * waves, 1, 1), lds, stream, p);
+}
+
+template <int BITS, int CPL>
+static hipError_t launch_decode_b(const GemmParams& p, hipStream_t stream)
+{
+    const bool grouped = p.group_size != 0;
+    if (p.m <= 16) return grouped ? launch_decode_t<BITS, CPL, 1, true>(p, stream) : launch_decode_t<BITS, CPL, 1, false>(p, stream);
+    return grouped ? launch_decode_t<BITS, CPL, 2, true>(p, stream) : launch_decode_t<BITS, CPL, 2, false>(p, stream);
 }
 
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)
 {
-    const bool grouped = p.group_size != 0;
-    const int mb = p.m <= 16 ? 1 : 2;
-    if (bits == 8) {
-        if (mb == 1) return grouped ? launch_decode_t<8, 1, true>(p, stream) : launch_decode_t<8, 1, false>(p, stream);
-        return grouped ? launch_decode_t<8, 2, true>(p, stream) : launch_decode_t<8, 2, false>(p, stream);
-    }
-    if (mb == 1) return grouped ? launch_decode_t<4, 1, true>(p, stream) : launch_decode_t<4, 1, false>(p, stream);
-    return grouped ? launch_decode_t<4, 2, true>(p, stream) : launch_decode_t<4, 2, false>(p, stream);
+    if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8>(p, stream) : launch_decode_b<8, 16>(p, stream);
+    return launch_decode_b<4, 16>(p, stream);
 }
 
 }  // namespace bfaintb

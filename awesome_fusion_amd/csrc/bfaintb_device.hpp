@@ -18,13 +18,21 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
-constexpr int kCounterSlots = 4096;  // arrival counters at the head of a workspace (uint32 each)
+// A split-K workspace word that holds no partial sum: an all-ones NaN.  Sums of products of bf16 numbers
+// are never this pattern (NaNs born in the arithmetic are the default quiet NaN; NaNs carried over from
+// bf16 inputs have zero low bits).
+constexpr uint32_t kEmptyWord = 0xffffffffu;
 
 template <typename Tuple, size_t... I>
 inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 {
     ((argv[I] = const_cast<void*>(static_cast<const void*>(&std::get<I>(t)))), ...);
 }
+
+// Decode variant: blocks of 32 rows of k a wave loads per pipeline step (cpl = weights per lane and
+// row).  Two blocks for the 8-byte-per-row layouts measured no faster than one: more bytes in flight
+// per wave, fewer waves per CU.
+__host__ __device__ constexpr int decode_blocks_per_step(int /*bits*/, int /*cpl*/) { return 1; }
 
 struct GemmParams {
     uint16_t* c;
@@ -38,12 +46,14 @@ struct GemmParams {
     uint32_t lds;        // elements per scale row (= n)
     uint32_t group_size; // rows of k per scale group; 0 = one group
     // split-K (decode variant only)
-    uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_waves)
+    uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_blocks_per_step * decode_waves)
     uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)
+    uint32_t decode_cols;  // columns per workgroup of the decode variant (256, or 128 for 8-bit codes)
     uint32_t splits;     // workgroups along k
-    unsigned long long* partials;  // [splits][m][n] slots of {fp32 value, uint32 tag}
-    uint32_t* counters;  // [column blocks] arrivals of the running launch (zero at rest)
-    uint32_t* epochs;    // [column blocks] tag of the last finished launch
+    unsigned long long* partials;  // [splits - 1][m][n] fp32 partial sums; kEmptyWord wherever none is waiting
+#ifdef BFAINTB_TRACE
+    unsigned long long* trace;  // timestamp sink (instrumented builds only)
+#endif
 };
 
 // Launch through hipLaunchKernel so that the error returned belongs to THIS launch:

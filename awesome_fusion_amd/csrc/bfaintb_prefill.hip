@@ -312,8 +312,8 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     if (kt < ksteps) step(C0{}, kt);
 
 #ifdef BFAINTB_TRACE
-    if (lane == 0 && p.partials != nullptr)
-        for (int i = 0; i < 5; ++i) p.partials[(size_t)(blockIdx.x * 8 + wave) * 8 + i] = (unsigned long long)tq[i];
+    if (lane == 0 && p.trace != nullptr)
+        for (int i = 0; i < 5; ++i) p.trace[(size_t)(blockIdx.x * 8 + wave) * 8 + i] = (unsigned long long)tq[i];
 #endif
     // ---- epilogue: bf16 tile through LDS (rows 64q..64q+63 in the q-th of the four arrays), then
     //      16-byte row-contiguous stores

@@ -76,9 +76,10 @@ enum {
  *   group_size    0: one scale per output channel (the reference's only mode);
  *                 otherwise rows per scale group along k (multiple of 32, divides k)
  *   workspace     device scratch of at least bfaintb_gemm_workspace_bytes(...) bytes that has been
- *                 passed through bfaintb_workspace_init once (or is all zero bytes).  The call
- *                 leaves it ready for the next call.  Two calls that may run concurrently must not
- *                 share a workspace.  May be NULL when the required size is 0.
+ *                 passed through bfaintb_workspace_init once (equivalently: every byte is 0xff).
+ *                 The call leaves it in that state again, ready for the next call of any shape.
+ *                 Two calls that may run concurrently must not share a workspace.  May be NULL
+ *                 when the required size is 0.
  */
 BFAINTB_API int bfaintb_gemm(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
                  uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
@@ -90,13 +91,15 @@ BFAINTB_API int bfaintb_gemm_ex(void* c, const void* a, const void* b, const voi
                     uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k);
 
-/* Scratch the GEMM needs for a shape: tagged split-K partial sums, arrival counters and epochs.  Depends only on
- * its arguments.  The reference kernel has no scratch (no split-K, bfAintBGemm.cc:107-109). */
+/* Scratch the GEMM needs for a shape: one fp32 word per (split but the last, row, column) of the
+ * split-K partial sums, rounded up to 256 bytes; 0 when the shape runs without split-K.  Depends only
+ * on its arguments.  The reference kernel has no scratch (no split-K, bfAintBGemm.cc:107-109). */
 BFAINTB_API size_t bfaintb_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 BFAINTB_API size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
                                        int variant, uint32_t split_k);
 
-/* Clears a freshly allocated workspace: arrival counters, epochs and partial-sum slots (stream-ordered). */
+/* Prepares a freshly allocated workspace: marks every word "no partial sum here" (all bits set).
+ * Stream-ordered, graph-capturable; workspace_bytes must be a multiple of 4. */
 BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */

@@ -35,8 +35,8 @@ def test_variant_choice_and_split():
     assert af.split_k(4096, 4096, 4096) == 1
     s = af.split_k(1, 4096, 4096)
     assert 1 < s <= 64 and 4096 % s == 0
-    # workspace = counters + epochs + splits * m * n tagged 8-byte slots; none for the prefill variant
-    assert af.workspace_bytes(1, 4096, 4096) == 2 * 4096 * 4 + s * 1 * 4096 * 8
+    # none for the prefill variant or without split-K
+    assert af.workspace_bytes(1, 4096, 4096) == (s - 1) * 1 * 4096 * 4   # one fp32 word per (split but the last, row, column)
     assert af.workspace_bytes(4096, 4096, 4096) == 0
     assert af.workspace_bytes(8, 4096, 4096, force_split_k=1) == 0
     assert af.kernel_name(1) == "bfaintb_decode_kernel" and af.kernel_name(4096) == "bfaintb_prefill_kernel"
@@ -65,8 +65,8 @@ def test_rejects_bad_arguments_without_launching():
     assert rc(b=P + 4) == -4
     assert rc(which=9) == -7
     assert rc(which=af.DECODE) == -7          # m = 64 cannot run the decode variant
-    assert rc(m=8, which=af.DECODE, force_split_k=2) == -6   # split-K needs a workspace
-    assert rc(m=8, which=af.DECODE, force_split_k=2, workspace=P, workspace_nbytes=64) == -6
+    assert rc(m=8, k=1024, which=af.DECODE, force_split_k=2) == -6   # split-K needs a workspace
+    assert rc(m=8, k=1024, which=af.DECODE, force_split_k=2, workspace=P, workspace_nbytes=64) == -6
     assert rc(m=0) == 0                       # nothing to do
     for code in (-1, -2, -3, -4, -5, -6, -7):
         assert len(af.error_string(code)) > 10
@@ -77,7 +77,7 @@ def test_rejects_bad_arguments_without_launching():
     assert af.dequant(P, P, P, 128, 256, stream=0, weight_bits=3, check=False) == -5
     assert af.dequant(P, P, P, 100, 256, stream=0, check=False) == -2
     assert af.dequant(P, P, None, 128, 256, stream=0, check=False) == -1
-    assert L.bfaintb_workspace_init(P, 64, None) == -6
+    assert L.bfaintb_workspace_init(P, 66, None) == -6   # not a whole number of words
     assert L.bfaintb_workspace_init(None, 0, None) == 0
 
 
