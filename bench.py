@@ -36,10 +36,10 @@ LLC_BYTES = 256 << 20
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
 MEASURED_TRAFFIC_BYTES = {
-    # fetch 8449.2 KiB x 1.997 + write 272.5 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
-    "decode_m1_n4096_k4096_int8_perchannel": 17557045,
-    # fetch 66957.3 KiB x 1.997 + write 35328.0 KiB
-    "prefill_m4096_n4096_k4096_int8_perchannel": 173098729,
+    # fetch 8404.8 KiB x 1.997 + write 456.0 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
+    "decode_m1_n4096_k4096_int8_perchannel": 17654154,
+    # fetch 65627.0 KiB x 1.997 + write 32768.0 KiB
+    "prefill_m4096_n4096_k4096_int8_perchannel": 167756921,
 }
 
 
@@ -123,6 +123,32 @@ def time_read_ceiling(af, w, steps, warmup):
     with torch.cuda.graph(g):
         for i in range(steps):
             af.probe_read(w.b[i % nb])
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def time_vendor_bf16_gemm(w, steps, warmup):
+    """Context for the prefill figure: the vendor library's plain bf16 x bf16 GEMM (torch.matmul, i.e.
+    hipBLASLt) on the same activations and the already dequantised weights, same graph protocol.  It does
+    none of the dequantisation work; it shows what a tuned MFMA kernel sustains on this machine at this shape."""
+    import torch
+    wq = torch.from_numpy(w.q.astype(np.float32)).cuda()
+    wb = (wq * w.s.float()[0][None, :]).to(torch.bfloat16)
+    del wq
+    out = torch.empty((w.m, w.n), dtype=torch.bfloat16, device="cuda")
+    for _ in range(warmup):
+        torch.matmul(w.a, wb, out=out)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(steps):
+            torch.matmul(w.a, wb, out=out)
     g.replay()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -287,6 +313,12 @@ def main():
         entry = {"value": round(w.flops / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "steps": pk,
                  "ms_per_step": round(wall_ms, 6), "GB/s": round(w.bytes / (wall_ms * 1e-3) / 1e9, 1),
                  "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma")}
+        try:
+            v_ms = time_vendor_bf16_gemm(w, pk, 5)
+            entry["vendor_bf16_gemm_same_shape"] = {"TFLOP/s": round(w.flops / (v_ms * 1e-3) / 1e12, 2), "kernel_us": round(v_ms * 1e3, 3),
+                                                    "note": "torch.matmul bf16 x bf16 on pre-dequantised weights (no dequantisation work): context, not a baseline"}
+        except Exception as exc:  # context only
+            entry["vendor_bf16_gemm_same_shape"] = {"error": str(exc)[:200]}
         out_extra["prefill_m4096"] = entry
         if res is None:
             res = {"metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=4096: TFLOP/s", "value": entry["value"], "unit": "TFLOP/s",

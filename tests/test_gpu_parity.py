@@ -172,10 +172,13 @@ def test_split_k_is_deterministic_and_consistent(af):
 
 def test_workspace_is_left_ready_for_the_next_call(af):
     # one workspace, back-to-back calls of different shapes and split factors, no re-initialisation
+    import helpers
     shapes = [(1, 4096, 4096), (16, 1024, 8192), (32, 272, 512), (1, 4096, 4096)]
     for i, (m, n, k) in enumerate(shapes):
         p = Problem(m, n, k, seed=i)
         assert_close_ulp(p, run_gemm(p), f"call {i}")
+        # every word of the workspace is back to "no partial sum here" (all bits set)
+        assert bool((helpers._ws.t == 0xFF).all()), f"workspace not restored after call {i}"
 
 
 def test_prefill_variant_on_small_m_matches_decode(af):
