@@ -23,7 +23,9 @@ namespace {
 using bfaintb::GemmParams;
 using bfaintb::kEmptyWord;
 
-constexpr uint32_t kDecodeMaxM = 32;
+constexpr uint32_t kDecodeAutoMaxM = 32;       // AUTO always runs the decode family up to this m
+constexpr uint32_t kDecodeFamilyAutoMaxM = 4096;  // ... and never beyond this one
+constexpr uint32_t kDecodeMaxM = 32768;        // what the decode family accepts when forced
 constexpr uint32_t kDecodeTargetWgs = 480;        // 4-wave workgroups: a little under two per CU on a 256-CU part
 constexpr uint32_t kDecodeTargetWgsNarrow = 256;  // 8-wave workgroups: one per CU
 constexpr uint32_t kMaxSplits = 64;
@@ -42,59 +44,137 @@ int check_shape(uint32_t m, uint32_t n, uint32_t k)
     return BFAINTB_OK;
 }
 
-int resolve_variant(uint32_t m, int variant)
-{
-    if (variant == BFAINTB_VARIANT_AUTO) return m <= kDecodeMaxM ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
-    if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
-    if (variant == BFAINTB_VARIANT_PREFILL) return variant;
-    return BFAINTB_ERR_BAD_VARIANT;
-}
-
-// Launch shape of the decode variant: columns and waves per workgroup, rows of k per workgroup, workgroups along k.
+// Launch shape of the decode variant: columns and waves per workgroup, blocks of 16 rows of A per workgroup,
+// rows of k per workgroup, workgroups along k.
 struct DecodePlan {
-    uint32_t cols, waves, k_per_wg, splits;
+    uint32_t cols, waves, mb, k_per_wg, splits;
 };
 
-DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
+// Rows of k per workgroup and the number of splits that results, for `splits` wanted.
+static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits)
 {
-    DecodePlan pl;
-    // 8-bit codes, 128 columns x 8 waves (a lane loads 8 bytes of a row, 16 lanes one 128-byte line): half
-    // the splits, so half the partial-sum traffic, for the same number of waves.  Measured faster than the
-    // wide block while the weights are few (the launch is latency-bound) and for the m where the partial
-    // sums weigh most; large weight matrices stream better in 256-byte row segments.
-    // Otherwise, and for 4-bit codes: 256 columns x 4 waves.
-    const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
-    const bool few = weight_bytes <= (32ull << 20);
-    const bool narrow = bits == 8 && (few || (m >= 8 && m <= 16));
-    pl.cols = narrow ? 128u : 256u;
-    pl.waves = narrow ? 8u : 4u;
-    uint32_t target = narrow ? (few ? kDecodeTargetWgsNarrow : kDecodeTargetWgsNarrow * 3u / 2u) : kDecodeTargetWgs;
-#ifdef BFAINTB_TUNE
-    if (const char* e = getenv("BFAINTB_DECODE_COLS")) {
-        if (atoi(e) == 256) { pl.cols = 256u; pl.waves = 4u; target = kDecodeTargetWgs; }
-    }
-    if (const char* e = getenv("BFAINTB_DECODE_WAVES")) pl.waves = (uint32_t)atoi(e);
-    if (const char* e = getenv("BFAINTB_DECODE_TARGET")) target = (uint32_t)atoi(e);
-#endif
     // rows one workgroup covers per pipeline step of its waves
     const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16) * pl.waves;
-    const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
-    uint32_t splits = forced_splits;
-    if (splits == 0) {
-        // about `target` workgroups: enough waves on every CU to keep the memory system busy ...
-        splits = (target + col_blocks / 2) / col_blocks;
-        // ... while the split-K partial sums (written and read back as fp32) stay below a quarter of the weight bytes
-        uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (256u * (m ? m : 1u)));
-        if (cap < 1) cap = 1;
-        if (splits > cap) splits = cap;
-    }
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
     uint32_t per = (k + splits - 1) / splits;
     per = (per + unit - 1) / unit * unit;
     pl.k_per_wg = per;
     pl.splits = (k + per - 1) / per;
+}
+
+// Rough time, in microseconds, of the decode family on a 256-CU part for more than 32 rows of A.
+// Every block of 16*mb rows streams and dequantises all weights again: measured 16, 22 and 35 cycles per
+// weight and lane for mb = 1, 2, 4 (the dequantisation plus mb matrix instructions per 8 weights, less well
+// overlapped the fewer waves a SIMD holds); repeats of the stream mostly hit in cache; split-K partial sums
+// are written, read and cleared, and cost two more trips to memory; with fewer than one wave per SIMD both the
+// arithmetic and the stream slow down in proportion.  Fitted to measurements at N = 4096, 11008 and 28672.
+static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
+{
+    const double weights = (double)n * k;
+    const double row_blocks = (double)((m + 16u * pl.mb - 1u) / (16u * pl.mb));
+    const double col_blocks = (double)((n + pl.cols - 1u) / pl.cols);
+    const double waves = row_blocks * col_blocks * pl.splits * pl.waves;
+    const double busy = waves >= 1024.0 ? 1.0 : waves / 1024.0;
+    const double cycles_per_weight = 10.0 + 6.25 * pl.mb;
+    const double compute = row_blocks * weights * cycles_per_weight / 65536.0 / 2000.0 / busy;
+    const double stream = weights * bits / 8.0 * (1.0 + 0.3 * (row_blocks - 1.0)) / 3.5e6 / busy;
+    const double partial = pl.splits > 1 ? 3.0 + 12.0 * (pl.splits - 1.0) * m * n / 1.5e6 : 0.0;
+    return 5.0 + (compute > stream ? compute : stream) + partial;
+}
+
+// Rough time of the prefill kernel: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of k.
+static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
+{
+    const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
+    const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
+    return 4.0 + rounds * (k / 64.0) * 1.33;
+}
+
+DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
+{
+    DecodePlan pl;
+    const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
+    if (m > 32) {
+        // More than 32 rows of A: grid z walks blocks of 16*mb rows.  128 columns x 64 rows (mb = 4, 4 waves: one
+        // wave per SIMD, 128 accumulator registers) amortises the dequantisation best; smaller row blocks give
+        // more workgroups when columns x row blocks alone do not fill the machine.  Pick by estimate.
+        DecodePlan best{};
+        double best_t = 0.0;
+        for (uint32_t mb = bits == 8 ? 4u : 2u; mb >= 1u; mb >>= 1) {
+            DecodePlan c;
+            c.cols = bits == 8 ? 128u : 256u;
+            c.waves = (bits == 8 && mb <= 2u) ? 8u : 4u;
+            c.mb = mb;
+            const uint32_t tiles = ((n + c.cols - 1u) / c.cols) * ((m + 16u * mb - 1u) / (16u * mb));
+            for (uint32_t s = 1; s <= 16u; s += (s < 4u ? 1u : s < 8u ? 2u : 4u)) {
+                if (forced_splits && s != 1u) break;
+                set_splits(c, k, bits, forced_splits ? forced_splits : s);
+                if (!forced_splits && c.splits != s && s != 1u) continue;  // k does not divide that way
+                if (!forced_splits && s > 1u && tiles * s > 768u) break;
+                const double t = decode_family_estimate_us(m, n, k, bits, c);
+                if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
+            }
+        }
+        pl = best;
+    } else {
+        // 8-bit codes, 128 columns x 8 waves (a lane loads 8 bytes of a row, 16 lanes one 128-byte line): half
+        // the splits, so half the partial-sum traffic, for the same number of waves.  Measured faster than the
+        // wide block while the weights are few (the launch is latency-bound) and for the m where the partial
+        // sums weigh most; large weight matrices stream better in 256-byte row segments.
+        // Otherwise, and for 4-bit codes: 256 columns x 4 waves.
+        const bool few = weight_bytes <= (32ull << 20);
+        const bool narrow = bits == 8 && (few || (m >= 8 && m <= 16));
+        pl.cols = narrow ? 128u : 256u;
+        pl.waves = narrow ? 8u : 4u;
+        pl.mb = m <= 16 ? 1u : 2u;
+        uint32_t target = narrow ? (few ? kDecodeTargetWgsNarrow : kDecodeTargetWgsNarrow * 3u / 2u) : kDecodeTargetWgs;
+        uint32_t capdiv = 256u;
+#ifdef BFAINTB_TUNE
+        if (const char* e = getenv("BFAINTB_DECODE_COLS")) {
+            if (atoi(e) == 256) { pl.cols = 256u; pl.waves = 4u; target = kDecodeTargetWgs; }
+        }
+        if (const char* e = getenv("BFAINTB_DECODE_TARGET")) target = (uint32_t)atoi(e);
+        if (const char* e = getenv("BFAINTB_DECODE_CAPDIV")) capdiv = (uint32_t)atoi(e);
+#endif
+        const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
+        uint32_t splits = forced_splits;
+        if (splits == 0) {
+            // about `target` workgroups: enough waves on every CU to keep the memory system busy ...
+            splits = (target + col_blocks / 2) / col_blocks;
+            // ... while the split-K partial sums (written, read back and cleared as fp32) stay below a quarter of the weight bytes
+            uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (capdiv * (m ? m : 1u)));
+            if (cap < 1) cap = 1;
+            if (splits > cap) splits = cap;
+        }
+        set_splits(pl, k, bits, splits);
+    }
+#ifdef BFAINTB_TUNE
+    if (const char* e = getenv("BFAINTB_DECODE_MB")) {
+        pl.mb = (uint32_t)atoi(e);
+        pl.waves = pl.mb > 2 ? 4u : 8u;
+        if (const char* w = getenv("BFAINTB_DECODE_WAVES")) pl.waves = (uint32_t)atoi(w);
+        if (pl.mb == 4 && pl.cols != 128u) pl.mb = 2u;
+        if (const char* sp = getenv("BFAINTB_DECODE_SPLITS")) set_splits(pl, k, bits, (uint32_t)atoi(sp));
+        else set_splits(pl, k, bits, pl.splits);
+    }
+#endif
     return pl;
+}
+
+// The decode family up to 32 rows of A; beyond that whichever of the two the estimates favour (the prefill
+// kernel's 256x256 tiles leave most of the machine idle until m*n reaches a few hundred tiles).
+int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
+{
+    if (variant == BFAINTB_VARIANT_AUTO) {
+        if (m <= kDecodeAutoMaxM) return BFAINTB_VARIANT_DECODE;
+        if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
+        const DecodePlan pl = decode_plan(m, n, k, bits, 0);
+        return decode_family_estimate_us(m, n, k, bits, pl) * 1.1 < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    }
+    if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
+    if (variant == BFAINTB_VARIANT_PREFILL) return variant;
+    return BFAINTB_ERR_BAD_VARIANT;
 }
 
 size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant, uint32_t forced_split)
@@ -137,7 +217,7 @@ int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, ui
     if (e) return e;
     e = check_shape(m, n, k);
     if (e) return e;
-    return resolve_variant(m, BFAINTB_VARIANT_AUTO);
+    return resolve_variant(m, n, k, weight_bits, BFAINTB_VARIANT_AUTO);
 }
 
 uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
@@ -150,7 +230,7 @@ size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int w
                                        uint32_t split_k)
 {
     if (check_format(k, weight_bits, group_size) || check_shape(m, n, k)) return 0;
-    const int v = resolve_variant(m, variant);
+    const int v = resolve_variant(m, n, k, weight_bits, variant);
     if (v < 0) return 0;
     return workspace_need(m, n, k, weight_bits, v, split_k);
 }
@@ -180,7 +260,7 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     e = check_shape(m, n, k);
     if (e) return e;
     if (lda < k || ldb < n || ldc < n || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
-    const int v = resolve_variant(m, variant);
+    const int v = resolve_variant(m, n, k, weight_bits, variant);
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
     if (c == nullptr || a == nullptr || b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
@@ -215,6 +295,7 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     p.splits = pl.splits;
     p.decode_waves = pl.waves;
     p.decode_cols = pl.cols;
+    p.decode_mb = pl.mb;
     if (p.splits > 1) {
         const size_t need = workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k);
         if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
@@ -262,7 +343,8 @@ int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream)
 
 const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m)
 {
-    const int v = resolve_variant(m, variant);
+    int v = variant;
+    if (v == BFAINTB_VARIANT_AUTO) v = m <= kDecodeAutoMaxM ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     if (v == BFAINTB_VARIANT_DECODE) return "bfaintb_decode_kernel";
     if (v == BFAINTB_VARIANT_PREFILL) return "bfaintb_prefill_kernel";
     (void)weight_bits;

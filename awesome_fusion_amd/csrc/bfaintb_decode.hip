@@ -134,26 +134,33 @@ __device__ __forceinline__ void apply_scales(float (&cs)[CPL], const uint4 (&sra
 
 constexpr uint32_t kMaxSlotRetries = 1u << 18;  // re-reads of a split-K word before giving up (each is a memory round trip)
 
-// Dynamic LDS of one workgroup, in floats: the waves' tiles [waves][m][COLS + 4].
-__host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t m, uint32_t cols)
+// Blocks of 16 rows whose per-wave tiles fit in LDS together (4 waves; 8 waves run MB <= 2).
+__host__ __device__ constexpr int decode_rows16_per_pass(int cpl, int mb)
 {
-    return waves * m * (cols + 4u);
+    const int fit = cpl == 8 ? 4 : 2;  // 4 waves x 64 rows x 132 floats, or 4 waves x 32 rows x 260 floats: 133 KiB
+    return mb < fit ? mb : fit;
 }
 
-// Split-K, the reducing workgroup's part for one thread: R rows (rs, rs + nrs, ...) of 4 columns.
-// Fetches the other splits' partial sums, adds them in split order with the thread's own sums last,
-// writes bf16 C and leaves the workspace words empty again.  sum[] may hold more than R rows; the
-// rest is not this launch's.
+// Dynamic LDS of one workgroup, in floats: the waves' tiles [waves][rows of one pass][COLS + 4].
+__host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t rows, uint32_t cols)
+{
+    return waves * rows * (cols + 4u);
+}
+
+// Split-K, the reducing workgroup's part for one thread: R rows (first_row + rs, + nrs, ...; `rows` of
+// them exist from first_row on) of 4 columns.  Fetches the other splits' partial sums, adds them in
+// split order with the thread's own sums last, writes bf16 C and leaves the workspace words empty
+// again.  sum[] may hold more than R rows; the rest is not this launch's.
 template <uint32_t R, uint32_t NSUM>
-__device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 (&sum)[NSUM], uint32_t rs, uint32_t nrs, uint32_t col, bool col_ok)
+__device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 (&sum)[NSUM], uint32_t first_row, uint32_t rows, uint32_t rs,
+                                              uint32_t nrs, uint32_t col, bool col_ok)
 {
     static_assert(R <= NSUM, "rows per thread");
     constexpr uint32_t kSplitBatch = 16u / R;  // splits whose partial sums a thread fetches together
     constexpr unsigned long long kEmptyPair = ((unsigned long long)kEmptyWord << 32) | kEmptyWord;
-    const uint32_t rows_out = p.m;
     const uint32_t others = p.splits - 1u;
     const size_t split_words = (size_t)p.m * p.n;
-    float* const words = reinterpret_cast<float*>(p.partials);
+    float* const words = reinterpret_cast<float*>(p.partials) + (size_t)first_row * p.n;
     float4 total[R];
 #pragma unroll
     for (uint32_t i = 0; i < R; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -161,7 +168,7 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
         unsigned long long v[kSplitBatch][R][2];
         // All words of the batch are fetched together, and fetched again together while any of them is
         // still empty: one memory round trip per attempt, however many words were late.
-        // Rows past m and splits past the last one re-read a word that exists; what they fetch is not used.
+        // Rows past the last and splits past the last one re-read a word that exists; what they fetch is not used.
         bool complete = false;
         for (uint32_t tries = 0; !complete && tries < kMaxSlotRetries; ++tries) {
             if (tries) __builtin_amdgcn_s_sleep(2);
@@ -171,7 +178,7 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 #pragma unroll
                 for (uint32_t i = 0; i < R; ++i) {
                     uint32_t row = rs + i * nrs;
-                    if (row >= rows_out) row = rows_out - 1u;
+                    if (row >= rows) row = rows - 1u;
                     const unsigned long long* src =
                         reinterpret_cast<const unsigned long long*>(words + (size_t)sp * split_words + (size_t)row * p.n + (col_ok ? col : 0u));
                     v[j][i][0] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -183,7 +190,7 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
             for (uint32_t j = 0; j < kSplitBatch; ++j)
 #pragma unroll
                 for (uint32_t i = 0; i < R; ++i)
-                    if (sp0 + j < others && rs + i * nrs < rows_out && col_ok)
+                    if (sp0 + j < others && rs + i * nrs < rows && col_ok)
 #pragma unroll
                         for (int h = 0; h < 2; ++h)
                             if ((uint32_t)v[j][i][h] == kEmptyWord || (uint32_t)(v[j][i][h] >> 32) == kEmptyWord) complete = false;
@@ -194,7 +201,7 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 #pragma unroll
             for (uint32_t i = 0; i < R; ++i) {
                 const uint32_t row = rs + i * nrs;
-                if (sp0 + j < others && row < rows_out && col_ok) {
+                if (sp0 + j < others && row < rows && col_ok) {
                     unsigned long long* src = reinterpret_cast<unsigned long long*>(words + (size_t)(sp0 + j) * split_words + (size_t)row * p.n + col);
                     __hip_atomic_store(src, kEmptyPair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(src + 1, kEmptyPair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -209,17 +216,17 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 #pragma unroll
     for (uint32_t i = 0; i < R; ++i) {
         const uint32_t row = rs + i * nrs;
-        if (row < rows_out && col_ok) {
+        if (row < rows && col_ok) {
             uint2 o;
             o.x = pack_bf16_rne(total[i].x + sum[i].x, total[i].y + sum[i].y);
             o.y = pack_bf16_rne(total[i].z + sum[i].z, total[i].w + sum[i].w);
-            *reinterpret_cast<uint2*>(p.c + (size_t)row * p.ldc + col) = o;
+            *reinterpret_cast<uint2*>(p.c + (size_t)(first_row + row) * p.ldc + col) = o;
         }
     }
 }
 
 template <int BITS, int CPL, int MB, bool GROUPED>
-__global__ void __launch_bounds__((CPL == 8 || MB == 1) ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
+__global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
 {
     constexpr int KB = decode_blocks_per_step(BITS, CPL);  // blocks of 32 rows per pipeline step
     constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
@@ -234,6 +241,9 @@ __global__ void __launch_bounds__((CPL == 8 || MB == 1) ? 512 : 256) bfaintb_dec
     const int kg = lane >> 4;
     const uint32_t cb = blockIdx.x;
     const uint32_t ks = blockIdx.y;
+    // rows of A and C this workgroup covers: block blockIdx.z of 16*MB rows
+    const uint32_t row0 = blockIdx.z * (16u * MB);
+    const uint32_t rows_here = p.m - row0 < 16u * MB ? p.m - row0 : 16u * MB;
 
     // ---- this lane's CPL weight columns.  A lane past the last column reads the last CPL columns
     //      instead (no predicated loads in the hot loop); what it computes is never stored.
@@ -253,14 +263,14 @@ __global__ void __launch_bounds__((CPL == 8 || MB == 1) ? 512 : 256) bfaintb_dec
     static_assert(kLaneBytes == 16 || kLaneBytes == 8, "lane loads 16 or 8 bytes of a row");
 
     // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg.
-    // Lanes whose row is past m re-read row m-1; their accumulator columns are never stored.
+    // Lanes whose row is past the last one re-read the last one; their accumulator columns are never stored.
     const uint16_t* aptr[MB];
     bool row_ok[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const uint32_t mi = 16u * mb + (uint32_t)nl;
-        row_ok[mb] = mi < p.m;
-        aptr[mb] = p.a + (size_t)(row_ok[mb] ? mi : p.m - 1u) * p.lda + kb + 8u * kg;
+        row_ok[mb] = mi < rows_here;
+        aptr[mb] = p.a + (size_t)(row0 + (row_ok[mb] ? mi : rows_here - 1u)) * p.lda + kb + 8u * kg;
     }
 
     f32x4_t acc[MB][CPL];
@@ -324,103 +334,115 @@ __global__ void __launch_bounds__((CPL == 8 || MB == 1) ? 512 : 256) bfaintb_dec
     }
     TRACE_MARK(2);
 
-    // ---- add the waves' partial sums through LDS: one barrier, then each thread finishes a few
-    //      neighbouring columns of some rows.  acc[mb][c][r] of lane (nl, kg) is row mi = 16*mb + nl,
-    //      local column (4*kg + r)*CPL + c.
-    const uint32_t rows_out = p.m;  // <= 16*MB
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        if (!row_ok[mb]) continue;
-        float* row = red + ((size_t)wave * rows_out + (mb * 16 + nl)) * kRedStride;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int c4 = 0; c4 < CPL / 4; ++c4) {
-                float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
-                                       acc[mb][4 * c4 + 3][r]);
-                *reinterpret_cast<float4*>(row + (4 * kg + r) * CPL + 4 * c4) = v;
-            }
-    }
-    __syncthreads();
-    TRACE_MARK(3);
-
-    // thread t: 4 consecutive columns (cg = t % (kCols/4)) of rows t / (kCols/4), + threads/(kCols/4), ...
+    // ---- add the waves' partial sums through LDS, kMBC blocks of 16 rows at a time (what fits): one barrier,
+    //      then each thread finishes 4 neighbouring columns of some rows.  acc[mb][c][r] of lane (nl, kg) is
+    //      row 16*mb + nl, local column (4*kg + r)*CPL + c.
+    constexpr int kMBC = decode_rows16_per_pass(CPL, MB);
     constexpr uint32_t kQuads = kCols / 4u;
-    constexpr uint32_t kMaxR = 16u * MB * kQuads / 256u;      // rows per thread with 4 waves (half that with 8)
+    constexpr uint32_t kMaxR = 16u * kMBC * kQuads / 256u;      // rows per thread and pass with 4 waves (half that with 8)
+    // thread t: 4 consecutive columns (cg = t % (kCols/4)) of rows t / (kCols/4), + threads/(kCols/4), ...
     const uint32_t cg = threadIdx.x % kQuads, rs = threadIdx.x / kQuads, nrs = blockDim.x / kQuads;
     const uint32_t col = cb * kCols + 4u * cg;
     const bool col_ok = col < p.n;
-    float4 sum[kMaxR];
-#pragma unroll
-    for (uint32_t i = 0; i < kMaxR; ++i) {
-        const uint32_t row = rs + i * nrs;
-        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (row < rows_out) {
-            const float* src = red + (size_t)row * kRedStride + 4u * cg;
-            for (uint32_t w = 0; w < nwaves; ++w) {  // fixed order: wave 0 first
-                const float4 v = *reinterpret_cast<const float4*>(src + (size_t)w * rows_out * kRedStride);
-                t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
-            }
-        }
-        sum[i] = t;
-    }
-    auto store_c = [&](uint32_t row, const float4& t) {
-        uint2 o;
-        o.x = pack_bf16_rne(t.x, t.y);
-        o.y = pack_bf16_rne(t.z, t.w);
-        *reinterpret_cast<uint2*>(p.c + (size_t)row * p.ldc + col) = o;
-    };
-    if (p.splits == 1) {
-#pragma unroll
-        for (uint32_t i = 0; i < kMaxR; ++i) {
-            const uint32_t row = rs + i * nrs;
-            if (row < rows_out && col_ok) store_c(row, sum[i]);
-        }
-        return;
-    }
-
-    // ---- split-K.  The workspace holds one fp32 word per (split, row, column); at rest every word is
-    // kEmptyWord, a NaN pattern no sum of products of bf16 numbers takes.  The workgroups of all splits
-    // but the last write their sums there with device-scope (write-through) stores and are done: they
-    // wait for nothing, not even the stores' acknowledgement.  The workgroup of the LAST split
-    // (dispatched after the others) fetches the words with device-scope loads, reads again whichever
-    // still shows kEmptyWord (a store in flight), adds them in split order with its own sums last,
-    // writes C and puts kEmptyWord back for the next launch.  No counter, no flag, no read-modify-write;
-    // only this workgroup ever waits, and only on workgroups that wait for nothing, so the wait ends
-    // whatever order they run in.  It is bounded all the same: a word that never arrives leaves a NaN
-    // in the output instead of hanging the kernel.
     const size_t split_words = (size_t)p.m * p.n;
     float* const words = reinterpret_cast<float*>(p.partials);
     auto pair_of = [](float lo, float hi) { return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32); };
-    if (ks != p.splits - 1u) {
+
+#pragma unroll
+    for (int mb0 = 0; mb0 < MB; mb0 += kMBC) {
+        const uint32_t pass_row0 = 16u * mb0;  // within the row block
+        if (pass_row0 >= rows_here) break;     // uniform over the workgroup
+        const uint32_t rows_out = rows_here - pass_row0 < 16u * kMBC ? rows_here - pass_row0 : 16u * kMBC;
+        if (mb0 > 0) __syncthreads();          // the previous pass's tiles have been read
+#pragma unroll
+        for (int mbi = 0; mbi < kMBC; ++mbi) {
+            const int mb = mb0 + mbi;
+            if (mb >= MB || !row_ok[mb]) continue;
+            float* row = red + ((size_t)wave * rows_out + (mbi * 16 + nl)) * kRedStride;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                    float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
+                                           acc[mb][4 * c4 + 3][r]);
+                    *reinterpret_cast<float4*>(row + (4 * kg + r) * CPL + 4 * c4) = v;
+                }
+        }
+        __syncthreads();
+        TRACE_MARK(3);
+
+        float4 sum[kMaxR];
 #pragma unroll
         for (uint32_t i = 0; i < kMaxR; ++i) {
             const uint32_t row = rs + i * nrs;
-            if (row < rows_out && col_ok) {
-                unsigned long long* dst = reinterpret_cast<unsigned long long*>(words + (size_t)ks * split_words + (size_t)row * p.n + col);
-                __hip_atomic_store(dst, pair_of(sum[i].x, sum[i].y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(dst + 1, pair_of(sum[i].z, sum[i].w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row < rows_out) {
+                const float* src = red + (size_t)row * kRedStride + 4u * cg;
+                for (uint32_t w = 0; w < nwaves; ++w) {  // fixed order: wave 0 first
+                    const float4 v = *reinterpret_cast<const float4*>(src + (size_t)w * rows_out * kRedStride);
+                    t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+                }
             }
+            sum[i] = t;
         }
-        TRACE_MARK(4);
-        return;
+        const uint32_t first_row = row0 + pass_row0;  // global row of this pass's row 0
+        if (p.splits == 1) {
+#pragma unroll
+            for (uint32_t i = 0; i < kMaxR; ++i) {
+                const uint32_t row = rs + i * nrs;
+                if (row < rows_out && col_ok) {
+                    uint2 o;
+                    o.x = pack_bf16_rne(sum[i].x, sum[i].y);
+                    o.y = pack_bf16_rne(sum[i].z, sum[i].w);
+                    *reinterpret_cast<uint2*>(p.c + (size_t)(first_row + row) * p.ldc + col) = o;
+                }
+            }
+        } else if (ks != p.splits - 1u) {
+            // ---- split-K.  The workspace holds one fp32 word per (split, row, column); at rest every word is
+            // kEmptyWord, a NaN pattern no sum of products of bf16 numbers takes.  The workgroups of all splits
+            // but the last write their sums there with device-scope (write-through) stores and are done: they
+            // wait for nothing, not even the stores' acknowledgement.
+#pragma unroll
+            for (uint32_t i = 0; i < kMaxR; ++i) {
+                const uint32_t row = rs + i * nrs;
+                if (row < rows_out && col_ok) {
+                    unsigned long long* dst =
+                        reinterpret_cast<unsigned long long*>(words + (size_t)ks * split_words + (size_t)(first_row + row) * p.n + col);
+                    __hip_atomic_store(dst, pair_of(sum[i].x, sum[i].y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(dst + 1, pair_of(sum[i].z, sum[i].w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            TRACE_MARK(4);
+        } else {
+            // The workgroup of the LAST split (dispatched after the others) fetches the words with device-scope
+            // loads, reads again whichever still shows kEmptyWord (a store in flight), adds them in split order
+            // with its own sums last, writes C and puts kEmptyWord back for the next launch.  No counter, no
+            // flag, no read-modify-write; only this workgroup ever waits, and only on workgroups that wait for
+            // nothing, so the wait ends whatever order they run in.  It is bounded all the same: a word that
+            // never arrives leaves a NaN in the output instead of hanging the kernel.
+            // Rows a thread has in this pass: a power of two up to kMaxR; the fewer, the more splits are fetched at once.
+            const uint32_t rows_per_thread = (rows_out + nrs - 1u) / nrs;
+            if (rows_per_thread <= 1u) reduce_splits<1>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
+            else if (rows_per_thread <= 2u) reduce_splits<(kMaxR < 2u ? kMaxR : 2u)>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
+            else if (rows_per_thread <= 4u) reduce_splits<(kMaxR < 4u ? kMaxR : 4u)>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
+            else reduce_splits<kMaxR>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
+            TRACE_MARK(5);
+        }
     }
-    // rows this launch gives a thread: a power of two up to kMaxR; the fewer, the more splits are fetched at once
-    const uint32_t rows_per_thread = (rows_out + nrs - 1u) / nrs;
-    if (rows_per_thread <= 1u) reduce_splits<1>(p, sum, rs, nrs, col, col_ok);
-    else if (rows_per_thread <= 2u) reduce_splits<(kMaxR < 2u ? kMaxR : 2u)>(p, sum, rs, nrs, col, col_ok);
-    else if (rows_per_thread <= 4u) reduce_splits<(kMaxR < 4u ? kMaxR : 4u)>(p, sum, rs, nrs, col, col_ok);
-    else reduce_splits<kMaxR>(p, sum, rs, nrs, col, col_ok);
-    TRACE_MARK(5);
 }
 
 template <int BITS, int CPL, int MB, bool GROUPED>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
     constexpr uint32_t kCols = 16u * CPL;
-    const dim3 grid((p.n + kCols - 1u) / kCols, p.splits, 1);
+    constexpr uint32_t kRows = 16u * MB;
     const uint32_t waves = p.decode_waves;
-    const size_t lds = (size_t)decode_red_floats(waves, p.m, kCols) * sizeof(float);
+    if (MB > 2 && waves != 4u) return hipErrorInvalidValue;  // MB = 4 needs the register budget of one wave per SIMD
+    const dim3 grid((p.n + kCols - 1u) / kCols, p.splits, (p.m + kRows - 1u) / kRows);
+    if (grid.z > 65535u) return hipErrorInvalidValue;
+    const uint32_t pass_rows = 16u * (uint32_t)decode_rows16_per_pass(CPL, MB);
+    const size_t lds = (size_t)decode_red_floats(waves, p.m < pass_rows ? p.m : pass_rows, kCols) * sizeof(float);
+    if (lds > 160 * 1024 - 64) return hipErrorInvalidValue;
     if (lds > 64 * 1024) {
         static bool attr_set = false;
         if (!attr_set) {
@@ -430,7 +452,6 @@ static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
             attr_set = true;
         }
     }
-    if (lds > 160 * 1024 - 64) return hipErrorInvalidValue;
     return launch_kernel(bfaintb_decode_kernel<BITS, CPL, MB, GROUPED>, grid, dim3(64 * waves, 1, 1), lds, stream, p);
 }
 
@@ -438,8 +459,15 @@ template <int BITS, int CPL>
 static hipError_t launch_decode_b(const GemmParams& p, hipStream_t stream)
 {
     const bool grouped = p.group_size != 0;
-    if (p.m <= 16) return grouped ? launch_decode_t<BITS, CPL, 1, true>(p, stream) : launch_decode_t<BITS, CPL, 1, false>(p, stream);
-    return grouped ? launch_decode_t<BITS, CPL, 2, true>(p, stream) : launch_decode_t<BITS, CPL, 2, false>(p, stream);
+    switch (p.decode_mb) {
+        case 1: return grouped ? launch_decode_t<BITS, CPL, 1, true>(p, stream) : launch_decode_t<BITS, CPL, 1, false>(p, stream);
+        case 2: return grouped ? launch_decode_t<BITS, CPL, 2, true>(p, stream) : launch_decode_t<BITS, CPL, 2, false>(p, stream);
+        case 4:  // 16 accumulators x 4 blocks x 8 columns = 128 registers: only the 128-column shape has room
+            if constexpr (CPL == 8) return grouped ? launch_decode_t<BITS, CPL, 4, true>(p, stream) : launch_decode_t<BITS, CPL, 4, false>(p, stream);
+            break;
+        default: break;
+    }
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)

@@ -49,6 +49,7 @@ struct GemmParams {
     uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_blocks_per_step * decode_waves)
     uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)
     uint32_t decode_cols;  // columns per workgroup of the decode variant (256, or 128 for 8-bit codes)
+    uint32_t decode_mb;    // blocks of 16 rows of A per workgroup of the decode variant (1, 2 or 4)
     uint32_t splits;     // workgroups along k
     unsigned long long* partials;  // [splits - 1][m][n] fp32 partial sums; kEmptyWord wherever none is waiting
 #ifdef BFAINTB_TRACE

@@ -189,10 +189,20 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
             // the reference's own criterion (exact small-integer data)
             res = valid_vector<CDataType>(c_ref.data(), c_dev.data(), m * n);
         } else {
-            const UlpReport rep = valid_vector_ulp(c_ref.data(), c_dev.data(), (long)m * n);
-            std::printf("ulp check: %ld of %ld outside 2 bf16 ULP (or 1e-2 relative below 1e-3), worst %.3f ULP at %ld\n", rep.failing,
-                        (long)m * n, rep.worst_ulp, rep.worst_index);
-            res = rep.failing == 0;
+            // sum_k |a*w| per output, from the same host routine, bounds the rounding noise of either side's fp32 sum
+            std::vector<float> noise((std::size_t)m * n);
+            for (auto& v : a_seen) v = std::fabs(v);
+            for (auto& v : w_seen) v = std::fabs(v);
+            checker->gemm_rrr(noise.data(), a_seen.data(), w_seen.data(), ones.data(), m, n, k, lda, n, n);
+            const float noise_scale = 2.0f * std::sqrt((float)k) * std::ldexp(1.0f, -24);
+            for (auto& v : noise) v *= noise_scale;
+            const UlpReport rep = valid_vector_ulp(c_ref.data(), c_dev.data(), (long)m * n, 2.0, 1e-3, 1e-2, noise.data());
+            // outputs that cancel to almost nothing: at most 2 in 10^4 (plus one), each within the noise bound
+            const long allowed = (long)((double)m * n * 2e-4) + 1;
+            std::printf("ulp check: %ld of %ld outside 2 bf16 ULP (or 1e-2 relative below 1e-3), %ld more only within the fp32 summation "
+                        "noise (allowed %ld), worst %.3f ULP at %ld\n", rep.failing, (long)m * n, rep.cancelling, allowed, rep.worst_ulp,
+                        rep.worst_index);
+            res = rep.failing == 0 && rep.cancelling <= allowed;
         }
         std::printf(",%s \n", res ? "valid" : "fail");
         if (result) result->validated = res ? 1 : 0;

@@ -43,12 +43,17 @@ inline bool valid_vector(const float* ref, const T* pred, int n, float nrms = 1e
 
 struct UlpReport {
     long failing = 0;
+    long cancelling = 0;  // outside the plain bound, inside the bound widened by the summation noise
     double worst_ulp = 0.0;
     long worst_index = 0;
 };
 
+// `noise`, if given, is a per-element bound on what the rounding of an fp32 sum may contribute on either
+// side (the caller passes 2 * sqrt(k) * 2^-24 * sum_k |a*w|): an output that cancels to almost nothing can
+// differ from the reference by more than two of ITS ULPs whatever order the device adds in.  Such elements
+// are counted separately; the caller decides how many it tolerates.
 inline UlpReport valid_vector_ulp(const float* ref, const bfloat16* pred, long n, double max_ulp = 2.0, double small_abs = 1e-3,
-                                  double small_rel = 1e-2)
+                                  double small_rel = 1e-2, const float* noise = nullptr)
 {
     UlpReport rep;
     for (long i = 0; i < n; ++i) {
@@ -63,6 +68,7 @@ inline UlpReport valid_vector_ulp(const float* ref, const bfloat16* pred, long n
         const double u = err / ulp;
         bool ok = (u <= max_ulp) || (std::fabs(r) < small_abs && err <= small_rel * std::fabs(r));
         if (!(p == p) || !(r == r)) ok = false;
+        else if (!ok && noise != nullptr && err <= max_ulp * ulp + noise[i]) { ok = true; rep.cancelling++; }
         if (!ok) rep.failing++;
         if (u > rep.worst_ulp || !(u == u)) { rep.worst_ulp = u; rep.worst_index = i; }
     }

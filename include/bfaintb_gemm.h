@@ -48,8 +48,8 @@ enum {
 
 /* Which kernel family runs a shape. */
 enum {
-    BFAINTB_VARIANT_AUTO = 0,
-    BFAINTB_VARIANT_DECODE = 1, /* split-K weight-streaming kernel, m <= 32 (HBM-bound) */
+    BFAINTB_VARIANT_AUTO = 0,   /* decode up to m = 32; beyond, whichever the library estimates faster for (m, n, k) */
+    BFAINTB_VARIANT_DECODE = 1, /* split-K weight-streaming kernel (HBM-bound); m > 32 in row blocks; accepts m <= 32768 */
     BFAINTB_VARIANT_PREFILL = 2 /* 256x256 LDS-tiled MFMA kernel (MFMA-bound) */
 };
 
@@ -124,8 +124,9 @@ BFAINTB_API int bfaintb_dequant(void* w, const void* b, const void* scale, uint3
  */
 BFAINTB_API int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream);
 
-/* Name of the __global__ function a variant launches for (weight_bits, group_size, m), as it
- * appears in a kernel trace. */
+/* Name of the __global__ function a variant launches, as it appears in a kernel trace.  Pass what
+ * bfaintb_gemm_variant returned; BFAINTB_VARIANT_AUTO is read as decode up to m = 32, else prefill,
+ * which for 32 < m <= 4096 need not be what bfaintb_gemm picks for a given n and k. */
 BFAINTB_API const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m);
 
 /* Text for a return code of this library (negative codes; positive ones are hipError_t values). */

