@@ -1,0 +1,137 @@
+"""PyTorch binding of the bfAintBGemm C ABI: a custom operator and a linear layer built on it.
+
+The reference is a stand-alone harness with no framework side; its README names the intended use
+("gemm fusion for llm", /root/reference/README.md:2) and its argument block is that of a linear layer's
+forward pass: activations A [m, k], weights B [k, n], per-output-channel scale, output C [m, n]
+(/root/reference/bfAintBGemm/bfAintBGemm.cc:17-28,119-133).  This module lets such a layer call the
+library:
+
+    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size) -> c
+
+``a`` bf16 [m, k] (row stride a multiple of 8 elements), ``b`` uint8 [k, n] (8-bit, excess-128) or
+[k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n]; returns bf16
+[m, n].  torch supplies the output tensor, the current stream and a per-(device, stream) split-K
+workspace; all arithmetic happens in ``libbfaintb_gemm.so``.  There is no CPU implementation: on a CPU
+tensor the operator raises.
+
+``quantize_weight`` (host-side helper, symmetric round-to-nearest) and ``QuantLinear`` are conveniences
+for trying the kernel on a float model; the quantiser is not part of the reference either.
+"""
+import torch
+
+from .gemm import gemm as _gemm, workspace_bytes as _workspace_bytes, workspace_init as _workspace_init
+
+_LIB_NAME = "awesome_fusion"
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    """One split-K workspace per (device, stream): calls ordered on a stream may share it, calls on
+    different streams may overlap and must not."""
+    if nbytes == 0:
+        return None
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 4 << 20), dtype=torch.uint8, device=device)
+        _workspace_init(ws)
+        _workspaces[key] = ws
+    return ws
+
+
+def _check(a, b, scale, weight_bits, group_size):
+    if a.dim() != 2 or b.dim() != 2 or scale.dim() != 2:
+        raise ValueError("bfaintb_gemm: a [m, k], b [k, n*bits/8], scale [groups, n] must be 2-D")
+    if a.dtype != torch.bfloat16 or scale.dtype != torch.bfloat16 or b.dtype != torch.uint8:
+        raise TypeError("bfaintb_gemm: a and scale must be bfloat16, b uint8")
+    if weight_bits not in (8, 4):
+        raise ValueError("bfaintb_gemm: weight_bits must be 8 or 4")
+    k = a.shape[1]
+    n = b.shape[1] * (8 // weight_bits)
+    groups = k // group_size if group_size else 1
+    if b.shape[0] != k or tuple(scale.shape) != (groups, n):
+        raise ValueError(f"bfaintb_gemm: shapes do not agree: a {tuple(a.shape)}, b {tuple(b.shape)}, scale {tuple(scale.shape)}")
+    return a.shape[0], n, k
+
+
+@torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm", mutates_args=())
+def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int) -> torch.Tensor:
+    m, n, k = _check(a, b, scale, weight_bits, group_size)
+    if not a.is_cuda:
+        raise RuntimeError("bfaintb_gemm runs on the GPU only (no CPU implementation)")
+    if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
+        a = a.contiguous()
+    b = b.contiguous()
+    scale = scale.contiguous()
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    if m == 0 or n == 0:
+        return c
+    with torch.cuda.device(a.device):
+        need = _workspace_bytes(m, n, k, weight_bits, group_size)
+        ws = _workspace(a.device, need)
+        _gemm(c, a, b, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, workspace=ws,
+                workspace_nbytes=0 if ws is None else ws.numel())
+    return c
+
+
+@bfaintb_gemm.register_fake
+def _(a, b, scale, weight_bits, group_size):
+    m, n, _k = _check(a, b, scale, weight_bits, group_size)
+    return a.new_empty((m, n))
+
+
+def quantize_weight(weight, weight_bits=8, group_size=0):
+    """float weight [n_out, k_in] (a torch Linear's layout) -> (b uint8 [k, n*bits/8], scale bf16 [groups, n]).
+
+    Symmetric: scale = max|w| over the group / qmax, rounded to bf16 first, q = round(w / scale) clamped to the
+    code range, stored in the library's wire format (excess-128 bytes; excess-8 nibbles, even column low)."""
+    w = weight.detach().float().t().contiguous()  # [k, n]
+    k, n = w.shape
+    g = group_size if group_size else k
+    if k % g or (weight_bits == 4 and n % 2):
+        raise ValueError("quantize_weight: group_size must divide k; 4-bit needs an even n")
+    qmax = 127 if weight_bits == 8 else 7
+    wg = w.view(k // g, g, n)
+    scale = (wg.abs().amax(dim=1) / qmax).clamp_min(1e-12).to(torch.bfloat16)  # [groups, n]
+    q = torch.round(wg / scale.float()[:, None, :]).clamp_(-qmax - 1, qmax).view(k, n).to(torch.int16)
+    if weight_bits == 8:
+        b = (q + 128).to(torch.uint8)
+    else:
+        u = (q + 8).to(torch.uint8)
+        b = (u[:, 0::2] | (u[:, 1::2] << 4)).contiguous()
+    return b, scale
+
+
+class QuantLinear(torch.nn.Module):
+    """y = x @ dequant(B, scale) (+ bias): a Linear whose weight lives as int8/int4 codes and bf16 scales.
+
+    The bias, if any, is added by torch after the GEMM (the library has no fused epilogue)."""
+
+    def __init__(self, in_features, out_features, weight_bits=8, group_size=0, bias=False, device=None):
+        super().__init__()
+        if out_features % 16 or in_features % 64:
+            raise ValueError("QuantLinear: the kernels need out_features % 16 == 0 and in_features % 64 == 0")
+        groups = in_features // group_size if group_size else 1
+        self.in_features, self.out_features = in_features, out_features
+        self.weight_bits, self.group_size = weight_bits, group_size
+        self.register_buffer("qweight", torch.zeros((in_features, out_features * weight_bits // 8), dtype=torch.uint8, device=device))
+        self.register_buffer("scales", torch.zeros((groups, out_features), dtype=torch.bfloat16, device=device))
+        self.bias = torch.nn.Parameter(torch.zeros(out_features, dtype=torch.bfloat16, device=device)) if bias else None
+
+    @classmethod
+    def from_float(cls, linear, weight_bits=8, group_size=0):
+        q = cls(linear.in_features, linear.out_features, weight_bits, group_size, linear.bias is not None, linear.weight.device)
+        b, s = quantize_weight(linear.weight, weight_bits, group_size)
+        q.qweight.copy_(b)
+        q.scales.copy_(s)
+        if linear.bias is not None:
+            q.bias.data.copy_(linear.bias.detach().to(torch.bfloat16))
+        return q
+
+    def forward(self, x):
+        lead = x.shape[:-1]
+        y = torch.ops.awesome_fusion.bfaintb_gemm(x.reshape(-1, self.in_features).to(torch.bfloat16), self.qweight, self.scales,
+                                                  self.weight_bits, self.group_size)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*lead, self.out_features)
