@@ -124,15 +124,16 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         // sums weigh most; large weight matrices stream better in 256-byte row segments.
         // Otherwise, and for 4-bit codes: 256 columns x 4 waves.
         const bool few = weight_bytes <= (32ull << 20);
-        const bool narrow = bits == 8 && (few || (m >= 8 && m <= 16));
+        const bool narrow = bits == 8 && (few || m >= 8);
         pl.cols = narrow ? 128u : 256u;
         pl.waves = narrow ? 8u : 4u;
         pl.mb = m <= 16 ? 1u : 2u;
-        uint32_t target = narrow ? (few ? kDecodeTargetWgsNarrow : kDecodeTargetWgsNarrow * 3u / 2u) : kDecodeTargetWgs;
+        uint32_t target = narrow ? kDecodeTargetWgsNarrow : kDecodeTargetWgs;
         uint32_t capdiv = 256u;
 #ifdef BFAINTB_TUNE
         if (const char* e = getenv("BFAINTB_DECODE_COLS")) {
             if (atoi(e) == 256) { pl.cols = 256u; pl.waves = 4u; target = kDecodeTargetWgs; }
+            if (atoi(e) == 128 && bits == 8) { pl.cols = 128u; pl.waves = 8u; target = kDecodeTargetWgsNarrow; }
         }
         if (const char* e = getenv("BFAINTB_DECODE_TARGET")) target = (uint32_t)atoi(e);
         if (const char* e = getenv("BFAINTB_DECODE_CAPDIV")) capdiv = (uint32_t)atoi(e);
@@ -140,12 +141,23 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
         uint32_t splits = forced_splits;
         if (splits == 0) {
-            // about `target` workgroups: enough waves on every CU to keep the memory system busy ...
-            splits = (target + col_blocks / 2) / col_blocks;
-            // ... while the split-K partial sums (written, read back and cleared as fp32) stay below a quarter of the weight bytes
+            // the split-K partial sums (written, read back and cleared as fp32) stay below a quarter of the weight bytes
             uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (capdiv * (m ? m : 1u)));
             if (cap < 1) cap = 1;
-            if (splits > cap) splits = cap;
+            if (pl.waves == 8u && !few) {
+                // 8-wave workgroups run one per CU: whole rounds of 256 count, and every further split costs
+                // partial-sum traffic and a longer reduction.  Measured at n = 11008, 8192, 28672 (m = 8..32).
+                double best = 0.0;
+                for (uint32_t s = 1; s <= cap && s <= 16u; ++s) {
+                    const double rounds = (double)((col_blocks * s + 255u) / 256u);
+                    const double g = rounds / s + 0.04 * s;
+                    if (best == 0.0 || g < best) { best = g; splits = s; }
+                }
+            } else {
+                // about `target` workgroups: enough waves on every CU to keep the memory system busy
+                splits = (target + col_blocks / 2) / col_blocks;
+                if (splits > cap) splits = cap;
+            }
         }
         set_splits(pl, k, bits, splits);
     }
