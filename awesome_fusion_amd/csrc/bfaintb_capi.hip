@@ -312,7 +312,9 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
         const size_t need = workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k);
         if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
         if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
+        if (need >= (1ull << 31)) return BFAINTB_ERR_BAD_VARIANT;  // the kernel addresses the workspace with 32-bit offsets
         p.partials = static_cast<unsigned long long*>(workspace);
+        p.partial_bytes = (uint32_t)need;
     }
 #ifdef BFAINTB_TRACE
     // timestamp sink: behind the split-K area (instrumented callers pass a larger workspace)

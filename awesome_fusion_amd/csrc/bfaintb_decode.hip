@@ -157,21 +157,25 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 {
     static_assert(R <= NSUM, "rows per thread");
     constexpr uint32_t kSplitBatch = 16u / R;  // splits whose partial sums a thread fetches together
-    constexpr unsigned long long kEmptyPair = ((unsigned long long)kEmptyWord << 32) | kEmptyWord;
     const uint32_t others = p.splits - 1u;
-    const size_t split_words = (size_t)p.m * p.n;
-    float* const words = reinterpret_cast<float*>(p.partials) + (size_t)first_row * p.n;
+    const uint32_t split_bytes = p.m * p.n * 4u;
+    // 16-byte device-scope accesses through a buffer resource over the workspace: four words of one row per
+    // access, each word judged on its own (a 32-bit word is never torn)
+    const __amdgpu_buffer_rsrc_t ws = __builtin_amdgcn_make_buffer_rsrc(p.partials, 0, (int)p.partial_bytes, kBufferFlags);
+    const uint32_t base = (first_row * p.n + (col_ok ? col : 0u)) * 4u;
+    const u32x4_t empty4 = {kEmptyWord, kEmptyWord, kEmptyWord, kEmptyWord};
     float4 total[R];
 #pragma unroll
     for (uint32_t i = 0; i < R; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     for (uint32_t sp0 = 0; sp0 < others; sp0 += kSplitBatch) {
-        unsigned long long v[kSplitBatch][R][2];
+        u32x4_t v[kSplitBatch][R];
         // All words of the batch are fetched together, and fetched again together while any of them is
         // still empty: one memory round trip per attempt, however many words were late.
         // Rows past the last and splits past the last one re-read a word that exists; what they fetch is not used.
         bool complete = false;
         for (uint32_t tries = 0; !complete && tries < kMaxSlotRetries; ++tries) {
             if (tries) __builtin_amdgcn_s_sleep(2);
+            asm volatile("" ::: "memory");  // other workgroups write these words: every attempt really loads
 #pragma unroll
             for (uint32_t j = 0; j < kSplitBatch; ++j) {
                 const uint32_t sp = sp0 + j < others ? sp0 + j : others - 1u;
@@ -179,10 +183,7 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
                 for (uint32_t i = 0; i < R; ++i) {
                     uint32_t row = rs + i * nrs;
                     if (row >= rows) row = rows - 1u;
-                    const unsigned long long* src =
-                        reinterpret_cast<const unsigned long long*>(words + (size_t)sp * split_words + (size_t)row * p.n + (col_ok ? col : 0u));
-                    v[j][i][0] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    v[j][i][1] = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    v[j][i] = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)(base + row * p.n * 4u), (int)(sp * split_bytes), kAuxDeviceScope);
                 }
             }
             complete = true;
@@ -192,8 +193,8 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
                 for (uint32_t i = 0; i < R; ++i)
                     if (sp0 + j < others && rs + i * nrs < rows && col_ok)
 #pragma unroll
-                        for (int h = 0; h < 2; ++h)
-                            if ((uint32_t)v[j][i][h] == kEmptyWord || (uint32_t)(v[j][i][h] >> 32) == kEmptyWord) complete = false;
+                        for (int h = 0; h < 4; ++h)
+                            if (v[j][i][h] == kEmptyWord) complete = false;
         }
         // a word that never arrived is still the empty pattern, a NaN, and turns its sum into one
 #pragma unroll
@@ -202,13 +203,11 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
             for (uint32_t i = 0; i < R; ++i) {
                 const uint32_t row = rs + i * nrs;
                 if (sp0 + j < others && row < rows && col_ok) {
-                    unsigned long long* src = reinterpret_cast<unsigned long long*>(words + (size_t)(sp0 + j) * split_words + (size_t)row * p.n + col);
-                    __hip_atomic_store(src, kEmptyPair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(src + 1, kEmptyPair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    total[i].x += __uint_as_float((uint32_t)v[j][i][0]);
-                    total[i].y += __uint_as_float((uint32_t)(v[j][i][0] >> 32));
-                    total[i].z += __uint_as_float((uint32_t)v[j][i][1]);
-                    total[i].w += __uint_as_float((uint32_t)(v[j][i][1] >> 32));
+                    __builtin_amdgcn_raw_buffer_store_b128(empty4, ws, (int)(base + row * p.n * 4u), (int)((sp0 + j) * split_bytes), kAuxDeviceScope);
+                    total[i].x += __uint_as_float(v[j][i][0]);
+                    total[i].y += __uint_as_float(v[j][i][1]);
+                    total[i].z += __uint_as_float(v[j][i][2]);
+                    total[i].w += __uint_as_float(v[j][i][3]);
                 }
             }
         }
@@ -344,9 +343,6 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
     const uint32_t cg = threadIdx.x % kQuads, rs = threadIdx.x / kQuads, nrs = blockDim.x / kQuads;
     const uint32_t col = cb * kCols + 4u * cg;
     const bool col_ok = col < p.n;
-    const size_t split_words = (size_t)p.m * p.n;
-    float* const words = reinterpret_cast<float*>(p.partials);
-    auto pair_of = [](float lo, float hi) { return (unsigned long long)__float_as_uint(lo) | ((unsigned long long)__float_as_uint(hi) << 32); };
 
 #pragma unroll
     for (int mb0 = 0; mb0 < MB; mb0 += kMBC) {
@@ -402,14 +398,13 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
             // kEmptyWord, a NaN pattern no sum of products of bf16 numbers takes.  The workgroups of all splits
             // but the last write their sums there with device-scope (write-through) stores and are done: they
             // wait for nothing, not even the stores' acknowledgement.
+            const __amdgpu_buffer_rsrc_t ws = __builtin_amdgcn_make_buffer_rsrc(p.partials, 0, (int)p.partial_bytes, kBufferFlags);
 #pragma unroll
             for (uint32_t i = 0; i < kMaxR; ++i) {
                 const uint32_t row = rs + i * nrs;
                 if (row < rows_out && col_ok) {
-                    unsigned long long* dst =
-                        reinterpret_cast<unsigned long long*>(words + (size_t)ks * split_words + (size_t)(first_row + row) * p.n + col);
-                    __hip_atomic_store(dst, pair_of(sum[i].x, sum[i].y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(dst + 1, pair_of(sum[i].z, sum[i].w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const u32x4_t w4 = {__float_as_uint(sum[i].x), __float_as_uint(sum[i].y), __float_as_uint(sum[i].z), __float_as_uint(sum[i].w)};
+                    __builtin_amdgcn_raw_buffer_store_b128(w4, ws, (int)(((first_row + row) * p.n + col) * 4u), (int)(ks * p.m * p.n * 4u), kAuxDeviceScope);
                 }
             }
             TRACE_MARK(4);

@@ -17,6 +17,12 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kBufferFlags = 0x00027000;  // buffer resource word 3: raw buffer, 32-bit data format
+// Cache-policy operand of the raw buffer load/store builtins: device scope (sc1: the store writes through to
+// where every XCD sees it, the load does not settle for a stale local copy).
+constexpr int kAuxDeviceScope = 16;
 
 // A split-K workspace word that holds no partial sum: an all-ones NaN.  Sums of products of bf16 numbers
 // are never this pattern (NaNs born in the arithmetic are the default quiet NaN; NaNs carried over from
@@ -52,6 +58,7 @@ struct GemmParams {
     uint32_t decode_mb;    // blocks of 16 rows of A per workgroup of the decode variant (1, 2 or 4)
     uint32_t splits;     // workgroups along k
     unsigned long long* partials;  // [splits - 1][m][n] fp32 partial sums; kEmptyWord wherever none is waiting
+    uint32_t partial_bytes;        // size of that area (below 2^31)
 #ifdef BFAINTB_TRACE
     unsigned long long* trace;  // timestamp sink (instrumented builds only)
 #endif

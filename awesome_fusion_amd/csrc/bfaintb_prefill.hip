@@ -42,9 +42,7 @@ namespace bfaintb {
 constexpr int kBM = 256, kBN = 256, kBK = 64;
 constexpr uint32_t kTileBytes = 256 * 128;              // one A or W tile in LDS
 constexpr int kCRowBytes = 256 * 2;                     // epilogue staging row: 64 rows fill one 32 KiB tile array
-constexpr int kBufferFlags = 0x00027000;                // raw buffer, 32-bit data format
 
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t swizzled_off(uint32_t row, uint32_t chunk)
 {
