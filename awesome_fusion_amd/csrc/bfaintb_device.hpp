@@ -104,11 +104,13 @@ __device__ __forceinline__ uint32_t codes4_even_to_s8x16(uint32_t x) { return ((
 __device__ __forceinline__ uint32_t codes4_odd_to_s8x16(uint32_t x) { return (x ^ 0x88888888u) & 0xf0f0f0f0u; }
 
 // 16 bits holding four consecutive 4-bit codes (column j in nibble j) -> dword whose byte j reads as int8(16*q_j).
+// Byte 0 of (x << 4) is code 0 in the high nibble over zeros; byte 0 of x has code 1 in its high nibble, byte 1 of
+// (x << 4) code 2, byte 1 of x code 3: one byte permute gathers them, one three-input bit operation clears the low
+// nibbles and flips each code's top bit (excess-8 -> two's complement).
 __device__ __forceinline__ uint32_t codes4_quad_to_s8x16(uint32_t x)
 {
-    const uint32_t y = (x & 0xffu) | ((x & 0xff00u) << 8);  // bytes {c1c0, 0, c3c2, 0}
-    const uint32_t t = y ^ 0x00880088u;
-    return ((t << 4) & 0x00f000f0u) | ((t & 0x00f000f0u) << 8);
+    const uint32_t mixed = __builtin_amdgcn_perm(x << 4, x, 0x01050004u);  // bytes {(x<<4).0, x.0, (x<<4).1, x.1}
+    return (mixed & 0xf0f0f0f0u) ^ 0x80808080u;
 }
 
 // A column's multiplier: the bf16 scale widened to fp32 (times 1/16 for 4-bit codes, see above).
