@@ -10,9 +10,9 @@ reported under "extra".  The metric definitions follow the reference driver's pr
 (/root/reference/bfAintBGemm/bfAintBGemm.cc:186-195: flops = 2mnk, bytes = 2(mk+mn) + nk) with two
 corrections stated in the output: decimal units, and the scale bytes are counted.
 
-Timing: W untimed warm-up launches, then exactly K launches recorded into one HIP graph and replayed
-once between a pair of events on the launch stream (and a host clock, after/before a device
-synchronize).  The graph keeps host launch overhead out of a microsecond-scale kernel's
+Timing: W untimed warm-up launches, then exactly K launches recorded into one HIP graph; the graph is
+replayed five times, each replay between its own pair of events on the launch stream (and a host
+clock, after/before a device synchronize), and the median replay is reported.  The graph keeps host launch overhead out of a microsecond-scale kernel's
 measurement; the reference's own protocol is the same minus the graph (10 launches in one event pair,
 bfAintBGemm.cc:171-186).  For the decode shape consecutive launches read DIFFERENT copies of B
 (enough copies to exceed the 256 MB last-level cache), so the figure is an HBM figure; the
@@ -32,12 +32,13 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 LLC_BYTES = 256 << 20
+REPLAYS = 5                   # timed replays of the K-launch graph; the median one is reported
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
 MEASURED_TRAFFIC_BYTES = {
-    # fetch 8404.8 KiB x 1.997 + write 456.0 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
-    "decode_m1_n4096_k4096_int8_perchannel": 17654154,
+    # fetch 8399.2 KiB x 1.997 + write 232.0 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
+    "decode_m1_n4096_k4096_int8_perchannel": 17413327,
     # fetch 65627.0 KiB x 1.997 + write 32768.0 KiB
     "prefill_m4096_n4096_k4096_int8_perchannel": 167756921,
 }
@@ -101,15 +102,20 @@ def time_graph(af, w, steps, warmup, rotate):
             launch(i)
     g.replay()  # untimed: first replay pays graph upload
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0.record()
-    g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    return e0.elapsed_time(e1) / steps, (t1 - t0) * 1e3 / steps
+    ev, wall = [], []
+    for _ in range(REPLAYS):  # each replay is exactly `steps` launches inside one event pair; the median replay is reported
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ev.append(e0.elapsed_time(e1) / steps)
+        wall.append((t1 - t0) * 1e3 / steps)
+    mid = sorted(range(REPLAYS), key=lambda i: ev[i])[REPLAYS // 2]
+    return ev[mid], wall[mid]
 
 
 def time_read_ceiling(af, w, steps, warmup):
@@ -252,7 +258,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (decode sweep, int4 group-128)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="time only this workload family: decode | prefill")
+    ap.add_argument("--only", default="", help="time only this workload family: decode | prefill | decode_cold "
+                    "(decode_cold: nothing but the headline's cold-B launches, for a kernel trace without the hot and eager variants)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM shards over n with no "
@@ -270,13 +277,14 @@ def main():
 
     # ---- headline: decode M=1, N=K=4096, int8 per-channel; cold B (rotating copies > last-level cache)
     res = None
-    if args.only in ("", "decode"):
+    cold_only = args.only == "decode_cold"
+    if args.only in ("", "decode", "decode_cold"):
         copies = LLC_BYTES * 2 // (4096 * 4096) + 8  # 40 copies = 640 MiB
         w = Workload("decode_m1_n4096_k4096_int8_perchannel", 1, 4096, 4096, copies=copies)
         ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True)
-        hot_ms, _ = time_graph(af, w, K, W, rotate=False)
-        eager_ms = time_eager(af, w, K, W)
-        read_ms = time_read_ceiling(af, w, K, W)
+        hot_ms, _ = (ev_ms, wall_ms) if cold_only else time_graph(af, w, K, W, rotate=False)
+        eager_ms = ev_ms if cold_only else time_eager(af, w, K, W)
+        read_ms = ev_ms if cold_only else time_read_ceiling(af, w, K, W)
         c_gpu = w.c.float().cpu().numpy()
         res = {
             "metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=1: effective HBM bandwidth (algorithmic bytes / time per launch, B cold)",
@@ -284,20 +292,21 @@ def main():
             "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic",
             "config": {"workload": w.name, "m": 1, "n": 4096, "k": 4096, "weight_bits": 8, "group_size": 0,
-                       "b_copies_rotated": copies, "split_k": af.split_k(1, 4096, 4096), "launch": "hip graph of K launches",
+                       "b_copies_rotated": copies, "split_k": af.split_k(1, 4096, 4096), "launch": "hip graph of K launches, median of 5 replays",
                        "units": "decimal; scale bytes counted"},
             "roofline": roofline_entry(w, ev_ms, "hbm"),
         }
         res["tflops"] = round(w.flops / (wall_ms * 1e-3) / 1e12, 4)
         b_bytes = w.b[0].numel()
-        res["roofline"]["fetch_only_kernel_us"] = round(read_ms * 1e3, 3)
-        res["roofline"]["fetch_only_GBps"] = round(b_bytes / read_ms / 1e6, 1)
-        res["roofline"]["frac_of_fetch_only"] = round(read_ms / ev_ms, 4)
-        out_extra["decode_m1_hot_same_buffer"] = {"kernel_us": round(hot_ms * 1e3, 3), "GB/s": round(w.bytes / hot_ms / 1e6, 1),
-                                                  "note": "B re-read from cache: not an HBM figure"}
-        out_extra["decode_m1_eager_launch_loop"] = {"us_per_launch": round(eager_ms * 1e3, 3),
-                                                    "note": "reference protocol (no graph): host launch rate included"}
-        if not args.no_cpu:
+        if not cold_only:
+            res["roofline"]["fetch_only_kernel_us"] = round(read_ms * 1e3, 3)
+            res["roofline"]["fetch_only_GBps"] = round(b_bytes / read_ms / 1e6, 1)
+            res["roofline"]["frac_of_fetch_only"] = round(read_ms / ev_ms, 4)
+            out_extra["decode_m1_hot_same_buffer"] = {"kernel_us": round(hot_ms * 1e3, 3), "GB/s": round(w.bytes / hot_ms / 1e6, 1),
+                                                      "note": "B re-read from cache: not an HBM figure"}
+            out_extra["decode_m1_eager_launch_loop"] = {"us_per_launch": round(eager_ms * 1e3, 3),
+                                                        "note": "reference protocol (no graph): host launch rate included"}
+        if not args.no_cpu and not cold_only:
             one, allc, nrms = cpu_baseline(w, c_gpu)
             res["cpu_baseline"] = one
             out_extra["cpu_baseline_all_cores"] = allc
