@@ -263,9 +263,9 @@ int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream
                                          static_cast<hipStream_t>(stream));
 }
 
-int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
-                    uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
-                    size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
+static int gemm_impl(void* c, const void* a, const void* b, const void* scale, const void* bias, uint32_t m, uint32_t n, uint32_t k,
+                     uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
 {
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
@@ -276,9 +276,10 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
     if (c == nullptr || a == nullptr || b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
-    if (misaligned16(c) || misaligned16(a) || misaligned16(b) || misaligned16(scale)) return BFAINTB_ERR_ALIGNMENT;
+    if (misaligned16(c) || misaligned16(a) || misaligned16(b) || misaligned16(scale) || misaligned16(bias)) return BFAINTB_ERR_ALIGNMENT;
 
     GemmParams p{};
+    p.bias = static_cast<const uint16_t*>(bias);
     p.c = static_cast<uint16_t*>(c);
     p.a = static_cast<const uint16_t*>(a);
     p.b = static_cast<const uint8_t*>(b);
@@ -321,6 +322,22 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
     p.trace = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + ((workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) + 255) & ~(size_t)255));
 #endif
     return (int)bfaintb::launch_decode(p, weight_bits, st);
+}
+
+int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
+                    uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                    size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
+{
+    return gemm_impl(c, a, b, scale, nullptr, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
+                     variant, split_k);
+}
+
+int bfaintb_gemm_bias(void* c, const void* a, const void* b, const void* scale, const void* bias, uint32_t m, uint32_t n,
+                      uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                      size_t workspace_bytes, void* stream)
+{
+    return gemm_impl(c, a, b, scale, bias, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
+                     BFAINTB_VARIANT_AUTO, 0);
 }
 
 int bfaintb_gemm(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,

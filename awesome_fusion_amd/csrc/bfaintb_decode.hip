@@ -147,6 +147,18 @@ __host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t r
     return waves * rows * (cols + 4u);
 }
 
+// t += bias[col .. col+3] (fp32), if the launch has a bias.
+__device__ __forceinline__ void add_bias4(const GemmParams& p, float4& t, uint32_t col)
+{
+    if (p.bias != nullptr) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(p.bias + col);
+        t.x += bf16_bits_to_f32(raw.x & 0xffffu);
+        t.y += bf16_bits_to_f32(raw.x >> 16);
+        t.z += bf16_bits_to_f32(raw.y & 0xffffu);
+        t.w += bf16_bits_to_f32(raw.y >> 16);
+    }
+}
+
 // Split-K, the reducing workgroup's part for one thread: R rows (first_row + rs, + nrs, ...; `rows` of
 // them exist from first_row on) of 4 columns.  Fetches the other splits' partial sums, adds them in
 // split order with the thread's own sums last, writes bf16 C and leaves the workspace words empty
@@ -216,9 +228,11 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
     for (uint32_t i = 0; i < R; ++i) {
         const uint32_t row = rs + i * nrs;
         if (row < rows && col_ok) {
+            float4 t = make_float4(total[i].x + sum[i].x, total[i].y + sum[i].y, total[i].z + sum[i].z, total[i].w + sum[i].w);
+            add_bias4(p, t, col);
             uint2 o;
-            o.x = pack_bf16_rne(total[i].x + sum[i].x, total[i].y + sum[i].y);
-            o.y = pack_bf16_rne(total[i].z + sum[i].z, total[i].w + sum[i].w);
+            o.x = pack_bf16_rne(t.x, t.y);
+            o.y = pack_bf16_rne(t.z, t.w);
             *reinterpret_cast<uint2*>(p.c + (size_t)(first_row + row) * p.ldc + col) = o;
         }
     }
@@ -387,9 +401,11 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
             for (uint32_t i = 0; i < kMaxR; ++i) {
                 const uint32_t row = rs + i * nrs;
                 if (row < rows_out && col_ok) {
+                    float4 t = sum[i];
+                    add_bias4(p, t, col);
                     uint2 o;
-                    o.x = pack_bf16_rne(sum[i].x, sum[i].y);
-                    o.y = pack_bf16_rne(sum[i].z, sum[i].w);
+                    o.x = pack_bf16_rne(t.x, t.y);
+                    o.y = pack_bf16_rne(t.z, t.w);
                     *reinterpret_cast<uint2*>(p.c + (size_t)(first_row + row) * p.ldc + col) = o;
                 }
             }

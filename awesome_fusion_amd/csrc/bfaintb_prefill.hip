@@ -321,13 +321,23 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     {
         const uint32_t jl = lane & 31u, half = lane >> 5;
         const uint32_t colbyte = 8u * (32u * (wn & 1u) + jl) + 4u * (wn >> 1);
+        // this lane's two columns of the tile are colbyte/2 and the next: their bias, if the launch has one
+        float bias0 = 0.f, bias1 = 0.f;
+        const bool has_bias = p.bias != nullptr;
+        if (has_bias && n0 + colbyte / 2u < p.n) {
+            const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.bias + n0 + colbyte / 2u);
+            bias0 = bf16_bits_to_f32(raw & 0xffffu);
+            bias1 = bf16_bits_to_f32(raw >> 16);
+        }
 #pragma unroll
         for (uint32_t mt = 0; mt < 4; ++mt) {
             uint8_t* base = c_rows(wm * 2u + (mt >> 1));
 #pragma unroll
             for (uint32_t i = 0; i < 16; ++i) {
                 const uint32_t row = 32u * (mt & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
-                *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) = pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                // without a bias the sums are stored as they are (adding +0 would turn a -0 sum into +0)
+                *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) =
+                    has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
             }
         }
     }

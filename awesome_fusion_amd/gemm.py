@@ -55,6 +55,9 @@ def lib():
                                    C.c_size_t, _vp]
         L.bfaintb_gemm_ex.restype = C.c_int
         L.bfaintb_gemm_ex.argtypes = L.bfaintb_gemm.argtypes + [C.c_int, _u32]
+        L.bfaintb_gemm_bias.restype = C.c_int
+        L.bfaintb_gemm_bias.argtypes = [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
+                                        C.c_size_t, _vp]
         L.bfaintb_gemm_workspace_bytes.restype = C.c_size_t
         L.bfaintb_gemm_workspace_bytes.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
         L.bfaintb_gemm_workspace_bytes_ex.restype = C.c_size_t
@@ -124,16 +127,22 @@ def workspace_init(workspace, nbytes=None, stream=None):
 
 
 def gemm(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, group_size=0, workspace=None,
-         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True):
-    """C = A x dequant(B, scale) through bfaintb_gemm_ex.  Returns the library's return code
-    (raises on non-zero when ``check``)."""
+         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True, bias=None):
+    """C = A x dequant(B, scale) through bfaintb_gemm_ex, or (+ bias, AUTO variant only) through
+    bfaintb_gemm_bias.  Returns the library's return code (raises on non-zero when ``check``)."""
     lda = k if lda is None else lda
     ldb = n if ldb is None else ldb
     ldc = n if ldc is None else ldc
     if workspace_nbytes is None:
         workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
-    rc = lib().bfaintb_gemm_ex(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), m, n, k, lda, ldb, ldc, weight_bits, group_size,
-                               _ptr(workspace), workspace_nbytes, _stream_handle(stream), which, force_split_k)
+    if bias is not None:
+        if which != AUTO or force_split_k:
+            raise ValueError("bfaintb_gemm_bias takes no forced variant or split factor")
+        rc = lib().bfaintb_gemm_bias(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), _ptr(bias), m, n, k, lda, ldb, ldc, weight_bits,
+                                     group_size, _ptr(workspace), workspace_nbytes, _stream_handle(stream))
+    else:
+        rc = lib().bfaintb_gemm_ex(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), m, n, k, lda, ldb, ldc, weight_bits, group_size,
+                                   _ptr(workspace), workspace_nbytes, _stream_handle(stream), which, force_split_k)
     if rc and check:
         raise BfaintbError(rc, "bfaintb_gemm")
     return rc

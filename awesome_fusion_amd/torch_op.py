@@ -6,17 +6,19 @@ forward pass: activations A [m, k], weights B [k, n], per-output-channel scale, 
 (/root/reference/bfAintBGemm/bfAintBGemm.cc:17-28,119-133).  This module lets such a layer call the
 library:
 
-    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size) -> c
+    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size, bias=None) -> c
 
 ``a`` bf16 [m, k] (row stride a multiple of 8 elements), ``b`` uint8 [k, n] (8-bit, excess-128) or
-[k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n]; returns bf16
-[m, n].  torch supplies the output tensor, the current stream and a per-(device, stream) split-K
+[k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n], ``bias`` bf16 [n]
+(added to the fp32 sums before the rounding, inside the kernel); returns bf16 [m, n].  torch supplies the output tensor, the current stream and a per-(device, stream) split-K
 workspace; all arithmetic happens in ``libbfaintb_gemm.so``.  There is no CPU implementation: on a CPU
 tensor the operator raises.
 
 ``quantize_weight`` (host-side helper, symmetric round-to-nearest) and ``QuantLinear`` are conveniences
 for trying the kernel on a float model; the quantiser is not part of the reference either.
 """
+from typing import Optional
+
 import torch
 
 from .gemm import gemm as _gemm, workspace_bytes as _workspace_bytes, workspace_init as _workspace_init
@@ -39,7 +41,7 @@ def _workspace(device, nbytes):
     return ws
 
 
-def _check(a, b, scale, weight_bits, group_size):
+def _check(a, b, scale, weight_bits, group_size, bias=None):
     if a.dim() != 2 or b.dim() != 2 or scale.dim() != 2:
         raise ValueError("bfaintb_gemm: a [m, k], b [k, n*bits/8], scale [groups, n] must be 2-D")
     if a.dtype != torch.bfloat16 or scale.dtype != torch.bfloat16 or b.dtype != torch.uint8:
@@ -51,18 +53,23 @@ def _check(a, b, scale, weight_bits, group_size):
     groups = k // group_size if group_size else 1
     if b.shape[0] != k or tuple(scale.shape) != (groups, n):
         raise ValueError(f"bfaintb_gemm: shapes do not agree: a {tuple(a.shape)}, b {tuple(b.shape)}, scale {tuple(scale.shape)}")
+    if bias is not None and (bias.dtype != torch.bfloat16 or tuple(bias.shape) != (n,)):
+        raise ValueError("bfaintb_gemm: bias must be bfloat16 [n]")
     return a.shape[0], n, k
 
 
 @torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm", mutates_args=())
-def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int) -> torch.Tensor:
-    m, n, k = _check(a, b, scale, weight_bits, group_size)
+def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
+                 bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    m, n, k = _check(a, b, scale, weight_bits, group_size, bias)
     if not a.is_cuda:
         raise RuntimeError("bfaintb_gemm runs on the GPU only (no CPU implementation)")
     if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
         a = a.contiguous()
     b = b.contiguous()
     scale = scale.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
     c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
     if m == 0 or n == 0:
         return c
@@ -70,13 +77,13 @@ def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_b
         need = _workspace_bytes(m, n, k, weight_bits, group_size)
         ws = _workspace(a.device, need)
         _gemm(c, a, b, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, workspace=ws,
-                workspace_nbytes=0 if ws is None else ws.numel())
+              workspace_nbytes=0 if ws is None else ws.numel(), bias=bias)
     return c
 
 
 @bfaintb_gemm.register_fake
-def _(a, b, scale, weight_bits, group_size):
-    m, n, _k = _check(a, b, scale, weight_bits, group_size)
+def _(a, b, scale, weight_bits, group_size, bias=None):
+    m, n, _k = _check(a, b, scale, weight_bits, group_size, bias)
     return a.new_empty((m, n))
 
 
@@ -105,7 +112,7 @@ def quantize_weight(weight, weight_bits=8, group_size=0):
 class QuantLinear(torch.nn.Module):
     """y = x @ dequant(B, scale) (+ bias): a Linear whose weight lives as int8/int4 codes and bf16 scales.
 
-    The bias, if any, is added by torch after the GEMM (the library has no fused epilogue)."""
+    The bias, if any, is added inside the kernel, to the fp32 sums."""
 
     def __init__(self, in_features, out_features, weight_bits=8, group_size=0, bias=False, device=None):
         super().__init__()
@@ -131,7 +138,5 @@ class QuantLinear(torch.nn.Module):
     def forward(self, x):
         lead = x.shape[:-1]
         y = torch.ops.awesome_fusion.bfaintb_gemm(x.reshape(-1, self.in_features).to(torch.bfloat16), self.qweight, self.scales,
-                                                  self.weight_bits, self.group_size)
-        if self.bias is not None:
-            y = y + self.bias
+                                                  self.weight_bits, self.group_size, self.bias)
         return y.reshape(*lead, self.out_features)

@@ -33,7 +33,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 100 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 101 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -90,6 +90,16 @@ BFAINTB_API int bfaintb_gemm(void* c, const void* a, const void* b, const void* 
 BFAINTB_API int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
                     uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k);
+
+/*
+ * The GEMM with a fused bias: C[m,n] = bf16_rne(sum_k A[m,k]*W[k,n] + bias[n]), the bias (bf16 [n], 16-byte
+ * aligned) added to the fp32 sum before the one rounding.  bias == NULL is bfaintb_gemm.  No counterpart in the
+ * reference, whose kernel stores the sums as they are (bf16gemm_kernel_gfx90a.s:594-630); it is the first of the
+ * epilogues a linear layer wants (the reference's stated purpose, README.md:2).  Same workspace as bfaintb_gemm.
+ */
+BFAINTB_API int bfaintb_gemm_bias(void* c, const void* a, const void* b, const void* scale, const void* bias, uint32_t m,
+                      uint32_t n, uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* Scratch the GEMM needs for a shape: one fp32 word per (split but the last, row, column) of the
  * split-K partial sums, rounded up to 256 bytes; 0 when the shape runs without split-K.  Depends only

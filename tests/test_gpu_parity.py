@@ -204,6 +204,29 @@ def test_decode_family_with_row_blocks_matches_oracle(af, m, n, k, bits, group, 
     assert np.array_equal(run_gemm(p, which=af.DECODE, force_split_k=split), c), "not reproducible"
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (1, 4096, 4096, 8, 0),      # decode, split-K: the bias joins in the reducing workgroup
+    (16, 528, 512, 4, 128),     # decode without split-K
+    (100, 1040, 1024, 8, 0),    # decode family in row blocks
+    (300, 784, 512, 8, 128),    # prefill kernel, ragged tile edges
+    (4096, 512, 256, 4, 0),
+])
+def test_fused_bias(af, m, n, k, bits, group):
+    """bfaintb_gemm_bias: C = bf16(sum + bias).  Checked against the oracle's fp32 sums plus the bias, and through
+    two closed forms: zero activations return the bias itself, and a zero bias returns bfaintb_gemm's bits."""
+    p = Problem(m, n, k, bits, group, seed=700 + m).with_bias(seed=m)
+    assert_close_ulp(p, run_gemm(p), f"bias m={m}")
+    plain = Problem(m, n, k, bits, group, seed=700 + m)
+    c_plain = run_gemm(plain)
+    p.bias_bf = np.zeros(n, np.uint16)
+    c_zero_bias = run_gemm(p)
+    # x + (+0) == x except that -0 becomes +0
+    assert np.array_equal(np.where(c_plain == 0x8000, 0, c_plain), c_zero_bias)
+    p.with_bias(seed=m)
+    p.a_bf = np.zeros_like(p.a_bf)
+    assert np.array_equal(run_gemm(p), np.broadcast_to(p.bias_bf, (m, n)))
+
+
 def test_row_permutation_permutes_output(af):
     # size-independent property at a prefill shape: rows of A are independent
     p = Problem(512, 512, 512, seed=5)

@@ -82,7 +82,7 @@ def test_quant_linear_forward():
     # comparison against the oracle is the operator test above
     q = ql.qweight.to(torch.int16) - 128
     w = (q.float() * ql.scales.float().repeat_interleave(128, dim=0)).to(torch.bfloat16).float()
-    ref = x.to(torch.bfloat16).float().reshape(-1, 512) @ w + ql.bias.float()
+    ref = x.to(torch.bfloat16).float().reshape(-1, 512) @ w + ql.bias.float()  # the kernel adds the bias to its fp32 sums
     assert torch.allclose(y.float().reshape(-1, 256), ref, rtol=2e-2, atol=2e-2)
     # and the quantised layer tracks the float layer it came from
     assert (y.float() - lin(x)).abs().max() < 0.05
