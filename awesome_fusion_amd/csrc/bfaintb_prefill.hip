@@ -226,6 +226,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         using Other = std::integral_constant<uint32_t, S ^ 1u>;
         uint32_t b_s8[8];
         // Q1
+        __builtin_amdgcn_s_setprio(0);
         dma_a(Other{}, kt + 1 < ksteps ? kt + 1 : kt);
         read_frags(stage_c, C1{}, af1, wf1);
         mma(af0, wf0);
@@ -275,6 +276,10 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         PF_MARK(2);
+        // From here to the end of the step this wave outranks its SIMD neighbour: past the barrier it holds the
+        // fragments of the next stage's first quarter and should start on them at once, ahead of a neighbour
+        // still converting weights (measured: 5-6 % at M = 4096 and 8192; raising other quarters gains less).
+        __builtin_amdgcn_s_setprio(1);
         // this wave's part of the next A tile has landed in LDS (the 8 W loads issued after it may still fly)
         asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         __syncthreads();
@@ -313,6 +318,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     if (lane == 0 && p.trace != nullptr)
         for (int i = 0; i < 5; ++i) p.trace[(size_t)(blockIdx.x * 8 + wave) * 8 + i] = (unsigned long long)tq[i];
 #endif
+    __builtin_amdgcn_s_setprio(0);
     // ---- epilogue: bf16 tile through LDS (rows 64q..64q+63 in the q-th of the four arrays), then
     //      16-byte row-contiguous stores
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
