@@ -236,7 +236,9 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         read_frags(stage_c, C2{}, af0, wf0);
         update_scales(kt + 1 < ksteps ? kt + 1 : kt);
         prepare(b_s8);
-        gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
+        // the raw W tile of step kt+2 goes into the registers just freed: here for 8-bit codes, a quarter later for
+        // 4-bit codes, whose conversion makes this quarter the longest (measured: each placement wins for its format)
+        if constexpr (BITS == 8) gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
         store_w_col(Other{}, J0{}, b_s8);
         store_w_col(Other{}, J1{}, b_s8);
         mma(af1, wf1);
@@ -247,7 +249,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);
+        if constexpr (BITS == 8) __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -262,10 +264,12 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         PF_MARK(1);
         // Q3
         read_frags(stage_c, C3{}, af1, wf1);
+        if constexpr (BITS == 4) gload(kt + 2 < ksteps ? kt + 2 : ksteps - 1);
         store_w_col(Other{}, J2{}, b_s8);
         store_w_col(Other{}, J3{}, b_s8);
         mma(af0, wf0);
         __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+        if constexpr (BITS == 4) __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
