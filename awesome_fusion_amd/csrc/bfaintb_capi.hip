@@ -118,59 +118,44 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         }
         pl = best;
     } else {
-        // 8-bit codes, 128 columns x 8 waves (a lane loads 8 bytes of a row, 16 lanes one 128-byte line): half
-        // the splits, so half the partial-sum traffic, for the same number of waves.  Measured faster than the
-        // wide block while the weights are few (the launch is latency-bound) and for the m where the partial
-        // sums weigh most; large weight matrices stream better in 256-byte row segments.
-        // Otherwise, and for 4-bit codes: 256 columns x 4 waves.
+        // 8-bit codes, 128 columns x 8 waves ("narrow": a lane loads 8 bytes of a row, 16 lanes one 128-byte line)
+        // needs half the splits of 256 columns x 4 waves ("wide") for the same number of waves, so half the
+        // partial-sum traffic.  Narrow workgroups run one per CU, so they pay for a ragged last round of 256.
+        // Measured (n = 4096, 8192, 11008, 28672): narrow wins while the weights are few (latency-bound
+        // launch), for m >= 8 (partial sums weigh most), and elsewhere when its best split factor fills whole
+        // rounds; otherwise large matrices stream better in 256-byte row segments.  4-bit codes: wide.
         const bool few = weight_bytes <= (32ull << 20);
-        const bool narrow = bits == 8 && (few || m >= 8);
+        // the split-K partial sums (written, read back and cleared as fp32) stay below a quarter of the weight bytes
+        uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (256u * (m ? m : 1u)));
+        if (cap < 1) cap = 1;
+        // narrow, large matrix: every further split costs traffic and a longer reduction; whole rounds count
+        const uint32_t narrow_blocks = (n + 127u) / 128u;
+        uint32_t narrow_splits = 1;
+        double best = 0.0;
+        for (uint32_t s = 1; s <= cap && s <= 16u; ++s) {
+            const double rounds = (double)((narrow_blocks * s + 255u) / 256u);
+            const double g = rounds / s + 0.04 * s * 4096.0 / k;  // time of the rounds + what a split costs, both relative to one pass over k
+            if (best == 0.0 || g < best) { best = g; narrow_splits = s; }
+        }
+        const uint32_t narrow_wgs = narrow_blocks * narrow_splits;
+        const bool fills_rounds = narrow_wgs * 20u >= ((narrow_wgs + 255u) / 256u) * 256u * 19u;  // >= 95 % of whole rounds
+        const bool narrow = bits == 8 && (few || m >= 8 || fills_rounds);
         pl.cols = narrow ? 128u : 256u;
         pl.waves = narrow ? 8u : 4u;
         pl.mb = m <= 16 ? 1u : 2u;
-        uint32_t target = narrow ? kDecodeTargetWgsNarrow : kDecodeTargetWgs;
-        uint32_t capdiv = 256u;
-#ifdef BFAINTB_TUNE
-        if (const char* e = getenv("BFAINTB_DECODE_COLS")) {
-            if (atoi(e) == 256) { pl.cols = 256u; pl.waves = 4u; target = kDecodeTargetWgs; }
-            if (atoi(e) == 128 && bits == 8) { pl.cols = 128u; pl.waves = 8u; target = kDecodeTargetWgsNarrow; }
-        }
-        if (const char* e = getenv("BFAINTB_DECODE_TARGET")) target = (uint32_t)atoi(e);
-        if (const char* e = getenv("BFAINTB_DECODE_CAPDIV")) capdiv = (uint32_t)atoi(e);
-#endif
-        const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
         uint32_t splits = forced_splits;
         if (splits == 0) {
-            // the split-K partial sums (written, read back and cleared as fp32) stay below a quarter of the weight bytes
-            uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (capdiv * (m ? m : 1u)));
-            if (cap < 1) cap = 1;
-            if (pl.waves == 8u && !few) {
-                // 8-wave workgroups run one per CU: whole rounds of 256 count, and every further split costs
-                // partial-sum traffic and a longer reduction.  Measured at n = 11008, 8192, 28672 (m = 8..32).
-                double best = 0.0;
-                for (uint32_t s = 1; s <= cap && s <= 16u; ++s) {
-                    const double rounds = (double)((col_blocks * s + 255u) / 256u);
-                    const double g = rounds / s + 0.04 * s;
-                    if (best == 0.0 || g < best) { best = g; splits = s; }
-                }
+            if (narrow && !few) {
+                splits = narrow_splits;
             } else {
-                // about `target` workgroups: enough waves on every CU to keep the memory system busy
-                splits = (target + col_blocks / 2) / col_blocks;
+                // about 256 narrow or 480 wide workgroups: enough waves on every CU to keep the memory system busy
+                const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
+                splits = ((narrow ? kDecodeTargetWgsNarrow : kDecodeTargetWgs) + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
             }
         }
         set_splits(pl, k, bits, splits);
     }
-#ifdef BFAINTB_TUNE
-    if (const char* e = getenv("BFAINTB_DECODE_MB")) {
-        pl.mb = (uint32_t)atoi(e);
-        pl.waves = pl.mb > 2 ? 4u : 8u;
-        if (const char* w = getenv("BFAINTB_DECODE_WAVES")) pl.waves = (uint32_t)atoi(w);
-        if (pl.mb == 4 && pl.cols != 128u) pl.mb = 2u;
-        if (const char* sp = getenv("BFAINTB_DECODE_SPLITS")) set_splits(pl, k, bits, (uint32_t)atoi(sp));
-        else set_splits(pl, k, bits, pl.splits);
-    }
-#endif
     return pl;
 }
 
