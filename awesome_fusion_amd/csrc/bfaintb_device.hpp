@@ -52,6 +52,8 @@ struct GemmParams {
     uint32_t ldc;        // elements
     uint32_t lds;        // elements per scale row (= n)
     uint32_t group_size; // rows of k per scale group; 0 = one group
+    // prefill variant: the logical 256x256 tiles one launch covers
+    uint32_t tile_first, tile_count;
     // split-K (decode variant only)
     uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_blocks_per_step * decode_waves)
     uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)

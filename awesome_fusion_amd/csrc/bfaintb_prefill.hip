@@ -49,9 +49,13 @@ __device__ __forceinline__ uint32_t swizzled_off(uint32_t row, uint32_t chunk)
     return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
 
-template <int BITS, bool GROUPED>
+// MT = blocks of 32 rows per wave along m: 4 for the 256-row tile, 2 for a 128-row half tile.  Half tiles take
+// over the tiles of a last, less than half full round of 256 workgroups: twice as many workgroups, each with half
+// the matrix instructions (and all of the weight conversion), finish sooner than half-idle CUs running whole tiles.
+template <int BITS, bool GROUPED, int MT>
 __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p)
 {
+    constexpr uint32_t kRows = 64u * MT;  // rows of C per workgroup
     // Four separate LDS arrays (A and W tiles, two stages each) rather than one block: the compiler
     // then knows that fragment reads of one stage cannot alias the asynchronous global->LDS writes
     // into the other, and does not make them wait for those writes.
@@ -70,21 +74,25 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 
     // ---- tile of this workgroup: ids that share an XCD (id mod 8) cover consecutive logical ids;
     //      logical ids walk groups of 4 tile-rows column by column
+    //      This launch covers logical tiles tile_first .. tile_first + tile_count - 1 (two workgroups per tile when MT = 2).
     const uint32_t tiles_m = (p.m + kBM - 1) / kBM, tiles_n = (p.n + kBN - 1) / kBN;
-    const uint32_t total = tiles_m * tiles_n;
-    const uint32_t per_xcd = (total + 7u) / 8u;
-    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
+    const uint32_t wgs = p.tile_count * (4u / MT);
+    const uint32_t per_xcd = (wgs + 7u) / 8u;
+    const uint32_t local = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if (local >= wgs) return;
+    const uint32_t logical = p.tile_first + local / (4u / MT);
+    const uint32_t mhalf = MT == 4 ? 0u : (local & 1u);
     const uint32_t group = logical / (4u * tiles_n);
     const uint32_t first_m = group * 4u;
     const uint32_t group_rows = tiles_m - first_m < 4u ? tiles_m - first_m : 4u;
     const uint32_t in_group = logical - group * 4u * tiles_n;
     const uint32_t tm = first_m + in_group % group_rows;
     const uint32_t tn = in_group / group_rows;
-    const uint32_t m0 = tm * kBM, n0 = tn * kBN;
+    const uint32_t m0 = tm * kBM + mhalf * kRows, n0 = tn * kBN;
+    if (m0 >= p.m) return;  // the lower half of a tile that ends in its upper half
 
     // ---- buffer resources over this tile's rows of A and columns of B
-    const uint32_t rows_valid = p.m - m0 < (uint32_t)kBM ? p.m - m0 : (uint32_t)kBM;
+    const uint32_t rows_valid = p.m - m0 < kRows ? p.m - m0 : kRows;
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)(((rows_valid - 1u) * p.lda + p.k) * 2u), kBufferFlags);
     const uint32_t cols_valid = p.n - n0 < (uint32_t)kBN ? p.n - n0 : (uint32_t)kBN;
@@ -93,12 +101,14 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         kBufferFlags);
 
     // A goes global -> LDS directly (buffer_load_dwordx4 ... lds): instruction j of wave w fills the 1 KiB
-    // of rows 32w + 8j .. +7; lane l lands at byte 16*l of it, i.e. row 32w + 8j + l/8, chunk POSITION l%8,
+    // of rows 8*MT*w + 8j .. +7; lane l lands at byte 16*l of it, i.e. row 8*MT*w + 8j + l/8, chunk POSITION l%8,
     // so the lane fetches the chunk that the swizzle puts there: chunk (l%8) ^ ((row >> 1) & 7).
+    // (arrays below keep the 256-row tile's extent whatever MT is: with array bounds that depend on MT this compiler's host
+    // pass stops emitting the kernel's launch stub; the unused elements cost nothing)
     uint32_t a_voff[4];
 #pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) {
-        const uint32_t row = 32u * wave + 8u * j + (lane >> 3);
+    for (uint32_t j = 0; j < MT; ++j) {
+        const uint32_t row = 8u * MT * wave + 8u * j + (lane >> 3);
         a_voff[j] = (row * p.lda + (((lane & 7u) ^ ((row >> 1) & 7u)) * 8u)) * 2u;
     }
     // W: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
@@ -109,7 +119,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 #pragma unroll
     for (uint32_t kk = 0; kk < 4; ++kk) {
         const uint32_t x = swizzled_off(lane & 31u, 2u * kk + (lane >> 5));
-        a_rd[kk] = wm * 16384u + x;  // + mt*4096
+        a_rd[kk] = wm * (MT * 4096u) + x;  // + mt*4096
         w_rd[kk] = wn * 8192u + x;   // + t*4096
     }
 
@@ -133,9 +143,9 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 
     // A tile of K-step `kt` -> LDS stage (asynchronous; counted by vmcnt like any other load)
     auto dma_a = [&](auto stage_c, uint32_t kt) {
-        uint8_t* base = a_tile(stage_c) + wave * 4096u;
+        uint8_t* base = a_tile(stage_c) + wave * (MT * 1024u);
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
+        for (uint32_t j = 0; j < MT; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
                                                      a_voff[j], kt * (uint32_t)kBK * 2u, 0, 0);
     };
@@ -174,7 +184,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 
     f32x16_t acc[4][2];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -183,13 +193,13 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     auto read_frags = [&](auto stage_c, auto kk_c, bf16x8_t (&af)[4], bf16x8_t (&wf)[2]) {
         constexpr uint32_t KK = decltype(kk_c)::value;
 #pragma unroll
-        for (uint32_t mt = 0; mt < 4; ++mt) af[mt] = *reinterpret_cast<const bf16x8_t*>(a_tile(stage_c) + a_rd[KK] + mt * 4096u);
+        for (uint32_t mt = 0; mt < MT; ++mt) af[mt] = *reinterpret_cast<const bf16x8_t*>(a_tile(stage_c) + a_rd[KK] + mt * 4096u);
 #pragma unroll
         for (uint32_t t = 0; t < 2; ++t) wf[t] = *reinterpret_cast<const bf16x8_t*>(w_tile(stage_c) + w_rd[KK] + t * 4096u);
     };
     auto mma = [&](const bf16x8_t (&af)[4], const bf16x8_t (&wf)[2]) {
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int t = 0; t < 2; ++t) acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mt], wf[t], acc[mt][t], 0, 0, 0);
     };
@@ -340,11 +350,12 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             bias1 = bf16_bits_to_f32(raw >> 16);
         }
 #pragma unroll
-        for (uint32_t mt = 0; mt < 4; ++mt) {
-            uint8_t* base = c_rows(wm * 2u + (mt >> 1));
+        for (uint32_t mt = 0; mt < MT; ++mt) {
+            const uint32_t block32 = wm * MT + mt;  // which 32 rows of the tile
+            uint8_t* base = c_rows(block32 >> 1);
 #pragma unroll
             for (uint32_t i = 0; i < 16; ++i) {
-                const uint32_t row = 32u * (mt & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
                 // without a bias the sums are stored as they are (adding +0 would turn a -0 sum into +0)
                 *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) =
                     has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
@@ -353,7 +364,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     }
     __syncthreads();
 #pragma unroll
-    for (uint32_t pass = 0; pass < 16; ++pass) {
+    for (uint32_t pass = 0; pass < 4u * MT; ++pass) {
         const uint32_t row = pass * 16u + (tid >> 5);
         const uint32_t ch = tid & 31u;
         const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
@@ -365,11 +376,31 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 }
 
 template <int BITS, bool GROUPED>
-static hipError_t launch_prefill_t(const GemmParams& p, hipStream_t stream)
+static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
 {
+    GemmParams p = p0;
     const uint32_t tiles = ((p.m + kBM - 1) / kBM) * ((p.n + kBN - 1) / kBN);
-    const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    return launch_kernel(bfaintb_prefill_kernel<BITS, GROUPED>, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
+    // whole rounds of 256 workgroups run 256-row tiles; a last round that would fill less than half of the
+    // CUs runs as twice as many 128-row half tiles instead (also when there is no whole round at all)
+    const uint32_t rest = tiles % 256u;
+    const uint32_t halves = (rest != 0u && rest <= 128u && p.m > 128u) ? rest : 0u;
+    const uint32_t whole = tiles - halves;
+    if (whole) {
+        p.tile_first = 0;
+        p.tile_count = whole;
+        const uint32_t grid = (whole + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
+        void (*whole_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 4>;
+        hipError_t e = launch_kernel(whole_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
+        if (e != hipSuccess) return e;
+    }
+    if (halves) {
+        p.tile_first = whole;
+        p.tile_count = halves;
+        const uint32_t grid = (2u * halves + 7u) / 8u * 8u;
+        void (*half_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 2>;
+        return launch_kernel(half_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
+    }
+    return hipSuccess;
 }
 
 hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream)
