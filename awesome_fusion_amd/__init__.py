@@ -14,11 +14,16 @@ from .gemm import (  # noqa: F401
     dequant,
     error_string,
     gemm,
+    gemm_prepacked,
     kernel_name,
     lib,
+    prepack,
+    prepack_bytes,
+    prepacked_variant,
     library_path,
     probe_read,
     split_k,
+    unpack,
     variant,
     workspace_bytes,
     workspace_init,

@@ -18,6 +18,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kBufferFlags = 0x00027000;  // buffer resource word 3: raw buffer, 32-bit data format
 // Cache-policy operand of the raw buffer load/store builtins: device scope (sc1: the store writes through to

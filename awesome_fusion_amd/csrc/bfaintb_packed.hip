@@ -1,0 +1,262 @@
+// Pre-packed weights: B reordered once, offline, into the operand order of v_mfma_f32_16x16x32_bf16, and the
+// decode kernel that streams that order.
+//
+// The reference ships B to the device exactly as the host wrote it, row-major K x N
+// (/root/reference/bfAintBGemm/include/mem_transfer.hpp:23-32, bfAintBGemm.cc:101-103), and its kernel re-reads
+// it with a row stride (bf16gemm_kernel_gfx90a.s:239-262).  Row-major B forces a decode workgroup to own at
+// least 128 columns (whole 128-byte lines per row), so n = 4096 yields 32 column blocks and the other CUs have
+// to be filled by splitting K, with a second pass over partial sums.  In the packed order a block of 16 columns
+// is one contiguous slab of k x 16 codes: n / 16 workgroups each stream their slab linearly and own their
+// outputs outright — no split, no workspace, no second pass.
+//
+// Packed order ("mfma16"): column block nb = col / 16; K-chunks of R rows, R = 64 for 8-bit and 128 for 4-bit
+// codes (k must be a multiple of R), kc = row / R, chunks = k / R.  Chunk (nb, kc) is 1024 bytes at
+// (nb * chunks + kc) * 1024; lane l = 16 * kg + nl of a wave owns bytes 16 l .. 16 l + 15 of it:
+//   8-bit codes: byte 8 h + r is B[64 kc + 32 h + 8 kg + r][16 nb + nl]                  (h = 0, 1; r = 0..7);
+//   4-bit codes: byte 4 h + r / 2 holds, in nibble r & 1 (0 = low), B[128 kc + 32 h + 8 kg + r][16 nb + nl]  (h = 0..3).
+//   So a lane's 16 bytes are, in order, its 8-element W operands of the chunk's K-blocks of 32 rows — column nl
+//   of the block, rows 8 kg .. 8 kg + 7 of each K-block: one 128-bit load, no shuffling.
+// Codes keep their stored form (excess-128 / excess-8); scales and bias are not reordered.
+#include <type_traits>
+#include "bfaintb_device.hpp"
+
+namespace bfaintb {
+
+namespace {
+
+template <int BITS>
+struct PackedFormat {
+    static constexpr uint32_t kChunkRows = BITS == 8 ? 64u : 128u;
+    static constexpr uint32_t kBlocks = kChunkRows / 32u;  // K-blocks (matrix instructions) per chunk
+};
+
+// byte offset in the packed payload of the code of (row, col); for 4-bit codes *nibble is 0 (low) or 1
+template <int BITS>
+__device__ __forceinline__ size_t packed_offset(uint32_t row, uint32_t col, uint32_t chunks, uint32_t* nibble)
+{
+    const uint32_t nb = col >> 4, nl = col & 15u;
+    const uint32_t kc = row / PackedFormat<BITS>::kChunkRows, h = (row % PackedFormat<BITS>::kChunkRows) >> 5;
+    const uint32_t kg = (row >> 3) & 3u, r = row & 7u;
+    const size_t lane_slot = ((size_t)nb * chunks + kc) * 64u + 16u * kg + nl;
+    if constexpr (BITS == 8) {
+        *nibble = 0;
+        return lane_slot * 16u + 8u * h + r;
+    } else {
+        *nibble = r & 1u;
+        return lane_slot * 16u + 4u * h + (r >> 1);
+    }
+}
+
+// one thread per packed byte: gathers its 1 or 2 codes from the row-major matrix
+template <int BITS>
+__global__ void __launch_bounds__(256) pack_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src, uint32_t n, uint32_t k,
+                                                   uint32_t ldb_bytes)
+{
+    const size_t total = (size_t)n * k * BITS / 8;
+    const uint32_t chunks = k / PackedFormat<BITS>::kChunkRows;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t lane_slot = i >> 4;
+        const uint32_t within = (uint32_t)(i & 15u);
+        const uint32_t lane = (uint32_t)(lane_slot & 63u);
+        const size_t chunk = lane_slot >> 6;
+        const uint32_t kc = (uint32_t)(chunk % chunks), nb = (uint32_t)(chunk / chunks);
+        const uint32_t nl = lane & 15u, kg = lane >> 4;
+        const uint32_t col = 16u * nb + nl;
+        if constexpr (BITS == 8) {
+            const uint32_t h = within >> 3, r = within & 7u;
+            const uint32_t row = 64u * kc + 32u * h + 8u * kg + r;
+            dst[i] = src[(size_t)row * ldb_bytes + col];
+        } else {
+            const uint32_t h = within >> 2, r0 = (within & 3u) * 2u;
+            const uint32_t row = 128u * kc + 32u * h + 8u * kg + r0;
+            const uint32_t shift = (col & 1u) * 4u;
+            const uint32_t lo = (src[(size_t)row * ldb_bytes + (col >> 1)] >> shift) & 15u;
+            const uint32_t hi = (src[(size_t)(row + 1u) * ldb_bytes + (col >> 1)] >> shift) & 15u;
+            dst[i] = (uint8_t)(lo | (hi << 4));
+        }
+    }
+}
+
+// one thread per row-major byte: the inverse
+template <int BITS>
+__global__ void __launch_bounds__(256) unpack_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src, uint32_t n, uint32_t k,
+                                                     uint32_t ldb_bytes)
+{
+    const uint32_t row_bytes = n * BITS / 8;
+    const size_t total = (size_t)row_bytes * k;
+    const uint32_t chunks = k / PackedFormat<BITS>::kChunkRows;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t row = (uint32_t)(i / row_bytes), j = (uint32_t)(i % row_bytes);
+        uint32_t nib;
+        if constexpr (BITS == 8) {
+            dst[(size_t)row * ldb_bytes + j] = src[packed_offset<8>(row, j, chunks, &nib)];
+        } else {
+            const size_t o0 = packed_offset<4>(row, 2u * j, chunks, &nib);
+            const uint32_t lo = (src[o0] >> (4u * nib)) & 15u;
+            const size_t o1 = packed_offset<4>(row, 2u * j + 1u, chunks, &nib);
+            const uint32_t hi = (src[o1] >> (4u * nib)) & 15u;
+            dst[(size_t)row * ldb_bytes + j] = (uint8_t)(lo | (hi << 4));
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k, uint32_t ldb_bytes, int bits, bool unpack,
+                       hipStream_t stream)
+{
+    const size_t total = (size_t)n * k * (uint32_t)bits / 8;
+    const uint32_t grid = (uint32_t)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+    void (*kernel)(uint8_t*, const uint8_t*, uint32_t, uint32_t, uint32_t) =
+        bits == 8 ? (unpack ? unpack_kernel<8> : pack_kernel<8>) : (unpack ? unpack_kernel<4> : pack_kernel<4>);
+    return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, dst, src, n, k, ldb_bytes);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Decode over packed weights.
+//   grid = (n / 16, 1, ceil(m / (16 MB))); block = 8 waves.  A workgroup owns one column block (16 columns) and
+//   MB blocks of 16 rows of A, over all of k; wave w takes the K-chunks w, w + 8, ... of the slab, a batch at a
+//   time: all weight loads of the batch (one 128-bit load per chunk) and their activation loads are issued before
+//   the first is used, so a wave keeps 8 KiB (8-bit) or 4 KiB (4-bit) of the slab in flight.  Per K-block of 32
+//   rows: one conversion of 8 weights and MB v_mfma_f32_16x16x32_bf16 with the operands swapped, as in the
+//   row-major decode kernel (lane (nl, kg): W column nl, A row nl, rows 8 kg .. 8 kg + 7 of the K-block).  The
+//   eight waves' accumulators meet in LDS and are added in wave order: the summation order is fixed.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kPackedWaves = 8;
+
+template <int BITS, bool GROUPED, int MB>
+__global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kernel(const GemmParams p)
+{
+    constexpr uint32_t kBlocks = PackedFormat<BITS>::kBlocks;
+    constexpr uint32_t kChunkRows = PackedFormat<BITS>::kChunkRows;
+    constexpr int kBatch = (BITS == 8 ? 8 : 4) / MB;  // chunks a wave has in flight: 16 activation loads per batch
+    __shared__ float red[kPackedWaves][MB][16][16 + 4];  // [wave][row block][A row][W column], rows padded
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t nl = lane & 15u, kg = lane >> 4;
+    const uint32_t nb = blockIdx.x, rb = blockIdx.z;
+    const uint32_t chunks = p.k / kChunkRows;
+
+    const uint8_t* slab = p.b + ((size_t)nb * chunks) * 1024u + lane * 16u;
+    const uint32_t col = 16u * nb + nl;
+    const uint16_t* aptr[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        uint32_t arow = 16u * (MB * rb + mb) + nl;
+        if (arow >= p.m) arow = p.m - 1u;  // rows past m repeat the last one; their sums are never stored
+        aptr[mb] = p.a + (size_t)arow * p.lda + 8u * kg;
+    }
+    const uint16_t* sptr = p.scale + col;
+    // one scale per chunk when groups are whole chunks, else one per K-block
+    const bool scale_per_chunk = GROUPED && p.group_size % kChunkRows == 0;
+
+    float cs = 0.f;
+    if constexpr (!GROUPED) cs = make_col_scale<BITS>(*sptr);
+
+    f32x4_t acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto batch = [&](uint32_t base, auto guarded_c) {
+        constexpr bool GUARDED = decltype(guarded_c)::value;
+        uint4 wraw[kBatch];
+        uint4 araw[kBatch][kBlocks][MB];
+        uint32_t sraw[kBatch][kBlocks];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const uint32_t c = base + (uint32_t)i * kPackedWaves;
+            if (!GUARDED || c < chunks) {  // wave-uniform
+                wraw[i] = *reinterpret_cast<const uint4*>(slab + (size_t)c * 1024u);
+#pragma unroll
+                for (uint32_t h = 0; h < kBlocks; ++h)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) araw[i][h][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + kChunkRows * c + 32u * h);
+                if constexpr (GROUPED) {
+                    if (scale_per_chunk) {
+                        sraw[i][0] = sptr[(size_t)((kChunkRows * c) / p.group_size) * p.lds];
+                    } else {
+#pragma unroll
+                        for (uint32_t h = 0; h < kBlocks; ++h) sraw[i][h] = sptr[(size_t)((kChunkRows * c + 32u * h) / p.group_size) * p.lds];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const uint32_t c = base + (uint32_t)i * kPackedWaves;
+            if (!GUARDED || c < chunks) {
+                const uint32_t wd[4] = {wraw[i].x, wraw[i].y, wraw[i].z, wraw[i].w};
+#pragma unroll
+                for (uint32_t h = 0; h < kBlocks; ++h) {
+                    float s = cs;
+                    if constexpr (GROUPED) s = make_col_scale<BITS>(scale_per_chunk ? sraw[i][0] : sraw[i][h]);
+                    uint4 w;
+                    if constexpr (BITS == 8) {
+                        const uint32_t lo = codes8_to_s8(wd[2 * h]), hi = codes8_to_s8(wd[2 * h + 1]);
+                        w.x = pack_bf16_rne(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
+                        w.y = pack_bf16_rne(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
+                        w.z = pack_bf16_rne(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
+                        w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
+                    } else {
+                        // nibble r of the dword is row r: even rows from the low nibbles, odd rows from the high ones
+                        const uint32_t ev = codes4_even_to_s8x16(wd[h]), od = codes4_odd_to_s8x16(wd[h]);
+                        w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
+                        w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
+                        w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
+                        w.w = pack_bf16_rne(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
+                    }
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w),
+                                                                          __builtin_bit_cast(bf16x8_t, araw[i][h][mb]), acc[mb], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    constexpr uint32_t kStride = kPackedWaves * kBatch;
+    uint32_t base = wave;
+    for (; base + kStride - kPackedWaves < chunks; base += kStride) batch(base, std::false_type{});  // whole batches
+    if (base < chunks) batch(base, std::true_type{});
+
+    // acc[mb][r] of lane (nl, kg) is the sum for A row nl of block mb, W column 4 kg + r of the column block
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+        *reinterpret_cast<float4*>(&red[wave][mb][nl][4u * kg]) = make_float4(acc[mb][0], acc[mb][1], acc[mb][2], acc[mb][3]);
+    __syncthreads();
+    for (uint32_t t = tid; t < 256u * MB; t += 64u * kPackedWaves) {
+        const uint32_t mb = t >> 8, j = (t >> 4) & 15u, i = t & 15u;  // row block, A row, W column
+        const uint32_t row = 16u * (MB * rb + mb) + j;
+        if (row < p.m) {
+            float sum = red[0][mb][j][i];
+#pragma unroll
+            for (int w = 1; w < kPackedWaves; ++w) sum += red[w][mb][j][i];
+            const uint32_t c = 16u * nb + i;
+            if (p.bias != nullptr) sum += bf16_bits_to_f32(p.bias[c]);
+            p.c[(size_t)row * p.ldc + c] = (uint16_t)(pack_bf16_rne(sum, 0.f) & 0xffffu);
+        }
+    }
+}
+
+template <int BITS, bool GROUPED>
+static hipError_t launch_decode_packed_t(const GemmParams& p, hipStream_t stream)
+{
+    // two row blocks per workgroup once there are more than 16 rows: the weights are converted once for both
+    if (p.m > 16u) {
+        void (*kernel)(const GemmParams) = bfaintb_decode_packed_kernel<BITS, GROUPED, 2>;
+        return launch_kernel(kernel, dim3(p.n / 16u, 1, (p.m + 31u) / 32u), dim3(64 * kPackedWaves, 1, 1), 0, stream, p);
+    }
+    void (*kernel)(const GemmParams) = bfaintb_decode_packed_kernel<BITS, GROUPED, 1>;
+    return launch_kernel(kernel, dim3(p.n / 16u, 1, 1), dim3(64 * kPackedWaves, 1, 1), 0, stream, p);
+}
+
+hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream)
+{
+    const bool grouped = p.group_size != 0;
+    if (bits == 8) return grouped ? launch_decode_packed_t<8, true>(p, stream) : launch_decode_packed_t<8, false>(p, stream);
+    return grouped ? launch_decode_packed_t<4, true>(p, stream) : launch_decode_packed_t<4, false>(p, stream);
+}
+
+}  // namespace bfaintb

@@ -52,7 +52,7 @@ __device__ __forceinline__ uint32_t swizzled_off(uint32_t row, uint32_t chunk)
 // MT = blocks of 32 rows per wave along m: 4 for the 256-row tile, 2 for a 128-row half tile.  Half tiles take
 // over the tiles of a last, less than half full round of 256 workgroups: twice as many workgroups, each with half
 // the matrix instructions (and all of the weight conversion), finish sooner than half-idle CUs running whole tiles.
-template <int BITS, bool GROUPED, int MT>
+template <int BITS, bool GROUPED, int MT, bool PACKED>
 __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p)
 {
     constexpr uint32_t kRows = 64u * MT;  // rows of C per workgroup
@@ -96,9 +96,15 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)(((rows_valid - 1u) * p.lda + p.k) * 2u), kBufferFlags);
     const uint32_t cols_valid = p.n - n0 < (uint32_t)kBN ? p.n - n0 : (uint32_t)kBN;
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
-        kBufferFlags);
+    // packed weights: the tile's column blocks of 16 are consecutive slabs of slab_bytes each; the buffer ends with the
+    // last valid one, so blocks past n read as zero
+    const uint32_t slab_bytes = p.k * 16u * BITS / 8u;
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b + (size_t)(n0 / 16u) * slab_bytes), 0,
+                                                   (int)((cols_valid / 16u) * slab_bytes), kBufferFlags)
+               : __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0,
+                                                   (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
+                                                   kBufferFlags);
 
     // A goes global -> LDS directly (buffer_load_dwordx4 ... lds): instruction j of wave w fills the 1 KiB
     // of rows 8*MT*w + 8j .. +7; lane l lands at byte 16*l of it, i.e. row 8*MT*w + 8j + l/8, chunk POSITION l%8,
@@ -111,9 +117,22 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         const uint32_t row = 8u * MT * wave + 8u * j + (lane >> 3);
         a_voff[j] = (row * p.lda + (((lane & 7u) ^ ((row >> 1) & 7u)) * 8u)) * 2u;
     }
-    // W: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
+    // W, row-major: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
     const uint32_t b_voff = BITS == 8 ? 4u * lane : 2u * lane;
     const uint32_t w_dst = swizzled_off((lane & 31u) + (lane >> 5) * 64u, wave);  // + (j&1)*4096 + (j>>1)*16384
+    // W, packed: wave w converts column blocks 2w and 2w+1 of the tile; lane (nl, kg) holds, per block, column nl, rows
+    // 8 kg .. +7 of both K-blocks of the step, and writes them as chunks kg and 4 + kg of the column's LDS row.  Column
+    // nl of block cb lives in LDS row (cb>>2)*64 + (cb&1)*32 + ((cb>>1)&1)*16 + nl: the 16 lanes that write one chunk
+    // hit 16 consecutive rows (distinct bank groups), and wave wn's accumulator t, MFMA column jl is tile column
+    // 16*(4 wn + 2 (jl>>4) + t) + (jl & 15).
+    uint32_t pk_voff[2], pk_dst[2];
+#pragma unroll
+    for (uint32_t i = 0; i < 2; ++i) {
+        const uint32_t cb = 2u * wave + i;
+        pk_voff[i] = cb * slab_bytes + lane * 16u;
+        const uint32_t rho = (cb >> 2) * 64u + (cb & 1u) * 32u + ((cb >> 1) & 1u) * 16u + (lane & 15u);
+        pk_dst[i] = swizzled_off(rho, lane >> 4);  // chunk kg; chunk 4 + kg is this address ^ 64
+    }
     // fragment reads: row (lane&31) of a 32-row block, chunk 2*kk + lane/32
     uint32_t a_rd[4], w_rd[4];
 #pragma unroll
@@ -126,15 +145,32 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     // ---- scales of this lane's 4 columns
     const uint32_t ncol = n0 + 4u * lane;
     const bool w_ok = ncol < p.n;
+    // row-major: cs[j] scales column 4*lane + j.  Packed: cs[2 i + h] scales column nl of block 2 wave + i in K-block h.
     float cs[4];
     uint32_t cur_group = 0xffffffffu;
     auto fetch_scales = [&](uint32_t g) {
-        uint2 sr = make_uint2(0, 0);
-        if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + ncol);
-        cs[0] = make_col_scale<BITS>(sr.x & 0xffffu);
-        cs[1] = make_col_scale<BITS>(sr.x >> 16);
-        cs[2] = make_col_scale<BITS>(sr.y & 0xffffu);
-        cs[3] = make_col_scale<BITS>(sr.y >> 16);
+        if constexpr (PACKED) {
+            // g = group of the step's first K-block; the second K-block is in the next group when groups are 32 rows
+            const uint32_t g1 = (GROUPED && p.group_size == 32u) ? g + 1u : g;
+#pragma unroll
+            for (uint32_t i = 0; i < 2; ++i) {
+                const uint32_t c = n0 + 16u * (2u * wave + i) + (lane & 15u);
+                uint32_t s0 = 0, s1 = 0;
+                if (c < p.n) {
+                    s0 = p.scale[(size_t)g * p.lds + c];
+                    s1 = p.scale[(size_t)g1 * p.lds + c];
+                }
+                cs[2 * i] = make_col_scale<BITS>(s0);
+                cs[2 * i + 1] = make_col_scale<BITS>(s1);
+            }
+        } else {
+            uint2 sr = make_uint2(0, 0);
+            if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + ncol);
+            cs[0] = make_col_scale<BITS>(sr.x & 0xffffu);
+            cs[1] = make_col_scale<BITS>(sr.x >> 16);
+            cs[2] = make_col_scale<BITS>(sr.y & 0xffffu);
+            cs[3] = make_col_scale<BITS>(sr.y >> 16);
+        }
     };
     if constexpr (!GROUPED) fetch_scales(0);
 
@@ -151,6 +187,19 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     };
     // raw W codes of K-step `kt` -> registers (kt is clamped by the callers, so every load is in range)
     auto gload = [&](uint32_t kt) {
+        if constexpr (PACKED) {
+#pragma unroll
+            for (uint32_t i = 0; i < 2; ++i) {
+                if constexpr (BITS == 8) {  // K-chunk = this step: the lane's 16 bytes
+                    const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, pk_voff[i], kt * 1024u, 0);
+                    b_reg[4 * i] = v[0]; b_reg[4 * i + 1] = v[1]; b_reg[4 * i + 2] = v[2]; b_reg[4 * i + 3] = v[3];
+                } else {  // K-chunk = two steps: the half of the lane's 16 bytes that belongs to this one
+                    const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_b, pk_voff[i], (kt >> 1) * 1024u + (kt & 1u) * 8u, 0);
+                    b_reg[2 * i] = v[0]; b_reg[2 * i + 1] = v[1];
+                }
+            }
+            return;
+        }
         const uint32_t row0 = (kt * (uint32_t)kBK + 8u * wave) * p.ldb_bytes;
 #pragma unroll
         for (uint32_t r = 0; r < 8; ++r) {
@@ -162,6 +211,26 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     auto store_w_col = [&](auto stage_c, auto j_c, const uint32_t (&b_s8)[8]) {
         constexpr int J = decltype(j_c)::value;
         uint4 w;
+        if constexpr (PACKED) {
+            // J = 2 i + h: column block i of this wave, K-block h of the step
+            constexpr int I = J >> 1, H = J & 1;
+            const float s = cs[J];
+            if constexpr (BITS == 8) {
+                const uint32_t lo = b_s8[4 * I + 2 * H], hi = b_s8[4 * I + 2 * H + 1];  // rows 0-3, rows 4-7
+                w.x = pack_bf16_rne(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
+                w.y = pack_bf16_rne(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
+                w.z = pack_bf16_rne(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
+                w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
+            } else {
+                const uint32_t ev = b_s8[2 * J], od = b_s8[2 * J + 1];  // rows 0,2,4,6 and rows 1,3,5,7
+                w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
+                w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
+                w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
+                w.w = pack_bf16_rne(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
+            }
+            *reinterpret_cast<uint4*>(w_tile(stage_c) + (pk_dst[I] ^ (H * 64u))) = w;
+            return;
+        }
         w.x = pack_bf16_rne(sbyte_to_f32<J>(b_s8[0]) * cs[J], sbyte_to_f32<J>(b_s8[1]) * cs[J]);
         w.y = pack_bf16_rne(sbyte_to_f32<J>(b_s8[2]) * cs[J], sbyte_to_f32<J>(b_s8[3]) * cs[J]);
         w.z = pack_bf16_rne(sbyte_to_f32<J>(b_s8[4]) * cs[J], sbyte_to_f32<J>(b_s8[5]) * cs[J]);
@@ -169,12 +238,20 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         *reinterpret_cast<uint4*>(w_tile(stage_c) + w_dst + (J & 1) * 4096u + (J >> 1) * 16384u) = w;
     };
     auto prepare = [&](uint32_t (&b_s8)[8]) {
+        if constexpr (PACKED && BITS == 4) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {  // dword d = 2 i + h: 8 nibbles = rows 0..7 of one column
+                b_s8[2 * d] = codes4_even_to_s8x16(b_reg[d]);
+                b_s8[2 * d + 1] = codes4_odd_to_s8x16(b_reg[d]);
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < 8; ++r) b_s8[r] = BITS == 8 ? codes8_to_s8(b_reg[r]) : codes4_quad_to_s8x16(b_reg[r]);
     };
     auto update_scales = [&](uint32_t kt) {
         if constexpr (GROUPED) {
-            const uint32_t g = (kt * (uint32_t)kBK + 8u * wave) / p.group_size;
+            const uint32_t g = (kt * (uint32_t)kBK + (PACKED ? 0u : 8u * wave)) / p.group_size;
             if (g != cur_group) {
                 cur_group = g;
                 fetch_scales(g);
@@ -259,7 +336,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
         }
-        if constexpr (BITS == 8) __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);
+        if constexpr (BITS == 8) __builtin_amdgcn_sched_group_barrier(0x020, PACKED ? 2 : 8, 0);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -279,7 +356,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         store_w_col(Other{}, J3{}, b_s8);
         mma(af0, wf0);
         __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-        if constexpr (BITS == 4) __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);
+        if constexpr (BITS == 4) __builtin_amdgcn_sched_group_barrier(0x020, PACKED ? 2 : 8, 0);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -295,7 +372,8 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         // still converting weights (measured: 5-6 % at M = 4096 and 8192; raising other quarters gains less).
         __builtin_amdgcn_s_setprio(1);
         // this wave's part of the next A tile has landed in LDS (the 8 W loads issued after it may still fly)
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        if constexpr (PACKED) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         __syncthreads();
         PF_MARK(3);
         // Q4
@@ -317,7 +395,8 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         store_w_col(C0{}, J3{}, b_s8);
     }
     gload(ksteps > 1 ? 1 : 0);
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    if constexpr (PACKED) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     __syncthreads();
     read_frags(C0{}, C0{}, af0, wf0);
 
@@ -338,6 +417,31 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
     __syncthreads();
     auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_w0 : lds_w1; };
+    if constexpr (PACKED) {
+        // accumulator t of this wave, MFMA column jl is tile column 16 * (4 wn + 2 (jl >> 4) + t) + (jl & 15): the two
+        // accumulators are 16 columns apart, so each value is staged on its own
+        const uint32_t jl = lane & 31u, half = lane >> 5;
+        const uint32_t col0 = 16u * (4u * wn + 2u * (jl >> 4)) + (jl & 15u);
+        float bias0 = 0.f, bias1 = 0.f;
+        const bool has_bias = p.bias != nullptr;
+        if (has_bias) {
+            if (n0 + col0 < p.n) bias0 = bf16_bits_to_f32(p.bias[n0 + col0]);
+            if (n0 + col0 + 16u < p.n) bias1 = bf16_bits_to_f32(p.bias[n0 + col0 + 16u]);
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < MT; ++mt) {
+            const uint32_t block32 = wm * MT + mt;
+            uint8_t* base = c_rows(block32 >> 1);
+#pragma unroll
+            for (uint32_t i = 0; i < 16; ++i) {
+                const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                const uint32_t both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1)
+                                               : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0) = (uint16_t)(both & 0xffffu);
+                *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0 + 32u) = (uint16_t)(both >> 16);
+            }
+        }
+    } else
     {
         const uint32_t jl = lane & 31u, half = lane >> 5;
         const uint32_t colbyte = 8u * (32u * (wn & 1u) + jl) + 4u * (wn >> 1);
@@ -375,7 +479,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     }
 }
 
-template <int BITS, bool GROUPED>
+template <int BITS, bool GROUPED, bool PACKED>
 static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
 {
     GemmParams p = p0;
@@ -389,7 +493,7 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
         p.tile_first = 0;
         p.tile_count = whole;
         const uint32_t grid = (whole + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-        void (*whole_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 4>;
+        void (*whole_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 4, PACKED>;
         hipError_t e = launch_kernel(whole_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
         if (e != hipSuccess) return e;
     }
@@ -397,7 +501,7 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
         p.tile_first = whole;
         p.tile_count = halves;
         const uint32_t grid = (2u * halves + 7u) / 8u * 8u;
-        void (*half_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 2>;
+        void (*half_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 2, PACKED>;
         return launch_kernel(half_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
     }
     return hipSuccess;
@@ -406,8 +510,16 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
 hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream)
 {
     const bool grouped = p.group_size != 0;
-    if (bits == 8) return grouped ? launch_prefill_t<8, true>(p, stream) : launch_prefill_t<8, false>(p, stream);
-    return grouped ? launch_prefill_t<4, true>(p, stream) : launch_prefill_t<4, false>(p, stream);
+    if (bits == 8) return grouped ? launch_prefill_t<8, true, false>(p, stream) : launch_prefill_t<8, false, false>(p, stream);
+    return grouped ? launch_prefill_t<4, true, false>(p, stream) : launch_prefill_t<4, false, false>(p, stream);
+}
+
+// The same kernel over weights in the packed order (p.b is the packed buffer; p.ldb_bytes is unused).
+hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream)
+{
+    const bool grouped = p.group_size != 0;
+    if (bits == 8) return grouped ? launch_prefill_t<8, true, true>(p, stream) : launch_prefill_t<8, false, true>(p, stream);
+    return grouped ? launch_prefill_t<4, true, true>(p, stream) : launch_prefill_t<4, false, true>(p, stream);
 }
 
 }  // namespace bfaintb

@@ -68,6 +68,18 @@ def lib():
         L.bfaintb_gemm_variant.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
         L.bfaintb_gemm_split_k.restype = _u32
         L.bfaintb_gemm_split_k.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
+        L.bfaintb_prepack_bytes.restype = C.c_size_t
+        L.bfaintb_prepack_bytes.argtypes = [_u32, _u32, C.c_int]
+        L.bfaintb_prepack.restype = C.c_int
+        L.bfaintb_prepack.argtypes = [_vp, _vp, _u32, _u32, _u32, C.c_int, _vp]
+        L.bfaintb_unpack.restype = C.c_int
+        L.bfaintb_unpack.argtypes = [_vp, _vp, _u32, _u32, _u32, C.c_int, _vp]
+        L.bfaintb_gemm_prepacked.restype = C.c_int
+        L.bfaintb_gemm_prepacked.argtypes = [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
+        L.bfaintb_gemm_prepacked_ex.restype = C.c_int
+        L.bfaintb_gemm_prepacked_ex.argtypes = L.bfaintb_gemm_prepacked.argtypes + [C.c_int]
+        L.bfaintb_gemm_prepacked_variant.restype = C.c_int
+        L.bfaintb_gemm_prepacked_variant.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
         L.bfaintb_dequant.restype = C.c_int
         L.bfaintb_dequant.argtypes = [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
         L.bfaintb_probe_read.restype = C.c_int
@@ -145,6 +157,40 @@ def gemm(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, g
                                    _ptr(workspace), workspace_nbytes, _stream_handle(stream), which, force_split_k)
     if rc and check:
         raise BfaintbError(rc, "bfaintb_gemm")
+    return rc
+
+
+def prepack_bytes(n, k, weight_bits=8):
+    return lib().bfaintb_prepack_bytes(n, k, weight_bits)
+
+
+def prepack(packed, b, n, k, ldb=None, weight_bits=8, stream=None, check=True):
+    """Row-major B -> the packed operand order (bfaintb_prepack); ``packed`` holds prepack_bytes(n, k, bits) bytes."""
+    rc = lib().bfaintb_prepack(_ptr(packed), _ptr(b), n, k, n if ldb is None else ldb, weight_bits, _stream_handle(stream))
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_prepack")
+    return rc
+
+
+def unpack(b, packed, n, k, ldb=None, weight_bits=8, stream=None, check=True):
+    rc = lib().bfaintb_unpack(_ptr(b), _ptr(packed), n, k, n if ldb is None else ldb, weight_bits, _stream_handle(stream))
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_unpack")
+    return rc
+
+
+def prepacked_variant(m, n, k, weight_bits=8, group_size=0):
+    return lib().bfaintb_gemm_prepacked_variant(m, n, k, weight_bits, group_size)
+
+
+def gemm_prepacked(c, a, packed_b, scale, m, n, k, lda=None, ldc=None, weight_bits=8, group_size=0, bias=None, stream=None,
+                   which=AUTO, check=True):
+    """C = A x dequant(B, scale) (+ bias) with B in the packed order, through bfaintb_gemm_prepacked_ex."""
+    rc = lib().bfaintb_gemm_prepacked_ex(_ptr(c), _ptr(a), _ptr(packed_b), _ptr(scale), _ptr(bias), m, n, k,
+                                         k if lda is None else lda, n if ldc is None else ldc, weight_bits, group_size,
+                                         _stream_handle(stream), which)
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_gemm_prepacked")
     return rc
 
 

@@ -144,6 +144,43 @@ def pack_int4(q):
     return out
 
 
+def pack_mfma16(b, k, n, bits=8):
+    """Row-major packed codes b (uint8 [k, n] for 8-bit, [k, n/2] for 4-bit, the wire formats above) -> the library's
+    pre-packed operand order, as a flat uint8 array of k * n * bits / 8 bytes.
+
+    No counterpart in the reference (it keeps B row-major, bfAintBGemm.cc:101-103); this restates the byte map that
+    awesome_fusion_amd/csrc/bfaintb_packed.hip documents, with array reshapes instead of the kernel's index
+    arithmetic: column blocks of 16, K-chunks of R rows (64 for 8-bit, 128 for 4-bit), and inside a chunk, for lane
+    16*kg + nl, the codes of column nl, rows 32*h + 8*kg + r in the order (h, r).  Pinned in the tests by
+    hand-computed positions and by its inverse."""
+    b = _c(b, np.uint8)
+    if bits == 8:
+        assert b.shape == (k, n) and k % 64 == 0 and n % 16 == 0
+        v = b.reshape(k // 64, 2, 4, 8, n // 16, 16)          # [kc, h, kg, r, nb, nl]
+        return np.ascontiguousarray(v.transpose(4, 0, 2, 5, 1, 3)).reshape(-1)   # [nb, kc, kg, nl, h, r]
+    assert bits == 4 and b.shape == (k, n // 2) and k % 128 == 0 and n % 16 == 0
+    codes = np.empty((k, n), np.uint8)
+    codes[:, 0::2] = b & 15
+    codes[:, 1::2] = b >> 4
+    v = codes.reshape(k // 128, 4, 4, 8, n // 16, 16).transpose(4, 0, 2, 5, 1, 3)   # [nb, kc, kg, nl, h, r]
+    v = np.ascontiguousarray(v)
+    return (v[..., 0::2] | (v[..., 1::2] << 4)).astype(np.uint8).reshape(-1)      # row r even in the low nibble
+
+
+def unpack_mfma16(packed, k, n, bits=8):
+    """Inverse of pack_mfma16."""
+    packed = _c(packed, np.uint8)
+    if bits == 8:
+        v = packed.reshape(n // 16, k // 64, 4, 16, 2, 8)      # [nb, kc, kg, nl, h, r]
+        return np.ascontiguousarray(v.transpose(1, 4, 2, 5, 0, 3)).reshape(k, n)
+    v = packed.reshape(n // 16, k // 128, 4, 16, 4, 4)
+    codes = np.empty(v.shape[:-1] + (8,), np.uint8)
+    codes[..., 0::2] = v & 15
+    codes[..., 1::2] = v >> 4
+    codes = np.ascontiguousarray(codes.transpose(1, 4, 2, 5, 0, 3)).reshape(k, n)
+    return (codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8)
+
+
 def dequant(b, scale, k, n, bits=8, group_size=0, rtz=False):
     """Dequantized weights as bf16 bit patterns [k, n].  scale: uint16 (bf16 bits) or float32,
     shape [groups, n] (or [n])."""

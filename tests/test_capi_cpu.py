@@ -19,7 +19,7 @@ def declared_symbols():
 
 def test_library_exports_every_declared_symbol():
     names = declared_symbols()
-    assert len(names) >= 11 and "bfaintb_gemm" in names and "bfaintb_dequant" in names
+    assert len(names) >= 17 and "bfaintb_gemm_prepacked" in names and "bfaintb_gemm" in names and "bfaintb_dequant" in names
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
@@ -84,6 +84,40 @@ def test_rejects_bad_arguments_without_launching():
     assert af.dequant(P, P, None, 128, 256, stream=0, check=False) == -1
     assert L.bfaintb_workspace_init(P, 66, None) == -6   # not a whole number of words
     assert L.bfaintb_workspace_init(None, 0, None) == 0
+
+
+def test_prepacked_entry_points_validate_before_launching():
+    L = af.lib()
+    assert af.prepack_bytes(4096, 4096, 8) == 4096 * 4096 and af.prepack_bytes(4096, 4096, 4) == 4096 * 4096 // 2
+    assert af.prepack_bytes(4096, 4160, 4) == 0          # 4-bit packed order has K-chunks of 128 rows
+    assert af.prepack_bytes(100, 4096, 8) == 0 and af.prepack_bytes(16, 64, 5) == 0
+    assert af.prepack(P, P, 128, 256, stream=0, weight_bits=3, check=False) == -5
+    assert af.prepack(P, P, 100, 256, stream=0, check=False) == -2
+    assert af.prepack(P, P, 128, 192, stream=0, weight_bits=4, check=False) == -2
+    assert af.prepack(P, P, 128, 256, ldb=64, stream=0, check=False) == -3
+    assert af.prepack(None, P, 128, 256, stream=0, check=False) == -1
+    assert af.prepack(P, P + 8, 128, 256, stream=0, check=False) == -4
+    assert af.unpack(P, None, 128, 256, stream=0, check=False) == -1
+
+    def rcp(**kw):
+        d = dict(c=P, a=P, packed_b=P, scale=P, m=64, n=128, k=256, stream=0, check=False)
+        d.update(kw)
+        return af.gemm_prepacked(d.pop("c"), d.pop("a"), d.pop("packed_b"), d.pop("scale"), d.pop("m"), d.pop("n"), d.pop("k"), **d)
+    assert rcp(weight_bits=5) == -5
+    assert rcp(group_size=48) == -5
+    assert rcp(n=100) == -2
+    assert rcp(k=192, weight_bits=4) == -2
+    assert rcp(lda=128) == -3
+    assert rcp(ldc=64) == -3
+    assert rcp(packed_b=None) == -1
+    assert rcp(bias=P + 2) == -4
+    assert rcp(which=7) == -7
+    assert rcp(m=0) == 0
+    assert af.prepacked_variant(1, 4096, 4096) == af.DECODE
+    assert af.prepacked_variant(64, 4096, 4096) == af.DECODE
+    assert af.prepacked_variant(4096, 4096, 4096) == af.PREFILL
+    assert af.prepacked_variant(1, 4096, 4160, 4, 0) == -2
+    assert L.bfaintb_gemm_prepacked_variant(1, 100, 4096, 8, 0) == -2
 
 
 def test_product_does_not_reach_for_the_oracle():

@@ -1,0 +1,133 @@
+"""Pre-packed weights on the GPU, through the C ABI: the packing kernels bit-exact against the oracle's restatement
+of the byte map, and bfaintb_gemm_prepacked (both kernels behind it) against the oracle GEMM on the same seeded
+inputs, to the bar of the row-major path (2 bf16 ULP of the fp32-accumulated reference)."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import Problem, assert_close_ulp, from_dev_u16, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def af():
+    import torch
+    import awesome_fusion_amd as af_
+    assert torch.cuda.is_available()
+    af_.lib()
+    return af_
+
+
+def packed_on_device(af, p):
+    import torch
+    pk = torch.zeros(af.prepack_bytes(p.n, p.k, p.bits), dtype=torch.uint8, device="cuda")
+    af.prepack(pk, to_dev(p.b_bytes), p.n, p.k, weight_bits=p.bits)
+    return pk
+
+
+def run_prepacked(af, p, which=0, pk=None, ldc=None):
+    import torch
+    pk = packed_on_device(af, p) if pk is None else pk
+    ldc_ = p.n if ldc is None else ldc
+    c = torch.full((p.m, ldc_), 0x7FC0, dtype=torch.int16, device="cuda")
+    bias = None if p.bias_bf is None else to_dev(p.bias_bf)
+    af.gemm_prepacked(c, to_dev(p.a_bf), pk, to_dev(p.s_bf), p.m, p.n, p.k, ldc=ldc, weight_bits=p.bits, group_size=p.group_size,
+                      bias=bias, which=which)
+    torch.cuda.synchronize()
+    return from_dev_u16(c)
+
+
+@pytest.mark.parametrize("bits,k,n", [(8, 64, 16), (8, 448, 272), (4, 128, 16), (4, 640, 304), (8, 4096, 4096)])
+def test_pack_kernels_bit_exact_and_inverse(af, bits, k, n):
+    import torch
+    p = Problem(1, n, k, bits, 0, seed=k + n)
+    pk = packed_on_device(af, p)
+    torch.cuda.synchronize()
+    assert np.array_equal(pk.cpu().numpy(), oracle.pack_mfma16(p.b_bytes, k, n, bits))
+    back = torch.zeros_like(to_dev(p.b_bytes))
+    af.unpack(back, pk, n, k, weight_bits=bits)
+    torch.cuda.synchronize()
+    assert np.array_equal(back.cpu().numpy(), p.b_bytes)
+
+
+def test_pack_honours_the_row_stride(af):
+    import torch
+    k, n, ldb = 128, 48, 64
+    p = Problem(1, n, k, 8, 0, seed=3)
+    wide = np.full((k, ldb), 0xEE, np.uint8)
+    wide[:, :n] = p.b_bytes
+    pk = torch.zeros(af.prepack_bytes(n, k, 8), dtype=torch.uint8, device="cuda")
+    af.prepack(pk, to_dev(wide), n, k, ldb=ldb, weight_bits=8)
+    back = torch.full((k, ldb), 0x11, dtype=torch.uint8, device="cuda")
+    af.unpack(back, pk, n, k, ldb=ldb, weight_bits=8)
+    torch.cuda.synchronize()
+    assert np.array_equal(pk.cpu().numpy(), oracle.pack_mfma16(p.b_bytes, k, n, 8))
+    got = back.cpu().numpy()
+    assert np.array_equal(got[:, :n], p.b_bytes) and np.all(got[:, n:] == 0x11)
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (1, 16, 64, 8, 0), (1, 256, 512, 8, 0), (3, 48, 192, 8, 64), (16, 64, 1024, 4, 0), (17, 80, 640, 4, 32),
+    (33, 96, 1152, 4, 128), (70, 64, 1600, 8, 32), (1, 32, 8256, 8, 0), (40, 128, 4096, 8, 128), (5, 1024, 2048, 4, 128)])
+def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    assert_close_ulp(p, run_prepacked(af, p, af.DECODE), f"packed decode {m}x{n}x{k} b{bits} g{group}")
+    p.with_bias()
+    assert_close_ulp(p, run_prepacked(af, p, af.DECODE), f"packed decode + bias {m}x{n}x{k} b{bits} g{group}")
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (256, 256, 64, 8, 0), (300, 272, 192, 8, 0), (64, 128, 256, 8, 0), (512, 512, 256, 4, 128), (1000, 1008, 384, 4, 0),
+    (513, 784, 448, 8, 64), (130, 528, 512, 8, 32), (260, 304, 512, 4, 32), (4160, 256, 256, 8, 0), (2304, 512, 512, 4, 128)])
+def test_tiled_kernel_matches_oracle(af, m, n, k, bits, group):
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    assert_close_ulp(p, run_prepacked(af, p, af.PREFILL), f"packed prefill {m}x{n}x{k} b{bits} g{group}")
+    p.with_bias()
+    assert_close_ulp(p, run_prepacked(af, p, af.PREFILL), f"packed prefill + bias {m}x{n}x{k} b{bits} g{group}")
+
+
+@pytest.mark.parametrize("bits,group", [(8, 0), (4, 128)])
+@pytest.mark.parametrize("which,m", [(1, 16), (1, 32), (2, 64)])
+def test_kernels_dequantise_bit_exact(af, bits, group, which, m):
+    """One-hot activations make C[i, :] = W[k_i, :] with nothing to round: the in-register conversion of both
+    kernels is observed exactly, against the oracle's dequantised weights."""
+    k, n = 256, 512
+    p = Problem(m, n, k, bits, group, seed=7)
+    pk = packed_on_device(af, p)
+    for base in range(0, k, m):
+        a = np.zeros((m, k), np.float32)
+        rows = (base + np.arange(m)) % k
+        a[np.arange(m), rows] = 1.0
+        p.a_bf = oracle.f32_to_bf16_rne(a)
+        assert np.array_equal(run_prepacked(af, p, which, pk=pk), p.w_bf[rows]), f"rows {base}.. differ"
+
+
+@pytest.mark.parametrize("m", [1, 16])
+def test_headline_shapes(af, m):
+    p = Problem(m, 4096, 4096, seed=20 + m)
+    assert af.prepacked_variant(m, 4096, 4096) == af.DECODE
+    assert_close_ulp(p, run_prepacked(af, p), f"packed 4096x4096 m={m}", threads=16)
+    p = Problem(m, 28672, 8192, 4, 128, seed=50 + m, scale_lo=0.001, scale_hi=0.02)
+    assert_close_ulp(p, run_prepacked(af, p), f"packed int4 g128 m={m}", threads=16)
+
+
+def test_tiled_full_size(af):
+    p = Problem(4096, 4096, 4096, seed=4)
+    assert af.prepacked_variant(4096, 4096, 4096) == af.PREFILL
+    assert_close_ulp(p, run_prepacked(af, p), "packed prefill 4096^3", threads=16, max_frac=1e-4)
+
+
+def test_matches_the_row_major_path_in_the_exact_regime(af):
+    """Small-integer data (the reference's own test regime) has exact sums: packed and row-major agree bit for bit."""
+    from helpers import run_gemm
+    for m in (1, 40, 300):
+        p = Problem(m, 272, 512, 8, 0, seed=m, regime="small_int")
+        assert np.array_equal(run_prepacked(af, p), run_gemm(p))
+
+
+def test_output_stride_and_padding(af):
+    p = Problem(5, 48, 128, 8, 0, seed=9)
+    c = run_prepacked(af, p, ldc=64)
+    assert_close_ulp(p, np.ascontiguousarray(c[:, :48]), "packed ldc")
+    assert np.all(c[:, 48:] == 0x7FC0)

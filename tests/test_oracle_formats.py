@@ -141,3 +141,32 @@ def test_int_times_bf16_scale_is_exact_exhaustive():
     sig = widen(np.arange(0x3F80, 0x4000, dtype=np.uint32).astype(np.uint16)).astype(np.float64)[None, :]
     exact = q * sig
     assert np.array_equal(exact.astype(np.float32).astype(np.float64), exact)
+
+
+def test_prepacked_order_positions_and_inverse():
+    # the packed operand order has no counterpart in the reference: pin the restatement by positions worked out by
+    # hand from the documented byte map, and by its inverse
+    rng = np.random.default_rng(5)
+    k, n = 192, 48
+    b = rng.integers(0, 256, size=(k, n), dtype=np.uint8)
+    pk = oracle.pack_mfma16(b, k, n, 8)
+    assert pk.size == k * n
+    # row 37 = chunk 0, K-block 1, kg 0, r 5; column 5 = block 0, nl 5: lane 5 -> byte 5*16 + 8*1 + 5
+    assert pk[93] == b[37, 5]
+    # row 150 = chunk 2 (128..191), h 0, kg 2 (rows 16..23 of the K-block), r 6; column 40 = block 2, nl 8:
+    # chunk index (2 * 3 + 2) = 8, lane 16*2 + 8 = 40 -> 8*1024 + 40*16 + 0*8 + 6
+    assert pk[8 * 1024 + 40 * 16 + 6] == b[150, 40]
+    assert np.array_equal(oracle.unpack_mfma16(pk, k, n, 8), b)
+
+    k, n = 256, 32
+    q = rng.integers(-8, 8, size=(k, n), dtype=np.int8)
+    b4 = oracle.pack_int4(q)
+    pk4 = oracle.pack_mfma16(b4, k, n, 4)
+    assert pk4.size == k * n // 2
+    code = lambda r, c: int(q[r, c]) + 8
+    # row 100 = chunk 0, h 3, kg 0, r 4; column 21 = block 1, nl 5: chunk index 1*2+0 = 2, lane 5
+    # -> byte 2*1024 + 5*16 + 4*3 + 4/2, low nibble (r even); the high nibble is row 101
+    assert pk4[2 * 1024 + 5 * 16 + 14] == (code(100, 21) | (code(101, 21) << 4))
+    # row 255 = chunk 1, h 3, kg 3, r 7; column 0: chunk index 1, lane 48 -> byte 1024 + 48*16 + 12 + 3, high nibble
+    assert pk4[1024 + 48 * 16 + 15] >> 4 == code(255, 0)
+    assert np.array_equal(oracle.unpack_mfma16(pk4, k, n, 4), b4)
