@@ -7,6 +7,9 @@ has no CPU fallback: without the built library every call raises.
 """
 from .gemm import (  # noqa: F401
     BfaintbError,
+    PackedHeader,
+    load_packed,
+    save_packed,
     DECODE,
     PREFILL,
     AUTO,

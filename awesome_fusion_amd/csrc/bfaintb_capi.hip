@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "bfaintb_device.hpp"
 #include "../../include/bfaintb_gemm.h"
@@ -325,6 +326,40 @@ size_t bfaintb_prepack_bytes(uint32_t n, uint32_t k, int weight_bits)
 {
     if ((weight_bits != 8 && weight_bits != 4) || check_packed_shape(n, k, weight_bits)) return 0;
     return (size_t)n * k * (uint32_t)weight_bits / 8u;
+}
+
+int bfaintb_packed_header_init(bfaintb_packed_header* h, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int has_bias)
+{
+    if (h == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    int e = check_format(k, weight_bits, group_size);
+    if (e) return e;
+    e = check_packed_shape(n, k, weight_bits);
+    if (e) return e;
+    memset(h, 0, sizeof(*h));
+    memcpy(h->magic, "BFAINTB1", 8);
+    h->header_bytes = (uint32_t)sizeof(*h);
+    h->layout = BFAINTB_LAYOUT_MFMA16;
+    h->weight_bits = (uint32_t)weight_bits;
+    h->group_size = group_size;
+    h->k = k;
+    h->n = n;
+    h->payload_bytes = (uint64_t)n * k * (uint32_t)weight_bits / 8u;
+    h->scale_bytes = (uint64_t)(group_size ? k / group_size : 1u) * n * 2u;
+    h->has_bias = has_bias ? 1u : 0u;
+    return BFAINTB_OK;
+}
+
+int bfaintb_packed_header_check(const bfaintb_packed_header* h)
+{
+    if (h == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    if (memcmp(h->magic, "BFAINTB1", 8) != 0 || h->header_bytes != sizeof(*h) || h->layout != BFAINTB_LAYOUT_MFMA16)
+        return BFAINTB_ERR_UNSUPPORTED;
+    bfaintb_packed_header want;
+    const int e = bfaintb_packed_header_init(&want, h->n, h->k, (int)h->weight_bits, h->group_size, (int)h->has_bias);
+    if (e) return e;
+    if (h->has_bias > 1u || h->reserved[0] || h->reserved[1] || h->reserved[2]) return BFAINTB_ERR_UNSUPPORTED;
+    if (h->payload_bytes != want.payload_bytes || h->scale_bytes != want.scale_bytes) return BFAINTB_ERR_BAD_SHAPE;
+    return BFAINTB_OK;
 }
 
 static int repack(void* dst, const void* src, uint32_t n, uint32_t k, uint32_t ldb, int weight_bits, void* stream, bool unpack)

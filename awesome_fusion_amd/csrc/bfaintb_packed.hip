@@ -115,21 +115,25 @@ hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k,
 // ---------------------------------------------------------------------------------------------------------------
 // Decode over packed weights.
 //   grid = (n / 16, 1, ceil(m / (16 MB))); block = 8 waves.  A workgroup owns one column block (16 columns) and
-//   MB blocks of 16 rows of A, over all of k; wave w takes the K-chunks w, w + 8, ... of the slab, a batch at a
-//   time: all weight loads of the batch (one 128-bit load per chunk) and their activation loads are issued before
-//   the first is used, so a wave keeps 8 KiB (8-bit) or 4 KiB (4-bit) of the slab in flight.  Per K-block of 32
+//   MB blocks of 16 rows of A, over all of k; wave w takes the K-chunks w, w + 8, ... of the slab in batches: the
+//   weight loads of a batch (one 128-bit load per chunk) and their activation loads are issued back to back, and
+//   a wave keeps 8 KiB (8-bit) or 4 KiB (4-bit) of the slab in flight — as one batch when that is all the wave has
+//   (k up to 4096 for 8-bit codes; measured 2 % faster at k = 4096), else as two half-size batches, the next one
+//   loaded before the current one is converted (9 % faster at k = 11008).  Per K-block of 32
 //   rows: one conversion of 8 weights and MB v_mfma_f32_16x16x32_bf16 with the operands swapped, as in the
 //   row-major decode kernel (lane (nl, kg): W column nl, A row nl, rows 8 kg .. 8 kg + 7 of the K-block).  The
 //   eight waves' accumulators meet in LDS and are added in wave order: the summation order is fixed.
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kPackedWaves = 8;
 
-template <int BITS, bool GROUPED, int MB>
+template <int BITS, bool GROUPED, int MB, bool WHOLE>
 __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kernel(const GemmParams p)
 {
     constexpr uint32_t kBlocks = PackedFormat<BITS>::kBlocks;
     constexpr uint32_t kChunkRows = PackedFormat<BITS>::kChunkRows;
-    constexpr int kBatch = (BITS == 8 ? 8 : 4) / MB;  // chunks a wave has in flight: 16 activation loads per batch
+    // WHOLE: one batch holds all of a wave's chunks (the launcher checks), loaded at once.  Otherwise half as many per
+    // batch and two batches in flight, the next one loaded before the current one is converted.
+    constexpr int kBatch = (BITS == 8 ? 4 : 2) * (WHOLE ? 2 : 1) / MB;
     __shared__ float red[kPackedWaves][MB][16][16 + 4];  // [wave][row block][A row][W column], rows padded
 
     const uint32_t tid = threadIdx.x;
@@ -159,39 +163,42 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    auto batch = [&](uint32_t base, auto guarded_c) {
-        constexpr bool GUARDED = decltype(guarded_c)::value;
-        uint4 wraw[kBatch];
-        uint4 araw[kBatch][kBlocks][MB];
-        uint32_t sraw[kBatch][kBlocks];
+    struct Batch {
+        uint4 w[kBatch];
+        uint4 a[kBatch][kBlocks][MB];
+        uint32_t s[kBatch][kBlocks];
+    };
+    // all loads of a batch, back to back (chunks past the end re-read the last one; compute() skips them)
+    auto load = [&](Batch& b, uint32_t base) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            const uint32_t c = base + (uint32_t)i * kPackedWaves;
-            if (!GUARDED || c < chunks) {  // wave-uniform
-                wraw[i] = *reinterpret_cast<const uint4*>(slab + (size_t)c * 1024u);
+            uint32_t c = base + (uint32_t)i * kPackedWaves;
+            if (c >= chunks) c = chunks - 1u;
+            b.w[i] = *reinterpret_cast<const uint4*>(slab + (size_t)c * 1024u);
 #pragma unroll
-                for (uint32_t h = 0; h < kBlocks; ++h)
+            for (uint32_t h = 0; h < kBlocks; ++h)
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) araw[i][h][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + kChunkRows * c + 32u * h);
-                if constexpr (GROUPED) {
-                    if (scale_per_chunk) {
-                        sraw[i][0] = sptr[(size_t)((kChunkRows * c) / p.group_size) * p.lds];
-                    } else {
+                for (int mb = 0; mb < MB; ++mb) b.a[i][h][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + kChunkRows * c + 32u * h);
+            if constexpr (GROUPED) {
+                if (scale_per_chunk) {
+                    b.s[i][0] = sptr[(size_t)((kChunkRows * c) / p.group_size) * p.lds];
+                } else {
 #pragma unroll
-                        for (uint32_t h = 0; h < kBlocks; ++h) sraw[i][h] = sptr[(size_t)((kChunkRows * c + 32u * h) / p.group_size) * p.lds];
-                    }
+                    for (uint32_t h = 0; h < kBlocks; ++h) b.s[i][h] = sptr[(size_t)((kChunkRows * c + 32u * h) / p.group_size) * p.lds];
                 }
             }
         }
+    };
+    auto compute = [&](const Batch& b, uint32_t base) {
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const uint32_t c = base + (uint32_t)i * kPackedWaves;
-            if (!GUARDED || c < chunks) {
-                const uint32_t wd[4] = {wraw[i].x, wraw[i].y, wraw[i].z, wraw[i].w};
+            if (c < chunks) {  // wave-uniform
+                const uint32_t wd[4] = {b.w[i].x, b.w[i].y, b.w[i].z, b.w[i].w};
 #pragma unroll
                 for (uint32_t h = 0; h < kBlocks; ++h) {
                     float s = cs;
-                    if constexpr (GROUPED) s = make_col_scale<BITS>(scale_per_chunk ? sraw[i][0] : sraw[i][h]);
+                    if constexpr (GROUPED) s = make_col_scale<BITS>(scale_per_chunk ? b.s[i][0] : b.s[i][h]);
                     uint4 w;
                     if constexpr (BITS == 8) {
                         const uint32_t lo = codes8_to_s8(wd[2 * h]), hi = codes8_to_s8(wd[2 * h + 1]);
@@ -210,16 +217,31 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb)
                         acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w),
-                                                                          __builtin_bit_cast(bf16x8_t, araw[i][h][mb]), acc[mb], 0, 0, 0);
+                                                                          __builtin_bit_cast(bf16x8_t, b.a[i][h][mb]), acc[mb], 0, 0, 0);
                 }
             }
         }
     };
 
+    // two batches in flight: the loads of the next batch are issued before the current one is converted
     constexpr uint32_t kStride = kPackedWaves * kBatch;
+    Batch b0;
     uint32_t base = wave;
-    for (; base + kStride - kPackedWaves < chunks; base += kStride) batch(base, std::false_type{});  // whole batches
-    if (base < chunks) batch(base, std::true_type{});
+    if (base < chunks) load(b0, base);
+    if constexpr (WHOLE) {
+        compute(b0, base);
+        base = chunks;
+    }
+    Batch b1;
+    while (base < chunks) {
+        if (base + kStride < chunks) load(b1, base + kStride);
+        compute(b0, base);
+        base += kStride;
+        if (base >= chunks) break;
+        if (base + kStride < chunks) load(b0, base + kStride);
+        compute(b1, base);
+        base += kStride;
+    }
 
     // acc[mb][r] of lane (nl, kg) is the sum for A row nl of block mb, W column 4 kg + r of the column block
 #pragma unroll
@@ -244,12 +266,14 @@ template <int BITS, bool GROUPED>
 static hipError_t launch_decode_packed_t(const GemmParams& p, hipStream_t stream)
 {
     // two row blocks per workgroup once there are more than 16 rows: the weights are converted once for both
-    if (p.m > 16u) {
-        void (*kernel)(const GemmParams) = bfaintb_decode_packed_kernel<BITS, GROUPED, 2>;
-        return launch_kernel(kernel, dim3(p.n / 16u, 1, (p.m + 31u) / 32u), dim3(64 * kPackedWaves, 1, 1), 0, stream, p);
-    }
-    void (*kernel)(const GemmParams) = bfaintb_decode_packed_kernel<BITS, GROUPED, 1>;
-    return launch_kernel(kernel, dim3(p.n / 16u, 1, 1), dim3(64 * kPackedWaves, 1, 1), 0, stream, p);
+    const uint32_t mb = p.m > 16u ? 2u : 1u;
+    // chunks per wave that fit the one-batch form: 8 / mb of 64 rows (8-bit) or 4 / mb of 128 rows (4-bit)
+    const uint32_t chunks = p.k / PackedFormat<BITS>::kChunkRows;
+    const bool whole = chunks <= kPackedWaves * (BITS == 8 ? 8u : 4u) / mb;
+    void (*kernel)(const GemmParams) =
+        mb == 2u ? (whole ? bfaintb_decode_packed_kernel<BITS, GROUPED, 2, true> : bfaintb_decode_packed_kernel<BITS, GROUPED, 2, false>)
+                 : (whole ? bfaintb_decode_packed_kernel<BITS, GROUPED, 1, true> : bfaintb_decode_packed_kernel<BITS, GROUPED, 1, false>);
+    return launch_kernel(kernel, dim3(p.n / 16u, 1, (p.m + 16u * mb - 1u) / (16u * mb)), dim3(64 * kPackedWaves, 1, 1), 0, stream, p);
 }
 
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream)

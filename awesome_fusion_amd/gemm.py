@@ -41,6 +41,13 @@ _u32 = C.c_uint32
 _vp = C.c_void_p
 
 
+class PackedHeader(C.Structure):
+    """bfaintb_packed_header of include/bfaintb_gemm.h: the 64-byte header of a pre-packed weight file."""
+    _fields_ = [("magic", C.c_char * 8), ("header_bytes", _u32), ("layout", _u32), ("weight_bits", _u32), ("group_size", _u32),
+                ("k", _u32), ("n", _u32), ("payload_bytes", C.c_uint64), ("scale_bytes", C.c_uint64), ("has_bias", _u32),
+                ("reserved", _u32 * 3)]
+
+
 def lib():
     """The loaded library.  Raises if it has not been built: there is no fallback path."""
     global _lib
@@ -80,6 +87,10 @@ def lib():
         L.bfaintb_gemm_prepacked_ex.argtypes = L.bfaintb_gemm_prepacked.argtypes + [C.c_int]
         L.bfaintb_gemm_prepacked_variant.restype = C.c_int
         L.bfaintb_gemm_prepacked_variant.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
+        L.bfaintb_packed_header_init.restype = C.c_int
+        L.bfaintb_packed_header_init.argtypes = [C.POINTER(PackedHeader), _u32, _u32, C.c_int, _u32, C.c_int]
+        L.bfaintb_packed_header_check.restype = C.c_int
+        L.bfaintb_packed_header_check.argtypes = [C.POINTER(PackedHeader)]
         L.bfaintb_dequant.restype = C.c_int
         L.bfaintb_dequant.argtypes = [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
         L.bfaintb_probe_read.restype = C.c_int
@@ -192,6 +203,57 @@ def gemm_prepacked(c, a, packed_b, scale, m, n, k, lda=None, ldc=None, weight_bi
     if rc and check:
         raise BfaintbError(rc, "bfaintb_gemm_prepacked")
     return rc
+
+
+def save_packed(path, packed, scale, n, k, weight_bits=8, group_size=0, bias=None):
+    """Writes header + packed codes + bf16 scales (+ bf16 bias) in the wire form the header declares."""
+    h = PackedHeader()
+    rc = lib().bfaintb_packed_header_init(C.byref(h), n, k, weight_bits, group_size, 0 if bias is None else 1)
+    if rc:
+        raise BfaintbError(rc, "bfaintb_packed_header_init")
+    parts = [bytes(h), packed.detach().cpu().contiguous().view(-1).numpy().tobytes(),
+             scale.detach().cpu().contiguous().view(-1).view(dtype=_torch().int16).numpy().tobytes()]
+    if len(parts[1]) != h.payload_bytes or len(parts[2]) != h.scale_bytes:
+        raise ValueError("save_packed: tensor sizes do not match the shape")
+    if bias is not None:
+        parts.append(bias.detach().cpu().contiguous().view(-1).view(dtype=_torch().int16).numpy().tobytes())
+        if len(parts[3]) != 2 * n:
+            raise ValueError("save_packed: bias must hold n bf16 values")
+    with open(path, "wb") as f:
+        for part in parts:
+            f.write(part)
+
+
+def load_packed(path, device="cuda"):
+    """Reads a file written by save_packed: (header, packed uint8 tensor, scale bf16 [groups, n], bias bf16 [n] or None)."""
+    import numpy as np
+    torch = _torch()
+    with open(path, "rb") as f:
+        raw = f.read()
+    if len(raw) < C.sizeof(PackedHeader):
+        raise ValueError("load_packed: file shorter than the header")
+    h = PackedHeader.from_buffer_copy(raw[:C.sizeof(PackedHeader)])
+    rc = lib().bfaintb_packed_header_check(C.byref(h))
+    if rc:
+        raise BfaintbError(rc, "bfaintb_packed_header_check")
+    o0 = h.header_bytes
+    o1 = o0 + h.payload_bytes
+    o2 = o1 + h.scale_bytes
+    o3 = o2 + (2 * h.n if h.has_bias else 0)
+    if len(raw) != o3:
+        raise ValueError("load_packed: file size does not match the header")
+    packed = torch.from_numpy(np.frombuffer(raw, np.uint8, h.payload_bytes, o0).copy()).to(device)
+    groups = h.k // h.group_size if h.group_size else 1
+    scale = torch.from_numpy(np.frombuffer(raw, np.int16, h.scale_bytes // 2, o1).copy()).view(torch.bfloat16).view(groups, h.n).to(device)
+    bias = None
+    if h.has_bias:
+        bias = torch.from_numpy(np.frombuffer(raw, np.int16, h.n, o2).copy()).view(torch.bfloat16).to(device)
+    return h, packed, scale, bias
+
+
+def _torch():
+    import torch
+    return torch
 
 
 def dequant(w, b, scale, n, k, ldb=None, ldw=None, weight_bits=8, group_size=0, stream=None, check=True):

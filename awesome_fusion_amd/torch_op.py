@@ -7,6 +7,7 @@ forward pass: activations A [m, k], weights B [k, n], per-output-channel scale, 
 library:
 
     torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size, bias=None) -> c
+    torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, scale, weight_bits, group_size, bias=None) -> c
 
 ``a`` bf16 [m, k] (row stride a multiple of 8 elements), ``b`` uint8 [k, n] (8-bit, excess-128) or
 [k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n], ``bias`` bf16 [n]
@@ -21,7 +22,8 @@ from typing import Optional
 
 import torch
 
-from .gemm import gemm as _gemm, workspace_bytes as _workspace_bytes, workspace_init as _workspace_init
+from .gemm import (gemm as _gemm, gemm_prepacked as _gemm_prepacked, prepack as _prepack, prepack_bytes as _prepack_bytes,
+                   workspace_bytes as _workspace_bytes, workspace_init as _workspace_init)
 
 _LIB_NAME = "awesome_fusion"
 _workspaces = {}
@@ -87,6 +89,63 @@ def _(a, b, scale, weight_bits, group_size, bias=None):
     return a.new_empty((m, n))
 
 
+@torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm_prepacked", mutates_args=())
+def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
+                           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same product with the weights in the library's pre-packed order (``prepack_weight``): ``packed`` is a flat
+    uint8 tensor of k * n * weight_bits / 8 bytes, n is taken from ``scale``.  Needs no workspace."""
+    m, n, k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
+    if not a.is_cuda:
+        raise RuntimeError("bfaintb_gemm_prepacked runs on the GPU only (no CPU implementation)")
+    if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
+        a = a.contiguous()
+    packed = packed.contiguous()
+    scale = scale.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    if m == 0 or n == 0:
+        return c
+    with torch.cuda.device(a.device):
+        _gemm_prepacked(c, a, packed, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, bias=bias)
+    return c
+
+
+def _check_prepacked(a, packed, scale, weight_bits, group_size, bias=None):
+    if a.dim() != 2 or scale.dim() != 2 or packed.dim() != 1:
+        raise ValueError("bfaintb_gemm_prepacked: a [m, k], packed [k*n*bits/8], scale [groups, n]")
+    if a.dtype != torch.bfloat16 or scale.dtype != torch.bfloat16 or packed.dtype != torch.uint8:
+        raise TypeError("bfaintb_gemm_prepacked: a and scale must be bfloat16, packed uint8")
+    if weight_bits not in (8, 4):
+        raise ValueError("bfaintb_gemm_prepacked: weight_bits must be 8 or 4")
+    k, n = a.shape[1], scale.shape[1]
+    groups = k // group_size if group_size else 1
+    if scale.shape[0] != groups or packed.numel() != k * n * weight_bits // 8:
+        raise ValueError(f"bfaintb_gemm_prepacked: shapes do not agree: a {tuple(a.shape)}, packed {packed.numel()} bytes, scale {tuple(scale.shape)}")
+    if bias is not None and (bias.dtype != torch.bfloat16 or tuple(bias.shape) != (n,)):
+        raise ValueError("bfaintb_gemm_prepacked: bias must be bfloat16 [n]")
+    return a.shape[0], n, k
+
+
+@bfaintb_gemm_prepacked.register_fake
+def _(a, packed, scale, weight_bits, group_size, bias=None):
+    m, n, _k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
+    return a.new_empty((m, n))
+
+
+def prepack_weight(b, weight_bits=8):
+    """Row-major codes ``b`` (uint8 [k, n*bits/8], on the GPU) -> flat packed tensor for ``bfaintb_gemm_prepacked``."""
+    k = b.shape[0]
+    n = b.shape[1] * (8 // weight_bits)
+    nbytes = _prepack_bytes(n, k, weight_bits)
+    if nbytes == 0:
+        raise ValueError("prepack_weight: the packed order needs n % 16 == 0 and k % 64 == 0 (k % 128 == 0 for 4-bit codes)")
+    packed = torch.empty(nbytes, dtype=torch.uint8, device=b.device)
+    with torch.cuda.device(b.device):
+        _prepack(packed, b.contiguous(), n, k, weight_bits=weight_bits)
+    return packed
+
+
 def quantize_weight(weight, weight_bits=8, group_size=0):
     """float weight [n_out, k_in] (a torch Linear's layout) -> (b uint8 [k, n*bits/8], scale bf16 [groups, n]).
 
@@ -121,6 +180,7 @@ class QuantLinear(torch.nn.Module):
         groups = in_features // group_size if group_size else 1
         self.in_features, self.out_features = in_features, out_features
         self.weight_bits, self.group_size = weight_bits, group_size
+        self.prepacked = False
         self.register_buffer("qweight", torch.zeros((in_features, out_features * weight_bits // 8), dtype=torch.uint8, device=device))
         self.register_buffer("scales", torch.zeros((groups, out_features), dtype=torch.bfloat16, device=device))
         self.bias = torch.nn.Parameter(torch.zeros(out_features, dtype=torch.bfloat16, device=device)) if bias else None
@@ -135,8 +195,16 @@ class QuantLinear(torch.nn.Module):
             q.bias.data.copy_(linear.bias.detach().to(torch.bfloat16))
         return q
 
+    def prepack(self):
+        """Switches the layer to the pre-packed weight order (on the GPU, once): the row-major codes are replaced."""
+        if not self.prepacked:
+            self.qweight = prepack_weight(self.qweight, self.weight_bits)
+            self.prepacked = True
+        return self
+
     def forward(self, x):
         lead = x.shape[:-1]
-        y = torch.ops.awesome_fusion.bfaintb_gemm(x.reshape(-1, self.in_features).to(torch.bfloat16), self.qweight, self.scales,
-                                                  self.weight_bits, self.group_size, self.bias)
+        op = torch.ops.awesome_fusion.bfaintb_gemm_prepacked if self.prepacked else torch.ops.awesome_fusion.bfaintb_gemm
+        y = op(x.reshape(-1, self.in_features).to(torch.bfloat16), self.qweight, self.scales, self.weight_bits, self.group_size,
+               self.bias)
         return y.reshape(*lead, self.out_features)

@@ -138,6 +138,31 @@ BFAINTB_API int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* pa
                               void* stream, int variant);
 BFAINTB_API int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 
+/*
+ * Wire / on-disk form of a pre-packed weight: this 64-byte little-endian header, then payload_bytes of packed codes
+ * (what bfaintb_prepack wrote), then scale_bytes of bf16 scales, row-major [groups][n], then, if has_bias, n bf16
+ * biases.  Sections follow one another without padding (all sizes are multiples of 32 bytes).  The two functions run
+ * on the host and touch no device: _init fills a header for a shape (same shape rules as bfaintb_prepack), _check
+ * returns BFAINTB_OK for a header this library can consume (magic, layout, shape rules, section sizes that agree
+ * with the shape) and a negative BFAINTB_ERR_* otherwise.
+ */
+typedef struct bfaintb_packed_header {
+    char magic[8];          /* "BFAINTB1" */
+    uint32_t header_bytes;  /* 64 */
+    uint32_t layout;        /* BFAINTB_LAYOUT_MFMA16 */
+    uint32_t weight_bits;   /* 8 or 4 */
+    uint32_t group_size;    /* rows of k per scale group; 0 = one scale per output channel */
+    uint32_t k, n;
+    uint64_t payload_bytes; /* n * k * weight_bits / 8 */
+    uint64_t scale_bytes;   /* groups * n * 2 */
+    uint32_t has_bias;      /* 0 or 1 */
+    uint32_t reserved[3];   /* zero */
+} bfaintb_packed_header;
+#define BFAINTB_LAYOUT_MFMA16 1u
+BFAINTB_API int bfaintb_packed_header_init(bfaintb_packed_header* h, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
+                               int has_bias);
+BFAINTB_API int bfaintb_packed_header_check(const bfaintb_packed_header* h);
+
 /* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */
 BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 

@@ -120,6 +120,40 @@ def test_prepacked_entry_points_validate_before_launching():
     assert L.bfaintb_gemm_prepacked_variant(1, 100, 4096, 8, 0) == -2
 
 
+def test_packed_file_header_and_round_trip(tmp_path):
+    import torch
+    L = af.lib()
+    h = af.PackedHeader()
+    assert C.sizeof(h) == 64
+    assert L.bfaintb_packed_header_init(C.byref(h), 4096, 8192, 4, 128, 1) == 0
+    assert (h.magic, h.header_bytes, h.layout, h.weight_bits, h.group_size, h.k, h.n) == (b"BFAINTB1", 64, 1, 4, 128, 8192, 4096)
+    assert h.payload_bytes == 4096 * 8192 // 2 and h.scale_bytes == 64 * 4096 * 2 and h.has_bias == 1
+    assert L.bfaintb_packed_header_check(C.byref(h)) == 0
+    assert L.bfaintb_packed_header_init(C.byref(h), 4096, 4160, 4, 0, 0) == -2     # 4-bit: k % 128
+    assert L.bfaintb_packed_header_init(C.byref(h), 4096, 4096, 8, 48, 0) == -5
+    assert L.bfaintb_packed_header_init(None, 16, 64, 8, 0, 0) == -1
+    L.bfaintb_packed_header_init(C.byref(h), 64, 128, 8, 0, 0)
+    for field, bad in (("magic", b"BFAINTB2"), ("layout", 2), ("payload_bytes", 1), ("scale_bytes", 64), ("n", 72), ("has_bias", 2)):
+        g = af.PackedHeader.from_buffer_copy(bytes(h))
+        setattr(g, field, bad)
+        assert L.bfaintb_packed_header_check(C.byref(g)) < 0, field
+    # file round trip (host tensors: nothing here touches a device)
+    n, k = 64, 128
+    packed = torch.arange(n * k, dtype=torch.int64).to(torch.uint8)
+    scale = torch.linspace(0.001, 0.01, n).to(torch.bfloat16).view(1, n)
+    bias = torch.linspace(-1, 1, n).to(torch.bfloat16)
+    path = str(tmp_path / "w.bfaintb")
+    af.save_packed(path, packed, scale, n, k, 8, 0, bias)
+    assert os.path.getsize(path) == 64 + n * k + 2 * n + 2 * n
+    h2, p2, s2, b2 = af.load_packed(path, device="cpu")
+    assert (h2.n, h2.k, h2.weight_bits, h2.has_bias) == (n, k, 8, 1)
+    assert torch.equal(p2, packed) and torch.equal(s2.view(torch.int16), scale.view(torch.int16)) and torch.equal(b2.view(torch.int16), bias.view(torch.int16))
+    with open(path, "ab") as f:
+        f.write(b"x")
+    with pytest.raises(ValueError):
+        af.load_packed(path, device="cpu")
+
+
 def test_product_does_not_reach_for_the_oracle():
     # the shipped package and the C/HIP sources must not import, include or link anything under oracle/
     pkg = os.path.join(ROOT, "awesome_fusion_amd")

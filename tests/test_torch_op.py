@@ -86,3 +86,40 @@ def test_quant_linear_forward():
     assert torch.allclose(y.float().reshape(-1, 256), ref, rtol=2e-2, atol=2e-2)
     # and the quantised layer tracks the float layer it came from
     assert (y.float() - lin(x)).abs().max() < 0.05
+
+
+def test_prepacked_operator_is_registered_and_infers_shapes():
+    a = torch.zeros((5, 128), dtype=torch.bfloat16, device="meta")
+    packed = torch.zeros(128 * 48 // 2, dtype=torch.uint8, device="meta")
+    s = torch.zeros((2, 48), dtype=torch.bfloat16, device="meta")
+    out = torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, s, 4, 64)
+    assert out.shape == (5, 48) and out.dtype == torch.bfloat16
+    with pytest.raises(Exception):
+        torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed[:-1], s, 4, 64)
+    with pytest.raises(RuntimeError):           # no CPU implementation
+        torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a.to("cpu"), packed.to("cpu"), s.to("cpu"), 4, 64)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k,bits,group", [(1, 4096, 4096, 8, 0), (7, 528, 1024, 4, 128), (600, 512, 512, 8, 0)])
+def test_prepacked_operator_matches_oracle(m, n, k, bits, group):
+    p = Problem(m, n, k, bits, group, seed=700 + m)
+    a = torch.from_numpy(p.a_bf.view(np.int16)).cuda().view(torch.bfloat16)
+    s = torch.from_numpy(p.s_bf.view(np.int16)).cuda().view(torch.bfloat16)
+    packed = top.prepack_weight(torch.from_numpy(p.b_bytes).cuda(), bits)
+    c = torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, s, bits, group)
+    torch.cuda.synchronize()
+    assert_close_ulp(p, c.view(torch.int16).cpu().numpy().view(np.uint16), f"prepacked torch operator m={m}")
+
+
+@pytest.mark.gpu
+def test_quant_linear_prepacked_matches_row_major_layer():
+    torch.manual_seed(1)
+    lin = torch.nn.Linear(512, 256, bias=True).cuda()
+    ql = top.QuantLinear.from_float(lin, weight_bits=4, group_size=128)
+    x = torch.randn((3, 512), device="cuda")
+    y_row = ql(x)
+    y_packed = ql.prepack()(x)
+    assert ql.prepacked and ql.qweight.dim() == 1
+    # same weights, same fp32 accumulation up to summation order: within a bf16 ULP or two of each other
+    assert torch.allclose(y_row.float(), y_packed.float(), rtol=2e-2, atol=2e-3)
