@@ -117,23 +117,38 @@ hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k,
 //   grid = (n / 16, 1, ceil(m / (16 MB))); block = 8 waves.  A workgroup owns one column block (16 columns) and
 //   MB blocks of 16 rows of A, over all of k; wave w takes the K-chunks w, w + 8, ... of the slab in batches: the
 //   weight loads of a batch (one 128-bit load per chunk) and their activation loads are issued back to back, and
-//   a wave keeps 8 KiB (8-bit) or 4 KiB (4-bit) of the slab in flight — as one batch when that is all the wave has
-//   (k up to 4096 for 8-bit codes; measured 2 % faster at k = 4096), else as two half-size batches, the next one
-//   loaded before the current one is converted (9 % faster at k = 11008).  Per K-block of 32
+//   a wave keeps up to 8 KiB (8-bit) or 4 KiB (4-bit) of the slab in flight — large batches one at a time, or (long
+//   k, per-channel scales) small batches with the next one loaded before the current one is converted.  Per K-block of 32
 //   rows: one conversion of 8 weights and MB v_mfma_f32_16x16x32_bf16 with the operands swapped, as in the
 //   row-major decode kernel (lane (nl, kg): W column nl, A row nl, rows 8 kg .. 8 kg + 7 of the K-block).  The
 //   eight waves' accumulators meet in LDS and are added in wave order: the summation order is fixed.
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kPackedWaves = 8;
+constexpr int kPackedWaves = 8;  // measured: 4 and 16 waves per workgroup are 12-19 % slower at n = k = 4096
 
-template <int BITS, bool GROUPED, int MB, bool WHOLE>
-__global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kernel(const GemmParams p)
+// Chunks per batch.  Plain form: large batches, loaded and converted one at a time (for k up to 4096 with 8-bit codes
+// a wave's only batch).  Pipelined form: small batches, two of them in flight, sized so that the raw chunks (4
+// registers of codes, 4 per K-block and row block of activations) stay under about 100 registers — that kernel is
+// held to 128 so that two workgroups share a CU.
+__host__ __device__ constexpr int packed_batch(int bits, int mb, bool pipelined)
+{
+    if (!pipelined) return (bits == 8 ? 8 : 4) / mb;
+    return bits == 8 ? (mb == 1 ? 3 : 2) : (mb == 1 ? 2 : 1);
+}
+// How a kernel instance finds its scales: one per output channel; one per K-chunk (groups are whole chunks), loaded
+// with the chunk; one per K-block of 32 rows (groups of 32 or 64 rows), also loaded with the chunk.
+enum { kScalePerChannel = 0, kScalePerChunk = 1, kScalePerBlock = 2 };
+
+enum { kPackedPlain = 0, kPackedPipelined = 1, kPackedOneBatch = 2 };
+
+template <int BITS, int SCALES, int MB, int MODE>
+__device__ __forceinline__ void decode_packed_body(const GemmParams& p)
 {
     constexpr uint32_t kBlocks = PackedFormat<BITS>::kBlocks;
     constexpr uint32_t kChunkRows = PackedFormat<BITS>::kChunkRows;
-    // WHOLE: one batch holds all of a wave's chunks (the launcher checks), loaded at once.  Otherwise half as many per
-    // batch and two batches in flight, the next one loaded before the current one is converted.
-    constexpr int kBatch = (BITS == 8 ? 4 : 2) * (WHOLE ? 2 : 1) / MB;
+    constexpr bool GROUPED = SCALES != kScalePerChannel;
+    constexpr uint32_t kScalesPerChunk = SCALES == kScalePerBlock ? PackedFormat<BITS>::kBlocks : 1u;
+    constexpr bool PIPELINED = MODE == kPackedPipelined;
+    constexpr int kBatch = packed_batch(BITS, MB, PIPELINED);
     __shared__ float red[kPackedWaves][MB][16][16 + 4];  // [wave][row block][A row][W column], rows padded
 
     const uint32_t tid = threadIdx.x;
@@ -153,8 +168,6 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
         aptr[mb] = p.a + (size_t)arow * p.lda + 8u * kg;
     }
     const uint16_t* sptr = p.scale + col;
-    // one scale per chunk when groups are whole chunks, else one per K-block
-    const bool scale_per_chunk = GROUPED && p.group_size % kChunkRows == 0;
 
     float cs = 0.f;
     if constexpr (!GROUPED) cs = make_col_scale<BITS>(*sptr);
@@ -166,7 +179,7 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
     struct Batch {
         uint4 w[kBatch];
         uint4 a[kBatch][kBlocks][MB];
-        uint32_t s[kBatch][kBlocks];
+        uint32_t s[kBatch][kScalesPerChunk];
     };
     // all loads of a batch, back to back (chunks past the end re-read the last one; compute() skips them)
     auto load = [&](Batch& b, uint32_t base) {
@@ -180,25 +193,23 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) b.a[i][h][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + kChunkRows * c + 32u * h);
             if constexpr (GROUPED) {
-                if (scale_per_chunk) {
-                    b.s[i][0] = sptr[(size_t)((kChunkRows * c) / p.group_size) * p.lds];
-                } else {
 #pragma unroll
-                    for (uint32_t h = 0; h < kBlocks; ++h) b.s[i][h] = sptr[(size_t)((kChunkRows * c + 32u * h) / p.group_size) * p.lds];
-                }
+                for (uint32_t h = 0; h < kScalesPerChunk; ++h) b.s[i][h] = sptr[(size_t)((kChunkRows * c + 32u * h) / p.group_size) * p.lds];
             }
         }
     };
-    auto compute = [&](const Batch& b, uint32_t base) {
+    // GUARDED: the batch may reach past the last chunk (wave-uniform tests); whole batches run as one straight block
+    auto compute = [&](const Batch& b, uint32_t base, auto guarded_c) {
+        constexpr bool GUARDED = decltype(guarded_c)::value;
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const uint32_t c = base + (uint32_t)i * kPackedWaves;
-            if (c < chunks) {  // wave-uniform
+            if (!GUARDED || c < chunks) {
                 const uint32_t wd[4] = {b.w[i].x, b.w[i].y, b.w[i].z, b.w[i].w};
 #pragma unroll
                 for (uint32_t h = 0; h < kBlocks; ++h) {
                     float s = cs;
-                    if constexpr (GROUPED) s = make_col_scale<BITS>(scale_per_chunk ? b.s[i][0] : b.s[i][h]);
+                    if constexpr (GROUPED) s = make_col_scale<BITS>(b.s[i][SCALES == kScalePerBlock ? h : 0u]);
                     uint4 w;
                     if constexpr (BITS == 8) {
                         const uint32_t lo = codes8_to_s8(wd[2 * h]), hi = codes8_to_s8(wd[2 * h + 1]);
@@ -223,24 +234,41 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
         }
     };
 
-    // two batches in flight: the loads of the next batch are issued before the current one is converted
     constexpr uint32_t kStride = kPackedWaves * kBatch;
-    Batch b0;
     uint32_t base = wave;
-    if (base < chunks) load(b0, base);
-    if constexpr (WHOLE) {
-        compute(b0, base);
-        base = chunks;
-    }
-    Batch b1;
-    while (base < chunks) {
-        if (base + kStride < chunks) load(b1, base + kStride);
-        compute(b0, base);
-        base += kStride;
-        if (base >= chunks) break;
-        if (base + kStride < chunks) load(b0, base + kStride);
-        compute(b1, base);
-        base += kStride;
+    if constexpr (MODE == kPackedOneBatch) {
+        // the launcher has checked that the slab is exactly one batch per wave: straight-line code, every load first
+        Batch b;
+        load(b, base);
+        compute(b, base, std::false_type{});
+    } else if constexpr (!PIPELINED) {
+        for (; base + kStride - kPackedWaves < chunks; base += kStride) {  // batches whose every chunk exists
+            Batch b;
+            load(b, base);
+            compute(b, base, std::false_type{});
+        }
+        if (base < chunks) {
+            Batch b;
+            load(b, base);
+            compute(b, base, std::true_type{});
+        }
+    } else {
+        // two batches in flight: the loads of the next batch are issued before the current one is converted
+        auto compute_any = [&](const Batch& b, uint32_t at) {
+            if (at + kStride - kPackedWaves < chunks) compute(b, at, std::false_type{});
+            else compute(b, at, std::true_type{});
+        };
+        Batch b0, b1;
+        if (base < chunks) load(b0, base);
+        while (base < chunks) {
+            if (base + kStride < chunks) load(b1, base + kStride);
+            compute_any(b0, base);
+            base += kStride;
+            if (base >= chunks) break;
+            if (base + kStride < chunks) load(b0, base + kStride);
+            compute_any(b1, base);
+            base += kStride;
+        }
     }
 
     // acc[mb][r] of lane (nl, kg) is the sum for A row nl of block mb, W column 4 kg + r of the column block
@@ -262,25 +290,61 @@ __global__ void __launch_bounds__(64 * kPackedWaves) bfaintb_decode_packed_kerne
     }
 }
 
-template <int BITS, bool GROUPED>
+// (no more than four waves per SIMD asked for: told that eight are possible, the compiler delays loads to save registers)
+template <int BITS, int SCALES, int MB>
+__global__ void __launch_bounds__(64 * kPackedWaves) __attribute__((amdgpu_waves_per_eu(2, 4)))
+bfaintb_decode_packed_kernel(const GemmParams p)
+{
+    decode_packed_body<BITS, SCALES, MB, kPackedPlain>(p);
+}
+
+// (the 128-register form of the attribute: measured 6 % faster here than the looser one above, which wins for the loop)
+template <int BITS, int SCALES, int MB>
+__global__ void __launch_bounds__(64 * kPackedWaves) __attribute__((amdgpu_waves_per_eu(4)))
+bfaintb_decode_packed_one_batch_kernel(const GemmParams p)
+{
+    decode_packed_body<BITS, SCALES, MB, kPackedOneBatch>(p);
+}
+
+// (at most 128 registers, so that two workgroups share a CU)
+template <int BITS, int MB>
+__global__ void __launch_bounds__(64 * kPackedWaves) __attribute__((amdgpu_waves_per_eu(4)))
+bfaintb_decode_packed_pipelined_kernel(const GemmParams p)
+{
+    decode_packed_body<BITS, kScalePerChannel, MB, kPackedPipelined>(p);
+}
+
+template <int BITS, int SCALES>
 static hipError_t launch_decode_packed_t(const GemmParams& p, hipStream_t stream)
 {
     // two row blocks per workgroup once there are more than 16 rows: the weights are converted once for both
     const uint32_t mb = p.m > 16u ? 2u : 1u;
-    // chunks per wave that fit the one-batch form: 8 / mb of 64 rows (8-bit) or 4 / mb of 128 rows (4-bit)
     const uint32_t chunks = p.k / PackedFormat<BITS>::kChunkRows;
-    const bool whole = chunks <= kPackedWaves * (BITS == 8 ? 8u : 4u) / mb;
+    // the pipelined form when a wave has more than one plain batch of chunks and scales are per channel (measured: 9 %
+    // faster at k = 11008 with per-channel scales, 10-25 % slower than the plain form with grouped ones)
+    const bool pipelined = SCALES == kScalePerChannel && chunks > (uint32_t)(kPackedWaves * packed_batch(BITS, (int)mb, false));
+    const bool one_batch = chunks == (uint32_t)(kPackedWaves * packed_batch(BITS, (int)mb, false));
     void (*kernel)(const GemmParams) =
-        mb == 2u ? (whole ? bfaintb_decode_packed_kernel<BITS, GROUPED, 2, true> : bfaintb_decode_packed_kernel<BITS, GROUPED, 2, false>)
-                 : (whole ? bfaintb_decode_packed_kernel<BITS, GROUPED, 1, true> : bfaintb_decode_packed_kernel<BITS, GROUPED, 1, false>);
+        mb == 2u ? (pipelined   ? bfaintb_decode_packed_pipelined_kernel<BITS, 2>
+                    : one_batch ? bfaintb_decode_packed_one_batch_kernel<BITS, SCALES, 2>
+                                : bfaintb_decode_packed_kernel<BITS, SCALES, 2>)
+                 : (pipelined   ? bfaintb_decode_packed_pipelined_kernel<BITS, 1>
+                    : one_batch ? bfaintb_decode_packed_one_batch_kernel<BITS, SCALES, 1>
+                                : bfaintb_decode_packed_kernel<BITS, SCALES, 1>);
     return launch_kernel(kernel, dim3(p.n / 16u, 1, (p.m + 16u * mb - 1u) / (16u * mb)), dim3(64 * kPackedWaves, 1, 1), 0, stream, p);
+}
+
+template <int BITS>
+static hipError_t launch_decode_packed_b(const GemmParams& p, hipStream_t stream)
+{
+    if (p.group_size == 0) return launch_decode_packed_t<BITS, kScalePerChannel>(p, stream);
+    if (p.group_size % PackedFormat<BITS>::kChunkRows == 0) return launch_decode_packed_t<BITS, kScalePerChunk>(p, stream);
+    return launch_decode_packed_t<BITS, kScalePerBlock>(p, stream);
 }
 
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream)
 {
-    const bool grouped = p.group_size != 0;
-    if (bits == 8) return grouped ? launch_decode_packed_t<8, true>(p, stream) : launch_decode_packed_t<8, false>(p, stream);
-    return grouped ? launch_decode_packed_t<4, true>(p, stream) : launch_decode_packed_t<4, false>(p, stream);
+    return bits == 8 ? launch_decode_packed_b<8>(p, stream) : launch_decode_packed_b<4>(p, stream);
 }
 
 }  // namespace bfaintb

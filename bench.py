@@ -84,14 +84,24 @@ class Workload:
         return ws
 
 
-def time_graph(af, w, steps, warmup, rotate):
-    """Returns (event_ms_per_step, wall_ms_per_step)."""
+def time_graph(af, w, steps, warmup, rotate, packed=False):
+    """Returns (event_ms_per_step, wall_ms_per_step).  packed: every copy of B is reordered once (untimed, as a model
+    loader would) and the launches go through bfaintb_gemm_prepacked."""
     import torch
     ws = w.workspace(af)
     nb = len(w.b) if rotate else 1
+    if packed:
+        pks = []
+        for i in range(nb):
+            pk = torch.empty(af.prepack_bytes(w.n, w.k, w.bits), dtype=torch.uint8, device="cuda")
+            af.prepack(pk, w.b[i], w.n, w.k, weight_bits=w.bits)
+            pks.append(pk)
 
     def launch(i):
-        af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
+        if packed:
+            af.gemm_prepacked(w.c, w.a, pks[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group)
+        else:
+            af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
 
     for i in range(warmup):
         launch(i)
@@ -258,8 +268,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (decode sweep, int4 group-128)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="time only this workload family: decode | prefill | decode_cold "
-                    "(decode_cold: nothing but the headline's cold-B launches, for a kernel trace without the hot and eager variants)")
+    ap.add_argument("--only", default="", help="time only this workload family: decode | prefill | decode_cold | decode_packed_cold "
+                    "(decode_cold: nothing but the headline's cold-B launches, for a kernel trace without the hot and eager variants; "
+                    "decode_packed_cold: the same launches over pre-packed weights)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM shards over n with no "
@@ -277,11 +288,13 @@ def main():
 
     # ---- headline: decode M=1, N=K=4096, int8 per-channel; cold B (rotating copies > last-level cache)
     res = None
-    cold_only = args.only == "decode_cold"
-    if args.only in ("", "decode", "decode_cold"):
+    cold_only = args.only in ("decode_cold", "decode_packed_cold")
+    if args.only in ("", "decode", "decode_cold", "decode_packed_cold"):
         copies = LLC_BYTES * 2 // (4096 * 4096) + 8  # 40 copies = 640 MiB
         w = Workload("decode_m1_n4096_k4096_int8_perchannel", 1, 4096, 4096, copies=copies)
-        ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True)
+        ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True, packed=args.only == "decode_packed_cold")
+        if args.only == "decode_packed_cold":
+            w.name += "_prepacked"
         hot_ms, _ = (ev_ms, wall_ms) if cold_only else time_graph(af, w, K, W, rotate=False)
         eager_ms = ev_ms if cold_only else time_eager(af, w, K, W)
         read_ms = ev_ms if cold_only else time_read_ceiling(af, w, K, W)
@@ -306,6 +319,11 @@ def main():
                                                       "note": "B re-read from cache: not an HBM figure"}
             out_extra["decode_m1_eager_launch_loop"] = {"us_per_launch": round(eager_ms * 1e3, 3),
                                                         "note": "reference protocol (no graph): host launch rate included"}
+            pk_ms, _ = time_graph(af, w, K, W, rotate=True, packed=True)
+            out_extra["decode_m1_prepacked"] = {
+                **roofline_entry(w, pk_ms, "hbm"), "frac_of_fetch_only": round(read_ms / pk_ms, 4),
+                "note": "same shape and cold-B rotation through bfaintb_gemm_prepacked (weights reordered once, offline): "
+                        "no split-K, no workspace; not the drop-in row-major path, so not `value`"}
         if not args.no_cpu and not cold_only:
             one, allc, nrms = cpu_baseline(w, c_gpu)
             res["cpu_baseline"] = one
@@ -328,6 +346,8 @@ def main():
                                                     "note": "torch.matmul bf16 x bf16 on pre-dequantised weights (no dequantisation work): context, not a baseline"}
         except Exception as exc:  # context only
             entry["vendor_bf16_gemm_same_shape"] = {"error": str(exc)[:200]}
+        pk_ms, _ = time_graph(af, w, pk, max(5, W // 4), rotate=True, packed=True)
+        entry["prepacked"] = {**roofline_entry(w, pk_ms, "mfma"), "note": "bfaintb_gemm_prepacked, same shape"}
         out_extra["prefill_m4096"] = entry
         if res is None:
             res = {"metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=4096: TFLOP/s", "value": entry["value"], "unit": "TFLOP/s",
@@ -343,12 +363,18 @@ def main():
             w = Workload(f"decode_m{m}_n11008_k4096_int8_perchannel", m, 11008, 4096, copies=14)
             ev_ms, _ = time_graph(af, w, min(K, 200), W, rotate=True)
             sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "hbm")})
+            if m <= 8:
+                pk_ms, _ = time_graph(af, w, min(K, 200), W, rotate=True, packed=True)
+                sweep.append({"workload": w.name + "_prepacked", **roofline_entry(w, pk_ms, "hbm")})
             del w
             torch.cuda.empty_cache()
         for m in (1, 16, 2048):
             w = Workload(f"m{m}_n28672_k8192_int4_group128", m, 28672, 8192, bits=4, group=128, copies=6 if m <= 32 else 1)
             ev_ms, _ = time_graph(af, w, min(K, 100) if m <= 32 else 10, min(W, 10), rotate=True)
             sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "hbm" if m <= 32 else "mfma")})
+            if m == 1:
+                pk_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True, packed=True)
+                sweep.append({"workload": w.name + "_prepacked", **roofline_entry(w, pk_ms, "hbm")})
             del w
             torch.cuda.empty_cache()
         out_extra["sweep"] = sweep

@@ -69,7 +69,10 @@ def test_pack_honours_the_row_stride(af):
 
 @pytest.mark.parametrize("m,n,k,bits,group", [
     (1, 16, 64, 8, 0), (1, 256, 512, 8, 0), (3, 48, 192, 8, 64), (16, 64, 1024, 4, 0), (17, 80, 640, 4, 32),
-    (33, 96, 1152, 4, 128), (70, 64, 1600, 8, 32), (1, 32, 8256, 8, 0), (40, 128, 4096, 8, 128), (5, 1024, 2048, 4, 128)])
+    (33, 96, 1152, 4, 128), (70, 64, 1600, 8, 32), (1, 32, 8256, 8, 0), (40, 128, 4096, 8, 128), (5, 1024, 2048, 4, 128),
+    # every launch form: one batch per wave (k = 4096 / 2048 for 8-bit with 1 / 2 row blocks, 4096 for 4-bit), pipelined
+    # (long k, per-channel scales), with one and two row blocks
+    (20, 48, 2048, 8, 0), (3, 32, 4096, 4, 128), (2, 32, 8192, 4, 0), (40, 32, 8256, 8, 0), (24, 32, 8192, 4, 0), (9, 64, 4096, 8, 0)])
 def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
     p = Problem(m, n, k, bits, group, seed=m + n + k)
     assert_close_ulp(p, run_prepacked(af, p, af.DECODE), f"packed decode {m}x{n}x{k} b{bits} g{group}")
