@@ -37,10 +37,13 @@ REPLAYS = 5                   # timed replays of the K-launch graph; the median 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
 MEASURED_TRAFFIC_BYTES = {
-    # fetch 8399.2 KiB x 1.997 + write 232.0 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
-    "decode_m1_n4096_k4096_int8_perchannel": 17413327,
-    # fetch 65627.0 KiB x 1.997 + write 32768.0 KiB
-    "prefill_m4096_n4096_k4096_int8_perchannel": 167756921,
+    # fetch 8392.4 KiB x 1.997 + write 232.0 KiB (profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
+    "decode_m1_n4096_k4096_int8_perchannel": 17399422,
+    # fetch 65640.5 KiB x 1.997 + write 32768.0 KiB
+    "prefill_m4096_n4096_k4096_int8_perchannel": 167784528,
+    # the same shapes through bfaintb_gemm_prepacked: fetch 8276.0 KiB x 1.997 + write 8.0 KiB; fetch 65648.5 KiB x 1.997 + write 32768.0 KiB
+    "decode_m1_n4096_k4096_int8_perchannel_prepacked": 16932016,
+    "prefill_m4096_n4096_k4096_int8_perchannel_prepacked": 167800888,
 }
 
 
@@ -191,7 +194,7 @@ def time_eager(af, w, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
-def roofline_entry(w, ms, bound):
+def roofline_entry(w, ms, bound, suffix=""):
     if bound == "hbm":
         achieved = w.bytes / (ms * 1e-3) / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
@@ -199,7 +202,7 @@ def roofline_entry(w, ms, bound):
         achieved = w.flops / (ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
     return {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name), "kernel_us": round(ms * 1e3, 3),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name + suffix), "kernel_us": round(ms * 1e3, 3),
             "algorithmic_bytes": w.bytes, "flops": w.flops}
 
 
@@ -321,7 +324,7 @@ def main():
                                                         "note": "reference protocol (no graph): host launch rate included"}
             pk_ms, _ = time_graph(af, w, K, W, rotate=True, packed=True)
             out_extra["decode_m1_prepacked"] = {
-                **roofline_entry(w, pk_ms, "hbm"), "frac_of_fetch_only": round(read_ms / pk_ms, 4),
+                **roofline_entry(w, pk_ms, "hbm", "_prepacked"), "frac_of_fetch_only": round(read_ms / pk_ms, 4),
                 "note": "same shape and cold-B rotation through bfaintb_gemm_prepacked (weights reordered once, offline): "
                         "no split-K, no workspace; not the drop-in row-major path, so not `value`"}
         if not args.no_cpu and not cold_only:
@@ -347,7 +350,7 @@ def main():
         except Exception as exc:  # context only
             entry["vendor_bf16_gemm_same_shape"] = {"error": str(exc)[:200]}
         pk_ms, _ = time_graph(af, w, pk, max(5, W // 4), rotate=True, packed=True)
-        entry["prepacked"] = {**roofline_entry(w, pk_ms, "mfma"), "note": "bfaintb_gemm_prepacked, same shape"}
+        entry["prepacked"] = {**roofline_entry(w, pk_ms, "mfma", "_prepacked"), "note": "bfaintb_gemm_prepacked, same shape"}
         out_extra["prefill_m4096"] = entry
         if res is None:
             res = {"metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=4096: TFLOP/s", "value": entry["value"], "unit": "TFLOP/s",
