@@ -23,6 +23,7 @@ from .gemm import (  # noqa: F401
     prepack,
     prepack_bytes,
     prepacked_variant,
+    prepacked_workspace_bytes,
     library_path,
     probe_read,
     split_k,

@@ -21,6 +21,7 @@ hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k,
                        hipStream_t stream);
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
 }  // namespace bfaintb
 
 namespace {
@@ -34,6 +35,7 @@ constexpr uint32_t kDecodeMaxM = 32768;        // what the decode family accepts
 constexpr uint32_t kDecodeTargetWgs = 480;        // 4-wave workgroups: a little under two per CU on a 256-CU part
 constexpr uint32_t kDecodeTargetWgsNarrow = 256;  // 8-wave workgroups: one per CU
 constexpr uint32_t kMaxSplits = 64;
+constexpr uint32_t kPackedSlabMaxM = 48;       // packed weights: the slab-streaming kernel up to this m, the row-blocked family beyond
 
 int check_format(uint32_t k, int bits, uint32_t group_size)
 {
@@ -385,19 +387,20 @@ int bfaintb_unpack(void* b, const void* packed, uint32_t n, uint32_t k, uint32_t
     return repack(b, packed, n, k, ldb, weight_bits, stream, true);
 }
 
-// Which kernel multiplies by packed weights.  The packed decode kernel streams the weights once per 16 (m <= 16)
-// or 32 rows of A and fetches A from cache for every matrix instruction: measured on a 256-CU part at n = k = 4096,
-// 3.5 us + 0.23 us per row of A (5.6, 7.1, 10.6, 18.2 us at m = 1, 16, 32, 64), taken to scale with n * k.
-static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int variant)
+// Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one up to kPackedSlabMaxM rows of A, the
+// row-blocked family without a split along k beyond) or the tiled kernel, by the estimates that choose for row-major weights.
+static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
-    if (variant == BFAINTB_VARIANT_DECODE || variant == BFAINTB_VARIANT_PREFILL) return variant;
+    if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
+    if (variant == BFAINTB_VARIANT_PREFILL) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
-    if (m <= kDecodeAutoMaxM) return BFAINTB_VARIANT_DECODE;
-    const double decode_us = 3.5 + 0.23 * m * ((double)n * k / (4096.0 * 4096.0));
+    if (m <= kPackedSlabMaxM) return BFAINTB_VARIANT_DECODE;
+    if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
+    const DecodePlan pl = decode_plan(m, n, k, bits, 0);
     // a lightly loaded machine runs the tiled kernel's steps faster (measured 57 us at m = 256 and 512, n = k = 4096)
     const uint32_t tiles = ((m + 255u) / 256u) * ((n + 255u) / 256u);
     const double prefill_us = tiles <= 64u ? 4.0 + (k / 64.0) * 0.85 : prefill_estimate_us(m, n, k);
-    return decode_us < prefill_us ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return decode_family_estimate_us(m, n, k, bits, pl) * 1.1 < prefill_us ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
@@ -408,12 +411,31 @@ int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weigh
     if (e) return e;
     e = check_packed_shape(n, k, weight_bits);
     if (e) return e;
-    return packed_variant(m, n, k, BFAINTB_VARIANT_AUTO);
+    return packed_variant(m, n, k, weight_bits, BFAINTB_VARIANT_AUTO);
+}
+
+// Scratch of the packed path: only the row-blocked decode family (more than kPackedSlabMaxM rows of A) splits along k.
+static size_t packed_workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int v)
+{
+    if (v != BFAINTB_VARIANT_DECODE || m <= kPackedSlabMaxM) return 0;
+    return workspace_need(m, n, k, bits, BFAINTB_VARIANT_DECODE, 0);
+}
+
+size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant)
+{
+    if (check_format(k, weight_bits, group_size) || check_shape(m, n, k) || check_packed_shape(n, k, weight_bits)) return 0;
+    const int v = packed_variant(m, n, k, weight_bits, variant);
+    return v < 0 ? 0 : packed_workspace_need(m, n, k, weight_bits, v);
+}
+
+size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
+{
+    return bfaintb_gemm_prepacked_workspace_bytes_ex(m, n, k, weight_bits, group_size, BFAINTB_VARIANT_AUTO);
 }
 
 int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
-                              uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size, void* stream,
-                              int variant)
+                              uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
+                              void* workspace, size_t workspace_bytes, void* stream, int variant)
 {
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
@@ -422,7 +444,7 @@ int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, cons
     e = check_packed_shape(n, k, weight_bits);
     if (e) return e;
     if (lda < k || ldc < n || lda % 8u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
-    const int v = packed_variant(m, n, k, variant);
+    const int v = packed_variant(m, n, k, weight_bits, variant);
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
     if (c == nullptr || a == nullptr || packed_b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
@@ -446,16 +468,36 @@ int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, cons
             return BFAINTB_ERR_BAD_SHAPE;
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st);
     }
-    // the decode kernel walks 16 (m <= 16) or 32 rows of A per grid step along z
-    if ((m + 31u) / 32u > 65535u) return BFAINTB_ERR_BAD_VARIANT;
+    if (m > kPackedSlabMaxM) {
+        // beyond a few dozen rows the row-blocked decode family (A reused across 128 or 256 columns) reads the packed
+        // slabs: measured at n = k = 4096 and m = 64, 128, 256: 16, 20, 22 us against 18, 34, 63 us for the slab kernel.
+        // Same plan as for row-major weights, split along k and workspace protocol included.
+        if (m > kDecodeMaxM) return BFAINTB_ERR_BAD_VARIANT;
+        const DecodePlan pl = decode_plan(m, n, k, weight_bits, 0);
+        p.k_per_wg = pl.k_per_wg;
+        p.splits = pl.splits;
+        p.decode_waves = pl.waves;
+        p.decode_cols = pl.cols;
+        p.decode_mb = pl.mb;
+        if (p.splits > 1) {
+            const size_t need = packed_workspace_need(m, n, k, weight_bits, v);
+            if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
+            if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
+            if (need >= (1ull << 31)) return BFAINTB_ERR_BAD_VARIANT;
+            p.partials = static_cast<unsigned long long*>(workspace);
+            p.partial_bytes = (uint32_t)need;
+        }
+        return (int)bfaintb::launch_decode_family_packed(p, weight_bits, st);
+    }
     return (int)bfaintb::launch_decode_packed(p, weight_bits, st);
 }
 
 int bfaintb_gemm_prepacked(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m, uint32_t n,
-                           uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size, void* stream)
+                           uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
+                           size_t workspace_bytes, void* stream)
 {
-    return bfaintb_gemm_prepacked_ex(c, a, packed_b, scale, bias, m, n, k, lda, ldc, weight_bits, group_size, stream,
-                                     BFAINTB_VARIANT_AUTO);
+    return bfaintb_gemm_prepacked_ex(c, a, packed_b, scale, bias, m, n, k, lda, ldc, weight_bits, group_size, workspace,
+                                     workspace_bytes, stream, BFAINTB_VARIANT_AUTO);
 }
 
 int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,

@@ -22,6 +22,7 @@
 //   block meet in the workspace and the workgroup of the last split adds them in split order and
 //   writes bf16 C — the summation order is fixed, so results are reproducible run to run.  The narrower block (CPL = 8)
 //   needs half the splits for the same number of workgroups, i.e. half the partial-sum traffic.
+#include <type_traits>
 #include <utility>
 #include "bfaintb_device.hpp"
 
@@ -102,6 +103,70 @@ __device__ __forceinline__ void mac_step(const RawStep<BITS, CPL>& raw, const fl
 #pragma unroll
     for (int r = 0; r < 8; ++r) prepare_row<BITS, CPL>(rows[r], raw.d[r]);
     (mac_column<BITS, CPL, MB, Cs>(rows, cs, afrag, acc), ...);
+}
+
+// ---- the same step over weights in the packed order (bfaintb_packed.hip): the workgroup's CPL column blocks of 16 take
+//      the place of a lane's CPL consecutive columns.  For column block c the lane holds the 8 codes of column nl, rows
+//      8 kg .. 8 kg + 7 of the K-block: two dwords (rows 0-3, 4-7) for 8-bit codes, one dword of 8 nibbles for 4-bit.
+template <int BITS, int CPL>
+struct PackedStep {
+    static constexpr int kDwords = BITS == 8 ? 2 : 1;
+    uint32_t d[CPL][kDwords];
+};
+
+// lane_off: where this lane's codes of the K-block sit inside a column block's slab; slab[c]: the slab of column block c
+template <int BITS, int CPL>
+__device__ __forceinline__ void load_packed(PackedStep<BITS, CPL>& raw, const uint8_t* const (&slab)[CPL], size_t lane_off)
+{
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        if constexpr (BITS == 8) {
+            const uint2 v = *reinterpret_cast<const uint2*>(slab[c] + lane_off);
+            raw.d[c][0] = v.x; raw.d[c][1] = v.y;
+        } else {
+            raw.d[c][0] = *reinterpret_cast<const uint32_t*>(slab[c] + lane_off);
+        }
+    }
+}
+
+template <int BITS, int CPL, int MB>
+__device__ __forceinline__ void mac_step_packed(const PackedStep<BITS, CPL>& raw, const float (&cs)[CPL], const uint4 (&afrag)[MB],
+                                                f32x4_t (&acc)[MB][CPL])
+{
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const float s = cs[c];
+        uint4 w;
+        if constexpr (BITS == 8) {
+            const uint32_t lo = codes8_to_s8(raw.d[c][0]), hi = codes8_to_s8(raw.d[c][1]);
+            w.x = pack_bf16_rne(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
+            w.y = pack_bf16_rne(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
+            w.z = pack_bf16_rne(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
+            w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
+        } else {
+            const uint32_t ev = codes4_even_to_s8x16(raw.d[c][0]), od = codes4_odd_to_s8x16(raw.d[c][0]);
+            w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
+            w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
+            w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
+            w.w = pack_bf16_rne(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
+        }
+        const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, w);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            acc[mb][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, __builtin_bit_cast(bf16x8_t, afrag[mb]), acc[mb][c], 0, 0, 0);
+    }
+}
+
+// the lane's CPL scales in packed mode: column col[c] of a scale row, as raw bf16 pairs in the layout load_scales
+// produces (scale c in half c % 2 of dword c / 2)
+template <int CPL>
+__device__ __forceinline__ void load_scales_packed(uint4 (&sraw)[CPL / 8], const uint16_t* srow, const uint32_t (&col)[CPL])
+{
+    uint32_t d[CPL / 2];
+#pragma unroll
+    for (int i = 0; i < CPL / 2; ++i) d[i] = (uint32_t)srow[col[2 * i]] | ((uint32_t)srow[col[2 * i + 1]] << 16);
+#pragma unroll
+    for (int i = 0; i < CPL / 8; ++i) sraw[i] = make_uint4(d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3]);
 }
 
 template <int CPL>
@@ -238,7 +303,9 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
     }
 }
 
-template <int BITS, int CPL, int MB, bool GROUPED>
+// PACKED: p.b holds the weights in the packed order; the workgroup's kCols columns are CPL column blocks of 16, and
+// accumulator c of a lane belongs to column block c (local column 16 c + 4 kg + r instead of (4 kg + r) CPL + c).
+template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED>
 __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
 {
     constexpr int KB = decode_blocks_per_step(BITS, CPL);  // blocks of 32 rows per pipeline step
@@ -273,6 +340,25 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
 
     const uint8_t* bptr = p.b + (size_t)(kb + 8u * kg) * p.ldb_bytes + (size_t)n_ld * BITS / 8;
     const size_t bstep = (size_t)32 * p.ldb_bytes;
+    // packed: K-chunks of 64 (8-bit) or 128 (4-bit) rows, 1024 bytes each, hold 2 or 4 K-blocks of 32 rows; a lane's 16
+    // bytes of a chunk are its K-blocks in order
+    constexpr uint32_t kBlocksPerChunk = BITS == 8 ? 2u : 4u;
+    constexpr uint32_t kBlockBytes = 16u / kBlocksPerChunk;
+    // column block c of the workgroup (blocks past the last one re-read it; what they compute is never stored)
+    const uint8_t* slab[CPL];
+    uint32_t pk_col[CPL];
+    if constexpr (PACKED) {
+        const size_t slab_bytes = (size_t)p.k * 16u * BITS / 8u;
+        const uint32_t nblocks = p.n / 16u;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            uint32_t gb = cb * CPL + (uint32_t)c;
+            if (gb >= nblocks) gb = nblocks - 1u;
+            slab[c] = p.b + (size_t)gb * slab_bytes + (size_t)lane * 16u;
+            pk_col[c] = 16u * gb + (uint32_t)nl;
+        }
+    }
+    const uint32_t kblock0 = kb / 32u;  // first K-block of this wave
     static_assert(kLaneBytes == 16 || kLaneBytes == 8, "lane loads 16 or 8 bytes of a row");
 
     // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg.
@@ -300,33 +386,73 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
         // derives are exact; a load behind a branch, or a stage copied into another, makes it wait
         // for the prefetch as well.
         struct Stage {
-            RawStep<BITS, CPL> raw[KB];
+            std::conditional_t<PACKED, PackedStep<BITS, CPL>, RawStep<BITS, CPL>> raw[KB];
             uint4 af[KB][MB];
             uint4 sraw[KB][CPL / 8];
         };
         float cs[CPL];
-        const uint16_t* sptr = p.scale + n_ld;
+        const uint16_t* sptr = p.scale + (PACKED ? 0u : n_ld);
+        // packed weights with grouped scales: the wave's transposition table in LDS, behind the reduction area, and
+        // the columns whose scales this lane fetches (kept inside the scale row)
+        uint16_t* sc_table = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(red) + p.decode_scale_lds) + (uint32_t)wave * 16u * CPL;
+        uint32_t sc_col = cb * kCols + 4u * (uint32_t)lane;
+        if (sc_col + 4u > p.n) sc_col = p.n - 4u;
         auto load_stage = [&](Stage& st, int step) {
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
                 const size_t blk = (size_t)step * KB + q;
-                load_raw<BITS, CPL>(st.raw[q], bptr + blk * bstep, p.ldb_bytes);
+                if constexpr (PACKED) {
+                    const uint32_t kblock = kblock0 + (uint32_t)blk;
+                    load_packed<BITS, CPL>(st.raw[q], slab, (size_t)(kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
+                } else {
+                    load_raw<BITS, CPL>(st.raw[q], bptr + blk * bstep, p.ldb_bytes);
+                }
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) st.af[q][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + blk * 32);
-                if constexpr (GROUPED) load_scales<CPL>(st.sraw[q], sptr + (size_t)((kb + 32u * (uint32_t)blk) / p.group_size) * p.lds);
+                if constexpr (GROUPED) {
+                    const uint16_t* srow = sptr + (size_t)((kb + 32u * (uint32_t)blk) / p.group_size) * p.lds;
+                    if constexpr (PACKED) {
+                        // lane j fetches the scales of the workgroup's columns 4j .. 4j+3 (one 8-byte load instead of CPL
+                        // 2-byte gathers); compute_stage turns them, through LDS, into this lane's CPL scales
+                        const uint2 v = *reinterpret_cast<const uint2*>(srow + sc_col);
+                        st.sraw[q][0].x = v.x;
+                        st.sraw[q][0].y = v.y;
+                    } else {
+                        load_scales<CPL>(st.sraw[q], srow);
+                    }
+                }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic that follows
         };
         auto compute_stage = [&](Stage& st) {
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
-                if constexpr (GROUPED) apply_scales<BITS, CPL>(cs, st.sraw[q]);
-                mac_step<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
+                if constexpr (GROUPED && PACKED) {
+                    // scale of column 4j + e goes to T[(4j + e) % 16][(4j + e) / 16]; lane (nl, kg) then reads row nl: its CPL
+                    // scales, in column-block order.  The table is this wave's own; LDS serves a wave's requests in order.
+                    if ((uint32_t)lane < kCols / 4u) {
+                        const uint32_t d[2] = {st.sraw[q][0].x, st.sraw[q][0].y};
+#pragma unroll
+                        for (uint32_t e = 0; e < 4; ++e) {
+                            const uint32_t cix = 4u * (uint32_t)lane + e;
+                            sc_table[(cix & 15u) * CPL + (cix >> 4)] = (uint16_t)(e & 1u ? d[e >> 1] >> 16 : d[e >> 1] & 0xffffu);
+                        }
+                    }
+                    uint4 mine[CPL / 8];
+#pragma unroll
+                    for (int i = 0; i < CPL / 8; ++i) mine[i] = *reinterpret_cast<const uint4*>(sc_table + (uint32_t)nl * CPL + 8u * i);
+                    apply_scales<BITS, CPL>(cs, mine);
+                } else if constexpr (GROUPED) {
+                    apply_scales<BITS, CPL>(cs, st.sraw[q]);
+                }
+                if constexpr (PACKED) mac_step_packed<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc);
+                else mac_step<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
             }
         };
         Stage s0, s1;
         if constexpr (!GROUPED) {
-            load_scales<CPL>(s0.sraw[0], sptr);
+            if constexpr (PACKED) load_scales_packed<CPL>(s0.sraw[0], sptr, pk_col);
+            else load_scales<CPL>(s0.sraw[0], sptr);
         }
         load_stage(s0, 0);
         if constexpr (!GROUPED) apply_scales<BITS, CPL>(cs, s0.sraw[0]);
@@ -369,14 +495,20 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
             const int mb = mb0 + mbi;
             if (mb >= MB || !row_ok[mb]) continue;
             float* row = red + ((size_t)wave * rows_out + (mbi * 16 + nl)) * kRedStride;
+            if constexpr (PACKED) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+                for (int c = 0; c < CPL; ++c)  // column block c, columns 4 kg .. 4 kg + 3 of it
+                    *reinterpret_cast<float4*>(row + 16 * c + 4 * kg) = make_float4(acc[mb][c][0], acc[mb][c][1], acc[mb][c][2], acc[mb][c][3]);
+            } else {
 #pragma unroll
-                for (int c4 = 0; c4 < CPL / 4; ++c4) {
-                    float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
-                                           acc[mb][4 * c4 + 3][r]);
-                    *reinterpret_cast<float4*>(row + (4 * kg + r) * CPL + 4 * c4) = v;
-                }
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                        float4 v = make_float4(acc[mb][4 * c4 + 0][r], acc[mb][4 * c4 + 1][r], acc[mb][4 * c4 + 2][r],
+                                               acc[mb][4 * c4 + 3][r]);
+                        *reinterpret_cast<float4*>(row + (4 * kg + r) * CPL + 4 * c4) = v;
+                    }
+            }
         }
         __syncthreads();
         TRACE_MARK(3);
@@ -442,7 +574,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
     }
 }
 
-template <int BITS, int CPL, int MB, bool GROUPED>
+template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
     constexpr uint32_t kCols = 16u * CPL;
@@ -452,29 +584,35 @@ static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
     const dim3 grid((p.n + kCols - 1u) / kCols, p.splits, (p.m + kRows - 1u) / kRows);
     if (grid.z > 65535u) return hipErrorInvalidValue;
     const uint32_t pass_rows = 16u * (uint32_t)decode_rows16_per_pass(CPL, MB);
-    const size_t lds = (size_t)decode_red_floats(waves, p.m < pass_rows ? p.m : pass_rows, kCols) * sizeof(float);
+    size_t lds = (size_t)decode_red_floats(waves, p.m < pass_rows ? p.m : pass_rows, kCols) * sizeof(float);
+    GemmParams q = p;
+    if (PACKED && GROUPED) {
+        q.decode_scale_lds = (uint32_t)lds;     // each wave's 16 x CPL table of bf16 scales sits behind the reduction area
+        lds += (size_t)waves * 16u * CPL * 2u;
+    }
     if (lds > 160 * 1024 - 64) return hipErrorInvalidValue;
     if (lds > 64 * 1024) {
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, CPL, MB, GROUPED>),
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, CPL, MB, GROUPED, PACKED>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
             if (e != hipSuccess) return e;
             attr_set = true;
         }
     }
-    return launch_kernel(bfaintb_decode_kernel<BITS, CPL, MB, GROUPED>, grid, dim3(64 * waves, 1, 1), lds, stream, p);
+    void (*kernel)(const GemmParams) = bfaintb_decode_kernel<BITS, CPL, MB, GROUPED, PACKED>;
+    return launch_kernel(kernel, grid, dim3(64 * waves, 1, 1), lds, stream, q);
 }
 
-template <int BITS, int CPL>
+template <int BITS, int CPL, bool PACKED>
 static hipError_t launch_decode_b(const GemmParams& p, hipStream_t stream)
 {
     const bool grouped = p.group_size != 0;
     switch (p.decode_mb) {
-        case 1: return grouped ? launch_decode_t<BITS, CPL, 1, true>(p, stream) : launch_decode_t<BITS, CPL, 1, false>(p, stream);
-        case 2: return grouped ? launch_decode_t<BITS, CPL, 2, true>(p, stream) : launch_decode_t<BITS, CPL, 2, false>(p, stream);
+        case 1: return grouped ? launch_decode_t<BITS, CPL, 1, true, PACKED>(p, stream) : launch_decode_t<BITS, CPL, 1, false, PACKED>(p, stream);
+        case 2: return grouped ? launch_decode_t<BITS, CPL, 2, true, PACKED>(p, stream) : launch_decode_t<BITS, CPL, 2, false, PACKED>(p, stream);
         case 4:  // 16 accumulators x 4 blocks x 8 columns = 128 registers: only the 128-column shape has room
-            if constexpr (CPL == 8) return grouped ? launch_decode_t<BITS, CPL, 4, true>(p, stream) : launch_decode_t<BITS, CPL, 4, false>(p, stream);
+            if constexpr (CPL == 8) return grouped ? launch_decode_t<BITS, CPL, 4, true, PACKED>(p, stream) : launch_decode_t<BITS, CPL, 4, false, PACKED>(p, stream);
             break;
         default: break;
     }
@@ -483,8 +621,16 @@ static hipError_t launch_decode_b(const GemmParams& p, hipStream_t stream)
 
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)
 {
-    if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8>(p, stream) : launch_decode_b<8, 16>(p, stream);
-    return launch_decode_b<4, 16>(p, stream);
+    if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8, false>(p, stream) : launch_decode_b<8, 16, false>(p, stream);
+    return launch_decode_b<4, 16, false>(p, stream);
+}
+
+// The same family over weights in the packed order (p.b = the packed buffer): the shapes the plan uses beyond 32 rows of A,
+// 128 columns for 8-bit and 256 for 4-bit codes.  n must hold at least one such group of column blocks.
+hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream)
+{
+    if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8, true>(p, stream) : hipErrorInvalidValue;
+    return launch_decode_b<4, 16, true>(p, stream);
 }
 
 }  // namespace bfaintb

@@ -60,6 +60,7 @@ struct GemmParams {
     uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)
     uint32_t decode_cols;  // columns per workgroup of the decode variant (256, or 128 for 8-bit codes)
     uint32_t decode_mb;    // blocks of 16 rows of A per workgroup of the decode variant (1, 2 or 4)
+    uint32_t decode_scale_lds;  // byte offset, in dynamic LDS, of the waves' scale tables (packed weights, grouped scales)
     uint32_t splits;     // workgroups along k
     unsigned long long* partials;  // [splits - 1][m][n] fp32 partial sums; kEmptyWord wherever none is waiting
     uint32_t partial_bytes;        // size of that area (below 2^31)

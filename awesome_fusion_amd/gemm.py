@@ -82,7 +82,9 @@ def lib():
         L.bfaintb_unpack.restype = C.c_int
         L.bfaintb_unpack.argtypes = [_vp, _vp, _u32, _u32, _u32, C.c_int, _vp]
         L.bfaintb_gemm_prepacked.restype = C.c_int
-        L.bfaintb_gemm_prepacked.argtypes = [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
+        L.bfaintb_gemm_prepacked.argtypes = [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp, C.c_size_t, _vp]
+        L.bfaintb_gemm_prepacked_workspace_bytes_ex.restype = C.c_size_t
+        L.bfaintb_gemm_prepacked_workspace_bytes_ex.argtypes = [_u32, _u32, _u32, C.c_int, _u32, C.c_int]
         L.bfaintb_gemm_prepacked_ex.restype = C.c_int
         L.bfaintb_gemm_prepacked_ex.argtypes = L.bfaintb_gemm_prepacked.argtypes + [C.c_int]
         L.bfaintb_gemm_prepacked_variant.restype = C.c_int
@@ -194,12 +196,18 @@ def prepacked_variant(m, n, k, weight_bits=8, group_size=0):
     return lib().bfaintb_gemm_prepacked_variant(m, n, k, weight_bits, group_size)
 
 
-def gemm_prepacked(c, a, packed_b, scale, m, n, k, lda=None, ldc=None, weight_bits=8, group_size=0, bias=None, stream=None,
-                   which=AUTO, check=True):
+def prepacked_workspace_bytes(m, n, k, weight_bits=8, group_size=0, which=AUTO):
+    return lib().bfaintb_gemm_prepacked_workspace_bytes_ex(m, n, k, weight_bits, group_size, which)
+
+
+def gemm_prepacked(c, a, packed_b, scale, m, n, k, lda=None, ldc=None, weight_bits=8, group_size=0, bias=None, workspace=None,
+                   workspace_nbytes=None, stream=None, which=AUTO, check=True):
     """C = A x dequant(B, scale) (+ bias) with B in the packed order, through bfaintb_gemm_prepacked_ex."""
+    if workspace_nbytes is None:
+        workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
     rc = lib().bfaintb_gemm_prepacked_ex(_ptr(c), _ptr(a), _ptr(packed_b), _ptr(scale), _ptr(bias), m, n, k,
                                          k if lda is None else lda, n if ldc is None else ldc, weight_bits, group_size,
-                                         _stream_handle(stream), which)
+                                         _ptr(workspace), workspace_nbytes, _stream_handle(stream), which)
     if rc and check:
         raise BfaintbError(rc, "bfaintb_gemm_prepacked")
     return rc

@@ -23,6 +23,7 @@ from typing import Optional
 import torch
 
 from .gemm import (gemm as _gemm, gemm_prepacked as _gemm_prepacked, prepack as _prepack, prepack_bytes as _prepack_bytes,
+                   prepacked_workspace_bytes as _prepacked_workspace_bytes,
                    workspace_bytes as _workspace_bytes, workspace_init as _workspace_init)
 
 _LIB_NAME = "awesome_fusion"
@@ -93,7 +94,7 @@ def _(a, b, scale, weight_bits, group_size, bias=None):
 def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
                            bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same product with the weights in the library's pre-packed order (``prepack_weight``): ``packed`` is a flat
-    uint8 tensor of k * n * weight_bits / 8 bytes, n is taken from ``scale``.  Needs no workspace."""
+    uint8 tensor of k * n * weight_bits / 8 bytes, n is taken from ``scale``."""
     m, n, k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
     if not a.is_cuda:
         raise RuntimeError("bfaintb_gemm_prepacked runs on the GPU only (no CPU implementation)")
@@ -107,7 +108,9 @@ def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.T
     if m == 0 or n == 0:
         return c
     with torch.cuda.device(a.device):
-        _gemm_prepacked(c, a, packed, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, bias=bias)
+        ws = _workspace(a.device, _prepacked_workspace_bytes(m, n, k, weight_bits, group_size))
+        _gemm_prepacked(c, a, packed, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, bias=bias,
+                        workspace=ws)
     return c
 
 

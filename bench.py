@@ -94,6 +94,11 @@ def time_graph(af, w, steps, warmup, rotate, packed=False):
     ws = w.workspace(af)
     nb = len(w.b) if rotate else 1
     if packed:
+        need = af.prepacked_workspace_bytes(w.m, w.n, w.k, w.bits, w.group)
+        pws = None
+        if need:
+            pws = torch.empty(need, dtype=torch.uint8, device="cuda")
+            af.workspace_init(pws)
         pks = []
         for i in range(nb):
             pk = torch.empty(af.prepack_bytes(w.n, w.k, w.bits), dtype=torch.uint8, device="cuda")
@@ -102,7 +107,7 @@ def time_graph(af, w, steps, warmup, rotate, packed=False):
 
     def launch(i):
         if packed:
-            af.gemm_prepacked(w.c, w.a, pks[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group)
+            af.gemm_prepacked(w.c, w.a, pks[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=pws)
         else:
             af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
 

@@ -5,7 +5,9 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Problem, assert_close_ulp, from_dev_u16, to_dev
+from helpers import Problem, Workspace, assert_close_ulp, from_dev_u16, to_dev
+
+_ws = Workspace()
 
 pytestmark = pytest.mark.gpu
 
@@ -32,8 +34,9 @@ def run_prepacked(af, p, which=0, pk=None, ldc=None):
     ldc_ = p.n if ldc is None else ldc
     c = torch.full((p.m, ldc_), 0x7FC0, dtype=torch.int16, device="cuda")
     bias = None if p.bias_bf is None else to_dev(p.bias_bf)
+    ws = _ws.get(af.prepacked_workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size, which))
     af.gemm_prepacked(c, to_dev(p.a_bf), pk, to_dev(p.s_bf), p.m, p.n, p.k, ldc=ldc, weight_bits=p.bits, group_size=p.group_size,
-                      bias=bias, which=which)
+                      bias=bias, workspace=ws, which=which)
     torch.cuda.synchronize()
     return from_dev_u16(c)
 
@@ -81,6 +84,20 @@ def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
 
 
 @pytest.mark.parametrize("m,n,k,bits,group", [
+    (49, 128, 512, 8, 0), (64, 4096, 1024, 8, 0), (100, 272, 448, 8, 64), (130, 48, 1024, 8, 32), (200, 1040, 256, 8, 0), (300, 144, 2048, 8, 128),
+    (64, 256, 512, 4, 0), (97, 528, 1024, 4, 128), (150, 80, 640, 4, 32), (260, 1296, 384, 4, 128),
+    # shapes whose plan splits along k (few column groups, long k): partial sums meet in the workspace
+    (64, 256, 4096, 4, 128), (80, 128, 8192, 8, 0), (100, 512, 4096, 4, 0)])
+def test_row_blocked_family_over_packed_weights(af, m, n, k, bits, group):
+    """Beyond 48 rows of A the forced DECODE variant is the row-blocked decode family reading packed slabs (8 column
+    blocks per workgroup for 8-bit codes, 16 for 4-bit; partial last groups re-read the last block)."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    assert_close_ulp(p, run_prepacked(af, p, af.DECODE), f"packed family {m}x{n}x{k} b{bits} g{group}")
+    p.with_bias()
+    assert_close_ulp(p, run_prepacked(af, p, af.DECODE), f"packed family + bias {m}x{n}x{k} b{bits} g{group}")
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [
     (256, 256, 64, 8, 0), (300, 272, 192, 8, 0), (64, 128, 256, 8, 0), (512, 512, 256, 4, 128), (1000, 1008, 384, 4, 0),
     (513, 784, 448, 8, 64), (130, 528, 512, 8, 32), (260, 304, 512, 4, 32), (4160, 256, 256, 8, 0), (2304, 512, 512, 4, 128)])
 def test_tiled_kernel_matches_oracle(af, m, n, k, bits, group):
@@ -91,7 +108,7 @@ def test_tiled_kernel_matches_oracle(af, m, n, k, bits, group):
 
 
 @pytest.mark.parametrize("bits,group", [(8, 0), (4, 128)])
-@pytest.mark.parametrize("which,m", [(1, 16), (1, 32), (2, 64)])
+@pytest.mark.parametrize("which,m", [(1, 16), (1, 32), (1, 64), (2, 64)])
 def test_kernels_dequantise_bit_exact(af, bits, group, which, m):
     """One-hot activations make C[i, :] = W[k_i, :] with nothing to round: the in-register conversion of both
     kernels is observed exactly, against the oracle's dequantised weights."""
@@ -129,6 +146,25 @@ def test_matches_the_row_major_path_in_the_exact_regime(af):
         assert np.array_equal(run_prepacked(af, p), run_gemm(p))
 
 
+def test_workspace_is_required_where_the_plan_splits_and_left_ready(af):
+    import torch
+    m, n, k, bits, g = 64, 256, 4096, 4, 128
+    need = af.prepacked_workspace_bytes(m, n, k, bits, g)
+    assert need > 0 and af.prepacked_workspace_bytes(1, n, k, bits, g) == 0 and af.prepacked_workspace_bytes(4096, 4096, 4096) == 0
+    p = Problem(m, n, k, bits, g, seed=11)
+    pk = packed_on_device(af, p)
+    c = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+    args = (c, to_dev(p.a_bf), pk, to_dev(p.s_bf), m, n, k)
+    assert af.gemm_prepacked(*args, weight_bits=bits, group_size=g, check=False) == -6
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    af.workspace_init(ws)
+    for _ in range(2):  # the second call finds the workspace as the first left it
+        af.gemm_prepacked(*args, weight_bits=bits, group_size=g, workspace=ws)
+        torch.cuda.synchronize()
+        assert_close_ulp(p, from_dev_u16(c), "packed split-K")
+    assert bool((ws == 0xFF).all())
+
+
 def test_output_stride_and_padding(af):
     p = Problem(5, 48, 128, 8, 0, seed=9)
     c = run_prepacked(af, p, ldc=64)
@@ -140,16 +176,21 @@ def test_hip_graph_replays_match_eager(af):
     """Packing and the packed GEMMs hold no memset and no scratch state: captured once, every replay reproduces the
     eager bits, with other work and synchronisations in between."""
     import torch
-    shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (40, 64, 8256, 8, 0), (600, 512, 512, 8, 0)]
+    shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (40, 64, 8256, 8, 0), (64, 256, 4096, 4, 128), (600, 512, 512, 8, 0)]
     probs = [Problem(m, n, k, bits, g, seed=190 + i) for i, (m, n, k, bits, g) in enumerate(shapes)]
     eager = [run_prepacked(af, p) for p in probs]
     bufs = [dict(a=to_dev(p.a_bf), b=to_dev(p.b_bytes), s=to_dev(p.s_bf), pk=torch.zeros(af.prepack_bytes(p.n, p.k, p.bits), dtype=torch.uint8, device="cuda"),
-                 c=torch.zeros((p.m, p.n), dtype=torch.int16, device="cuda")) for p in probs]
+                 c=torch.zeros((p.m, p.n), dtype=torch.int16, device="cuda"), w=None) for p in probs]
+    for p, d in zip(probs, bufs):
+        need = af.prepacked_workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size)
+        if need:
+            d["w"] = torch.empty(need, dtype=torch.uint8, device="cuda")
+            af.workspace_init(d["w"])
 
     def run_all():
         for p, d in zip(probs, bufs):
             af.prepack(d["pk"], d["b"], p.n, p.k, weight_bits=p.bits)
-            af.gemm_prepacked(d["c"], d["a"], d["pk"], d["s"], p.m, p.n, p.k, weight_bits=p.bits, group_size=p.group_size)
+            af.gemm_prepacked(d["c"], d["a"], d["pk"], d["s"], p.m, p.n, p.k, weight_bits=p.bits, group_size=p.group_size, workspace=d["w"])
 
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
