@@ -20,18 +20,21 @@
 // The buffers' extents end with the tile's last valid row of A and the last row of B (gfx9-family
 // range checks add the SGPR offset to the lane offset): rows of A past m read as zero; columns of B
 // past n read whatever lies there, or zero past the end of B, and feed only columns that are never stored.
-// A path: 16-byte loads (8 lanes per row) -> registers -> ds_write_b128.
-// W path: wave w loads rows 8w..8w+7 of the step, one dword (4 codes) per lane per row, so a lane
+// A path: global -> LDS directly (buffer_load ... lds, 16 bytes per lane, 8 lanes per row), each lane fetching the chunk
+//   that the swizzle places at its LDS position.
+// W path (row-major B; the PACKED instantiation reads the packed order instead, see the kernel): wave w loads rows 8w..8w+7 of the step, one dword (4 codes) per lane per row, so a lane
 //   ends up with 8 consecutive k of 4 columns; it dequantises them (xor, cvt with sign-extending
 //   byte select, multiply, cvt_pk) and writes one 16-byte chunk per column.  Column (4*lane + j)
 //   goes to LDS row rho = (j>>1)*128 + (j&1)*32 + (lane&31) + (lane>>5)*64, so consecutive lanes
 //   write consecutive rows.  The MFMA "column" index is the LDS row: wave wn, accumulator t, lane
 //   column jl hold tile column 4*(32*(wn&1) + jl) + 2*(wn>>1) + t.
-// Pipeline per step (registers hold the raw tile of step+1, loaded one step earlier): the 32 MFMAs
+// Pipeline per step (registers hold the raw W tile of step+1, loaded one step earlier): the 32 MFMAs
 //   of the current stage run in four quarters; the raw tile is converted and written to the other
 //   stage between the MFMAs of the second and third quarter, the registers it frees are refilled
 //   with step+2 at once, and the barrier sits before the last quarter so that the first fragments
 //   of the next stage are fetched behind those MFMAs.
+// Launches: whole 256-row tiles, then (a last round of 256 workgroups that would be less than half full, or fewer
+//   than 128 tiles in all) 128-row half tiles, MT = 2.
 // Epilogue: accumulators are rounded to bf16 (v_cvt_pk_bf16_f32; t = 0,1 are neighbouring columns
 //   and share a dword), staged in LDS in true [m][n] order and stored with 16-byte row-contiguous writes.
 #include <utility>
