@@ -7,6 +7,7 @@ has no CPU fallback: without the built library every call raises.
 """
 from .gemm import (  # noqa: F401
     BfaintbError,
+    Epilogue,
     PackedHeader,
     load_packed,
     save_packed,

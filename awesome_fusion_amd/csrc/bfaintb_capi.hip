@@ -255,10 +255,29 @@ int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream
                                          static_cast<hipStream_t>(stream));
 }
 
-static int gemm_impl(void* c, const void* a, const void* b, const void* scale, const void* bias, uint32_t m, uint32_t n, uint32_t k,
+// what the epilogue descriptor asks for, checked: bias and residual pointers (either may be null) and the residual's row stride
+struct Epilogue {
+    const void* bias = nullptr;
+    const void* residual = nullptr;
+    uint32_t ldr = 0;
+};
+
+static int read_epilogue(Epilogue& out, const bfaintb_epilogue* ep, uint32_t n)
+{
+    if (ep == nullptr) return BFAINTB_OK;
+    if (ep->reserved != 0) return BFAINTB_ERR_UNSUPPORTED;
+    out.bias = ep->bias;
+    out.residual = ep->residual;
+    out.ldr = ep->ldr;
+    if (ep->residual != nullptr && (ep->ldr < n || ep->ldr % 8u != 0)) return BFAINTB_ERR_BAD_LD;
+    return BFAINTB_OK;
+}
+
+static int gemm_impl(void* c, const void* a, const void* b, const void* scale, const Epilogue& ep, uint32_t m, uint32_t n, uint32_t k,
                      uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                      size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
 {
+    const void* bias = ep.bias;
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
     e = check_shape(m, n, k);
@@ -268,10 +287,13 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
     if (c == nullptr || a == nullptr || b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
-    if (misaligned16(c) || misaligned16(a) || misaligned16(b) || misaligned16(scale) || misaligned16(bias)) return BFAINTB_ERR_ALIGNMENT;
+    if (misaligned16(c) || misaligned16(a) || misaligned16(b) || misaligned16(scale) || misaligned16(bias) || misaligned16(ep.residual))
+        return BFAINTB_ERR_ALIGNMENT;
 
     GemmParams p{};
     p.bias = static_cast<const uint16_t*>(bias);
+    p.residual = static_cast<const uint16_t*>(ep.residual);
+    p.ldr = ep.ldr;
     p.c = static_cast<uint16_t*>(c);
     p.a = static_cast<const uint16_t*>(a);
     p.b = static_cast<const uint8_t*>(b);
@@ -433,10 +455,11 @@ size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n, uint32_t k
     return bfaintb_gemm_prepacked_workspace_bytes_ex(m, n, k, weight_bits, group_size, BFAINTB_VARIANT_AUTO);
 }
 
-int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
-                              uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
-                              void* workspace, size_t workspace_bytes, void* stream, int variant)
+static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, const void* scale, const Epilogue& ep, uint32_t m,
+                               uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
+                               void* workspace, size_t workspace_bytes, void* stream, int variant)
 {
+    const void* bias = ep.bias;
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
     e = check_shape(m, n, k);
@@ -448,9 +471,12 @@ int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, cons
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
     if (c == nullptr || a == nullptr || packed_b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;
-    if (misaligned16(c) || misaligned16(a) || misaligned16(packed_b) || misaligned16(scale) || misaligned16(bias))
+    if (misaligned16(c) || misaligned16(a) || misaligned16(packed_b) || misaligned16(scale) || misaligned16(bias) ||
+        misaligned16(ep.residual))
         return BFAINTB_ERR_ALIGNMENT;
     GemmParams p{};
+    p.residual = static_cast<const uint16_t*>(ep.residual);
+    p.ldr = ep.ldr;
     p.c = static_cast<uint16_t*>(c);
     p.a = static_cast<const uint16_t*>(a);
     p.b = static_cast<const uint8_t*>(packed_b);
@@ -492,6 +518,27 @@ int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, cons
     return (int)bfaintb::launch_decode_packed(p, weight_bits, st);
 }
 
+int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
+                              uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
+                              void* workspace, size_t workspace_bytes, void* stream, int variant)
+{
+    Epilogue ep;
+    ep.bias = bias;
+    return gemm_prepacked_impl(c, a, packed_b, scale, ep, m, n, k, lda, ldc, weight_bits, group_size, workspace, workspace_bytes,
+                               stream, variant);
+}
+
+int bfaintb_gemm_prepacked_fused(void* c, const void* a, const void* packed_b, const void* scale, const bfaintb_epilogue* epilogue,
+                                 uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
+                                 void* workspace, size_t workspace_bytes, void* stream)
+{
+    Epilogue ep;
+    const int e = read_epilogue(ep, epilogue, n);
+    if (e) return e;
+    return gemm_prepacked_impl(c, a, packed_b, scale, ep, m, n, k, lda, ldc, weight_bits, group_size, workspace, workspace_bytes,
+                               stream, BFAINTB_VARIANT_AUTO);
+}
+
 int bfaintb_gemm_prepacked(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m, uint32_t n,
                            uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                            size_t workspace_bytes, void* stream)
@@ -504,7 +551,7 @@ int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, ui
                     uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
 {
-    return gemm_impl(c, a, b, scale, nullptr, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
+    return gemm_impl(c, a, b, scale, Epilogue{}, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
                      variant, split_k);
 }
 
@@ -512,7 +559,20 @@ int bfaintb_gemm_bias(void* c, const void* a, const void* b, const void* scale, 
                       uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                       size_t workspace_bytes, void* stream)
 {
-    return gemm_impl(c, a, b, scale, bias, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
+    Epilogue ep;
+    ep.bias = bias;
+    return gemm_impl(c, a, b, scale, ep, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
+                     BFAINTB_VARIANT_AUTO, 0);
+}
+
+int bfaintb_gemm_fused(void* c, const void* a, const void* b, const void* scale, const bfaintb_epilogue* epilogue, uint32_t m,
+                       uint32_t n, uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size,
+                       void* workspace, size_t workspace_bytes, void* stream)
+{
+    Epilogue ep;
+    const int e = read_epilogue(ep, epilogue, n);
+    if (e) return e;
+    return gemm_impl(c, a, b, scale, ep, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
                      BFAINTB_VARIANT_AUTO, 0);
 }
 

@@ -212,11 +212,18 @@ __host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t r
     return waves * rows * (cols + 4u);
 }
 
-// t += bias[col .. col+3] (fp32), if the launch has a bias.
-__device__ __forceinline__ void add_bias4(const GemmParams& p, float4& t, uint32_t col)
+// t += bias[col .. col+3], then += residual[row][col .. col+3] (fp32 additions), for what the launch has of them.
+__device__ __forceinline__ void add_epilogue4(const GemmParams& p, float4& t, uint32_t row, uint32_t col)
 {
     if (p.bias != nullptr) {
         const uint2 raw = *reinterpret_cast<const uint2*>(p.bias + col);
+        t.x += bf16_bits_to_f32(raw.x & 0xffffu);
+        t.y += bf16_bits_to_f32(raw.x >> 16);
+        t.z += bf16_bits_to_f32(raw.y & 0xffffu);
+        t.w += bf16_bits_to_f32(raw.y >> 16);
+    }
+    if (p.residual != nullptr) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(p.residual + (size_t)row * p.ldr + col);
         t.x += bf16_bits_to_f32(raw.x & 0xffffu);
         t.y += bf16_bits_to_f32(raw.x >> 16);
         t.z += bf16_bits_to_f32(raw.y & 0xffffu);
@@ -294,7 +301,7 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
         const uint32_t row = rs + i * nrs;
         if (row < rows && col_ok) {
             float4 t = make_float4(total[i].x + sum[i].x, total[i].y + sum[i].y, total[i].z + sum[i].z, total[i].w + sum[i].w);
-            add_bias4(p, t, col);
+            add_epilogue4(p, t, first_row + row, col);
             uint2 o;
             o.x = pack_bf16_rne(t.x, t.y);
             o.y = pack_bf16_rne(t.z, t.w);
@@ -534,7 +541,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
                 const uint32_t row = rs + i * nrs;
                 if (row < rows_out && col_ok) {
                     float4 t = sum[i];
-                    add_bias4(p, t, col);
+                    add_epilogue4(p, t, first_row + row, col);
                     uint2 o;
                     o.x = pack_bf16_rne(t.x, t.y);
                     o.y = pack_bf16_rne(t.z, t.w);

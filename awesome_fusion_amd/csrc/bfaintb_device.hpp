@@ -47,6 +47,8 @@ struct GemmParams {
     const uint8_t* b;
     const uint16_t* scale;
     const uint16_t* bias;  // bf16 [n] added to the fp32 sums before the one rounding to bf16, or null
+    const uint16_t* residual;  // bf16 [m, ldr] added after the bias, before the rounding, or null
+    uint32_t ldr;              // elements per row of residual
     uint32_t m, n, k;
     uint32_t lda;        // elements
     uint32_t ldb_bytes;  // bytes per row of packed weights

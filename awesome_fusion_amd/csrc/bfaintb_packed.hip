@@ -285,6 +285,7 @@ __device__ __forceinline__ void decode_packed_body(const GemmParams& p)
             for (int w = 1; w < kPackedWaves; ++w) sum += red[w][mb][j][i];
             const uint32_t c = 16u * nb + i;
             if (p.bias != nullptr) sum += bf16_bits_to_f32(p.bias[c]);
+            if (p.residual != nullptr) sum += bf16_bits_to_f32(p.residual[(size_t)row * p.ldr + c]);
             p.c[(size_t)row * p.ldc + c] = (uint16_t)(pack_bf16_rne(sum, 0.f) & 0xffffu);
         }
     }

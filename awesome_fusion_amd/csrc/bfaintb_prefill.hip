@@ -426,7 +426,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         const uint32_t jl = lane & 31u, half = lane >> 5;
         const uint32_t col0 = 16u * (4u * wn + 2u * (jl >> 4)) + (jl & 15u);
         float bias0 = 0.f, bias1 = 0.f;
-        const bool has_bias = p.bias != nullptr;
+        const bool has_bias = p.bias != nullptr, has_res = p.residual != nullptr;
         if (has_bias) {
             if (n0 + col0 < p.n) bias0 = bf16_bits_to_f32(p.bias[n0 + col0]);
             if (n0 + col0 + 16u < p.n) bias1 = bf16_bits_to_f32(p.bias[n0 + col0 + 16u]);
@@ -438,8 +438,18 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 #pragma unroll
             for (uint32_t i = 0; i < 16; ++i) {
                 const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
-                const uint32_t both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1)
-                                               : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                uint32_t both;
+                if (has_res) {
+                    const uint32_t gm = m0 + 64u * (block32 >> 1) + row;
+                    float v0 = acc[mt][0][i] + bias0, v1 = acc[mt][1][i] + bias1;  // bias0/1 are +0 without a bias: a sum that
+                    if (gm < p.m) {                                                 // gets a residual added need not keep -0
+                        if (n0 + col0 < p.n) v0 += bf16_bits_to_f32(p.residual[(size_t)gm * p.ldr + n0 + col0]);
+                        if (n0 + col0 + 16u < p.n) v1 += bf16_bits_to_f32(p.residual[(size_t)gm * p.ldr + n0 + col0 + 16u]);
+                    }
+                    both = pack_bf16_rne(v0, v1);
+                } else {
+                    both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                }
                 *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0) = (uint16_t)(both & 0xffffu);
                 *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0 + 32u) = (uint16_t)(both >> 16);
             }
@@ -450,7 +460,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         const uint32_t colbyte = 8u * (32u * (wn & 1u) + jl) + 4u * (wn >> 1);
         // this lane's two columns of the tile are colbyte/2 and the next: their bias, if the launch has one
         float bias0 = 0.f, bias1 = 0.f;
-        const bool has_bias = p.bias != nullptr;
+        const bool has_bias = p.bias != nullptr, has_res = p.residual != nullptr;
         if (has_bias && n0 + colbyte / 2u < p.n) {
             const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.bias + n0 + colbyte / 2u);
             bias0 = bf16_bits_to_f32(raw & 0xffffu);
@@ -464,8 +474,20 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             for (uint32_t i = 0; i < 16; ++i) {
                 const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
                 // without a bias the sums are stored as they are (adding +0 would turn a -0 sum into +0)
-                *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) =
-                    has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                uint32_t both;
+                if (has_res) {
+                    const uint32_t gm = m0 + 64u * (block32 >> 1) + row;
+                    float v0 = acc[mt][0][i] + bias0, v1 = acc[mt][1][i] + bias1;
+                    if (gm < p.m && n0 + colbyte / 2u < p.n) {
+                        const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.residual + (size_t)gm * p.ldr + n0 + colbyte / 2u);
+                        v0 += bf16_bits_to_f32(raw & 0xffffu);
+                        v1 += bf16_bits_to_f32(raw >> 16);
+                    }
+                    both = pack_bf16_rne(v0, v1);
+                } else {
+                    both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                }
+                *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) = both;
             }
         }
     }

@@ -41,6 +41,11 @@ _u32 = C.c_uint32
 _vp = C.c_void_p
 
 
+class Epilogue(C.Structure):
+    """bfaintb_epilogue of include/bfaintb_gemm.h."""
+    _fields_ = [("bias", C.c_void_p), ("residual", C.c_void_p), ("ldr", C.c_uint32), ("reserved", C.c_uint32)]
+
+
 class PackedHeader(C.Structure):
     """bfaintb_packed_header of include/bfaintb_gemm.h: the 64-byte header of a pre-packed weight file."""
     _fields_ = [("magic", C.c_char * 8), ("header_bytes", _u32), ("layout", _u32), ("weight_bits", _u32), ("group_size", _u32),
@@ -65,6 +70,12 @@ def lib():
         L.bfaintb_gemm_bias.restype = C.c_int
         L.bfaintb_gemm_bias.argtypes = [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
                                         C.c_size_t, _vp]
+        L.bfaintb_gemm_fused.restype = C.c_int
+        L.bfaintb_gemm_fused.argtypes = [_vp, _vp, _vp, _vp, C.POINTER(Epilogue), _u32, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
+                                         C.c_size_t, _vp]
+        L.bfaintb_gemm_prepacked_fused.restype = C.c_int
+        L.bfaintb_gemm_prepacked_fused.argtypes = [_vp, _vp, _vp, _vp, C.POINTER(Epilogue), _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
+                                                   C.c_size_t, _vp]
         L.bfaintb_gemm_workspace_bytes.restype = C.c_size_t
         L.bfaintb_gemm_workspace_bytes.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
         L.bfaintb_gemm_workspace_bytes_ex.restype = C.c_size_t
@@ -151,16 +162,30 @@ def workspace_init(workspace, nbytes=None, stream=None):
         raise BfaintbError(rc, "bfaintb_workspace_init")
 
 
+def _epilogue(bias, residual, ldr, n):
+    ep = Epilogue()
+    ep.bias = _ptr(bias)
+    ep.residual = _ptr(residual)
+    ep.ldr = n if ldr is None else ldr
+    return ep
+
+
 def gemm(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, group_size=0, workspace=None,
-         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True, bias=None):
-    """C = A x dequant(B, scale) through bfaintb_gemm_ex, or (+ bias, AUTO variant only) through
-    bfaintb_gemm_bias.  Returns the library's return code (raises on non-zero when ``check``)."""
+         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True, bias=None, residual=None, ldr=None):
+    """C = A x dequant(B, scale) through bfaintb_gemm_ex, or (AUTO variant only) + bias through bfaintb_gemm_bias,
+    + bias + residual through bfaintb_gemm_fused.  Returns the library's return code (raises on non-zero when ``check``)."""
     lda = k if lda is None else lda
     ldb = n if ldb is None else ldb
     ldc = n if ldc is None else ldc
     if workspace_nbytes is None:
         workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
-    if bias is not None:
+    if residual is not None:
+        if which != AUTO or force_split_k:
+            raise ValueError("bfaintb_gemm_fused takes no forced variant or split factor")
+        ep = _epilogue(bias, residual, ldr, n)
+        rc = lib().bfaintb_gemm_fused(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), C.byref(ep), m, n, k, lda, ldb, ldc, weight_bits, group_size,
+                                      _ptr(workspace), workspace_nbytes, _stream_handle(stream))
+    elif bias is not None:
         if which != AUTO or force_split_k:
             raise ValueError("bfaintb_gemm_bias takes no forced variant or split factor")
         rc = lib().bfaintb_gemm_bias(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), _ptr(bias), m, n, k, lda, ldb, ldc, weight_bits,
@@ -201,10 +226,21 @@ def prepacked_workspace_bytes(m, n, k, weight_bits=8, group_size=0, which=AUTO):
 
 
 def gemm_prepacked(c, a, packed_b, scale, m, n, k, lda=None, ldc=None, weight_bits=8, group_size=0, bias=None, workspace=None,
-                   workspace_nbytes=None, stream=None, which=AUTO, check=True):
-    """C = A x dequant(B, scale) (+ bias) with B in the packed order, through bfaintb_gemm_prepacked_ex."""
+                   workspace_nbytes=None, stream=None, which=AUTO, check=True, residual=None, ldr=None):
+    """C = A x dequant(B, scale) (+ bias) with B in the packed order, through bfaintb_gemm_prepacked_ex; with a residual
+    (AUTO variant only) through bfaintb_gemm_prepacked_fused."""
     if workspace_nbytes is None:
         workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
+    if residual is not None:
+        if which != AUTO:
+            raise ValueError("bfaintb_gemm_prepacked_fused takes no forced variant")
+        ep = _epilogue(bias, residual, ldr, n)
+        rc = lib().bfaintb_gemm_prepacked_fused(_ptr(c), _ptr(a), _ptr(packed_b), _ptr(scale), C.byref(ep), m, n, k,
+                                                k if lda is None else lda, n if ldc is None else ldc, weight_bits, group_size,
+                                                _ptr(workspace), workspace_nbytes, _stream_handle(stream))
+        if rc and check:
+            raise BfaintbError(rc, "bfaintb_gemm_prepacked_fused")
+        return rc
     rc = lib().bfaintb_gemm_prepacked_ex(_ptr(c), _ptr(a), _ptr(packed_b), _ptr(scale), _ptr(bias), m, n, k,
                                          k if lda is None else lda, n if ldc is None else ldc, weight_bits, group_size,
                                          _ptr(workspace), workspace_nbytes, _stream_handle(stream), which)

@@ -6,12 +6,12 @@ forward pass: activations A [m, k], weights B [k, n], per-output-channel scale, 
 (/root/reference/bfAintBGemm/bfAintBGemm.cc:17-28,119-133).  This module lets such a layer call the
 library:
 
-    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size, bias=None) -> c
-    torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, scale, weight_bits, group_size, bias=None) -> c
+    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size, bias=None, residual=None) -> c
+    torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, scale, weight_bits, group_size, bias=None, residual=None) -> c
 
 ``a`` bf16 [m, k] (row stride a multiple of 8 elements), ``b`` uint8 [k, n] (8-bit, excess-128) or
-[k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n], ``bias`` bf16 [n]
-(added to the fp32 sums before the rounding, inside the kernel); returns bf16 [m, n].  torch supplies the output tensor, the current stream and a per-(device, stream) split-K
+[k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n], ``bias`` bf16 [n] and
+``residual`` bf16 [m, n] (added to the fp32 sums before the one rounding, inside the kernel); returns bf16 [m, n].  torch supplies the output tensor, the current stream and a per-(device, stream) split-K
 workspace; all arithmetic happens in ``libbfaintb_gemm.so``.  There is no CPU implementation: on a CPU
 tensor the operator raises.
 
@@ -61,10 +61,19 @@ def _check(a, b, scale, weight_bits, group_size, bias=None):
     return a.shape[0], n, k
 
 
+def _check_residual(residual, m, n):
+    if residual is None:
+        return None
+    if residual.dtype != torch.bfloat16 or tuple(residual.shape) != (m, n):
+        raise ValueError("bfaintb_gemm: residual must be bfloat16 [m, n]")
+    return residual.contiguous()
+
+
 @torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm", mutates_args=())
 def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
-                 bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     m, n, k = _check(a, b, scale, weight_bits, group_size, bias)
+    residual = _check_residual(residual, m, n)
     if not a.is_cuda:
         raise RuntimeError("bfaintb_gemm runs on the GPU only (no CPU implementation)")
     if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
@@ -80,22 +89,24 @@ def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_b
         need = _workspace_bytes(m, n, k, weight_bits, group_size)
         ws = _workspace(a.device, need)
         _gemm(c, a, b, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, workspace=ws,
-              workspace_nbytes=0 if ws is None else ws.numel(), bias=bias)
+              workspace_nbytes=0 if ws is None else ws.numel(), bias=bias, residual=residual)
     return c
 
 
 @bfaintb_gemm.register_fake
-def _(a, b, scale, weight_bits, group_size, bias=None):
+def _(a, b, scale, weight_bits, group_size, bias=None, residual=None):
     m, n, _k = _check(a, b, scale, weight_bits, group_size, bias)
+    _check_residual(residual, m, n)
     return a.new_empty((m, n))
 
 
 @torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm_prepacked", mutates_args=())
 def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
-                           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same product with the weights in the library's pre-packed order (``prepack_weight``): ``packed`` is a flat
     uint8 tensor of k * n * weight_bits / 8 bytes, n is taken from ``scale``."""
     m, n, k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
+    residual = _check_residual(residual, m, n)
     if not a.is_cuda:
         raise RuntimeError("bfaintb_gemm_prepacked runs on the GPU only (no CPU implementation)")
     if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
@@ -110,7 +121,7 @@ def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.T
     with torch.cuda.device(a.device):
         ws = _workspace(a.device, _prepacked_workspace_bytes(m, n, k, weight_bits, group_size))
         _gemm_prepacked(c, a, packed, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, bias=bias,
-                        workspace=ws)
+                        workspace=ws, residual=residual)
     return c
 
 
@@ -131,8 +142,9 @@ def _check_prepacked(a, packed, scale, weight_bits, group_size, bias=None):
 
 
 @bfaintb_gemm_prepacked.register_fake
-def _(a, packed, scale, weight_bits, group_size, bias=None):
+def _(a, packed, scale, weight_bits, group_size, bias=None, residual=None):
     m, n, _k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
+    _check_residual(residual, m, n)
     return a.new_empty((m, n))
 
 
@@ -205,9 +217,12 @@ class QuantLinear(torch.nn.Module):
             self.prepacked = True
         return self
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """``residual`` (same shape as the output, bf16) is added inside the kernel, before the rounding."""
         lead = x.shape[:-1]
         op = torch.ops.awesome_fusion.bfaintb_gemm_prepacked if self.prepacked else torch.ops.awesome_fusion.bfaintb_gemm
+        if residual is not None:
+            residual = residual.reshape(-1, self.out_features).to(torch.bfloat16)
         y = op(x.reshape(-1, self.in_features).to(torch.bfloat16), self.qweight, self.scales, self.weight_bits, self.group_size,
-               self.bias)
+               self.bias, residual)
         return y.reshape(*lead, self.out_features)

@@ -33,7 +33,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 101 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 102 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -101,6 +101,26 @@ BFAINTB_API int bfaintb_gemm_bias(void* c, const void* a, const void* b, const v
                       uint32_t n, uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * The GEMM with a fused epilogue, described by a struct so that it can grow:
+ *     C[m,n] = bf16_rne( sum_k A[m,k]*W[k,n]  + bias[n]  + residual[m,n] )
+ * each term that is present added in fp32, in this order, before the one rounding.  bias: bf16 [n]; residual: bf16
+ * [m, ldr] (ldr in elements, >= n, a multiple of 8); both 16-byte aligned; either may be NULL; epilogue == NULL is
+ * bfaintb_gemm.  `reserved` must be 0.  The reference kernel stores the bare sums (bf16gemm_kernel_gfx90a.s:594-630);
+ * these are the first epilogues of the reference's stated purpose, "gemm fusion for llm" (README.md:2): a linear layer's
+ * bias and a transformer block's residual connection, without a second pass over C.  The residual may alias c when
+ * ldr == ldc (every element is read by the thread that then writes it).
+ */
+typedef struct bfaintb_epilogue {
+    const void* bias;
+    const void* residual;
+    uint32_t ldr;
+    uint32_t reserved;
+} bfaintb_epilogue;
+BFAINTB_API int bfaintb_gemm_fused(void* c, const void* a, const void* b, const void* scale, const bfaintb_epilogue* epilogue, uint32_t m,
+                       uint32_t n, uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
 /* Scratch the GEMM needs for a shape: one fp32 word per (split but the last, row, column) of the
  * split-K partial sums, rounded up to 256 bytes; 0 when the shape runs without split-K.  Depends only
  * on its arguments.  The reference kernel has no scratch (no split-K, bfAintBGemm.cc:107-109). */
@@ -131,6 +151,10 @@ BFAINTB_API int bfaintb_unpack(void* b, const void* packed, uint32_t n, uint32_t
 BFAINTB_API int bfaintb_gemm_prepacked(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
                            uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
                            void* workspace, size_t workspace_bytes, void* stream);
+/* The packed-weight GEMM with the epilogue descriptor of bfaintb_gemm_fused. */
+BFAINTB_API int bfaintb_gemm_prepacked_fused(void* c, const void* a, const void* packed_b, const void* scale,
+                                 const bfaintb_epilogue* epilogue, uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc,
+                                 int weight_bits, uint32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 /* Scratch bfaintb_gemm_prepacked needs: 0 up to 48 rows of A (the slab-streaming kernel) and for the tiled kernel; in
  * between, what the row-blocked decode family needs when it splits along k.  Same workspace protocol as bfaintb_gemm
  * (bfaintb_workspace_init once; one workspace may serve both entry points). */

@@ -40,10 +40,16 @@ class Problem:
             self.b_bytes = oracle.pack_int4(q)
         self._w = None
         self.bias_bf = None  # optional bf16 [n] bias (set by with_bias)
+        self.residual_bf = None  # optional bf16 [m, n] residual (set by with_residual)
 
     def with_bias(self, seed=1, lo=-1.0, hi=1.0):
         rng = np.random.Generator(np.random.PCG64(seed))
         self.bias_bf = oracle.f32_to_bf16_rne(rng.uniform(lo, hi, size=(self.n,)).astype(np.float32))
+        return self
+
+    def with_residual(self, seed=2, lo=-2.0, hi=2.0):
+        rng = np.random.Generator(np.random.PCG64(seed))
+        self.residual_bf = oracle.f32_to_bf16_rne(rng.uniform(lo, hi, size=(self.m, self.n)).astype(np.float32))
         return self
 
     @property
@@ -101,8 +107,9 @@ def run_gemm(p, which=0, force_split_k=0, lda=None, ldb=None, ldc=None, a_dev=No
     c_dev = torch.full((m, ldc_), 0x7FC0 if c_fill is None else c_fill, dtype=torch.int16, device="cuda")
     ws = _ws.get(af.workspace_bytes(m, n, k, p.bits, p.group_size, which, force_split_k))
     bias_dev = None if p.bias_bf is None else to_dev(p.bias_bf)
+    res_dev = None if p.residual_bf is None else to_dev(p.residual_bf)
     af.gemm(c_dev, a_dev, b_dev, s_dev, m, n, k, lda, ldb, ldc, p.bits, p.group_size, ws, None, None, which, force_split_k,
-            bias=bias_dev)
+            bias=bias_dev, residual=res_dev)
     torch.cuda.synchronize()
     return from_dev_u16(c_dev)
 
@@ -135,6 +142,9 @@ def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
     bias = None if p.bias_bf is None else widen(p.bias_bf)
     if bias is not None:
         c_ref = (c_ref + bias[None, :]).astype(np.float32)  # one fp32 addition after the sum, before the rounding to bf16
+    res = None if p.residual_bf is None else widen(p.residual_bf if rows is None else p.residual_bf[rows])
+    if res is not None:
+        c_ref = (c_ref + res).astype(np.float32)            # and one more for the residual
     bad, ulps = ulp_violations(c_ref, c_bits)
     nbad_c, _, _ = oracle.check_ulp(c_ref, c_bits)
     assert nbad_c == len(bad), "C and numpy acceptance checks disagree"
@@ -147,7 +157,7 @@ def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
         for flat, g in zip(bad, got):
             i, j = divmod(int(flat), n)
             terms = af_[i] * wf_[:, j]
-            exact = terms.sum() + (0.0 if bias is None else float(bias[j]))
+            exact = terms.sum() + (0.0 if bias is None else float(bias[j])) + (0.0 if res is None else float(res[i, j]))
             _, e = np.frexp(abs(exact))
             tol = 2.0 * np.ldexp(1.0, max(int(e) - 1, -126) - 7) + np.sqrt(p.k) * 2.0 ** -24 * np.abs(terms).sum()
             assert abs(g - exact) <= tol, f"{what}: output ({i},{j}) = {g!r}, exact {exact!r}, fp32 oracle " \

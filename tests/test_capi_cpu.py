@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
-    assert af.lib().bfaintb_version() == 101
+    assert af.lib().bfaintb_version() == 102
     assert "bfaintb_gemm_bias" in names
 
 
@@ -73,6 +73,9 @@ def test_rejects_bad_arguments_without_launching():
     assert rc(m=8, k=1024, which=af.DECODE, force_split_k=2, workspace=P, workspace_nbytes=64) == -6
     assert rc(m=0) == 0                       # nothing to do
     assert rc(bias=P + 2) == -4               # bias must be 16-byte aligned too
+    assert rc(residual=P + 2) == -4           # and the residual
+    assert rc(residual=P, ldr=64) == -3       # ldr < n
+    assert rc(residual=P, ldr=132) == -3      # rows of the residual would lose 16-byte alignment
     for code in (-1, -2, -3, -4, -5, -6, -7):
         assert len(af.error_string(code)) > 10
     with pytest.raises(af.BfaintbError) as e:

@@ -227,6 +227,47 @@ def test_fused_bias(af, m, n, k, bits, group):
     assert np.array_equal(run_gemm(p), np.broadcast_to(p.bias_bf, (m, n)))
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (1, 4096, 4096, 8, 0),      # decode, split-K: the reducing workgroup adds the residual
+    (7, 528, 1024, 4, 128),     # decode, 4-bit
+    (24, 272, 512, 8, 0),       # decode, no split
+    (80, 1040, 2048, 8, 64),    # row-blocked decode family
+    (300, 272, 192, 8, 0),      # row-blocked family, ragged rows and columns
+    (4200, 272, 256, 8, 0),     # tiled kernel, ragged rows and columns, half tiles
+    (4200, 528, 256, 4, 128),   # tiled kernel, 4-bit
+])
+def test_fused_residual(af, m, n, k, bits, group):
+    """C = bf16(sum + bias + residual): against the oracle's fp32 sums plus the two fp32 additions, with and without the
+    bias, and in place (residual == c)."""
+    import torch
+    p = Problem(m, n, k, bits, group, seed=m + k).with_residual()
+    assert_close_ulp(p, run_gemm(p), f"residual {m}x{n}x{k}")
+    p.with_bias()
+    want = run_gemm(p)
+    assert_close_ulp(p, want, f"bias + residual {m}x{n}x{k}")
+    # in place: the residual is the output buffer
+    from helpers import Workspace
+    c = to_dev(p.residual_bf).clone()
+    ws = Workspace().get(af.workspace_bytes(m, n, k, bits, group))
+    af.gemm(c, to_dev(p.a_bf), to_dev(p.b_bytes), to_dev(p.s_bf), m, n, k, weight_bits=bits, group_size=group, workspace=ws,
+            bias=to_dev(p.bias_bf), residual=c)
+    torch.cuda.synchronize()
+    assert np.array_equal(from_dev_u16(c), want)
+
+
+def test_residual_closed_forms(af):
+    """Zero activations: C = bf16(bias + residual) exactly; zero residual: the bits of the bias-only call."""
+    p = Problem(40, 272, 256, seed=8).with_bias().with_residual()
+    base = Problem(40, 272, 256, seed=8).with_bias()
+    p.a_bf = np.zeros_like(p.a_bf)
+    want = oracle.f32_to_bf16_rne((widen(p.bias_bf)[None, :] + widen(p.residual_bf)).astype(np.float32))
+    assert np.array_equal(run_gemm(p), want)
+    q = Problem(40, 272, 256, seed=8).with_bias().with_residual()
+    q.residual_bf = np.zeros_like(q.residual_bf)
+    got, ref = run_gemm(q), run_gemm(base)
+    assert np.array_equal(got & 0x7FFF, ref & 0x7FFF) and np.all((got == ref) | ((ref & 0x7FFF) == 0))  # up to the sign of zero
+
+
 def test_row_permutation_permutes_output(af):
     # size-independent property at a prefill shape: rows of A are independent
     p = Problem(512, 512, 512, seed=5)

@@ -35,8 +35,9 @@ def run_prepacked(af, p, which=0, pk=None, ldc=None):
     c = torch.full((p.m, ldc_), 0x7FC0, dtype=torch.int16, device="cuda")
     bias = None if p.bias_bf is None else to_dev(p.bias_bf)
     ws = _ws.get(af.prepacked_workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size, which))
+    res = None if p.residual_bf is None else to_dev(p.residual_bf)
     af.gemm_prepacked(c, to_dev(p.a_bf), pk, to_dev(p.s_bf), p.m, p.n, p.k, ldc=ldc, weight_bits=p.bits, group_size=p.group_size,
-                      bias=bias, workspace=ws, which=which)
+                      bias=bias, workspace=ws, which=which, residual=res)
     torch.cuda.synchronize()
     return from_dev_u16(c)
 
@@ -163,6 +164,18 @@ def test_workspace_is_required_where_the_plan_splits_and_left_ready(af):
         torch.cuda.synchronize()
         assert_close_ulp(p, from_dev_u16(c), "packed split-K")
     assert bool((ws == 0xFF).all())
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (1, 4096, 4096, 8, 0), (20, 528, 1024, 4, 128),   # slab kernel
+    (80, 1040, 2048, 8, 64), (64, 256, 4096, 4, 128),  # row-blocked family, without and with a split along k
+    (4200, 272, 256, 8, 0), (4200, 528, 256, 4, 128),  # tiled kernel over packed weights
+])
+def test_fused_residual(af, m, n, k, bits, group):
+    p = Problem(m, n, k, bits, group, seed=m + k).with_residual()
+    assert_close_ulp(p, run_prepacked(af, p), f"packed residual {m}x{n}x{k}")
+    p.with_bias()
+    assert_close_ulp(p, run_prepacked(af, p), f"packed bias + residual {m}x{n}x{k}")
 
 
 def test_output_stride_and_padding(af):

@@ -123,3 +123,21 @@ def test_quant_linear_prepacked_matches_row_major_layer():
     assert ql.prepacked and ql.qweight.dim() == 1
     # same weights, same fp32 accumulation up to summation order: within a bf16 ULP or two of each other
     assert torch.allclose(y_row.float(), y_packed.float(), rtol=2e-2, atol=2e-3)
+
+
+@pytest.mark.gpu
+def test_quant_linear_residual_is_added_before_the_rounding():
+    torch.manual_seed(2)
+    lin = torch.nn.Linear(512, 256, bias=True).cuda()
+    ql = top.QuantLinear.from_float(lin, weight_bits=8, group_size=0)
+    x = torch.randn((6, 512), device="cuda")
+    r = torch.randn((6, 256), device="cuda").to(torch.bfloat16)
+    y = ql(x, residual=r)
+    q = ql.qweight.to(torch.int16) - 128
+    w = (q.float() * ql.scales.float()).to(torch.bfloat16).float()
+    ref = x.to(torch.bfloat16).float() @ w + ql.bias.float() + r.float()
+    assert torch.allclose(y.float(), ref, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(ql.prepack()(x, residual=r).float(), y.float(), rtol=2e-2, atol=2e-3)
+    out = torch.ops.awesome_fusion.bfaintb_gemm(torch.zeros((6, 512), dtype=torch.bfloat16, device="meta"), ql.qweight.to("meta") if not ql.prepacked else torch.zeros((512, 256), dtype=torch.uint8, device="meta"),
+                                                ql.scales.to("meta"), 8, 0, None, torch.zeros((6, 256), dtype=torch.bfloat16, device="meta"))
+    assert out.shape == (6, 256)
