@@ -431,27 +431,43 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             if (n0 + col0 < p.n) bias0 = bf16_bits_to_f32(p.bias[n0 + col0]);
             if (n0 + col0 + 16u < p.n) bias1 = bf16_bits_to_f32(p.bias[n0 + col0 + 16u]);
         }
+        // the residual of this lane's outputs (two columns each) is fetched for two 32-row blocks at a time, before the first
+        // value is used: the epilogue has the registers the main loop's fragments have freed, and pays two memory
+        // latencies instead of one per block
 #pragma unroll
-        for (uint32_t mt = 0; mt < MT; ++mt) {
-            const uint32_t block32 = wm * MT + mt;
-            uint8_t* base = c_rows(block32 >> 1);
+        for (uint32_t mt0 = 0; mt0 < MT; mt0 += 2) {
+            uint32_t rres[2][16];
+            if (has_res) {
 #pragma unroll
-            for (uint32_t i = 0; i < 16; ++i) {
-                const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
-                uint32_t both;
-                if (has_res) {
-                    const uint32_t gm = m0 + 64u * (block32 >> 1) + row;
-                    float v0 = acc[mt][0][i] + bias0, v1 = acc[mt][1][i] + bias1;  // bias0/1 are +0 without a bias: a sum that
-                    if (gm < p.m) {                                                 // gets a residual added need not keep -0
-                        if (n0 + col0 < p.n) v0 += bf16_bits_to_f32(p.residual[(size_t)gm * p.ldr + n0 + col0]);
-                        if (n0 + col0 + 16u < p.n) v1 += bf16_bits_to_f32(p.residual[(size_t)gm * p.ldr + n0 + col0 + 16u]);
+                for (uint32_t mt = mt0; mt < mt0 + 2; ++mt)
+#pragma unroll
+                    for (uint32_t i = 0; i < 16; ++i) {
+                        const uint32_t gm = m0 + 32u * (wm * MT + mt) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                        uint32_t lo = 0, hi = 0;
+                        if (gm < p.m) {
+                            if (n0 + col0 < p.n) lo = p.residual[(size_t)gm * p.ldr + n0 + col0];
+                            if (n0 + col0 + 16u < p.n) hi = p.residual[(size_t)gm * p.ldr + n0 + col0 + 16u];
+                        }
+                        rres[mt - mt0][i] = lo | (hi << 16);
                     }
-                    both = pack_bf16_rne(v0, v1);
-                } else {
-                    both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+            }
+#pragma unroll
+            for (uint32_t mt = mt0; mt < mt0 + 2; ++mt) {
+                const uint32_t block32 = wm * MT + mt;
+                uint8_t* base = c_rows(block32 >> 1);
+#pragma unroll
+                for (uint32_t i = 0; i < 16; ++i) {
+                    const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                    uint32_t both;
+                    if (has_res) {  // bias0/1 are +0 without a bias: a sum that gets a residual added need not keep -0
+                        both = pack_bf16_rne(acc[mt][0][i] + bias0 + bf16_bits_to_f32(rres[mt - mt0][i] & 0xffffu),
+                                             acc[mt][1][i] + bias1 + bf16_bits_to_f32(rres[mt - mt0][i] >> 16));
+                    } else {
+                        both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                    }
+                    *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0) = (uint16_t)(both & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0 + 32u) = (uint16_t)(both >> 16);
                 }
-                *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0) = (uint16_t)(both & 0xffffu);
-                *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0 + 32u) = (uint16_t)(both >> 16);
             }
         }
     } else
@@ -466,6 +482,19 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             bias0 = bf16_bits_to_f32(raw & 0xffffu);
             bias1 = bf16_bits_to_f32(raw >> 16);
         }
+        // the residual of this lane's 32 x MT outputs (two neighbouring columns each), fetched in one go before the first
+        // is used (see the packed branch)
+        uint32_t rres[4][16];
+        if (has_res) {
+#pragma unroll
+            for (uint32_t mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (uint32_t i = 0; i < 16; ++i) {
+                    const uint32_t gm = m0 + 32u * (wm * MT + mt) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                    rres[mt][i] = (gm < p.m && n0 + colbyte / 2u < p.n)
+                                      ? *reinterpret_cast<const uint32_t*>(p.residual + (size_t)gm * p.ldr + n0 + colbyte / 2u) : 0u;
+                }
+        }
 #pragma unroll
         for (uint32_t mt = 0; mt < MT; ++mt) {
             const uint32_t block32 = wm * MT + mt;  // which 32 rows of the tile
@@ -473,17 +502,11 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 #pragma unroll
             for (uint32_t i = 0; i < 16; ++i) {
                 const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
-                // without a bias the sums are stored as they are (adding +0 would turn a -0 sum into +0)
+                // without a bias or residual the sums are stored as they are (adding +0 would turn a -0 sum into +0)
                 uint32_t both;
                 if (has_res) {
-                    const uint32_t gm = m0 + 64u * (block32 >> 1) + row;
-                    float v0 = acc[mt][0][i] + bias0, v1 = acc[mt][1][i] + bias1;
-                    if (gm < p.m && n0 + colbyte / 2u < p.n) {
-                        const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.residual + (size_t)gm * p.ldr + n0 + colbyte / 2u);
-                        v0 += bf16_bits_to_f32(raw & 0xffffu);
-                        v1 += bf16_bits_to_f32(raw >> 16);
-                    }
-                    both = pack_bf16_rne(v0, v1);
+                    both = pack_bf16_rne(acc[mt][0][i] + bias0 + bf16_bits_to_f32(rres[mt][i] & 0xffffu),
+                                         acc[mt][1][i] + bias1 + bf16_bits_to_f32(rres[mt][i] >> 16));
                 } else {
                     both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
                 }

@@ -136,6 +136,44 @@ def time_graph(af, w, steps, warmup, rotate, packed=False):
     return ev[mid], wall[mid]
 
 
+def time_fused_epilogue(af, w, steps, warmup):
+    """(fused_ms, unfused_ms): C = A.W + bias + residual in one launch (bfaintb_gemm_fused), against the plain GEMM
+    followed by torch's elementwise bias and residual additions on the bf16 output (two more passes over C)."""
+    import torch
+    ws = w.workspace(af)
+    bias = torch.randn(w.n, device="cuda").to(torch.bfloat16)
+    res = torch.randn((w.m, w.n), device="cuda").to(torch.bfloat16)
+
+    def fused(i):
+        af.gemm(w.c, w.a, w.b[i % len(w.b)], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws, bias=bias, residual=res)
+
+    def unfused(i):
+        af.gemm(w.c, w.a, w.b[i % len(w.b)], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
+        w.c.add_(bias).add_(res)
+
+    out = []
+    for launch in (fused, unfused):
+        for i in range(warmup):
+            launch(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(steps):
+                launch(i)
+        g.replay()
+        torch.cuda.synchronize()
+        ev = []
+        for _ in range(REPLAYS):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            ev.append(e0.elapsed_time(e1) / steps)
+        out.append(sorted(ev)[REPLAYS // 2])
+    return out[0], out[1]
+
+
 def time_read_ceiling(af, w, steps, warmup):
     """The same rotation of B copies through a kernel that only fetches the bytes."""
     import torch
@@ -327,6 +365,9 @@ def main():
                                                       "note": "B re-read from cache: not an HBM figure"}
             out_extra["decode_m1_eager_launch_loop"] = {"us_per_launch": round(eager_ms * 1e3, 3),
                                                         "note": "reference protocol (no graph): host launch rate included"}
+            f_ms, u_ms = time_fused_epilogue(af, w, K, W)
+            out_extra["decode_m1_bias_residual"] = {"fused_kernel_us": round(f_ms * 1e3, 3), "gemm_then_two_elementwise_us": round(u_ms * 1e3, 3),
+                                                    "note": "C = A.W + bias + residual: one bfaintb_gemm_fused launch against bfaintb_gemm + torch add_ x2"}
             pk_ms, _ = time_graph(af, w, K, W, rotate=True, packed=True)
             out_extra["decode_m1_prepacked"] = {
                 **roofline_entry(w, pk_ms, "hbm", "_prepacked"), "frac_of_fetch_only": round(read_ms / pk_ms, 4),
@@ -354,6 +395,9 @@ def main():
                                                     "note": "torch.matmul bf16 x bf16 on pre-dequantised weights (no dequantisation work): context, not a baseline"}
         except Exception as exc:  # context only
             entry["vendor_bf16_gemm_same_shape"] = {"error": str(exc)[:200]}
+        f_ms, u_ms = time_fused_epilogue(af, w, pk, max(5, W // 4))
+        entry["bias_residual"] = {"fused_kernel_us": round(f_ms * 1e3, 3), "gemm_then_two_elementwise_us": round(u_ms * 1e3, 3),
+                                  "note": "C = A.W + bias + residual: one bfaintb_gemm_fused launch against bfaintb_gemm + torch add_ x2"}
         pk_ms, _ = time_graph(af, w, pk, max(5, W // 4), rotate=True, packed=True)
         entry["prepacked"] = {**roofline_entry(w, pk_ms, "mfma", "_prepacked"), "note": "bfaintb_gemm_prepacked, same shape"}
         out_extra["prefill_m4096"] = entry
