@@ -14,6 +14,8 @@ from .gemm import (  # noqa: F401
     DECODE,
     PREFILL,
     AUTO,
+    ACT_NONE,
+    ACT_SILU_GATE,
     build_library,
     dequant,
     error_string,

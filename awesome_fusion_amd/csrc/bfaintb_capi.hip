@@ -260,16 +260,20 @@ struct Epilogue {
     const void* bias = nullptr;
     const void* residual = nullptr;
     uint32_t ldr = 0;
+    uint32_t activation = BFAINTB_ACT_NONE;
+    // columns of C (and of the residual) for n columns of B
+    uint32_t out_cols(uint32_t n) const { return activation == BFAINTB_ACT_SILU_GATE ? n / 2u : n; }
 };
 
 static int read_epilogue(Epilogue& out, const bfaintb_epilogue* ep, uint32_t n)
 {
     if (ep == nullptr) return BFAINTB_OK;
-    if (ep->reserved != 0) return BFAINTB_ERR_UNSUPPORTED;
+    if (ep->activation != BFAINTB_ACT_NONE && ep->activation != BFAINTB_ACT_SILU_GATE) return BFAINTB_ERR_UNSUPPORTED;
     out.bias = ep->bias;
     out.residual = ep->residual;
     out.ldr = ep->ldr;
-    if (ep->residual != nullptr && (ep->ldr < n || ep->ldr % 8u != 0)) return BFAINTB_ERR_BAD_LD;
+    out.activation = ep->activation;
+    if (ep->residual != nullptr && (ep->ldr < out.out_cols(n) || ep->ldr % 8u != 0)) return BFAINTB_ERR_BAD_LD;
     return BFAINTB_OK;
 }
 
@@ -282,7 +286,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     if (e) return e;
     e = check_shape(m, n, k);
     if (e) return e;
-    if (lda < k || ldb < n || ldc < n || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
+    if (lda < k || ldb < n || ldc < ep.out_cols(n) || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
     const int v = resolve_variant(m, n, k, weight_bits, variant);
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
@@ -294,6 +298,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.bias = static_cast<const uint16_t*>(bias);
     p.residual = static_cast<const uint16_t*>(ep.residual);
     p.ldr = ep.ldr;
+    p.activation = ep.activation;
     p.c = static_cast<uint16_t*>(c);
     p.a = static_cast<const uint16_t*>(a);
     p.b = static_cast<const uint8_t*>(b);
@@ -466,7 +471,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
     if (e) return e;
     e = check_packed_shape(n, k, weight_bits);
     if (e) return e;
-    if (lda < k || ldc < n || lda % 8u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
+    if (lda < k || ldc < ep.out_cols(n) || lda % 8u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
     const int v = packed_variant(m, n, k, weight_bits, variant);
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;
@@ -477,6 +482,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
     GemmParams p{};
     p.residual = static_cast<const uint16_t*>(ep.residual);
     p.ldr = ep.ldr;
+    p.activation = ep.activation;
     p.c = static_cast<uint16_t*>(c);
     p.a = static_cast<const uint16_t*>(a);
     p.b = static_cast<const uint8_t*>(packed_b);

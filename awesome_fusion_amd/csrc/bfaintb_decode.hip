@@ -212,8 +212,10 @@ __host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t r
     return waves * rows * (cols + 4u);
 }
 
-// t += bias[col .. col+3], then += residual[row][col .. col+3] (fp32 additions), for what the launch has of them.
-__device__ __forceinline__ void add_epilogue4(const GemmParams& p, float4& t, uint32_t row, uint32_t col)
+// Finishes four neighbouring columns of one row: t += bias[col .. col+3]; then either += residual[row][col .. col+3] and
+// four bf16 outputs at C[row][col ..], or (gated) the two outputs silu(t.x) * t.y and silu(t.z) * t.w, += residual[row]
+// [col/2 ..], at C[row][col/2 ..].  All additions in fp32, one rounding.
+__device__ __forceinline__ void finish_row4(const GemmParams& p, float4 t, uint32_t row, uint32_t col)
 {
     if (p.bias != nullptr) {
         const uint2 raw = *reinterpret_cast<const uint2*>(p.bias + col);
@@ -222,6 +224,16 @@ __device__ __forceinline__ void add_epilogue4(const GemmParams& p, float4& t, ui
         t.z += bf16_bits_to_f32(raw.y & 0xffffu);
         t.w += bf16_bits_to_f32(raw.y >> 16);
     }
+    if (p.activation == kActSiluGate) {
+        float o0 = silu_gate(t.x, t.y), o1 = silu_gate(t.z, t.w);
+        if (p.residual != nullptr) {
+            const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.residual + (size_t)row * p.ldr + col / 2u);
+            o0 += bf16_bits_to_f32(raw & 0xffffu);
+            o1 += bf16_bits_to_f32(raw >> 16);
+        }
+        *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col / 2u) = pack_bf16_rne(o0, o1);
+        return;
+    }
     if (p.residual != nullptr) {
         const uint2 raw = *reinterpret_cast<const uint2*>(p.residual + (size_t)row * p.ldr + col);
         t.x += bf16_bits_to_f32(raw.x & 0xffffu);
@@ -229,6 +241,10 @@ __device__ __forceinline__ void add_epilogue4(const GemmParams& p, float4& t, ui
         t.z += bf16_bits_to_f32(raw.y & 0xffffu);
         t.w += bf16_bits_to_f32(raw.y >> 16);
     }
+    uint2 o;
+    o.x = pack_bf16_rne(t.x, t.y);
+    o.y = pack_bf16_rne(t.z, t.w);
+    *reinterpret_cast<uint2*>(p.c + (size_t)row * p.ldc + col) = o;
 }
 
 // Split-K, the reducing workgroup's part for one thread: R rows (first_row + rs, + nrs, ...; `rows` of
@@ -300,12 +316,8 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
     for (uint32_t i = 0; i < R; ++i) {
         const uint32_t row = rs + i * nrs;
         if (row < rows && col_ok) {
-            float4 t = make_float4(total[i].x + sum[i].x, total[i].y + sum[i].y, total[i].z + sum[i].z, total[i].w + sum[i].w);
-            add_epilogue4(p, t, first_row + row, col);
-            uint2 o;
-            o.x = pack_bf16_rne(t.x, t.y);
-            o.y = pack_bf16_rne(t.z, t.w);
-            *reinterpret_cast<uint2*>(p.c + (size_t)(first_row + row) * p.ldc + col) = o;
+            finish_row4(p, make_float4(total[i].x + sum[i].x, total[i].y + sum[i].y, total[i].z + sum[i].z, total[i].w + sum[i].w),
+                        first_row + row, col);
         }
     }
 }
@@ -540,12 +552,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
             for (uint32_t i = 0; i < kMaxR; ++i) {
                 const uint32_t row = rs + i * nrs;
                 if (row < rows_out && col_ok) {
-                    float4 t = sum[i];
-                    add_epilogue4(p, t, first_row + row, col);
-                    uint2 o;
-                    o.x = pack_bf16_rne(t.x, t.y);
-                    o.y = pack_bf16_rne(t.z, t.w);
-                    *reinterpret_cast<uint2*>(p.c + (size_t)(first_row + row) * p.ldc + col) = o;
+                    finish_row4(p, sum[i], first_row + row, col);
                 }
             }
         } else if (ks != p.splits - 1u) {

@@ -25,6 +25,16 @@ constexpr int kBufferFlags = 0x00027000;  // buffer resource word 3: raw buffer,
 // where every XCD sees it, the load does not settle for a stale local copy).
 constexpr int kAuxDeviceScope = 16;
 
+// Epilogue activations (values of bfaintb_epilogue.activation).
+constexpr uint32_t kActNone = 0, kActSiluGate = 1;
+
+// silu(g) * u in fp32: g / (1 + exp(-g)) * u.  exp through the hardware's base-2 exponential, the quotient through its
+// reciprocal: a few units in the last place of fp32, far below the bf16 rounding that follows.  g -> -inf gives -0 * u.
+__device__ __forceinline__ float silu_gate(float g, float u)
+{
+    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
+}
+
 // A split-K workspace word that holds no partial sum: an all-ones NaN.  Sums of products of bf16 numbers
 // are never this pattern (NaNs born in the arithmetic are the default quiet NaN; NaNs carried over from
 // bf16 inputs have zero low bits).
@@ -49,6 +59,7 @@ struct GemmParams {
     const uint16_t* bias;  // bf16 [n] added to the fp32 sums before the one rounding to bf16, or null
     const uint16_t* residual;  // bf16 [m, ldr] added after the bias, before the rounding, or null
     uint32_t ldr;              // elements per row of residual
+    uint32_t activation;       // kActNone, or kActSiluGate: columns (2j, 2j+1) of the sums are (gate, up) of output column j
     uint32_t m, n, k;
     uint32_t lda;        // elements
     uint32_t ldb_bytes;  // bytes per row of packed weights

@@ -276,15 +276,34 @@ __device__ __forceinline__ void decode_packed_body(const GemmParams& p)
     for (int mb = 0; mb < MB; ++mb)
         *reinterpret_cast<float4*>(&red[wave][mb][nl][4u * kg]) = make_float4(acc[mb][0], acc[mb][1], acc[mb][2], acc[mb][3]);
     __syncthreads();
+    auto wave_sum = [&](uint32_t mb, uint32_t j, uint32_t i) {
+        float sum = red[0][mb][j][i];
+#pragma unroll
+        for (int w = 1; w < kPackedWaves; ++w) sum += red[w][mb][j][i];
+        const uint32_t c = 16u * nb + i;
+        if (p.bias != nullptr) sum += bf16_bits_to_f32(p.bias[c]);
+        return sum;
+    };
+    if (p.activation == kActSiluGate) {
+        // columns (2 ip, 2 ip + 1) of the block are (gate, up) of output column 8 nb + ip
+        for (uint32_t t = tid; t < 128u * MB; t += 64u * kPackedWaves) {
+            const uint32_t mb = t >> 7, j = (t >> 3) & 15u, ip = t & 7u;
+            const uint32_t row = 16u * (MB * rb + mb) + j;
+            if (row < p.m) {
+                float out = silu_gate(wave_sum(mb, j, 2u * ip), wave_sum(mb, j, 2u * ip + 1u));
+                const uint32_t c = 8u * nb + ip;
+                if (p.residual != nullptr) out += bf16_bits_to_f32(p.residual[(size_t)row * p.ldr + c]);
+                p.c[(size_t)row * p.ldc + c] = (uint16_t)(pack_bf16_rne(out, 0.f) & 0xffffu);
+            }
+        }
+        return;
+    }
     for (uint32_t t = tid; t < 256u * MB; t += 64u * kPackedWaves) {
         const uint32_t mb = t >> 8, j = (t >> 4) & 15u, i = t & 15u;  // row block, A row, W column
         const uint32_t row = 16u * (MB * rb + mb) + j;
         if (row < p.m) {
-            float sum = red[0][mb][j][i];
-#pragma unroll
-            for (int w = 1; w < kPackedWaves; ++w) sum += red[w][mb][j][i];
+            float sum = wave_sum(mb, j, i);
             const uint32_t c = 16u * nb + i;
-            if (p.bias != nullptr) sum += bf16_bits_to_f32(p.bias[c]);
             if (p.residual != nullptr) sum += bf16_bits_to_f32(p.residual[(size_t)row * p.ldr + c]);
             p.c[(size_t)row * p.ldc + c] = (uint16_t)(pack_bf16_rne(sum, 0.f) & 0xffffu);
         }

@@ -420,6 +420,8 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
     __syncthreads();
     auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_w0 : lds_w1; };
+    // gated: columns (2j, 2j+1) of the sums are (gate, up) of output column j; the staged tile is then 128 columns wide
+    const bool gated = p.activation == kActSiluGate;
     if constexpr (PACKED) {
         // accumulator t of this wave, MFMA column jl is tile column 16 * (4 wn + 2 (jl >> 4) + t) + (jl & 15): the two
         // accumulators are 16 columns apart, so each value is staged on its own
@@ -431,6 +433,46 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             if (n0 + col0 < p.n) bias0 = bf16_bits_to_f32(p.bias[n0 + col0]);
             if (n0 + col0 + 16u < p.n) bias1 = bf16_bits_to_f32(p.bias[n0 + col0 + 16u]);
         }
+        if (gated) {
+            // neighbouring columns (gate, up) sit in neighbouring lanes: even lanes fetch the partner's sums with a DPP swap and
+            // produce output columns (n0 + col0) / 2 and (n0 + col0 + 16) / 2
+            const bool is_gate = (lane & 1u) == 0u;
+#pragma unroll
+            for (uint32_t mt = 0; mt < MT; ++mt) {
+                const uint32_t block32 = wm * MT + mt;
+                uint8_t* base = c_rows(block32 >> 1);
+                uint32_t rres[16];
+                if (has_res && is_gate) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 16; ++i) {
+                        const uint32_t gm = m0 + 32u * block32 + 8u * (i >> 2) + 4u * half + (i & 3u);
+                        uint32_t lo = 0, hi = 0;
+                        if (gm < p.m) {
+                            if (n0 + col0 < p.n) lo = p.residual[(size_t)gm * p.ldr + (n0 + col0) / 2u];
+                            if (n0 + col0 + 16u < p.n) hi = p.residual[(size_t)gm * p.ldr + (n0 + col0 + 16u) / 2u];
+                        }
+                        rres[i] = lo | (hi << 16);
+                    }
+                }
+#pragma unroll
+                for (uint32_t i = 0; i < 16; ++i) {
+                    const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                    const float x0 = acc[mt][0][i] + bias0, x1 = acc[mt][1][i] + bias1;
+                    const float y0 = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x0), 0xB1, 0xF, 0xF, true));
+                    const float y1 = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x1), 0xB1, 0xF, 0xF, true));
+                    if (is_gate) {
+                        float o0 = silu_gate(x0, y0), o1 = silu_gate(x1, y1);
+                        if (has_res) {
+                            o0 += bf16_bits_to_f32(rres[i] & 0xffffu);
+                            o1 += bf16_bits_to_f32(rres[i] >> 16);
+                        }
+                        const uint32_t both = pack_bf16_rne(o0, o1);
+                        *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + col0) = (uint16_t)(both & 0xffffu);
+                        *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + col0 + 16u) = (uint16_t)(both >> 16);
+                    }
+                }
+            }
+        } else
         // the residual of this lane's outputs (two columns each) is fetched for two 32-row blocks at a time, before the first
         // value is used: the epilogue has the registers the main loop's fragments have freed, and pays two memory
         // latencies instead of one per block
@@ -482,6 +524,29 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             bias0 = bf16_bits_to_f32(raw & 0xffffu);
             bias1 = bf16_bits_to_f32(raw >> 16);
         }
+        if (gated) {
+            // the lane's two neighbouring columns are (gate, up) of tile output column colbyte / 4
+#pragma unroll
+            for (uint32_t mt = 0; mt < MT; ++mt) {
+                const uint32_t block32 = wm * MT + mt;
+                uint8_t* base = c_rows(block32 >> 1);
+                uint32_t rres[16];
+                if (has_res) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 16; ++i) {
+                        const uint32_t gm = m0 + 32u * block32 + 8u * (i >> 2) + 4u * half + (i & 3u);
+                        rres[i] = (gm < p.m && n0 + colbyte / 2u < p.n) ? p.residual[(size_t)gm * p.ldr + (n0 + colbyte / 2u) / 2u] : 0u;
+                    }
+                }
+#pragma unroll
+                for (uint32_t i = 0; i < 16; ++i) {
+                    const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
+                    float o = silu_gate(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1);
+                    if (has_res) o += bf16_bits_to_f32(rres[i]);
+                    *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + colbyte / 2u) = (uint16_t)(pack_bf16_rne(o, 0.f) & 0xffffu);
+                }
+            }
+        } else {
         // the residual of this lane's 32 x MT outputs (two neighbouring columns each), fetched in one go before the first
         // is used (see the packed branch)
         uint32_t rres[4][16];
@@ -513,14 +578,16 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                 *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) = both;
             }
         }
+        }
     }
     __syncthreads();
 #pragma unroll
     for (uint32_t pass = 0; pass < 4u * MT; ++pass) {
         const uint32_t row = pass * 16u + (tid >> 5);
         const uint32_t ch = tid & 31u;
-        const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
-        if (gm < p.m && gn < p.n) {
+        const uint32_t gm = m0 + row;
+        const uint32_t gn = gated ? n0 / 2u + ch * 8u : n0 + ch * 8u;  // gated rows hold 128 outputs: chunks 0..15
+        if (gm < p.m && (gated ? (ch < 16u && gn < p.n / 2u) : gn < p.n)) {
             const uint4 v = *reinterpret_cast<const uint4*>(c_rows(pass >> 2) + (row & 63u) * kCRowBytes + ch * 16u);
             *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) = v;
         }

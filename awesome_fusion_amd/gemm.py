@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = os.path.join(_HERE, "libbfaintb_gemm.so")
 
 AUTO, DECODE, PREFILL = 0, 1, 2
+ACT_NONE, ACT_SILU_GATE = 0, 1
 
 
 class BfaintbError(RuntimeError):
@@ -43,7 +44,7 @@ _vp = C.c_void_p
 
 class Epilogue(C.Structure):
     """bfaintb_epilogue of include/bfaintb_gemm.h."""
-    _fields_ = [("bias", C.c_void_p), ("residual", C.c_void_p), ("ldr", C.c_uint32), ("reserved", C.c_uint32)]
+    _fields_ = [("bias", C.c_void_p), ("residual", C.c_void_p), ("ldr", C.c_uint32), ("activation", C.c_uint32)]
 
 
 class PackedHeader(C.Structure):
@@ -162,27 +163,29 @@ def workspace_init(workspace, nbytes=None, stream=None):
         raise BfaintbError(rc, "bfaintb_workspace_init")
 
 
-def _epilogue(bias, residual, ldr, n):
+def _epilogue(bias, residual, ldr, n, activation=ACT_NONE):
     ep = Epilogue()
     ep.bias = _ptr(bias)
     ep.residual = _ptr(residual)
-    ep.ldr = n if ldr is None else ldr
+    ep.ldr = (n // 2 if activation == ACT_SILU_GATE else n) if ldr is None else ldr
+    ep.activation = activation
     return ep
 
 
 def gemm(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, group_size=0, workspace=None,
-         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True, bias=None, residual=None, ldr=None):
+         workspace_nbytes=None, stream=None, which=AUTO, force_split_k=0, check=True, bias=None, residual=None, ldr=None,
+         activation=ACT_NONE):
     """C = A x dequant(B, scale) through bfaintb_gemm_ex, or (AUTO variant only) + bias through bfaintb_gemm_bias,
     + bias + residual through bfaintb_gemm_fused.  Returns the library's return code (raises on non-zero when ``check``)."""
     lda = k if lda is None else lda
     ldb = n if ldb is None else ldb
-    ldc = n if ldc is None else ldc
+    ldc = (n // 2 if activation == ACT_SILU_GATE else n) if ldc is None else ldc
     if workspace_nbytes is None:
         workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
-    if residual is not None:
+    if residual is not None or activation != ACT_NONE:
         if which != AUTO or force_split_k:
             raise ValueError("bfaintb_gemm_fused takes no forced variant or split factor")
-        ep = _epilogue(bias, residual, ldr, n)
+        ep = _epilogue(bias, residual, ldr, n, activation)
         rc = lib().bfaintb_gemm_fused(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), C.byref(ep), m, n, k, lda, ldb, ldc, weight_bits, group_size,
                                       _ptr(workspace), workspace_nbytes, _stream_handle(stream))
     elif bias is not None:
@@ -226,17 +229,18 @@ def prepacked_workspace_bytes(m, n, k, weight_bits=8, group_size=0, which=AUTO):
 
 
 def gemm_prepacked(c, a, packed_b, scale, m, n, k, lda=None, ldc=None, weight_bits=8, group_size=0, bias=None, workspace=None,
-                   workspace_nbytes=None, stream=None, which=AUTO, check=True, residual=None, ldr=None):
+                   workspace_nbytes=None, stream=None, which=AUTO, check=True, residual=None, ldr=None, activation=ACT_NONE):
     """C = A x dequant(B, scale) (+ bias) with B in the packed order, through bfaintb_gemm_prepacked_ex; with a residual
     (AUTO variant only) through bfaintb_gemm_prepacked_fused."""
     if workspace_nbytes is None:
         workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
-    if residual is not None:
+    if residual is not None or activation != ACT_NONE:
         if which != AUTO:
             raise ValueError("bfaintb_gemm_prepacked_fused takes no forced variant")
-        ep = _epilogue(bias, residual, ldr, n)
+        ep = _epilogue(bias, residual, ldr, n, activation)
+        out_n = n // 2 if activation == ACT_SILU_GATE else n
         rc = lib().bfaintb_gemm_prepacked_fused(_ptr(c), _ptr(a), _ptr(packed_b), _ptr(scale), C.byref(ep), m, n, k,
-                                                k if lda is None else lda, n if ldc is None else ldc, weight_bits, group_size,
+                                                k if lda is None else lda, out_n if ldc is None else ldc, weight_bits, group_size,
                                                 _ptr(workspace), workspace_nbytes, _stream_handle(stream))
         if rc and check:
             raise BfaintbError(rc, "bfaintb_gemm_prepacked_fused")

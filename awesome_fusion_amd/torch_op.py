@@ -6,8 +6,8 @@ forward pass: activations A [m, k], weights B [k, n], per-output-channel scale, 
 (/root/reference/bfAintBGemm/bfAintBGemm.cc:17-28,119-133).  This module lets such a layer call the
 library:
 
-    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size, bias=None, residual=None) -> c
-    torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, scale, weight_bits, group_size, bias=None, residual=None) -> c
+    torch.ops.awesome_fusion.bfaintb_gemm(a, b, scale, weight_bits, group_size, bias=None, residual=None, activation=0) -> c
+    torch.ops.awesome_fusion.bfaintb_gemm_prepacked(a, packed, scale, weight_bits, group_size, bias=None, residual=None, activation=0) -> c
 
 ``a`` bf16 [m, k] (row stride a multiple of 8 elements), ``b`` uint8 [k, n] (8-bit, excess-128) or
 [k, n/2] (4-bit, excess-8, even column in the low nibble), ``scale`` bf16 [groups, n], ``bias`` bf16 [n] and
@@ -61,6 +61,14 @@ def _check(a, b, scale, weight_bits, group_size, bias=None):
     return a.shape[0], n, k
 
 
+def _out_cols(n, activation):
+    """Columns of the output: n, or n / 2 for the SiLU-gate epilogue (activation = 1: columns 2j and 2j+1 of the weights
+    are the gate and up projections of output column j)."""
+    if activation not in (0, 1):
+        raise ValueError("bfaintb_gemm: activation must be 0 (none) or 1 (SiLU gate)")
+    return n // 2 if activation == 1 else n
+
+
 def _check_residual(residual, m, n):
     if residual is None:
         return None
@@ -71,9 +79,10 @@ def _check_residual(residual, m, n):
 
 @torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm", mutates_args=())
 def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
-                 bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None, activation: int = 0) -> torch.Tensor:
     m, n, k = _check(a, b, scale, weight_bits, group_size, bias)
-    residual = _check_residual(residual, m, n)
+    n_out = _out_cols(n, activation)
+    residual = _check_residual(residual, m, n_out)
     if not a.is_cuda:
         raise RuntimeError("bfaintb_gemm runs on the GPU only (no CPU implementation)")
     if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
@@ -82,31 +91,33 @@ def bfaintb_gemm(a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, weight_b
     scale = scale.contiguous()
     if bias is not None:
         bias = bias.contiguous()
-    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    c = torch.empty((m, n_out), dtype=torch.bfloat16, device=a.device)
     if m == 0 or n == 0:
         return c
     with torch.cuda.device(a.device):
         need = _workspace_bytes(m, n, k, weight_bits, group_size)
         ws = _workspace(a.device, need)
         _gemm(c, a, b, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, workspace=ws,
-              workspace_nbytes=0 if ws is None else ws.numel(), bias=bias, residual=residual)
+              workspace_nbytes=0 if ws is None else ws.numel(), bias=bias, residual=residual, activation=activation)
     return c
 
 
 @bfaintb_gemm.register_fake
-def _(a, b, scale, weight_bits, group_size, bias=None, residual=None):
+def _(a, b, scale, weight_bits, group_size, bias=None, residual=None, activation=0):
     m, n, _k = _check(a, b, scale, weight_bits, group_size, bias)
-    _check_residual(residual, m, n)
-    return a.new_empty((m, n))
+    _check_residual(residual, m, _out_cols(n, activation))
+    return a.new_empty((m, _out_cols(n, activation)))
 
 
 @torch.library.custom_op(f"{_LIB_NAME}::bfaintb_gemm_prepacked", mutates_args=())
 def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, weight_bits: int, group_size: int,
-                           bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
+                           activation: int = 0) -> torch.Tensor:
     """The same product with the weights in the library's pre-packed order (``prepack_weight``): ``packed`` is a flat
     uint8 tensor of k * n * weight_bits / 8 bytes, n is taken from ``scale``."""
     m, n, k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
-    residual = _check_residual(residual, m, n)
+    n_out = _out_cols(n, activation)
+    residual = _check_residual(residual, m, n_out)
     if not a.is_cuda:
         raise RuntimeError("bfaintb_gemm_prepacked runs on the GPU only (no CPU implementation)")
     if a.stride(1) != 1 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
@@ -115,13 +126,13 @@ def bfaintb_gemm_prepacked(a: torch.Tensor, packed: torch.Tensor, scale: torch.T
     scale = scale.contiguous()
     if bias is not None:
         bias = bias.contiguous()
-    c = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    c = torch.empty((m, n_out), dtype=torch.bfloat16, device=a.device)
     if m == 0 or n == 0:
         return c
     with torch.cuda.device(a.device):
         ws = _workspace(a.device, _prepacked_workspace_bytes(m, n, k, weight_bits, group_size))
         _gemm_prepacked(c, a, packed, scale, m, n, k, lda=a.stride(0), weight_bits=weight_bits, group_size=group_size, bias=bias,
-                        workspace=ws, residual=residual)
+                        workspace=ws, residual=residual, activation=activation)
     return c
 
 
@@ -142,10 +153,10 @@ def _check_prepacked(a, packed, scale, weight_bits, group_size, bias=None):
 
 
 @bfaintb_gemm_prepacked.register_fake
-def _(a, packed, scale, weight_bits, group_size, bias=None, residual=None):
+def _(a, packed, scale, weight_bits, group_size, bias=None, residual=None, activation=0):
     m, n, _k = _check_prepacked(a, packed, scale, weight_bits, group_size, bias)
-    _check_residual(residual, m, n)
-    return a.new_empty((m, n))
+    _check_residual(residual, m, _out_cols(n, activation))
+    return a.new_empty((m, _out_cols(n, activation)))
 
 
 def prepack_weight(b, weight_bits=8):

@@ -103,10 +103,16 @@ BFAINTB_API int bfaintb_gemm_bias(void* c, const void* a, const void* b, const v
 
 /*
  * The GEMM with a fused epilogue, described by a struct so that it can grow:
- *     C[m,n] = bf16_rne( sum_k A[m,k]*W[k,n]  + bias[n]  + residual[m,n] )
- * each term that is present added in fp32, in this order, before the one rounding.  bias: bf16 [n]; residual: bf16
- * [m, ldr] (ldr in elements, >= n, a multiple of 8); both 16-byte aligned; either may be NULL; epilogue == NULL is
- * bfaintb_gemm.  `reserved` must be 0.  The reference kernel stores the bare sums (bf16gemm_kernel_gfx90a.s:594-630);
+ *     activation == BFAINTB_ACT_NONE:
+ *         C[m,n] = bf16_rne( sum_k A[m,k]*W[k,n]  + bias[n]  + residual[m,n] )
+ *     activation == BFAINTB_ACT_SILU_GATE (the gated MLP of LLaMA-style models: gate and up projections in one GEMM):
+ *         S[m,c] = sum_k A[m,k]*W[k,c] + bias[c]          for the n columns of B, scale and bias, where column 2j is
+ *                                                         "gate" and column 2j+1 is "up" of output column j;
+ *         C[m,j] = bf16_rne( silu(S[m,2j]) * S[m,2j+1] + residual[m,j] ),   silu(x) = x / (1 + exp(-x)),   j < n/2
+ *         (C and residual have n/2 columns: ldc, ldr >= n/2).
+ * Each term that is present is added in fp32, in this order, before the one rounding.  bias: bf16 [n]; residual: bf16
+ * [m, ldr] (ldr in elements, a multiple of 8); both 16-byte aligned; either may be NULL; epilogue == NULL is
+ * bfaintb_gemm.  The reference kernel stores the bare sums (bf16gemm_kernel_gfx90a.s:594-630);
  * these are the first epilogues of the reference's stated purpose, "gemm fusion for llm" (README.md:2): a linear layer's
  * bias and a transformer block's residual connection, without a second pass over C.  The residual may alias c when
  * ldr == ldc (every element is read by the thread that then writes it).
@@ -115,8 +121,10 @@ typedef struct bfaintb_epilogue {
     const void* bias;
     const void* residual;
     uint32_t ldr;
-    uint32_t reserved;
+    uint32_t activation; /* BFAINTB_ACT_* */
 } bfaintb_epilogue;
+#define BFAINTB_ACT_NONE 0u
+#define BFAINTB_ACT_SILU_GATE 1u
 BFAINTB_API int bfaintb_gemm_fused(void* c, const void* a, const void* b, const void* scale, const bfaintb_epilogue* epilogue, uint32_t m,
                        uint32_t n, uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size,
                        void* workspace, size_t workspace_bytes, void* stream);

@@ -95,7 +95,7 @@ class Workspace:
 _ws = Workspace()
 
 
-def run_gemm(p, which=0, force_split_k=0, lda=None, ldb=None, ldc=None, a_dev=None, b_dev=None, s_dev=None, c_fill=None):
+def run_gemm(p, which=0, force_split_k=0, lda=None, ldb=None, ldc=None, a_dev=None, b_dev=None, s_dev=None, c_fill=None, activation=0):
     """Runs the library on Problem p; returns C as uint16 bits [m, ldc or n]."""
     import torch
     import awesome_fusion_amd as af
@@ -103,13 +103,13 @@ def run_gemm(p, which=0, force_split_k=0, lda=None, ldb=None, ldc=None, a_dev=No
     a_dev = to_dev(p.a_bf) if a_dev is None else a_dev
     b_dev = to_dev(p.b_bytes) if b_dev is None else b_dev
     s_dev = to_dev(p.s_bf) if s_dev is None else s_dev
-    ldc_ = n if ldc is None else ldc
+    ldc_ = (n // 2 if activation else n) if ldc is None else ldc
     c_dev = torch.full((m, ldc_), 0x7FC0 if c_fill is None else c_fill, dtype=torch.int16, device="cuda")
     ws = _ws.get(af.workspace_bytes(m, n, k, p.bits, p.group_size, which, force_split_k))
     bias_dev = None if p.bias_bf is None else to_dev(p.bias_bf)
     res_dev = None if p.residual_bf is None else to_dev(p.residual_bf)
     af.gemm(c_dev, a_dev, b_dev, s_dev, m, n, k, lda, ldb, ldc, p.bits, p.group_size, ws, None, None, which, force_split_k,
-            bias=bias_dev, residual=res_dev)
+            bias=bias_dev, residual=res_dev, activation=activation)
     torch.cuda.synchronize()
     return from_dev_u16(c_dev)
 
@@ -164,3 +164,37 @@ def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
                                           f"{c_ref[i, j]!r}: off by {abs(g - exact):.3e} > {tol:.3e}"
     ok_ulps = np.delete(ulps, bad)
     return (float(ok_ulps.max()) if ok_ulps.size else 0.0), len(bad)
+
+
+def gated_reference(p, rows=None, threads=8):
+    """fp64 silu(gate) * up (+ residual) from the oracle's fp32 sums (+ bias): columns (2j, 2j+1) of the problem are
+    (gate, up) of output column j.  Also returns the tolerance that goes with it: 2 bf16 ULP of the result plus what
+    the fp32 summation noise of either sum (sqrt(K) * 2^-24 * sum_k |a_k w_k|) can move it by, plus 4e-6 relative
+    for the device's fast exponential and reciprocal, plus an absolute floor of 1e-30 * (1 + |gate * up|): the hardware's
+    exponential and reciprocal flush subnormal results, so silu of a gate below about -87 comes out as zero where the
+    exact value is of the order of 1e-36."""
+    a = p.a_bf if rows is None else p.a_bf[rows]
+    s_ref = oracle.gemm_bf16_rows(a, p.w_bf, threads=threads)
+    if p.bias_bf is not None:
+        s_ref = (s_ref + widen(p.bias_bf)[None, :]).astype(np.float32)
+    absum = oracle.gemm_bf16_rows(a & 0x7FFF, p.w_bf & 0x7FFF, threads=threads).astype(np.float64)
+    noise = np.sqrt(p.k) * 2.0 ** -24 * absum + np.abs(s_ref) * 2.0 ** -23
+    g, u = s_ref[:, 0::2].astype(np.float64), s_ref[:, 1::2].astype(np.float64)
+    sig = 1.0 / (1.0 + np.exp(-g))
+    out = g * sig * u
+    dsilu = sig * (1.0 + g * (1.0 - sig))
+    moved = np.abs(dsilu * u) * noise[:, 0::2] + np.abs(g * sig) * noise[:, 1::2]
+    if p.residual_bf is not None:
+        out = out + widen(p.residual_bf if rows is None else p.residual_bf[rows]).astype(np.float64)
+    _, e = np.frexp(np.abs(out))
+    ulp = np.ldexp(1.0, np.maximum(e - 1, -126) - 7)
+    return out, 2.0 * ulp + 1.1 * moved + 4e-6 * np.abs(out) + 1e-30 * (1.0 + np.abs(g * u))
+
+
+def assert_close_gated(p, c_bits, what, rows=None, threads=8):
+    out, tol = gated_reference(p, rows, threads)
+    got = widen(np.asarray(c_bits, np.uint16)).astype(np.float64)
+    assert got.shape == out.shape, f"{what}: shape {got.shape} against {out.shape}"
+    bad = np.abs(got - out) > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {out.size} gated outputs off; worst {np.max(np.abs(got - out) / tol):.2f} x tolerance"
+    return float(np.max(np.abs(got - out) / tol))

@@ -75,6 +75,9 @@ def test_rejects_bad_arguments_without_launching():
     assert rc(bias=P + 2) == -4               # bias must be 16-byte aligned too
     assert rc(residual=P + 2) == -4           # and the residual
     assert rc(residual=P, ldr=64) == -3       # ldr < n
+    assert rc(activation=7) == -5             # unknown activation
+    assert rc(activation=af.ACT_SILU_GATE, ldc=56) == -3   # gated C has n/2 = 64 columns
+    assert rc(activation=af.ACT_SILU_GATE, residual=P, ldr=56) == -3
     assert rc(residual=P, ldr=132) == -3      # rows of the residual would lose 16-byte alignment
     for code in (-1, -2, -3, -4, -5, -6, -7):
         assert len(af.error_string(code)) > 10

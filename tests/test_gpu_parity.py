@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Problem, assert_close_ulp, from_dev_u16, run_gemm, to_dev, widen
+from helpers import Problem, assert_close_gated, assert_close_ulp, from_dev_u16, run_gemm, to_dev, widen
 
 pytestmark = pytest.mark.gpu
 
@@ -266,6 +266,62 @@ def test_residual_closed_forms(af):
     q.residual_bf = np.zeros_like(q.residual_bf)
     got, ref = run_gemm(q), run_gemm(base)
     assert np.array_equal(got & 0x7FFF, ref & 0x7FFF) and np.all((got == ref) | ((ref & 0x7FFF) == 0))  # up to the sign of zero
+
+
+GATED_SHAPES = [
+    (1, 4096, 4096, 8, 0),      # decode, split-K
+    (7, 544, 1024, 4, 128),     # decode, 4-bit
+    (24, 288, 512, 8, 0),       # decode, no split
+    (80, 1056, 2048, 8, 64),    # row-blocked decode family
+    (4200, 288, 256, 8, 0),     # tiled kernel, ragged rows and columns, half tiles
+    (4200, 544, 256, 4, 128),   # tiled kernel, 4-bit
+]
+
+
+def gated_problem(m, n, k, bits, group, seed):
+    # sums of a few units, so that silu is exercised on both sides of zero and in its curved part
+    return Problem(m, n, k, bits, group, seed=seed, scale_lo=0.002, scale_hi=0.02 if bits == 8 else 0.2)
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", GATED_SHAPES)
+def test_silu_gate_epilogue(af, m, n, k, bits, group):
+    """C[m, j] = bf16(silu(S[m, 2j]) * S[m, 2j+1] (+ residual)), S = A.W + bias: against fp64 arithmetic on the oracle's
+    fp32 sums, with the tolerance gated_reference states."""
+    p = gated_problem(m, n, k, bits, group, seed=m + k)
+    c = run_gemm(p, activation=af.ACT_SILU_GATE)
+    assert c.shape == (m, n // 2)
+    assert_close_gated(p, c, f"gated {m}x{n}x{k}")
+    p.with_bias()
+    p.residual_bf = oracle.f32_to_bf16_rne(np.random.default_rng(3).uniform(-2, 2, size=(m, n // 2)).astype(np.float32))
+    worst = assert_close_gated(p, run_gemm(p, activation=af.ACT_SILU_GATE), f"gated + bias + residual {m}x{n}x{k}")
+    print(f"gated {m}x{n}x{k}: worst {worst:.2f} x tolerance")
+
+
+def test_silu_gate_closed_forms(af):
+    """What the mathematics fixes, independent of the oracle's formula: with zero up-weights and an up-bias of 1 the output
+    is silu(gate) (checked against torch's own silu on exactly known gates); a zero gate gives 0; a large gate lets the
+    up value through; a very negative one gives 0."""
+    import torch
+    m, n, k = 8, 32, 64
+    p = Problem(m, n, k, 8, 0, seed=1)
+    gates = np.array([-30.0, -4.0, -1.0, -0.25, 0.0, 0.5, 2.0, 40.0], np.float32)
+    a = np.zeros((m, k), np.float32)
+    a[:, 0] = gates                                   # A[i, 0] = gate_i, everything else 0
+    p.a_bf = oracle.f32_to_bf16_rne(a)
+    q = np.zeros((k, n), np.int8)
+    q[0, 0::2] = 64                                   # gate columns: W[0, 2j] = 64 * (1/64) = 1, so S[i, 2j] = gate_i
+    p.q = q
+    p.b_bytes = oracle.mem_transfer_int8(q.astype(np.float32))
+    p.s_bf = oracle.f32_to_bf16_rne(np.full((1, n), 1.0 / 64, np.float32))
+    p._w = None
+    bias = np.zeros(n, np.float32)
+    bias[1::2] = 1.0                                  # up columns: S[i, 2j+1] = 0 + 1
+    p.bias_bf = oracle.f32_to_bf16_rne(bias)
+    c = widen(run_gemm(p, activation=af.ACT_SILU_GATE))
+    want = torch.nn.functional.silu(torch.from_numpy(gates)).to(torch.bfloat16).float().numpy()
+    for j in range(n // 2):
+        assert np.allclose(c[:, j], want, rtol=2 ** -7, atol=1e-12), (c[:, j], want)
+    assert np.all(c[4] == 0.0) and np.all(np.abs(c[0]) < 1e-11) and np.all(c[7] == 40.0)
 
 
 def test_row_permutation_permutes_output(af):

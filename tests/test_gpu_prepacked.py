@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Problem, Workspace, assert_close_ulp, from_dev_u16, to_dev
+from helpers import Problem, Workspace, assert_close_gated, assert_close_ulp, from_dev_u16, to_dev
 
 _ws = Workspace()
 
@@ -28,16 +28,16 @@ def packed_on_device(af, p):
     return pk
 
 
-def run_prepacked(af, p, which=0, pk=None, ldc=None):
+def run_prepacked(af, p, which=0, pk=None, ldc=None, activation=0):
     import torch
     pk = packed_on_device(af, p) if pk is None else pk
-    ldc_ = p.n if ldc is None else ldc
+    ldc_ = (p.n // 2 if activation else p.n) if ldc is None else ldc
     c = torch.full((p.m, ldc_), 0x7FC0, dtype=torch.int16, device="cuda")
     bias = None if p.bias_bf is None else to_dev(p.bias_bf)
     ws = _ws.get(af.prepacked_workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size, which))
     res = None if p.residual_bf is None else to_dev(p.residual_bf)
     af.gemm_prepacked(c, to_dev(p.a_bf), pk, to_dev(p.s_bf), p.m, p.n, p.k, ldc=ldc, weight_bits=p.bits, group_size=p.group_size,
-                      bias=bias, workspace=ws, which=which, residual=res)
+                      bias=bias, workspace=ws, which=which, residual=res, activation=activation)
     torch.cuda.synchronize()
     return from_dev_u16(c)
 
@@ -176,6 +176,21 @@ def test_fused_residual(af, m, n, k, bits, group):
     assert_close_ulp(p, run_prepacked(af, p), f"packed residual {m}x{n}x{k}")
     p.with_bias()
     assert_close_ulp(p, run_prepacked(af, p), f"packed bias + residual {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (1, 4096, 4096, 8, 0), (20, 544, 1024, 4, 128),    # slab kernel
+    (80, 1056, 2048, 8, 64), (64, 256, 4096, 4, 128),   # row-blocked family, without and with a split along k
+    (4200, 288, 256, 8, 0), (4200, 544, 256, 4, 128),   # tiled kernel over packed weights
+])
+def test_silu_gate_epilogue(af, m, n, k, bits, group):
+    p = Problem(m, n, k, bits, group, seed=m + k, scale_lo=0.002, scale_hi=0.02 if bits == 8 else 0.2)
+    c = run_prepacked(af, p, activation=af.ACT_SILU_GATE)
+    assert c.shape == (m, n // 2)
+    assert_close_gated(p, c, f"packed gated {m}x{n}x{k}")
+    p.with_bias()
+    p.residual_bf = oracle.f32_to_bf16_rne(np.random.default_rng(3).uniform(-2, 2, size=(m, n // 2)).astype(np.float32))
+    assert_close_gated(p, run_prepacked(af, p, activation=af.ACT_SILU_GATE), f"packed gated + bias + residual {m}x{n}x{k}")
 
 
 def test_output_stride_and_padding(af):

@@ -141,3 +141,30 @@ def test_quant_linear_residual_is_added_before_the_rounding():
     out = torch.ops.awesome_fusion.bfaintb_gemm(torch.zeros((6, 512), dtype=torch.bfloat16, device="meta"), ql.qweight.to("meta") if not ql.prepacked else torch.zeros((512, 256), dtype=torch.uint8, device="meta"),
                                                 ql.scales.to("meta"), 8, 0, None, torch.zeros((6, 256), dtype=torch.bfloat16, device="meta"))
     assert out.shape == (6, 256)
+
+
+def test_gated_operator_infers_half_width():
+    a, b, s_, bits, g = _args(5, 64, 128, 8, 0, device="meta")
+    out = torch.ops.awesome_fusion.bfaintb_gemm(a, b, s_, bits, g, None, None, 1)
+    assert out.shape == (5, 32)
+    with pytest.raises(Exception):
+        torch.ops.awesome_fusion.bfaintb_gemm(a, b, s_, bits, g, None, None, 2)
+
+
+@pytest.mark.gpu
+def test_gated_mlp_against_torch():
+    """A LLaMA-style gated MLP front half, y = silu(x Wg) * (x Wu), as one GEMM over interleaved (gate, up) columns."""
+    torch.manual_seed(3)
+    k, n = 512, 256
+    wg, wu = torch.randn((n, k)) * 0.05, torch.randn((n, k)) * 0.05
+    w = torch.stack((wg, wu), dim=1).reshape(2 * n, k)            # rows 2j, 2j+1 = gate_j, up_j  ->  columns of B
+    b, s = top.quantize_weight(w, 8, 0)
+    x = torch.randn((9, k)).to(torch.bfloat16)
+    y = torch.ops.awesome_fusion.bfaintb_gemm(x.cuda(), b.cuda(), s.cuda(), 8, 0, None, None, 1)
+    assert y.shape == (9, n)
+    wq = ((b.to(torch.int16) - 128).float() * s.float()).to(torch.bfloat16).float()   # [k, 2n]
+    sums = x.float() @ wq
+    ref = torch.nn.functional.silu(sums[:, 0::2]) * sums[:, 1::2]
+    assert torch.allclose(y.float().cpu(), ref, rtol=2e-2, atol=2e-3)
+    yp = torch.ops.awesome_fusion.bfaintb_gemm_prepacked(x.cuda(), top.prepack_weight(b.cuda(), 8), s.cuda(), 8, 0, None, None, 1)
+    assert torch.allclose(yp.float(), y.float(), rtol=2e-2, atol=2e-3)
