@@ -174,6 +174,59 @@ def time_fused_epilogue(af, w, steps, warmup):
     return out[0], out[1]
 
 
+def time_gated(af, w, steps, warmup, packed):
+    """(fused_ms, unfused_ms) for silu(A.Wg) * (A.Wu) with interleaved (gate, up) columns in w: one launch with the
+    SiLU-gate epilogue, against the plain GEMM followed by torch's silu and multiply on the strided halves."""
+    import torch
+    ws = w.workspace(af)
+    nb = len(w.b)
+    out = torch.zeros((w.m, w.n // 2), dtype=torch.bfloat16, device="cuda")
+    if packed:
+        pks = []
+        for i in range(nb):
+            pk = torch.empty(af.prepack_bytes(w.n, w.k, w.bits), dtype=torch.uint8, device="cuda")
+            af.prepack(pk, w.b[i], w.n, w.k, weight_bits=w.bits)
+            pks.append(pk)
+        need = af.prepacked_workspace_bytes(w.m, w.n, w.k, w.bits, w.group)
+        pws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        af.workspace_init(pws)
+
+    def plain(i, c, act):
+        if packed:
+            af.gemm_prepacked(c, w.a, pks[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=pws, activation=act)
+        else:
+            af.gemm(c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws, activation=act)
+
+    def fused(i):
+        plain(i, out, af.ACT_SILU_GATE)
+
+    def unfused(i):
+        plain(i, w.c, af.ACT_NONE)
+        torch.mul(torch.nn.functional.silu(w.c[:, 0::2]), w.c[:, 1::2], out=out)
+
+    res = []
+    for launch in (fused, unfused):
+        for i in range(warmup):
+            launch(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(steps):
+                launch(i)
+        g.replay()
+        torch.cuda.synchronize()
+        ev = []
+        for _ in range(REPLAYS):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            ev.append(e0.elapsed_time(e1) / steps)
+        res.append(sorted(ev)[REPLAYS // 2])
+    return res[0], res[1]
+
+
 def time_read_ceiling(af, w, steps, warmup):
     """The same rotation of B copies through a kernel that only fetches the bytes."""
     import torch
@@ -427,6 +480,16 @@ def main():
             if m == 1:
                 pk_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True, packed=True)
                 sweep.append({"workload": w.name + "_prepacked", **roofline_entry(w, pk_ms, "hbm")})
+            del w
+            torch.cuda.empty_cache()
+        # gated MLP, LLaMA-7B shape: 2 x 11008 interleaved (gate, up) columns over k = 4096
+        for m in (1, 2048):
+            w = Workload(f"gated_mlp_m{m}_n22016_k4096_int8_perchannel", m, 22016, 4096, copies=8 if m == 1 else 1)
+            for packed in (False, True):
+                f_ms, u_ms = time_gated(af, w, min(K, 100) if m == 1 else 10, min(W, 10), packed)
+                sweep.append({"workload": w.name + ("_prepacked" if packed else ""), "fused_kernel_us": round(f_ms * 1e3, 3),
+                              "gemm_then_silu_mul_us": round(u_ms * 1e3, 3),
+                              "note": "silu(A.Wgate) * (A.Wup): one launch with the SiLU-gate epilogue against GEMM + torch silu, mul"})
             del w
             torch.cuda.empty_cache()
         out_extra["sweep"] = sweep
