@@ -13,6 +13,8 @@ from .gemm import (  # noqa: F401
     save_packed,
     DECODE,
     PREFILL,
+    PREFILL_128,
+    PREFILL_256,
     AUTO,
     ACT_NONE,
     ACT_SILU_GATE,
@@ -23,6 +25,7 @@ from .gemm import (  # noqa: F401
     gemm_prepacked,
     kernel_name,
     lib,
+    prefill_tile,
     prepack,
     prepack_bytes,
     prepacked_variant,

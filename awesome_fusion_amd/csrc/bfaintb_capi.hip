@@ -21,6 +21,7 @@ hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k,
                        hipStream_t stream);
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
 }  // namespace bfaintb
 
@@ -84,15 +85,44 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
     const double waves = row_blocks * col_blocks * pl.splits * pl.waves;
     const double busy = waves >= 1024.0 ? 1.0 : waves / 1024.0;
     const double cycles_per_weight = 10.0 + 6.25 * pl.mb;
-    const double compute = row_blocks * weights * cycles_per_weight / 65536.0 / 2000.0 / busy;
+    // workgroups beyond one per CU share a CU's arithmetic: the last, partly filled round costs a whole one
+    // (measured at n = k = 4096, 64-row blocks: m = 512 -> 256 workgroups, 35 us; m = 640 -> 320 workgroups, 61 us)
+    const double wgs = row_blocks * col_blocks * pl.splits;
+    const double ragged = wgs > 256.0 ? (double)(uint64_t)((wgs + 255.0) / 256.0) * 256.0 / wgs : 1.0;
+    const double compute = row_blocks * weights * cycles_per_weight / 65536.0 / 2000.0 / busy * ragged;
     const double stream = weights * bits / 8.0 * (1.0 + 0.3 * (row_blocks - 1.0)) / 3.5e6 / busy;
     const double partial = pl.splits > 1 ? 3.0 + 12.0 * (pl.splits - 1.0) * m * n / 1.5e6 : 0.0;
     return 5.0 + (compute > stream ? compute : stream) + partial;
 }
 
-// Rough time of the prefill kernel: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of k.
+// The tiled variant runs 128x128 tiles while those fit one per CU (at most 256 of them): four times the workgroups of
+// 256x256 tiles, each with a quarter of the work per K-step.  Measured against the large tiles (8-bit, k = 4096, us):
+// m x n = 256 x 4096: 48 / 59, 1024 x 4096: 58 / 66, 512 x 8192 (4-bit, k = 8192): 112 / 137; with more tiles the
+// large ones win (1536 x 4096: 81 / 72, 512 x 11008: 80 / 68).
+static bool prefill_small_tiles(uint32_t m, uint32_t n)
+{
+    return (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u) <= 256u;
+}
+
+static bool is_prefill(int v)
+{
+    return v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256 || v == BFAINTB_VARIANT_PREFILL_128;
+}
+
+// tile size of a tiled-variant launch: forced, or by shape
+static bool use_small_tiles(int v, uint32_t m, uint32_t n)
+{
+    return v == BFAINTB_VARIANT_PREFILL_128 || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n));
+}
+
+// Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
+// k.  Small tiles: a K-step takes 0.7 us on an empty machine and 0.9 us with a workgroup on every CU.
 static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
 {
+    if (prefill_small_tiles(m, n)) {
+        const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
+        return 4.0 + (k / 64.0) * (0.70 + 0.0008 * tiles);
+    }
     const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
     const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
     return 4.0 + rounds * (k / 64.0) * 1.33;
@@ -177,7 +207,7 @@ int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
         return decode_family_estimate_us(m, n, k, bits, pl) * 1.1 < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     }
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
-    if (variant == BFAINTB_VARIANT_PREFILL) return variant;
+    if (is_prefill(variant)) return variant;
     return BFAINTB_ERR_BAD_VARIANT;
 }
 
@@ -313,11 +343,13 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.splits = 1;
     hipStream_t st = static_cast<hipStream_t>(stream);
 
-    if (v == BFAINTB_VARIANT_PREFILL) {
+    if (is_prefill(v)) {
         // the prefill kernel addresses B and a 256-row panel of A through 32-bit buffer extents
         if ((uint64_t)k * p.ldb_bytes >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
 #ifdef BFAINTB_TRACE
         p.trace = static_cast<unsigned long long*>(workspace);  // per-quarter cycle totals, 8 words per wave
+#else
+        if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
 #endif
         return (int)bfaintb::launch_prefill(p, weight_bits, st);
     }
@@ -419,15 +451,12 @@ int bfaintb_unpack(void* b, const void* packed, uint32_t n, uint32_t k, uint32_t
 static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
-    if (variant == BFAINTB_VARIANT_PREFILL) return variant;
+    if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
     if (m <= kPackedSlabMaxM) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = decode_plan(m, n, k, bits, 0);
-    // a lightly loaded machine runs the tiled kernel's steps faster (measured 57 us at m = 256 and 512, n = k = 4096)
-    const uint32_t tiles = ((m + 255u) / 256u) * ((n + 255u) / 256u);
-    const double prefill_us = tiles <= 64u ? 4.0 + (k / 64.0) * 0.85 : prefill_estimate_us(m, n, k);
-    return decode_family_estimate_us(m, n, k, bits, pl) * 1.1 < prefill_us ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return decode_family_estimate_us(m, n, k, bits, pl) * 1.1 < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
@@ -494,10 +523,11 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
     p.lds = n;
     p.group_size = group_size;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (v == BFAINTB_VARIANT_PREFILL) {
+    if (is_prefill(v)) {
         // a tile's 16 column blocks and a 256-row panel of A are addressed through 32-bit buffer extents
         if ((uint64_t)k * 256u * (uint32_t)weight_bits / 8u >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31))
             return BFAINTB_ERR_BAD_SHAPE;
+        if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st);
     }
     if (m > kPackedSlabMaxM) {
@@ -614,12 +644,15 @@ int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream)
     return (int)bfaintb::launch_probe_read(src, bytes, sink, static_cast<hipStream_t>(stream));
 }
 
+uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n) { return prefill_small_tiles(m, n) ? 128u : 256u; }
+
 const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m)
 {
     int v = variant;
     if (v == BFAINTB_VARIANT_AUTO) v = m <= kDecodeAutoMaxM ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     if (v == BFAINTB_VARIANT_DECODE) return "bfaintb_decode_kernel";
-    if (v == BFAINTB_VARIANT_PREFILL) return "bfaintb_prefill_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256) return "bfaintb_prefill_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL_128) return "bfaintb_prefill128_kernel";
     (void)weight_bits;
     (void)group_size;
     return "";

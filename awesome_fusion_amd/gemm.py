@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = os.path.join(_HERE, "libbfaintb_gemm.so")
 
 AUTO, DECODE, PREFILL = 0, 1, 2
+PREFILL_256, PREFILL_128 = 3, 4  # the tiled variant with its tile size forced (tests, tuning)
 ACT_NONE, ACT_SILU_GATE = 0, 1
 
 
@@ -109,6 +110,8 @@ def lib():
         L.bfaintb_dequant.argtypes = [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
         L.bfaintb_probe_read.restype = C.c_int
         L.bfaintb_probe_read.argtypes = [_vp, C.c_size_t, _vp, _vp]
+        L.bfaintb_prefill_tile.restype = _u32
+        L.bfaintb_prefill_tile.argtypes = [_u32, _u32]
         L.bfaintb_kernel_name.restype = C.c_char_p
         L.bfaintb_kernel_name.argtypes = [C.c_int, C.c_int, _u32, _u32]
         L.bfaintb_error_string.restype = C.c_char_p
@@ -145,6 +148,11 @@ def variant(m, n, k, weight_bits=8, group_size=0):
 
 def split_k(m, n, k, weight_bits=8, group_size=0):
     return lib().bfaintb_gemm_split_k(m, n, k, weight_bits, group_size)
+
+
+def prefill_tile(m, n):
+    """Tile edge (128 or 256) the PREFILL variant uses for an m x n output."""
+    return lib().bfaintb_prefill_tile(m, n)
 
 
 def kernel_name(m, weight_bits=8, group_size=0, which=AUTO):

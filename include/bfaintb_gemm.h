@@ -33,7 +33,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 102 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 103 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -50,7 +50,10 @@ enum {
 enum {
     BFAINTB_VARIANT_AUTO = 0,   /* decode up to m = 32; beyond, whichever the library estimates faster for (m, n, k) */
     BFAINTB_VARIANT_DECODE = 1, /* split-K weight-streaming kernel (HBM-bound); m > 32 in row blocks; accepts m <= 32768 */
-    BFAINTB_VARIANT_PREFILL = 2 /* 256x256 LDS-tiled MFMA kernel (MFMA-bound) */
+    BFAINTB_VARIANT_PREFILL = 2, /* LDS-tiled MFMA kernels (MFMA-bound): 256x256 tiles, or 128x128 tiles while m x n
+                                  * holds at most 256 of those (the large tiles would leave most CUs idle) */
+    BFAINTB_VARIANT_PREFILL_256 = 3, /* the tiled kernel with 256x256 tiles, whatever the shape (tests, tuning) */
+    BFAINTB_VARIANT_PREFILL_128 = 4  /* the tiled kernel with 128x128 tiles, whatever the shape (tests, tuning) */
 };
 
 /*
@@ -170,7 +173,7 @@ BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
                                                  int variant);
 /* Same with the kernel family forced (BFAINTB_VARIANT_*: DECODE = the slab-streaming kernel up to 48 rows of A and the
- * row-blocked decode family beyond, m <= 32768; PREFILL = the 256x256 tiled kernel reading packed weights), and which of
+ * row-blocked decode family beyond, m <= 32768; PREFILL[_256|_128] = the tiled kernels reading packed weights), and which of
  * the two bfaintb_gemm_prepacked would run. */
 BFAINTB_API int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
                               uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
@@ -204,6 +207,10 @@ BFAINTB_API int bfaintb_packed_header_check(const bfaintb_packed_header* h);
 
 /* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */
 BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
+
+/* Edge of the square tiles BFAINTB_VARIANT_PREFILL runs an m x n output with: 128 while that makes at most 256 tiles
+ * (one per CU), else 256.  Depends only on its arguments. */
+BFAINTB_API uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n);
 
 /* The split-K factor the decode variant would use for a shape (1 for the prefill variant). */
 BFAINTB_API uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);

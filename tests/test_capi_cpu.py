@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
-    assert af.lib().bfaintb_version() == 102
+    assert af.lib().bfaintb_version() == 103
     assert "bfaintb_gemm_bias" in names
 
 
@@ -36,6 +36,14 @@ def test_variant_choice_and_split():
     assert af.variant(512, 28672, 8192, 4, 128) == af.PREFILL
     assert af.variant(4096, 4096, 4096) == af.PREFILL
     assert af.variant(1, 28672, 8192, 4, 128) == af.DECODE
+    # the tiled variant where the row-blocked family's last round would be mostly empty (320 workgroups on 256 CUs)
+    assert af.variant(512, 4096, 4096) == af.DECODE and af.variant(640, 4096, 4096) == af.PREFILL
+    # 128x128 tiles up to one per CU, 256x256 beyond; forced forms are accepted as variants and need no workspace
+    assert af.prefill_tile(1024, 4096) == 128 and af.prefill_tile(1025, 4096) == 256
+    assert af.prefill_tile(128, 28672) == 128 and af.prefill_tile(4096, 4096) == 256 and af.prefill_tile(1, 16) == 128
+    assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128) == 0 == af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_256)
+    assert af.kernel_name(64, which=af.PREFILL_128) == "bfaintb_prefill128_kernel"
+    assert af.kernel_name(64, which=af.PREFILL_256) == af.kernel_name(64, which=af.PREFILL) == "bfaintb_prefill_kernel"
     assert af.split_k(4096, 4096, 4096) == 1
     s = af.split_k(1, 4096, 4096)
     assert 1 < s <= 64 and 4096 % s == 0

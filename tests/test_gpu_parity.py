@@ -42,11 +42,12 @@ def test_dequant_dump_bit_exact(af, bits, group):
 
 
 @pytest.mark.parametrize("bits,group", [(8, 0), (4, 128)])
-@pytest.mark.parametrize("which_m", [("decode", 16), ("decode", 32), ("prefill", 64)])
+@pytest.mark.parametrize("which_m", [("decode", 16), ("decode", 32), ("prefill_256", 64), ("prefill_128", 64)])
 def test_gemm_kernels_dequantise_bit_exact(af, bits, group, which_m):
     """One-hot activations make C[i,:] = W[k_i,:] with nothing to round: the GEMM kernels' own
     in-register dequantisation is observed exactly."""
-    _, m = which_m
+    which, m = which_m
+    which = {"decode": af.DECODE, "prefill_256": af.PREFILL_256, "prefill_128": af.PREFILL_128}[which]
     k, n = 256, 512
     p = Problem(m, n, k, bits, group, seed=7)
     seen = np.zeros(k, bool)
@@ -55,7 +56,7 @@ def test_gemm_kernels_dequantise_bit_exact(af, bits, group, which_m):
         rows = (base + np.arange(m)) % k
         a[np.arange(m), rows] = 1.0
         p.a_bf = oracle.f32_to_bf16_rne(a)
-        c = run_gemm(p)
+        c = run_gemm(p, which=which)
         assert np.array_equal(c, p.w_bf[rows]), f"rows {base}.. differ"
         seen[rows] = True
     assert seen.all()
@@ -147,6 +148,27 @@ def test_ragged_shapes(af, m, n, k, bits, group):
     assert_close_ulp(p, c, f"ragged {m}x{n}x{k} bits={bits}")
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 48, 128), (257, 528, 192), (100, 1040, 320), (300, 272, 448), (1000, 1008, 384), (130, 4112, 256)])
+@pytest.mark.parametrize("bits,group", [(8, 0), (8, 64), (4, 0), (4, 64)])
+@pytest.mark.parametrize("tile", [256, 128])
+def test_tiled_kernels_on_ragged_shapes(af, m, n, k, bits, group, tile):
+    """The tiled variant with either tile size forced: partial tiles in m and n, odd numbers of K-steps, column counts
+    that end inside a 16-column block of a tile."""
+    p = Problem(m, n, k, bits, group, seed=m * 3 + n + tile)
+    assert_close_ulp(p, run_gemm(p, which=af.PREFILL_256 if tile == 256 else af.PREFILL_128), f"tile {tile}: {m}x{n}x{k} bits={bits} g={group}")
+
+
+def test_tiled_variant_picks_its_tile_size_by_shape(af):
+    """PREFILL runs 128x128 tiles while m x n holds at most 256 of them, 256x256 tiles beyond; either way the result
+    meets the oracle and is the forced form's, bit for bit."""
+    for (m, n, tile) in [(1024, 4096, 128), (2048, 2048, 128), (2064, 2048, 256), (1024, 4224, 256)]:
+        assert af.prefill_tile(m, n) == tile
+        p = Problem(m, n, 256, 8, 0, seed=m + n)
+        c = run_gemm(p, which=af.PREFILL)
+        assert_close_ulp(p, c, f"{m}x{n}")
+        assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128 if tile == 128 else af.PREFILL_256)), f"{m}x{n}"
+
+
 @pytest.mark.parametrize("m", [5, 80])
 def test_leading_dimensions_and_untouched_padding(af, m):
     import torch
@@ -233,8 +255,10 @@ def test_fused_bias(af, m, n, k, bits, group):
     (24, 272, 512, 8, 0),       # decode, no split
     (80, 1040, 2048, 8, 64),    # row-blocked decode family
     (300, 272, 192, 8, 0),      # row-blocked family, ragged rows and columns
-    (4200, 272, 256, 8, 0),     # tiled kernel, ragged rows and columns, half tiles
-    (4200, 528, 256, 4, 128),   # tiled kernel, 4-bit
+    (4200, 272, 256, 8, 0),     # tiled kernel (128x128 tiles), ragged rows and columns, half tiles
+    (4200, 528, 256, 4, 128),   # tiled kernel (128x128 tiles), 4-bit
+    (4200, 1040, 128, 8, 0),    # more than 256 small tiles: 256x256 tiles, ragged rows and columns
+    (4200, 1296, 256, 4, 128),  # 256x256 tiles, 4-bit
 ])
 def test_fused_residual(af, m, n, k, bits, group):
     """C = bf16(sum + bias + residual): against the oracle's fp32 sums plus the two fp32 additions, with and without the
@@ -273,8 +297,10 @@ GATED_SHAPES = [
     (7, 544, 1024, 4, 128),     # decode, 4-bit
     (24, 288, 512, 8, 0),       # decode, no split
     (80, 1056, 2048, 8, 64),    # row-blocked decode family
-    (4200, 288, 256, 8, 0),     # tiled kernel, ragged rows and columns, half tiles
-    (4200, 544, 256, 4, 128),   # tiled kernel, 4-bit
+    (4200, 288, 256, 8, 0),     # tiled kernel (128x128 tiles), ragged rows and columns, half tiles
+    (4200, 544, 256, 4, 128),   # tiled kernel (128x128 tiles), 4-bit
+    (4200, 1056, 128, 8, 0),    # more than 256 small tiles: 256x256 tiles
+    (4200, 1312, 256, 4, 128),  # 256x256 tiles, 4-bit
 ]
 
 

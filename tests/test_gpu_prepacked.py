@@ -101,15 +101,21 @@ def test_row_blocked_family_over_packed_weights(af, m, n, k, bits, group):
 @pytest.mark.parametrize("m,n,k,bits,group", [
     (256, 256, 64, 8, 0), (300, 272, 192, 8, 0), (64, 128, 256, 8, 0), (512, 512, 256, 4, 128), (1000, 1008, 384, 4, 0),
     (513, 784, 448, 8, 64), (130, 528, 512, 8, 32), (260, 304, 512, 4, 32), (4160, 256, 256, 8, 0), (2304, 512, 512, 4, 128)])
-def test_tiled_kernel_matches_oracle(af, m, n, k, bits, group):
+@pytest.mark.parametrize("tile", [256, 128])
+def test_tiled_kernel_matches_oracle(af, m, n, k, bits, group, tile):
+    """Both tile sizes of the tiled variant, each forced (left to itself the library runs 128x128 tiles on all of these
+    shapes: none has more than 256 of them)."""
+    which = af.PREFILL_256 if tile == 256 else af.PREFILL_128
     p = Problem(m, n, k, bits, group, seed=m + n + k)
-    assert_close_ulp(p, run_prepacked(af, p, af.PREFILL), f"packed prefill {m}x{n}x{k} b{bits} g{group}")
+    assert_close_ulp(p, run_prepacked(af, p, which), f"packed prefill{tile} {m}x{n}x{k} b{bits} g{group}")
     p.with_bias()
-    assert_close_ulp(p, run_prepacked(af, p, af.PREFILL), f"packed prefill + bias {m}x{n}x{k} b{bits} g{group}")
+    assert_close_ulp(p, run_prepacked(af, p, which), f"packed prefill{tile} + bias {m}x{n}x{k} b{bits} g{group}")
+    if tile == 128:
+        assert np.array_equal(run_prepacked(af, p, which), run_prepacked(af, p, af.PREFILL)), "PREFILL picks 128x128 tiles here"
 
 
 @pytest.mark.parametrize("bits,group", [(8, 0), (4, 128)])
-@pytest.mark.parametrize("which,m", [(1, 16), (1, 32), (1, 64), (2, 64)])
+@pytest.mark.parametrize("which,m", [(1, 16), (1, 32), (1, 64), (3, 64), (4, 64)])
 def test_kernels_dequantise_bit_exact(af, bits, group, which, m):
     """One-hot activations make C[i, :] = W[k_i, :] with nothing to round: the in-register conversion of both
     kernels is observed exactly, against the oracle's dequantised weights."""
@@ -169,7 +175,8 @@ def test_workspace_is_required_where_the_plan_splits_and_left_ready(af):
 @pytest.mark.parametrize("m,n,k,bits,group", [
     (1, 4096, 4096, 8, 0), (20, 528, 1024, 4, 128),   # slab kernel
     (80, 1040, 2048, 8, 64), (64, 256, 4096, 4, 128),  # row-blocked family, without and with a split along k
-    (4200, 272, 256, 8, 0), (4200, 528, 256, 4, 128),  # tiled kernel over packed weights
+    (4200, 272, 256, 8, 0), (4200, 528, 256, 4, 128),  # tiled kernel over packed weights, 128x128 tiles
+    (4200, 1040, 128, 8, 0), (4200, 1296, 256, 4, 128),  # more than 256 of those: 256x256 tiles
 ])
 def test_fused_residual(af, m, n, k, bits, group):
     p = Problem(m, n, k, bits, group, seed=m + k).with_residual()
@@ -181,7 +188,8 @@ def test_fused_residual(af, m, n, k, bits, group):
 @pytest.mark.parametrize("m,n,k,bits,group", [
     (1, 4096, 4096, 8, 0), (20, 544, 1024, 4, 128),    # slab kernel
     (80, 1056, 2048, 8, 64), (64, 256, 4096, 4, 128),   # row-blocked family, without and with a split along k
-    (4200, 288, 256, 8, 0), (4200, 544, 256, 4, 128),   # tiled kernel over packed weights
+    (4200, 288, 256, 8, 0), (4200, 544, 256, 4, 128),   # tiled kernel over packed weights, 128x128 tiles
+    (4200, 1056, 128, 8, 0), (4200, 1312, 256, 4, 128),  # more than 256 of those: 256x256 tiles
 ])
 def test_silu_gate_epilogue(af, m, n, k, bits, group):
     p = Problem(m, n, k, bits, group, seed=m + k, scale_lo=0.002, scale_hi=0.02 if bits == 8 else 0.2)
