@@ -482,6 +482,15 @@ def main():
                 sweep.append({"workload": w.name + "_prepacked", **roofline_entry(w, pk_ms, "hbm")})
             del w
             torch.cuda.empty_cache()
+        # between decode and prefill: what AUTO picks for a few hundred rows of A (row-blocked decode family, then 128x128 tiles)
+        for m in (64, 256, 640, 1024):
+            w = Workload(f"mid_m{m}_n4096_k4096_int8_perchannel", m, 4096, 4096, copies=4)
+            ev_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True)
+            v = af.variant(m, 4096, 4096)
+            sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "mfma"),
+                          "kernel": "row-blocked decode family" if v == af.DECODE else f"tiled, {af.prefill_tile(m, 4096)}x{af.prefill_tile(m, 4096)} tiles"})
+            del w
+            torch.cuda.empty_cache()
         # gated MLP, LLaMA-7B shape: 2 x 11008 interleaved (gate, up) columns over k = 4096
         for m in (1, 2048):
             w = Workload(f"gated_mlp_m{m}_n22016_k4096_int8_perchannel", m, 22016, 4096, copies=8 if m == 1 else 1)
