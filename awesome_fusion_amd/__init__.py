@@ -23,6 +23,7 @@ from .gemm import (  # noqa: F401
     error_string,
     gemm,
     gemm_prepacked,
+    gemm_reference,
     kernel_name,
     lib,
     prefill_tile,

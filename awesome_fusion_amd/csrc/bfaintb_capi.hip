@@ -291,6 +291,8 @@ struct Epilogue {
     const void* residual = nullptr;
     uint32_t ldr = 0;
     uint32_t activation = BFAINTB_ACT_NONE;
+    // not an epilogue but set the same way: the reference kernel's arithmetic (fp32 scales, W and C narrowed by truncation)
+    bool reference_arith = false;
     // columns of C (and of the residual) for n columns of B
     uint32_t out_cols(uint32_t n) const { return activation == BFAINTB_ACT_SILU_GATE ? n / 2u : n; }
 };
@@ -314,6 +316,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     const void* bias = ep.bias;
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
+    if (ep.reference_arith && (weight_bits != 8 || group_size != 0)) return BFAINTB_ERR_UNSUPPORTED;
     e = check_shape(m, n, k);
     if (e) return e;
     if (lda < k || ldb < n || ldc < ep.out_cols(n) || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
@@ -329,6 +332,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.residual = static_cast<const uint16_t*>(ep.residual);
     p.ldr = ep.ldr;
     p.activation = ep.activation;
+    p.reference_arith = ep.reference_arith ? 1u : 0u;
     p.c = static_cast<uint16_t*>(c);
     p.a = static_cast<const uint16_t*>(a);
     p.b = static_cast<const uint8_t*>(b);
@@ -610,6 +614,20 @@ int bfaintb_gemm_fused(void* c, const void* a, const void* b, const void* scale,
     if (e) return e;
     return gemm_impl(c, a, b, scale, ep, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes, stream,
                      BFAINTB_VARIANT_AUTO, 0);
+}
+
+int bfaintb_gemm_reference_ex(void* c, const void* a, const void* b, const float* scale, uint32_t m, uint32_t n, uint32_t k, uint32_t lda,
+                              uint32_t ldb, uint32_t ldc, void* workspace, size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
+{
+    Epilogue ep;
+    ep.reference_arith = true;
+    return gemm_impl(c, a, b, scale, ep, m, n, k, lda, ldb, ldc, 8, 0, workspace, workspace_bytes, stream, variant, split_k);
+}
+
+int bfaintb_gemm_reference(void* c, const void* a, const void* b, const float* scale, uint32_t m, uint32_t n, uint32_t k, uint32_t lda,
+                           uint32_t ldb, uint32_t ldc, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return bfaintb_gemm_reference_ex(c, a, b, scale, m, n, k, lda, ldb, ldc, workspace, workspace_bytes, stream, BFAINTB_VARIANT_AUTO, 0);
 }
 
 int bfaintb_gemm(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,

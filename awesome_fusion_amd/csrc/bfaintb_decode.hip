@@ -78,16 +78,16 @@ __device__ __forceinline__ void prepare_row(uint32_t (&out)[CPL / 4], const uint
     }
 }
 
-template <int BITS, int CPL, int MB, int C>
+template <int BITS, int CPL, int MB, bool REF, int C>
 __device__ __forceinline__ void mac_column(const uint32_t (&rows)[8][CPL / 4], const float (&cs)[CPL], const uint4 (&afrag)[MB],
                                            f32x4_t (&acc)[MB][CPL])
 {
     constexpr int PD = CPL / 4;
     uint4 w;
-    w.x = pack_bf16_rne(value_f32<BITS, C, PD>(rows[0]) * cs[C], value_f32<BITS, C, PD>(rows[1]) * cs[C]);
-    w.y = pack_bf16_rne(value_f32<BITS, C, PD>(rows[2]) * cs[C], value_f32<BITS, C, PD>(rows[3]) * cs[C]);
-    w.z = pack_bf16_rne(value_f32<BITS, C, PD>(rows[4]) * cs[C], value_f32<BITS, C, PD>(rows[5]) * cs[C]);
-    w.w = pack_bf16_rne(value_f32<BITS, C, PD>(rows[6]) * cs[C], value_f32<BITS, C, PD>(rows[7]) * cs[C]);
+    w.x = pack_bf16<REF>(value_f32<BITS, C, PD>(rows[0]) * cs[C], value_f32<BITS, C, PD>(rows[1]) * cs[C]);
+    w.y = pack_bf16<REF>(value_f32<BITS, C, PD>(rows[2]) * cs[C], value_f32<BITS, C, PD>(rows[3]) * cs[C]);
+    w.z = pack_bf16<REF>(value_f32<BITS, C, PD>(rows[4]) * cs[C], value_f32<BITS, C, PD>(rows[5]) * cs[C]);
+    w.w = pack_bf16<REF>(value_f32<BITS, C, PD>(rows[6]) * cs[C], value_f32<BITS, C, PD>(rows[7]) * cs[C]);
     const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, w);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -95,14 +95,14 @@ __device__ __forceinline__ void mac_column(const uint32_t (&rows)[8][CPL / 4], c
     }
 }
 
-template <int BITS, int CPL, int MB, int... Cs>
+template <int BITS, int CPL, int MB, bool REF, int... Cs>
 __device__ __forceinline__ void mac_step(const RawStep<BITS, CPL>& raw, const float (&cs)[CPL], const uint4 (&afrag)[MB],
                                          f32x4_t (&acc)[MB][CPL], std::integer_sequence<int, Cs...>)
 {
     uint32_t rows[8][CPL / 4];
 #pragma unroll
     for (int r = 0; r < 8; ++r) prepare_row<BITS, CPL>(rows[r], raw.d[r]);
-    (mac_column<BITS, CPL, MB, Cs>(rows, cs, afrag, acc), ...);
+    (mac_column<BITS, CPL, MB, REF, Cs>(rows, cs, afrag, acc), ...);
 }
 
 // ---- the same step over weights in the packed order (bfaintb_packed.hip): the workgroup's CPL column blocks of 16 take
@@ -214,7 +214,7 @@ __host__ __device__ inline uint32_t decode_red_floats(uint32_t waves, uint32_t r
 
 // Finishes four neighbouring columns of one row: t += bias[col .. col+3]; then either += residual[row][col .. col+3] and
 // four bf16 outputs at C[row][col ..], or (gated) the two outputs silu(t.x) * t.y and silu(t.z) * t.w, += residual[row]
-// [col/2 ..], at C[row][col/2 ..].  All additions in fp32, one rounding.
+// [col/2 ..], at C[row][col/2 ..].  All additions in fp32, one rounding (a truncation with the reference's arithmetic).
 __device__ __forceinline__ void finish_row4(const GemmParams& p, float4 t, uint32_t row, uint32_t col)
 {
     if (p.bias != nullptr) {
@@ -231,7 +231,7 @@ __device__ __forceinline__ void finish_row4(const GemmParams& p, float4 t, uint3
             o0 += bf16_bits_to_f32(raw & 0xffffu);
             o1 += bf16_bits_to_f32(raw >> 16);
         }
-        *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col / 2u) = pack_bf16_rne(o0, o1);
+        *reinterpret_cast<uint32_t*>(p.c + (size_t)row * p.ldc + col / 2u) = p.reference_arith ? pack_bf16_rtz(o0, o1) : pack_bf16_rne(o0, o1);
         return;
     }
     if (p.residual != nullptr) {
@@ -242,8 +242,8 @@ __device__ __forceinline__ void finish_row4(const GemmParams& p, float4 t, uint3
         t.w += bf16_bits_to_f32(raw.y >> 16);
     }
     uint2 o;
-    o.x = pack_bf16_rne(t.x, t.y);
-    o.y = pack_bf16_rne(t.z, t.w);
+    o.x = p.reference_arith ? pack_bf16_rtz(t.x, t.y) : pack_bf16_rne(t.x, t.y);
+    o.y = p.reference_arith ? pack_bf16_rtz(t.z, t.w) : pack_bf16_rne(t.z, t.w);
     *reinterpret_cast<uint2*>(p.c + (size_t)row * p.ldc + col) = o;
 }
 
@@ -324,9 +324,12 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 
 // PACKED: p.b holds the weights in the packed order; the workgroup's kCols columns are CPL column blocks of 16, and
 // accumulator c of a lane belongs to column block c (local column 16 c + 4 kg + r instead of (4 kg + r) CPL + c).
-template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED>
+// REF: the reference kernel's arithmetic (p.reference_arith): p.scale holds one fp32 scale per column, W is narrowed by
+// truncation.
+template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED, bool REF>
 __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
 {
+    static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
     constexpr int KB = decode_blocks_per_step(BITS, CPL);  // blocks of 32 rows per pipeline step
     constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
     constexpr uint32_t kRedStride = kCols + 4u;       // floats per row of a wave's tile in LDS (+4: spreads rows over banks)
@@ -465,16 +468,23 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
                     apply_scales<BITS, CPL>(cs, st.sraw[q]);
                 }
                 if constexpr (PACKED) mac_step_packed<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc);
-                else mac_step<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
+                else mac_step<BITS, CPL, MB, REF>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
             }
         };
         Stage s0, s1;
-        if constexpr (!GROUPED) {
+        if constexpr (REF) {
+            const float4* sf = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.scale) + n_ld);
+#pragma unroll
+            for (int i = 0; i < CPL / 4; ++i) {
+                const float4 v = sf[i];
+                cs[4 * i] = v.x; cs[4 * i + 1] = v.y; cs[4 * i + 2] = v.z; cs[4 * i + 3] = v.w;
+            }
+        } else if constexpr (!GROUPED) {
             if constexpr (PACKED) load_scales_packed<CPL>(s0.sraw[0], sptr, pk_col);
             else load_scales<CPL>(s0.sraw[0], sptr);
         }
         load_stage(s0, 0);
-        if constexpr (!GROUPED) apply_scales<BITS, CPL>(cs, s0.sraw[0]);
+        if constexpr (!GROUPED && !REF) apply_scales<BITS, CPL>(cs, s0.sraw[0]);
         int s = 0;
         for (; s + 2 < nsteps; s += 2) {
             load_stage(s1, s + 1);
@@ -588,7 +598,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
     }
 }
 
-template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED>
+template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED, bool REF = false>
 static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
 {
     constexpr uint32_t kCols = 16u * CPL;
@@ -608,13 +618,13 @@ static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
     if (lds > 64 * 1024) {
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, CPL, MB, GROUPED, PACKED>),
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&bfaintb_decode_kernel<BITS, CPL, MB, GROUPED, PACKED, REF>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64);
             if (e != hipSuccess) return e;
             attr_set = true;
         }
     }
-    void (*kernel)(const GemmParams) = bfaintb_decode_kernel<BITS, CPL, MB, GROUPED, PACKED>;
+    void (*kernel)(const GemmParams) = bfaintb_decode_kernel<BITS, CPL, MB, GROUPED, PACKED, REF>;
     return launch_kernel(kernel, grid, dim3(64 * waves, 1, 1), lds, stream, q);
 }
 
@@ -633,8 +643,27 @@ static hipError_t launch_decode_b(const GemmParams& p, hipStream_t stream)
     return hipErrorInvalidValue;
 }
 
+// The reference's arithmetic: 8-bit codes, one fp32 scale per column.
+template <int CPL>
+static hipError_t launch_decode_ref(const GemmParams& p, hipStream_t stream)
+{
+    switch (p.decode_mb) {
+        case 1: return launch_decode_t<8, CPL, 1, false, false, true>(p, stream);
+        case 2: return launch_decode_t<8, CPL, 2, false, false, true>(p, stream);
+        case 4:
+            if constexpr (CPL == 8) return launch_decode_t<8, CPL, 4, false, false, true>(p, stream);
+            break;
+        default: break;
+    }
+    return hipErrorInvalidValue;
+}
+
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)
 {
+    if (p.reference_arith) {
+        if (bits != 8 || p.group_size != 0) return hipErrorInvalidValue;
+        return p.decode_cols == 128u ? launch_decode_ref<8>(p, stream) : launch_decode_ref<16>(p, stream);
+    }
     if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8, false>(p, stream) : launch_decode_b<8, 16, false>(p, stream);
     return launch_decode_b<4, 16, false>(p, stream);
 }

@@ -4,7 +4,8 @@
 // (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:18-55): integer code -> fp32, times the
 // column's scale, narrowed to bf16.  Differences by contract: scales are bf16 (so the product is
 // exact in fp32), the narrowing rounds to nearest even (v_cvt_pk_bf16_f32) instead of truncating,
-// and 4-bit codes exist.
+// and 4-bit codes exist.  GemmParams.reference_arith selects the reference's own arithmetic instead
+// (fp32 scales, truncation) in the kernels that read row-major 8-bit weights with one scale per column.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -55,10 +56,12 @@ struct GemmParams {
     uint16_t* c;
     const uint16_t* a;
     const uint8_t* b;
-    const uint16_t* scale;
+    const uint16_t* scale;  // bf16 scales; with reference_arith: fp32 scales, one per column
     const uint16_t* bias;  // bf16 [n] added to the fp32 sums before the one rounding to bf16, or null
     const uint16_t* residual;  // bf16 [m, ldr] added after the bias, before the rounding, or null
     uint32_t ldr;              // elements per row of residual
+    uint32_t reference_arith;  // non-zero: the reference kernel's arithmetic — fp32 per-column scales, W and C narrowed by
+                               // truncation (8-bit codes, row-major B, no groups); zero: bf16 scales, round to nearest even
     uint32_t activation;       // kActNone, or kActSiluGate: columns (2j, 2j+1) of the sums are (gate, up) of output column j
     uint32_t m, n, k;
     uint32_t lda;        // elements
@@ -103,6 +106,22 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi)
     v[0] = (__bf16)lo;
     v[1] = (__bf16)hi;
     return __builtin_bit_cast(uint32_t, v);
+}
+
+// Two fp32 -> one dword of two bf16 by truncation (the high halves of the two words): how the reference kernel narrows,
+// both where it forms W (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:29-35, v_pack_b32_f16 with op_sel:[1,1])
+// and where it stores C (.s:597-611, ds_write_b16_d16_hi).
+__device__ __forceinline__ uint32_t pack_bf16_rtz(float lo, float hi)
+{
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);  // bytes {lo.2, lo.3, hi.2, hi.3}
+}
+
+// RTZ = the reference kernel's arithmetic (fp32 scales, truncation), else this library's contract (round to nearest even).
+template <bool RTZ>
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
+{
+    if constexpr (RTZ) return pack_bf16_rtz(lo, hi);
+    else return pack_bf16_rne(lo, hi);
 }
 
 // Signed byte `I` of a dword as fp32: one v_cvt_f32_i32 with an SDWA sign-extending byte select.

@@ -55,9 +55,11 @@ __device__ __forceinline__ uint32_t swizzled_off(uint32_t row, uint32_t chunk)
 // MT = blocks of 32 rows per wave along m: 4 for the 256-row tile, 2 for a 128-row half tile.  Half tiles take
 // over the tiles of a last, less than half full round of 256 workgroups: twice as many workgroups, each with half
 // the matrix instructions (and all of the weight conversion), finish sooner than half-idle CUs running whole tiles.
-template <int BITS, bool GROUPED, int MT, bool PACKED>
+// REF: the reference kernel's arithmetic (p.reference_arith): one fp32 scale per column, W and C narrowed by truncation.
+template <int BITS, bool GROUPED, int MT, bool PACKED, bool REF>
 __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p)
 {
+    static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
     constexpr uint32_t kRows = 64u * MT;  // rows of C per workgroup
     // Four separate LDS arrays (A and W tiles, two stages each) rather than one block: the compiler
     // then knows that fragment reads of one stage cannot alias the asynchronous global->LDS writes
@@ -166,6 +168,10 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                 cs[2 * i] = make_col_scale<BITS>(s0);
                 cs[2 * i + 1] = make_col_scale<BITS>(s1);
             }
+        } else if constexpr (REF) {
+            float4 sf = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (w_ok) sf = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.scale) + ncol);
+            cs[0] = sf.x; cs[1] = sf.y; cs[2] = sf.z; cs[3] = sf.w;
         } else {
             uint2 sr = make_uint2(0, 0);
             if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + ncol);
@@ -220,24 +226,24 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             const float s = cs[J];
             if constexpr (BITS == 8) {
                 const uint32_t lo = b_s8[4 * I + 2 * H], hi = b_s8[4 * I + 2 * H + 1];  // rows 0-3, rows 4-7
-                w.x = pack_bf16_rne(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
-                w.y = pack_bf16_rne(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
-                w.z = pack_bf16_rne(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
-                w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
+                w.x = pack_bf16<REF>(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
+                w.y = pack_bf16<REF>(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
+                w.z = pack_bf16<REF>(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
+                w.w = pack_bf16<REF>(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
             } else {
                 const uint32_t ev = b_s8[2 * J], od = b_s8[2 * J + 1];  // rows 0,2,4,6 and rows 1,3,5,7
-                w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
-                w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
-                w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
-                w.w = pack_bf16_rne(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
+                w.x = pack_bf16<REF>(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
+                w.y = pack_bf16<REF>(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
+                w.z = pack_bf16<REF>(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
+                w.w = pack_bf16<REF>(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
             }
             *reinterpret_cast<uint4*>(w_tile(stage_c) + (pk_dst[I] ^ (H * 64u))) = w;
             return;
         }
-        w.x = pack_bf16_rne(sbyte_to_f32<J>(b_s8[0]) * cs[J], sbyte_to_f32<J>(b_s8[1]) * cs[J]);
-        w.y = pack_bf16_rne(sbyte_to_f32<J>(b_s8[2]) * cs[J], sbyte_to_f32<J>(b_s8[3]) * cs[J]);
-        w.z = pack_bf16_rne(sbyte_to_f32<J>(b_s8[4]) * cs[J], sbyte_to_f32<J>(b_s8[5]) * cs[J]);
-        w.w = pack_bf16_rne(sbyte_to_f32<J>(b_s8[6]) * cs[J], sbyte_to_f32<J>(b_s8[7]) * cs[J]);
+        w.x = pack_bf16<REF>(sbyte_to_f32<J>(b_s8[0]) * cs[J], sbyte_to_f32<J>(b_s8[1]) * cs[J]);
+        w.y = pack_bf16<REF>(sbyte_to_f32<J>(b_s8[2]) * cs[J], sbyte_to_f32<J>(b_s8[3]) * cs[J]);
+        w.z = pack_bf16<REF>(sbyte_to_f32<J>(b_s8[4]) * cs[J], sbyte_to_f32<J>(b_s8[5]) * cs[J]);
+        w.w = pack_bf16<REF>(sbyte_to_f32<J>(b_s8[6]) * cs[J], sbyte_to_f32<J>(b_s8[7]) * cs[J]);
         *reinterpret_cast<uint4*>(w_tile(stage_c) + w_dst + (J & 1) * 4096u + (J >> 1) * 16384u) = w;
     };
     auto prepare = [&](uint32_t (&b_s8)[8]) {
@@ -466,7 +472,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                             o0 += bf16_bits_to_f32(rres[i] & 0xffffu);
                             o1 += bf16_bits_to_f32(rres[i] >> 16);
                         }
-                        const uint32_t both = pack_bf16_rne(o0, o1);
+                        const uint32_t both = pack_bf16<REF>(o0, o1);
                         *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + col0) = (uint16_t)(both & 0xffffu);
                         *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + col0 + 16u) = (uint16_t)(both >> 16);
                     }
@@ -502,10 +508,10 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                     const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
                     uint32_t both;
                     if (has_res) {  // bias0/1 are +0 without a bias: a sum that gets a residual added need not keep -0
-                        both = pack_bf16_rne(acc[mt][0][i] + bias0 + bf16_bits_to_f32(rres[mt - mt0][i] & 0xffffu),
+                        both = pack_bf16<REF>(acc[mt][0][i] + bias0 + bf16_bits_to_f32(rres[mt - mt0][i] & 0xffffu),
                                              acc[mt][1][i] + bias1 + bf16_bits_to_f32(rres[mt - mt0][i] >> 16));
                     } else {
-                        both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                        both = has_bias ? pack_bf16<REF>(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16<REF>(acc[mt][0][i], acc[mt][1][i]);
                     }
                     *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0) = (uint16_t)(both & 0xffffu);
                     *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + 2u * col0 + 32u) = (uint16_t)(both >> 16);
@@ -543,7 +549,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                     const uint32_t row = 32u * (block32 & 1u) + 8u * (i >> 2) + 4u * half + (i & 3u);
                     float o = silu_gate(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1);
                     if (has_res) o += bf16_bits_to_f32(rres[i]);
-                    *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + colbyte / 2u) = (uint16_t)(pack_bf16_rne(o, 0.f) & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(base + row * kCRowBytes + colbyte / 2u) = (uint16_t)(pack_bf16<REF>(o, 0.f) & 0xffffu);
                 }
             }
         } else {
@@ -570,10 +576,10 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
                 // without a bias or residual the sums are stored as they are (adding +0 would turn a -0 sum into +0)
                 uint32_t both;
                 if (has_res) {
-                    both = pack_bf16_rne(acc[mt][0][i] + bias0 + bf16_bits_to_f32(rres[mt][i] & 0xffffu),
+                    both = pack_bf16<REF>(acc[mt][0][i] + bias0 + bf16_bits_to_f32(rres[mt][i] & 0xffffu),
                                          acc[mt][1][i] + bias1 + bf16_bits_to_f32(rres[mt][i] >> 16));
                 } else {
-                    both = has_bias ? pack_bf16_rne(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16_rne(acc[mt][0][i], acc[mt][1][i]);
+                    both = has_bias ? pack_bf16<REF>(acc[mt][0][i] + bias0, acc[mt][1][i] + bias1) : pack_bf16<REF>(acc[mt][0][i], acc[mt][1][i]);
                 }
                 *reinterpret_cast<uint32_t*>(base + row * kCRowBytes + colbyte) = both;
             }
@@ -594,7 +600,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     }
 }
 
-template <int BITS, bool GROUPED, bool PACKED>
+template <int BITS, bool GROUPED, bool PACKED, bool REF = false>
 static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
 {
     GemmParams p = p0;
@@ -608,7 +614,7 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
         p.tile_first = 0;
         p.tile_count = whole;
         const uint32_t grid = (whole + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-        void (*whole_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 4, PACKED>;
+        void (*whole_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 4, PACKED, REF>;
         hipError_t e = launch_kernel(whole_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
         if (e != hipSuccess) return e;
     }
@@ -616,7 +622,7 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
         p.tile_first = whole;
         p.tile_count = halves;
         const uint32_t grid = (2u * halves + 7u) / 8u * 8u;
-        void (*half_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 2, PACKED>;
+        void (*half_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 2, PACKED, REF>;
         return launch_kernel(half_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
     }
     return hipSuccess;
@@ -625,6 +631,7 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream)
 hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream)
 {
     const bool grouped = p.group_size != 0;
+    if (p.reference_arith) return (bits == 8 && !grouped) ? launch_prefill_t<8, false, false, true>(p, stream) : hipErrorInvalidValue;
     if (bits == 8) return grouped ? launch_prefill_t<8, true, false>(p, stream) : launch_prefill_t<8, false, false>(p, stream);
     return grouped ? launch_prefill_t<4, true, false>(p, stream) : launch_prefill_t<4, false, false>(p, stream);
 }

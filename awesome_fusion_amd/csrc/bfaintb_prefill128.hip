@@ -42,10 +42,12 @@ __device__ __forceinline__ uint32_t swz128(uint32_t row, uint32_t chunk)
 }
 }  // namespace
 
-template <int BITS, bool GROUPED, bool PACKED>
+// REF: the reference kernel's arithmetic (p.reference_arith): one fp32 scale per column, W and C narrowed by truncation.
+template <int BITS, bool GROUPED, bool PACKED, bool REF>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
 bfaintb_prefill128_kernel(const GemmParams p)
 {
+    static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kStage128];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kStage128];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_w0[kStage128];
@@ -113,6 +115,13 @@ bfaintb_prefill128_kernel(const GemmParams p)
     float cs[2];
     uint32_t cur_group = 0xffffffffu;
     auto fetch_scales = [&](uint32_t g) {
+        if constexpr (REF) {
+            float2 sf = make_float2(0.f, 0.f);
+            if (w_ok) sf = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.scale) + ncol);
+            cs[0] = sf.x;
+            cs[1] = sf.y;
+            return;
+        }
         uint32_t s0 = 0, s1 = 0;
         if (w_ok) {
             if constexpr (PACKED) {
@@ -176,16 +185,16 @@ bfaintb_prefill128_kernel(const GemmParams p)
                 const float s = cs[h];
                 if constexpr (BITS == 8) {
                     const uint32_t lo = codes8_to_s8(b_reg[2 * h]), hi = codes8_to_s8(b_reg[2 * h + 1]);
-                    w[h].x = pack_bf16_rne(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
-                    w[h].y = pack_bf16_rne(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
-                    w[h].z = pack_bf16_rne(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
-                    w[h].w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
+                    w[h].x = pack_bf16<REF>(sbyte_to_f32<0>(lo) * s, sbyte_to_f32<1>(lo) * s);
+                    w[h].y = pack_bf16<REF>(sbyte_to_f32<2>(lo) * s, sbyte_to_f32<3>(lo) * s);
+                    w[h].z = pack_bf16<REF>(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
+                    w[h].w = pack_bf16<REF>(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
                 } else {
                     const uint32_t ev = codes4_even_to_s8x16(b_reg[h]), od = codes4_odd_to_s8x16(b_reg[h]);
-                    w[h].x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
-                    w[h].y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
-                    w[h].z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
-                    w[h].w = pack_bf16_rne(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
+                    w[h].x = pack_bf16<REF>(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
+                    w[h].y = pack_bf16<REF>(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
+                    w[h].z = pack_bf16<REF>(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
+                    w[h].w = pack_bf16<REF>(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
                 }
             }
             *reinterpret_cast<uint4*>(w_tile(stage_c) + w_dst) = w[0];
@@ -195,14 +204,14 @@ bfaintb_prefill128_kernel(const GemmParams p)
             uint32_t s8[8];
 #pragma unroll
             for (int r = 0; r < 8; ++r) s8[r] = BITS == 8 ? codes8_to_s8(b_reg[r]) : codes4_quad_to_s8x16(b_reg[r]);
-            w[0].x = pack_bf16_rne(sbyte_to_f32<0>(s8[0]) * cs[0], sbyte_to_f32<0>(s8[1]) * cs[0]);
-            w[0].y = pack_bf16_rne(sbyte_to_f32<0>(s8[2]) * cs[0], sbyte_to_f32<0>(s8[3]) * cs[0]);
-            w[0].z = pack_bf16_rne(sbyte_to_f32<0>(s8[4]) * cs[0], sbyte_to_f32<0>(s8[5]) * cs[0]);
-            w[0].w = pack_bf16_rne(sbyte_to_f32<0>(s8[6]) * cs[0], sbyte_to_f32<0>(s8[7]) * cs[0]);
-            w[1].x = pack_bf16_rne(sbyte_to_f32<1>(s8[0]) * cs[1], sbyte_to_f32<1>(s8[1]) * cs[1]);
-            w[1].y = pack_bf16_rne(sbyte_to_f32<1>(s8[2]) * cs[1], sbyte_to_f32<1>(s8[3]) * cs[1]);
-            w[1].z = pack_bf16_rne(sbyte_to_f32<1>(s8[4]) * cs[1], sbyte_to_f32<1>(s8[5]) * cs[1]);
-            w[1].w = pack_bf16_rne(sbyte_to_f32<1>(s8[6]) * cs[1], sbyte_to_f32<1>(s8[7]) * cs[1]);
+            w[0].x = pack_bf16<REF>(sbyte_to_f32<0>(s8[0]) * cs[0], sbyte_to_f32<0>(s8[1]) * cs[0]);
+            w[0].y = pack_bf16<REF>(sbyte_to_f32<0>(s8[2]) * cs[0], sbyte_to_f32<0>(s8[3]) * cs[0]);
+            w[0].z = pack_bf16<REF>(sbyte_to_f32<0>(s8[4]) * cs[0], sbyte_to_f32<0>(s8[5]) * cs[0]);
+            w[0].w = pack_bf16<REF>(sbyte_to_f32<0>(s8[6]) * cs[0], sbyte_to_f32<0>(s8[7]) * cs[0]);
+            w[1].x = pack_bf16<REF>(sbyte_to_f32<1>(s8[0]) * cs[1], sbyte_to_f32<1>(s8[1]) * cs[1]);
+            w[1].y = pack_bf16<REF>(sbyte_to_f32<1>(s8[2]) * cs[1], sbyte_to_f32<1>(s8[3]) * cs[1]);
+            w[1].z = pack_bf16<REF>(sbyte_to_f32<1>(s8[4]) * cs[1], sbyte_to_f32<1>(s8[5]) * cs[1]);
+            w[1].w = pack_bf16<REF>(sbyte_to_f32<1>(s8[6]) * cs[1], sbyte_to_f32<1>(s8[7]) * cs[1]);
             *reinterpret_cast<uint4*>(w_tile(stage_c) + w_dst) = w[0];
             *reinterpret_cast<uint4*>(w_tile(stage_c) + w_dst + 8192u) = w[1];
         }
@@ -319,7 +328,7 @@ bfaintb_prefill128_kernel(const GemmParams p)
                 o[2] += bf16_bits_to_f32(r.y & 0xffffu);
                 o[3] += bf16_bits_to_f32(r.y >> 16);
             }
-            *reinterpret_cast<uint2*>(p.c + (size_t)gm * p.ldc + gn / 2u) = make_uint2(pack_bf16_rne(o[0], o[1]), pack_bf16_rne(o[2], o[3]));
+            *reinterpret_cast<uint2*>(p.c + (size_t)gm * p.ldc + gn / 2u) = make_uint2(pack_bf16<REF>(o[0], o[1]), pack_bf16<REF>(o[2], o[3]));
         } else {
             if (p.residual != nullptr) {
                 const uint4 r = *reinterpret_cast<const uint4*>(p.residual + (size_t)gm * p.ldr + gn);
@@ -331,23 +340,24 @@ bfaintb_prefill128_kernel(const GemmParams p)
                 }
             }
             *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) =
-                make_uint4(pack_bf16_rne(v[0], v[1]), pack_bf16_rne(v[2], v[3]), pack_bf16_rne(v[4], v[5]), pack_bf16_rne(v[6], v[7]));
+                make_uint4(pack_bf16<REF>(v[0], v[1]), pack_bf16<REF>(v[2], v[3]), pack_bf16<REF>(v[4], v[5]), pack_bf16<REF>(v[6], v[7]));
         }
     }
 }
 
-template <int BITS, bool GROUPED, bool PACKED>
+template <int BITS, bool GROUPED, bool PACKED, bool REF = false>
 static hipError_t launch_prefill128_t(const GemmParams& p, hipStream_t stream)
 {
     const uint32_t tiles = ((p.m + kT128 - 1) / kT128) * ((p.n + kT128 - 1) / kT128);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    void (*kernel)(const GemmParams) = bfaintb_prefill128_kernel<BITS, GROUPED, PACKED>;
+    void (*kernel)(const GemmParams) = bfaintb_prefill128_kernel<BITS, GROUPED, PACKED, REF>;
     return launch_kernel(kernel, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
 }
 
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream)
 {
     const bool grouped = p.group_size != 0;
+    if (p.reference_arith) return (bits == 8 && !grouped && !packed) ? launch_prefill128_t<8, false, false, true>(p, stream) : hipErrorInvalidValue;
     if (packed) {
         if (bits == 8) return grouped ? launch_prefill128_t<8, true, true>(p, stream) : launch_prefill128_t<8, false, true>(p, stream);
         return grouped ? launch_prefill128_t<4, true, true>(p, stream) : launch_prefill128_t<4, false, true>(p, stream);

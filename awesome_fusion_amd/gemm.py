@@ -78,6 +78,10 @@ def lib():
         L.bfaintb_gemm_prepacked_fused.restype = C.c_int
         L.bfaintb_gemm_prepacked_fused.argtypes = [_vp, _vp, _vp, _vp, C.POINTER(Epilogue), _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
                                                    C.c_size_t, _vp]
+        L.bfaintb_gemm_reference.restype = C.c_int
+        L.bfaintb_gemm_reference.argtypes = [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp, C.c_size_t, _vp]
+        L.bfaintb_gemm_reference_ex.restype = C.c_int
+        L.bfaintb_gemm_reference_ex.argtypes = L.bfaintb_gemm_reference.argtypes + [C.c_int, _u32]
         L.bfaintb_gemm_workspace_bytes.restype = C.c_size_t
         L.bfaintb_gemm_workspace_bytes.argtypes = [_u32, _u32, _u32, C.c_int, _u32]
         L.bfaintb_gemm_workspace_bytes_ex.restype = C.c_size_t
@@ -206,6 +210,23 @@ def gemm(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, g
                                    _ptr(workspace), workspace_nbytes, _stream_handle(stream), which, force_split_k)
     if rc and check:
         raise BfaintbError(rc, "bfaintb_gemm")
+    return rc
+
+
+def gemm_reference(c, a, b, scale_f32, m, n, k, lda=None, ldb=None, ldc=None, workspace=None, workspace_nbytes=None, stream=None,
+                   which=AUTO, force_split_k=0, check=True):
+    """The reference kernel's arithmetic through bfaintb_gemm_reference[_ex]: fp32 scales [n], 8-bit codes, W and C
+    narrowed by truncation.  Workspace as for gemm(..., weight_bits=8, group_size=0)."""
+    if workspace_nbytes is None:
+        workspace_nbytes = 0 if workspace is None or isinstance(workspace, int) else workspace.numel() * workspace.element_size()
+    args = (_ptr(c), _ptr(a), _ptr(b), _ptr(scale_f32), m, n, k, k if lda is None else lda, n if ldb is None else ldb,
+            n if ldc is None else ldc, _ptr(workspace), workspace_nbytes, _stream_handle(stream))
+    if which != AUTO or force_split_k:
+        rc = lib().bfaintb_gemm_reference_ex(*args, which, force_split_k)
+    else:
+        rc = lib().bfaintb_gemm_reference(*args)
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_gemm_reference")
     return rc
 
 

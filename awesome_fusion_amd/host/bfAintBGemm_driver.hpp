@@ -1,7 +1,7 @@
 // The bfAintBGemm driver: command line, buffers, data, timing, metrics and (optionally) validation.
 // Same flow and positional command line as /root/reference/bfAintBGemm/bfAintBGemm.cc:36-217:
 //
-//   bfAintBGemm [validation] [m n k] [lda ldb ldc] [weight_bits group_size data seed loops]
+//   bfAintBGemm [validation] [m n k] [lda ldb ldc] [weight_bits group_size data seed loops arith]
 //
 // with the reference's defaults (validation 0, m 32, n 128, k 512, ld = k, n, n; 10 warm-up and 10
 // timed launches inside one event pair on the null stream, :103-104,151-186).  Where the reference
@@ -10,6 +10,10 @@
 //   data = 0  the reference's test regime: A, B and scale all integers in {-2,-1,0,1} (random_gen.hpp:24,37,50)
 //   data = 1  A ~ N(0,1); B uniform integers over the code range; scale uniform in [0.001, 0.01] (8-bit)
 //             or [0.001, 0.02] (4-bit); scales per column or per group of `group_size` rows
+//   arith = 0 this library's contract: bf16 scales, round-to-nearest-even conversions on host and device
+//   arith = 1 the reference's own: A narrowed by truncation (mem_transfer<bfloat16, float>, bfAintBGemm.cc:88), fp32 scales
+//             on the device (:27,101), bfaintb_gemm_reference (truncating kernel arithmetic); 8-bit codes, per column only.
+//             With data = 0 the validation is the reference's, operand for operand (:198-214).
 // Metrics are the reference's (:186-195) in decimal units with the scale bytes counted.
 // Validation needs a host GEMM to compare with; it is supplied by the caller of driver_main (the
 // test build passes one); the plain binary has none and refuses `validation`.
@@ -71,6 +75,9 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
     if (argc >= 11) data = std::atoi(argv[10]);
     if (argc >= 12) seed = std::strtoull(argv[11], nullptr, 10);
     if (argc >= 13) total_loop = std::atoi(argv[12]);
+    const bool ref_arith = argc >= 14 && std::atoi(argv[13]) != 0;
+    if (ref_arith && (weight_bits != 8 || group_size != 0)) { std::printf("arith 1 is 8-bit codes with one scale per column\n"); return 2; }
+    const std::size_t scale_elem_bytes = ref_arith ? sizeof(float) : sizeof(ScaleDataType);
     const int warm_ups = 10;
     if (m <= 0 || n <= 0 || k <= 0 || total_loop <= 0) { std::printf("bad sizes\n"); return 2; }
     if (validation && (checker == nullptr || checker->gemm_rrr == nullptr)) {
@@ -92,7 +99,7 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
     SimpleDeviceMem a_device_buf(sizeof(ADataType) * a_elems);
     SimpleDeviceMem b_device_buf(b_bytes);
     SimpleDeviceMem c_device_buf(sizeof(CDataType) * c_elems);
-    SimpleDeviceMem scale_device_buf(sizeof(ScaleDataType) * s_elems);
+    SimpleDeviceMem scale_device_buf(scale_elem_bytes * s_elems);
     GPU_CHECK_ERROR(a_device_buf.Status()); GPU_CHECK_ERROR(b_device_buf.Status());
     GPU_CHECK_ERROR(c_device_buf.Status()); GPU_CHECK_ERROR(scale_device_buf.Status());
 
@@ -116,14 +123,16 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
 
     SimpleHostMem a_host_buf_to_device(sizeof(ADataType) * a_elems), b_host_buf_to_device(b_bytes);
     SimpleHostMem scale_host_buf_to_device(sizeof(ScaleDataType) * s_elems), c_host_buf_from_device(sizeof(CDataType) * c_elems);
-    mem_transfer_bf16_rne(a_host_buf_to_device, a_host_buf, a_elems);
-    mem_transfer_bf16_rne(scale_host_buf_to_device, scale_host_buf, s_elems);
+    if (ref_arith) mem_transfer<ADataType, float, SimpleHostMem, SimpleHostMem>(a_host_buf_to_device, a_host_buf, a_elems);
+    else mem_transfer_bf16_rne(a_host_buf_to_device, a_host_buf, a_elems);
+    mem_transfer_bf16_rne(scale_host_buf_to_device, scale_host_buf, s_elems);  // unused with arith 1: the fp32 scales go as they are
     if (weight_bits == 8) mem_transfer<BDataType, float, SimpleHostMem, SimpleHostMem>(b_host_buf_to_device, b_host_buf, b_elems);
     else mem_transfer_int4(b_host_buf_to_device, b_host_buf, k, n, ldb);
 
     GPU_CHECK_ERROR(hipMemcpy(a_device_buf.GetBuffer(), a_host_buf_to_device.GetBuffer(), sizeof(ADataType) * a_elems, hipMemcpyHostToDevice));
     GPU_CHECK_ERROR(hipMemcpy(b_device_buf.GetBuffer(), b_host_buf_to_device.GetBuffer(), b_bytes, hipMemcpyHostToDevice));
-    GPU_CHECK_ERROR(hipMemcpy(scale_device_buf.GetBuffer(), scale_host_buf_to_device.GetBuffer(), sizeof(ScaleDataType) * s_elems, hipMemcpyHostToDevice));
+    GPU_CHECK_ERROR(hipMemcpy(scale_device_buf.GetBuffer(), ref_arith ? scale_host_buf.GetBuffer() : scale_host_buf_to_device.GetBuffer(),
+                              scale_elem_bytes * s_elems, hipMemcpyHostToDevice));
     GPU_CHECK_ERROR(hipMemset(c_device_buf.GetBuffer(), 0, sizeof(CDataType) * c_elems));
 
     const std::size_t ws_bytes = bfaintb_gemm_workspace_bytes(m, n, k, weight_bits, group_size);
@@ -133,6 +142,10 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
     if (rc) { std::printf("bfaintb_workspace_init: %s\n", bfaintb_error_string(rc)); return 1; }
 
     auto launch = [&]() {
+        if (ref_arith)
+            return bfaintb_gemm_reference(c_device_buf.GetBuffer(), a_device_buf.GetBuffer(), b_device_buf.GetBuffer(),
+                                          static_cast<const float*>(scale_device_buf.GetBuffer()), m, n, k, lda, ldb, ldc,
+                                          workspace.GetBuffer(), ws_bytes, nullptr);
         return bfaintb_gemm(c_device_buf.GetBuffer(), a_device_buf.GetBuffer(), b_device_buf.GetBuffer(), scale_device_buf.GetBuffer(),
                             m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace.GetBuffer(), ws_bytes, nullptr);
     };
@@ -162,7 +175,7 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
     std::printf("m: %d, n: %d, k: %d, time: %.3f ms, tflops: %.3f, bw: %.3f GB/s\n", m, n, k, time_per_loop, tflops, bw_gbs);
     const bool decode = bfaintb_gemm_variant(m, n, k, weight_bits, group_size) == BFAINTB_VARIANT_DECODE;
     std::cout << "layouts A/B/scale/C: " << ALayout{} << "/" << BLayout{} << "/" << ScaleLayout{} << "/" << CLayout{}
-              << ", weight_bits " << weight_bits << ", group_size " << group_size << ", variant " << (decode ? "decode" : "prefill")
+              << ", weight_bits " << weight_bits << ", group_size " << group_size << (ref_arith ? ", reference arithmetic" : "") << ", variant " << (decode ? "decode" : "prefill")
               << ", roofline: " << (decode ? 100.0 * bw_gbs / 8000.0 : 100.0 * tflops / 2500.0) << " % of "
               << (decode ? "8000 GB/s HBM" : "2500 TFLOP/s bf16 MFMA") << " (cache-hot: the same buffers every launch)\n\n";
     if (result) { result->ms_per_launch = time_per_loop; result->tflops = tflops; result->gbs = bw_gbs; }
@@ -176,10 +189,23 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
         for (std::size_t i = 0; i < a_elems; ++i) a_seen[i] = type_convert<float>(a_dev[i]);
         for (int ik = 0; ik < k; ++ik)
             for (int in = 0; in < n; ++in) {
-                const float s = type_convert<float>(s_dev[(std::size_t)(group_size ? ik / group_size : 0) * n + in]);
-                w_seen[(std::size_t)ik * n + in] = type_convert<float>(bf16_convert_rtn<bfloat16, float>(b_f[(std::size_t)ik * ldb + in] * s));
+                const float q = b_f[(std::size_t)ik * ldb + in];
+                if (ref_arith) {  // fp32 scale, product narrowed by truncation
+                    w_seen[(std::size_t)ik * n + in] = type_convert<float>(type_convert<bfloat16, float>(q * s_f[in]));
+                } else {
+                    const float s = type_convert<float>(s_dev[(std::size_t)(group_size ? ik / group_size : 0) * n + in]);
+                    w_seen[(std::size_t)ik * n + in] = type_convert<float>(bf16_convert_rtn<bfloat16, float>(q * s));
+                }
             }
-        checker->gemm_rrr(c_ref.data(), a_seen.data(), w_seen.data(), ones.data(), m, n, k, lda, n, n);
+        if (ref_arith && data == 0) {
+            // the reference's own check, operand for operand: the host's float A, float B and float scales (bfAintBGemm.cc:200-209)
+            std::vector<float> b_dense((std::size_t)k * n);
+            for (int ik = 0; ik < k; ++ik)
+                for (int in = 0; in < n; ++in) b_dense[(std::size_t)ik * n + in] = b_f[(std::size_t)ik * ldb + in];
+            checker->gemm_rrr(c_ref.data(), a_f, b_dense.data(), s_f, m, n, k, lda, n, n);
+        } else {
+            checker->gemm_rrr(c_ref.data(), a_seen.data(), w_seen.data(), ones.data(), m, n, k, lda, n, n);
+        }
         std::vector<bfloat16> c_dev((std::size_t)m * n);
         const bfloat16* c_raw = static_cast<const bfloat16*>(c_host_buf_from_device.GetBuffer());
         for (int im = 0; im < m; ++im)

@@ -33,7 +33,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 103 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 104 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -131,6 +131,27 @@ typedef struct bfaintb_epilogue {
 BFAINTB_API int bfaintb_gemm_fused(void* c, const void* a, const void* b, const void* scale, const bfaintb_epilogue* epilogue, uint32_t m,
                        uint32_t n, uint32_t k, uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size,
                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The reference kernel's launch, argument for argument, with the reference kernel's own arithmetic: for a caller that
+ * keeps the reference's buffers exactly as they are.  The arguments are the kernarg block of bfAintBGemm.cc:119-133
+ * (c, a, b, scale, m, n, k, lda, ldb, ldc); scale is fp32 [n] (ScaleDataType = float, bfAintBGemm.cc:27), not bf16;
+ *     W[k,n] = truncate_to_bf16( float(q[k,n]) * scale[n] )      (bf16gemm_kernel_gfx90a.s:18-55: fp32 product, the
+ *                                                                 high halves kept by v_pack_b32_f16 op_sel:[1,1])
+ *     C[m,n] = truncate_to_bf16( sum_k A[m,k] * W[k,n] )         (fp32 accumulation; the store keeps the high halves,
+ *                                                                 .s:597-611, "rtz mode")
+ * 8-bit excess-128 codes with one scale per column: the reference's only format.  Same kernels, variant choice,
+ * workspace (bfaintb_gemm_workspace_bytes(m, n, k, 8, 0)) and stream semantics as bfaintb_gemm; the order in which the
+ * fp32 sums are formed differs from the reference kernel's (as it does between any two tilings), so results agree with
+ * it to the last bit only where the sums are exact — as in the reference's own test data (random_gen.hpp:24,37,50) —
+ * and otherwise to one bf16 unit.  scale must be 16-byte aligned.
+ */
+BFAINTB_API int bfaintb_gemm_reference(void* c, const void* a, const void* b, const float* scale, uint32_t m, uint32_t n, uint32_t k,
+                           uint32_t lda, uint32_t ldb, uint32_t ldc, void* workspace, size_t workspace_bytes, void* stream);
+/* Same with the variant and split factor forced, as bfaintb_gemm_ex. */
+BFAINTB_API int bfaintb_gemm_reference_ex(void* c, const void* a, const void* b, const float* scale, uint32_t m, uint32_t n, uint32_t k,
+                              uint32_t lda, uint32_t ldb, uint32_t ldc, void* workspace, size_t workspace_bytes, void* stream,
+                              int variant, uint32_t split_k);
 
 /* Scratch the GEMM needs for a shape: one fp32 word per (split but the last, row, column) of the
  * split-K partial sums, rounded up to 256 bytes; 0 when the shape runs without split-K.  Depends only

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
-    assert af.lib().bfaintb_version() == 103
+    assert af.lib().bfaintb_version() == 104
     assert "bfaintb_gemm_bias" in names
 
 
@@ -92,6 +92,14 @@ def test_rejects_bad_arguments_without_launching():
     with pytest.raises(af.BfaintbError) as e:
         rc(n=100, check=True)
     assert e.value.code == -2
+    # the reference-arithmetic entry point: same validation, fp32 scales
+    def ref_rc(**kw):
+        d = dict(c=P, a=P, b=P, scale=P, m=64, n=128, k=256, stream=0, check=False)
+        d.update(kw)
+        return af.gemm_reference(d.pop("c"), d.pop("a"), d.pop("b"), d.pop("scale"), d.pop("m"), d.pop("n"), d.pop("k"), **d)
+    assert ref_rc(n=100) == -2 and ref_rc(k=96) == -2 and ref_rc(ldb=64) == -3 and ref_rc(ldc=120) == -3
+    assert ref_rc(scale=None) == -1 and ref_rc(scale=P + 4) == -4 and ref_rc(which=9) == -7 and ref_rc(m=0) == 0
+    assert ref_rc(m=8, k=1024, which=af.DECODE, force_split_k=2) == -6
     # dequant entry point
     assert af.dequant(P, P, P, 128, 256, stream=0, weight_bits=3, check=False) == -5
     assert af.dequant(P, P, P, 100, 256, stream=0, check=False) == -2

@@ -39,6 +39,13 @@ def run(exe, *args):
     (1, 1, 4096, 4096, 4096, 4096, 4096, 8, 0, 1, 0),  # config 2: decode
     (1, 16, 1024, 2048, 2048, 1024, 1024, 4, 128, 1, 3),   # int4, group 128, decode
     (1, 96, 512, 1024, 1032, 528, 520, 4, 128, 1, 4),  # int4 prefill with padded leading dimensions
+    # arith = 1: the reference's harness as it is — truncated A, fp32 scales on the device, bfaintb_gemm_reference
+    (1, 32, 128, 512, 512, 128, 128, 8, 0, 0, 0, 10, 1),       # its defaults and data: validated exactly as bfAintBGemm.cc:198-214 does
+    (1, 300, 528, 256, 256, 528, 528, 8, 0, 0, 5, 10, 1),      # the same regime on the tiled kernel (k small enough that every
+                                                               # sum fits bf16: truncated larger sums fail the reference's 1e-3
+                                                               # criterion, for its own kernel as for this one)
+    (1, 64, 128, 256, 256, 128, 128, 8, 0, 1, 0, 10, 1),       # config 1 data
+    (1, 1, 4096, 4096, 4096, 4096, 4096, 8, 0, 1, 0, 10, 1),   # config 2: decode
 ])
 def test_driver_validates_against_host_gemm(args):
     assert os.path.exists(CHECK), "build tests/driver_check first (make -C tests/driver_check)"
