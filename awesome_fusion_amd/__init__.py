@@ -29,6 +29,7 @@ from .gemm import (  # noqa: F401
     prefill_tile,
     prepack,
     prepack_bytes,
+    prepack_colmajor,
     prepacked_variant,
     prepacked_workspace_bytes,
     library_path,

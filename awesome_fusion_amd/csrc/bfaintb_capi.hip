@@ -17,6 +17,7 @@ hipError_t launch_dequant(uint16_t* w, const uint8_t* b, const uint16_t* scale, 
                           uint32_t ldw, int bits, uint32_t group_size, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* dst, uint32_t count, uint32_t value, hipStream_t stream);
 hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, hipStream_t stream);
+hipError_t launch_pack_colmajor(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k, uint32_t ldb_bytes, int bits, hipStream_t stream);
 hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k, uint32_t ldb_bytes, int bits, bool unpack,
                        hipStream_t stream);
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream);
@@ -448,6 +449,19 @@ int bfaintb_prepack(void* packed, const void* b, uint32_t n, uint32_t k, uint32_
 int bfaintb_unpack(void* b, const void* packed, uint32_t n, uint32_t k, uint32_t ldb, int weight_bits, void* stream)
 {
     return repack(b, packed, n, k, ldb, weight_bits, stream, true);
+}
+
+int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k, uint32_t ldb, int weight_bits, void* stream)
+{
+    if (weight_bits != 8 && weight_bits != 4) return BFAINTB_ERR_UNSUPPORTED;
+    const int e = check_packed_shape(n, k, weight_bits);
+    if (e) return e;
+    if (ldb < k || ldb % 16u != 0) return BFAINTB_ERR_BAD_LD;  // elements between columns
+    if (n == 0) return BFAINTB_OK;
+    if (packed == nullptr || b == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    if (misaligned16(packed) || misaligned16(b)) return BFAINTB_ERR_ALIGNMENT;
+    return (int)bfaintb::launch_pack_colmajor(static_cast<uint8_t*>(packed), static_cast<const uint8_t*>(b), n, k,
+                                              weight_bits == 8 ? ldb : ldb / 2u, weight_bits, static_cast<hipStream_t>(stream));
 }
 
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one up to kPackedSlabMaxM rows of A, the

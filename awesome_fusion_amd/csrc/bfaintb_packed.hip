@@ -100,7 +100,44 @@ __global__ void __launch_bounds__(256) unpack_kernel(uint8_t* __restrict__ dst, 
     }
 }
 
+// Column-major B (n rows of k codes, k contiguous; 4-bit: byte j of a column holds rows 2j and 2j+1, low nibble first)
+// -> the packed order.  A lane's 16 bytes of a chunk are whole runs of its column: 2 x 8 bytes (8-bit) or 4 x 4 bytes
+// (4-bit, already in the packed nibble order), so this is a gather of aligned words.
+template <int BITS>
+__global__ void __launch_bounds__(256) pack_colmajor_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src, uint32_t n, uint32_t k,
+                                                            uint32_t ldb_bytes)
+{
+    const size_t slots = (size_t)n * k * BITS / 8 / 16;
+    const uint32_t chunks = k / PackedFormat<BITS>::kChunkRows;
+    for (size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x; slot < slots; slot += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t lane = (uint32_t)(slot & 63u);
+        const size_t chunk = slot >> 6;
+        const uint32_t kc = (uint32_t)(chunk % chunks), nb = (uint32_t)(chunk / chunks);
+        const uint32_t nl = lane & 15u, kg = lane >> 4;
+        const uint8_t* col = src + (size_t)(16u * nb + nl) * ldb_bytes;
+        uint4 out;
+        if constexpr (BITS == 8) {
+            const uint2 h0 = *reinterpret_cast<const uint2*>(col + 64u * kc + 8u * kg);
+            const uint2 h1 = *reinterpret_cast<const uint2*>(col + 64u * kc + 32u + 8u * kg);
+            out = make_uint4(h0.x, h0.y, h1.x, h1.y);
+        } else {
+            const uint8_t* base = col + (128u * kc + 8u * kg) / 2u;
+            out = make_uint4(*reinterpret_cast<const uint32_t*>(base), *reinterpret_cast<const uint32_t*>(base + 16u),
+                             *reinterpret_cast<const uint32_t*>(base + 32u), *reinterpret_cast<const uint32_t*>(base + 48u));
+        }
+        *reinterpret_cast<uint4*>(dst + slot * 16u) = out;
+    }
+}
+
 }  // namespace
+
+hipError_t launch_pack_colmajor(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k, uint32_t ldb_bytes, int bits, hipStream_t stream)
+{
+    const size_t slots = (size_t)n * k * (uint32_t)bits / 8 / 16;
+    const uint32_t grid = (uint32_t)((slots + 255) / 256 < 65536 ? (slots + 255) / 256 : 65536);
+    void (*kernel)(uint8_t*, const uint8_t*, uint32_t, uint32_t, uint32_t) = bits == 8 ? pack_colmajor_kernel<8> : pack_colmajor_kernel<4>;
+    return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, dst, src, n, k, ldb_bytes);
+}
 
 hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k, uint32_t ldb_bytes, int bits, bool unpack,
                        hipStream_t stream)

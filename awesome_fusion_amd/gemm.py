@@ -96,6 +96,8 @@ def lib():
         L.bfaintb_prepack_bytes.argtypes = [_u32, _u32, C.c_int]
         L.bfaintb_prepack.restype = C.c_int
         L.bfaintb_prepack.argtypes = [_vp, _vp, _u32, _u32, _u32, C.c_int, _vp]
+        L.bfaintb_prepack_colmajor.restype = C.c_int
+        L.bfaintb_prepack_colmajor.argtypes = [_vp, _vp, _u32, _u32, _u32, C.c_int, _vp]
         L.bfaintb_unpack.restype = C.c_int
         L.bfaintb_unpack.argtypes = [_vp, _vp, _u32, _u32, _u32, C.c_int, _vp]
         L.bfaintb_gemm_prepacked.restype = C.c_int
@@ -239,6 +241,14 @@ def prepack(packed, b, n, k, ldb=None, weight_bits=8, stream=None, check=True):
     rc = lib().bfaintb_prepack(_ptr(packed), _ptr(b), n, k, n if ldb is None else ldb, weight_bits, _stream_handle(stream))
     if rc and check:
         raise BfaintbError(rc, "bfaintb_prepack")
+    return rc
+
+
+def prepack_colmajor(packed, b, n, k, ldb=None, weight_bits=8, stream=None, check=True):
+    """Column-major B ([n, ldb] codes, k contiguous; 4-bit: two rows per byte) -> the packed order (bfaintb_prepack_colmajor)."""
+    rc = lib().bfaintb_prepack_colmajor(_ptr(packed), _ptr(b), n, k, k if ldb is None else ldb, weight_bits, _stream_handle(stream))
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_prepack_colmajor")
     return rc
 
 

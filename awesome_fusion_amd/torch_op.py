@@ -23,6 +23,7 @@ from typing import Optional
 import torch
 
 from .gemm import (gemm as _gemm, gemm_prepacked as _gemm_prepacked, prepack as _prepack, prepack_bytes as _prepack_bytes,
+                   prepack_colmajor as _prepack_colmajor,
                    prepacked_workspace_bytes as _prepacked_workspace_bytes,
                    workspace_bytes as _workspace_bytes, workspace_init as _workspace_init)
 
@@ -159,16 +160,24 @@ def _(a, packed, scale, weight_bits, group_size, bias=None, residual=None, activ
     return a.new_empty((m, _out_cols(n, activation)))
 
 
-def prepack_weight(b, weight_bits=8):
-    """Row-major codes ``b`` (uint8 [k, n*bits/8], on the GPU) -> flat packed tensor for ``bfaintb_gemm_prepacked``."""
-    k = b.shape[0]
-    n = b.shape[1] * (8 // weight_bits)
+def prepack_weight(b, weight_bits=8, column_major=False):
+    """Codes ``b`` on the GPU -> flat packed tensor for ``bfaintb_gemm_prepacked``.  Row-major: uint8 [k, n*bits/8];
+    ``column_major``: uint8 [n, k*bits/8] — one row per output feature, the way a Linear keeps its weight (4-bit: two
+    consecutive k per byte, low nibble first)."""
+    per_byte = 8 // weight_bits
+    if column_major:
+        n, k = b.shape[0], b.shape[1] * per_byte
+    else:
+        k, n = b.shape[0], b.shape[1] * per_byte
     nbytes = _prepack_bytes(n, k, weight_bits)
     if nbytes == 0:
         raise ValueError("prepack_weight: the packed order needs n % 16 == 0 and k % 64 == 0 (k % 128 == 0 for 4-bit codes)")
     packed = torch.empty(nbytes, dtype=torch.uint8, device=b.device)
     with torch.cuda.device(b.device):
-        _prepack(packed, b.contiguous(), n, k, weight_bits=weight_bits)
+        if column_major:
+            _prepack_colmajor(packed, b.contiguous(), n, k, weight_bits=weight_bits)
+        else:
+            _prepack(packed, b.contiguous(), n, k, weight_bits=weight_bits)
     return packed
 
 

@@ -33,7 +33,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 104 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 105 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -180,6 +180,12 @@ BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, 
 BFAINTB_API size_t bfaintb_prepack_bytes(uint32_t n, uint32_t k, int weight_bits);
 BFAINTB_API int bfaintb_prepack(void* packed, const void* b, uint32_t n, uint32_t k, uint32_t ldb, int weight_bits, void* stream);
 BFAINTB_API int bfaintb_unpack(void* b, const void* packed, uint32_t n, uint32_t k, uint32_t ldb, int weight_bits, void* stream);
+/* The same packed buffer from column-major B ("rcr"): n columns stored one after the other, k codes each, ldb elements
+ * (>= k, a multiple of 16) from one column to the next — the layout tag the reference declares and never uses
+ * (gemm_tensor_layout.hpp:16-19, bfAintBGemm.cc:18), and how a [out_features, in_features] weight lies in memory.
+ * 8-bit: byte i of a column is row i's code.  4-bit: byte j of a column holds rows 2j (low nibble) and 2j+1 (high
+ * nibble).  The result is byte for byte what bfaintb_prepack makes of the row-major form of the same codes. */
+BFAINTB_API int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k, uint32_t ldb, int weight_bits, void* stream);
 BFAINTB_API int bfaintb_gemm_prepacked(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
                            uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,
                            void* workspace, size_t workspace_bytes, void* stream);

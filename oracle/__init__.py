@@ -144,6 +144,18 @@ def pack_int4(q):
     return out
 
 
+def colmajor_codes(q, bits=8):
+    """Integer weights q [k, n] -> the column-major device bytes [n, k*bits/8]: one row per column, k contiguous;
+    8-bit excess-128, 4-bit excess-8 with row 2j in the low and row 2j+1 in the high nibble of byte j.  (No counterpart in
+    the reference, which declares the ColumnMajor tag, gemm_tensor_layout.hpp:16-19, and never stores B that way; pinned by
+    hand-computed positions in tests/test_oracle_formats.py.)"""
+    q = np.asarray(q).astype(np.int64).T  # [n, k]
+    if bits == 8:
+        return np.ascontiguousarray((q + 128).astype(np.uint8))
+    u = (q + 8).astype(np.uint8)
+    return np.ascontiguousarray(u[:, 0::2] | (u[:, 1::2] << 4))
+
+
 def pack_mfma16(b, k, n, bits=8):
     """Row-major packed codes b (uint8 [k, n] for 8-bit, [k, n/2] for 4-bit, the wire formats above) -> the library's
     pre-packed operand order, as a flat uint8 array of k * n * bits / 8 bytes.

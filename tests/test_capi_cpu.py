@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
-    assert af.lib().bfaintb_version() == 104
+    assert af.lib().bfaintb_version() == 105
     assert "bfaintb_gemm_bias" in names
 
 
@@ -119,6 +119,14 @@ def test_prepacked_entry_points_validate_before_launching():
     assert af.prepack(P, P, 128, 256, ldb=64, stream=0, check=False) == -3
     assert af.prepack(None, P, 128, 256, stream=0, check=False) == -1
     assert af.prepack(P, P + 8, 128, 256, stream=0, check=False) == -4
+    # column-major source: ldb counts the elements between columns (>= k)
+    assert af.prepack_colmajor(P, P, 128, 256, stream=0, weight_bits=3, check=False) == -5
+    assert af.prepack_colmajor(P, P, 100, 256, stream=0, check=False) == -2
+    assert af.prepack_colmajor(P, P, 128, 256, ldb=128, stream=0, check=False) == -3
+    assert af.prepack_colmajor(P, P, 128, 256, ldb=264, stream=0, check=False) == -3
+    assert af.prepack_colmajor(P, None, 128, 256, stream=0, check=False) == -1
+    assert af.prepack_colmajor(P + 4, P, 128, 256, stream=0, check=False) == -4
+    assert af.prepack_colmajor(P, P, 0, 256, stream=0, check=False) == 0
     assert af.unpack(P, None, 128, 256, stream=0, check=False) == -1
 
     def rcp(**kw):

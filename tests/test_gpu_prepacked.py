@@ -55,6 +55,25 @@ def test_pack_kernels_bit_exact_and_inverse(af, bits, k, n):
     assert np.array_equal(back.cpu().numpy(), p.b_bytes)
 
 
+@pytest.mark.parametrize("bits,k,n,ldb", [(8, 64, 16, None), (8, 448, 272, 512), (4, 128, 16, None), (4, 640, 304, 768), (8, 4096, 4096, None)])
+def test_pack_from_column_major_is_the_same_buffer(af, bits, k, n, ldb):
+    """bfaintb_prepack_colmajor on [n, ldb] codes (k contiguous) gives byte for byte what bfaintb_prepack gives on the
+    row-major form of the same weights (= the oracle's packed order); a GEMM over it meets the oracle."""
+    import torch
+    p = Problem(64, n, k, bits, 0, seed=k + n + 1)
+    cm = oracle.colmajor_codes(p.q, bits)                     # [n, k * bits / 8]
+    if ldb is not None:                                       # padded columns: the padding must not be read as codes
+        wide = np.full((n, ldb * bits // 8), 0xAB, np.uint8)
+        wide[:, :cm.shape[1]] = cm
+        cm = wide
+    pk = torch.zeros(af.prepack_bytes(n, k, bits), dtype=torch.uint8, device="cuda")
+    af.prepack_colmajor(pk, to_dev(cm), n, k, ldb=ldb, weight_bits=bits)
+    torch.cuda.synchronize()
+    assert np.array_equal(pk.cpu().numpy(), oracle.pack_mfma16(p.b_bytes, k, n, bits))
+    if k <= 640:
+        assert_close_ulp(p, run_prepacked(af, p, pk=pk), f"GEMM over column-major-packed weights {n}x{k} b{bits}")
+
+
 def test_pack_honours_the_row_stride(af):
     import torch
     k, n, ldb = 128, 48, 64

@@ -170,3 +170,26 @@ def test_prepacked_order_positions_and_inverse():
     # row 255 = chunk 1, h 3, kg 3, r 7; column 0: chunk index 1, lane 48 -> byte 1024 + 48*16 + 12 + 3, high nibble
     assert pk4[1024 + 48 * 16 + 15] >> 4 == code(255, 0)
     assert np.array_equal(oracle.unpack_mfma16(pk4, k, n, 4), b4)
+
+
+def test_colmajor_codes_positions():
+    # column-major device bytes (no counterpart in the reference): positions worked out by hand from the stated format
+    q = np.zeros((8, 4), np.int8)
+    q[3, 2], q[4, 2], q[5, 2], q[0, 1] = -128, 127, -1, 5
+    b = oracle.colmajor_codes(q, 8)
+    assert b.shape == (4, 8) and b[2, 3] == 0 and b[2, 4] == 255 and b[2, 5] == 127 and b[1, 0] == 133 and b[0, 0] == 128
+    q4 = np.zeros((8, 4), np.int8)
+    q4[4, 3], q4[5, 3], q4[0, 0], q4[7, 1] = -8, 7, 3, -1
+    b4 = oracle.colmajor_codes(q4, 4)
+    assert b4.shape == (4, 4)
+    assert b4[3, 2] == 0xF0            # rows 4 (code 0, low nibble) and 5 (code 15, high nibble) of column 3
+    assert b4[0, 0] == (8 << 4 | 11)   # row 0: 3 + 8 = 11 low; row 1: zero -> 8 high
+    assert b4[1, 3] == (7 << 4 | 8)    # row 7 of column 1: -1 + 8 = 7 in the high nibble of byte 3
+    # and it is the transpose of the row-major form, code by code
+    rng = np.random.default_rng(9)
+    q = rng.integers(-8, 8, size=(64, 32), dtype=np.int8)
+    rm, cm = oracle.pack_int4(q), oracle.colmajor_codes(q, 4)
+    for (r, c) in [(0, 0), (13, 7), (63, 31), (20, 30), (41, 1)]:
+        row_code = (rm[r, c // 2] >> (4 * (c % 2))) & 15
+        col_code = (cm[c, r // 2] >> (4 * (r % 2))) & 15
+        assert row_code == col_code == q[r, c] + 8
