@@ -135,6 +135,25 @@ def test_dequant_against_numpy(bits, group):
     assert (w_rtz != w).any()
 
 
+def test_dequant_with_the_reference_kernels_arithmetic():
+    # fp32 scales, product rounded to fp32 by the multiply, then the high 16 bits (bf16gemm_kernel_gfx90a.s:29-35):
+    # independent statement in numpy float32 arithmetic, exhaustive over the 256 codes for scales with full mantissas
+    rng = np.random.Generator(np.random.PCG64(6))
+    k, n = 256, 48
+    q = np.tile(np.arange(-128, 128, dtype=np.int64)[:, None], (1, n)).astype(np.int8)
+    s = rng.uniform(-0.02, 0.02, size=n).astype(np.float32)
+    s[:4] = np.array([1.0, -1.0, 0.0, 3.0000002], np.float32)
+    b = oracle.mem_transfer_int8(q.astype(np.float32))
+    w = oracle.dequant(b, s, k, n, 8, 0, rtz=True)
+    prod = q.astype(np.float32) * s[None, :]                 # one IEEE fp32 multiply per weight
+    assert np.array_equal(w, (prod.view(np.uint32) >> 16).astype(np.uint16))
+    assert np.array_equal(w[:, 0], oracle.f32_to_bf16_rtz(q[:, 0].astype(np.float32)))   # unit scale: the code itself
+    # truncation never grows a magnitude, and it differs from both other contracts on this data
+    assert np.all(np.abs(widen(w)) <= np.abs(prod))
+    assert (w != oracle.dequant(b, s, k, n, 8, 0, rtz=False)).any()
+    assert (w != oracle.dequant(b, oracle.f32_to_bf16_rne(s.reshape(1, n)), k, n, 8, 0, rtz=True)).any()
+
+
 def test_int_times_bf16_scale_is_exact_exhaustive():
     # every 8-bit integer times every positive normal bf16 significand pattern: the fp32 product equals the exact one
     q = np.arange(-128, 128, dtype=np.float64)[:, None]
