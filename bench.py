@@ -37,13 +37,13 @@ REPLAYS = 5                   # timed replays of the K-launch graph; the median 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
 MEASURED_TRAFFIC_BYTES = {
-    # fetch 8378.0 KiB x 1.997 + write 232.0 KiB (plain launches; profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
-    "decode_m1_n4096_k4096_int8_perchannel": 17369975,
-    # fetch 65685.5 KiB x 1.997 + write 32768.0 KiB (plain launches)
-    "prefill_m4096_n4096_k4096_int8_perchannel": 167876550,
-    # the same shapes through bfaintb_gemm_prepacked: fetch 8281.0 KiB x 1.997 + write 8.0 KiB; fetch 65705.5 KiB x 1.997 + write 32768.0 KiB
-    "decode_m1_n4096_k4096_int8_perchannel_prepacked": 16942241,
-    "prefill_m4096_n4096_k4096_int8_perchannel_prepacked": 167917449,
+    # fetch 8392.5 KiB x 1.997 + write 232.0 KiB (plain launches; profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
+    "decode_m1_n4096_k4096_int8_perchannel": 17398385,
+    # fetch 65698.5 KiB x 1.997 + write 32768.0 KiB (plain launches)
+    "prefill_m4096_n4096_k4096_int8_perchannel": 167893415,
+    # the same shapes through bfaintb_gemm_prepacked: fetch 8273.0 KiB x 1.997 + write 8.0 KiB; fetch 65712.0 KiB x 1.997 + write 32768.0 KiB
+    "decode_m1_n4096_k4096_int8_perchannel_prepacked": 16924658,
+    "prefill_m4096_n4096_k4096_int8_perchannel_prepacked": 167921020,
 }
 
 
