@@ -372,8 +372,8 @@ def main():
                     "decode_packed_cold: the same launches over pre-packed weights)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM shards over n with no "
-              "exchange; see DESIGN.md).  Run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM would shard over the columns "
+              "of B with no exchange between GPUs).  Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch

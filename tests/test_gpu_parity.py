@@ -94,7 +94,7 @@ def test_power_of_two_scaling_commutes(af):
     assert np.array_equal(widen(c4), widen(c1) * 4.0)
 
 
-# ---------------------------------------------------------------------------- BASELINE configs
+# ---------------------------------------------------------------------------- the headline configurations
 
 def test_config1_golden(af, golden_dir):
     g = np.load(f"{golden_dir}/c1_seed0.npz")
