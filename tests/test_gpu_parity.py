@@ -158,6 +158,15 @@ def test_tiled_kernels_on_ragged_shapes(af, m, n, k, bits, group, tile):
     assert_close_ulp(p, run_gemm(p, which=af.PREFILL_256 if tile == 256 else af.PREFILL_128), f"tile {tile}: {m}x{n}x{k} bits={bits} g={group}")
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [(4160, 256, 256, 8, 0), (1000, 1008, 384, 4, 0), (300, 528, 512, 8, 64), (130, 4112, 256, 4, 128)])
+def test_tile_sizes_agree_bit_for_bit(af, m, n, k, bits, group):
+    """Both tiled kernels add the products of an output in the same order (ascending k through one chain of matrix
+    instructions per 64 rows of k), so they must agree in every bit, near-cancelling outputs included: an indexing
+    slip in either one shows here even where it would stay inside the 2-ULP bound."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    assert np.array_equal(run_gemm(p, which=af.PREFILL_128), run_gemm(p, which=af.PREFILL_256))
+
+
 def test_tiled_variant_picks_its_tile_size_by_shape(af):
     """PREFILL runs 128x128 tiles while m x n holds at most 256 of them, 256x256 tiles beyond; either way the result
     meets the oracle and is the forced form's, bit for bit."""

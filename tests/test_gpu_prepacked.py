@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import Problem, Workspace, assert_close_gated, assert_close_ulp, from_dev_u16, to_dev
+from helpers import Problem, Workspace, assert_close_gated, assert_close_ulp, from_dev_u16, run_gemm, to_dev
 
 _ws = Workspace()
 
@@ -131,6 +131,17 @@ def test_tiled_kernel_matches_oracle(af, m, n, k, bits, group, tile):
     assert_close_ulp(p, run_prepacked(af, p, which), f"packed prefill{tile} + bias {m}x{n}x{k} b{bits} g{group}")
     if tile == 128:
         assert np.array_equal(run_prepacked(af, p, which), run_prepacked(af, p, af.PREFILL)), "PREFILL picks 128x128 tiles here"
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [(4160, 256, 256, 8, 0), (1000, 1008, 384, 4, 0), (300, 528, 512, 8, 64), (130, 4112, 256, 4, 128)])
+def test_tile_sizes_and_weight_orders_agree_bit_for_bit(af, m, n, k, bits, group):
+    """The tiled kernels add an output's products in the same order whatever the tile size and whichever order the
+    weights are stored in: four launches, one result, bias included."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    want = run_gemm(p, which=af.PREFILL_256)
+    assert np.array_equal(run_prepacked(af, p, af.PREFILL_128), want) and np.array_equal(run_prepacked(af, p, af.PREFILL_256), want)
+    p.with_bias()
+    assert np.array_equal(run_prepacked(af, p, af.PREFILL_128), run_prepacked(af, p, af.PREFILL_256))
 
 
 @pytest.mark.parametrize("bits,group", [(8, 0), (4, 128)])
