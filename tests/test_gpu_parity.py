@@ -374,7 +374,8 @@ def test_hip_graph_replays_match_eager(af):
     synchronisations in between."""
     import torch
     from helpers import Workspace
-    shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (16, 768, 1024, 8, 0), (96, 512, 512, 8, 0)]
+    shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (16, 768, 1024, 8, 0), (96, 512, 512, 8, 0),
+              (4200, 272, 256, 8, 0), (4200, 1040, 128, 4, 64)]   # the tiled kernels: 128x128 tiles, 256x256 tiles (two launches)
     probs = [Problem(m, n, k, bits, g, seed=90 + i) for i, (m, n, k, bits, g) in enumerate(shapes)]
     eager = [run_gemm(p) for p in probs]
     ws = Workspace()
