@@ -409,6 +409,36 @@ def test_hip_graph_replays_match_eager(af):
         torch.cuda.synchronize()
 
 
+def test_two_streams_with_their_own_workspaces(af):
+    """Launches are stream-ordered and keep no state outside their arguments: GEMMs issued alternately on two streams,
+    each stream with its own workspace and output, give the single-stream results."""
+    import torch
+    shapes = [(1, 4096, 4096, 8, 0), (8, 1040, 4096, 4, 128), (200, 528, 1024, 8, 0), (4200, 272, 256, 8, 0)]
+    probs = [Problem(m, n, k, bits, g, seed=300 + i) for i, (m, n, k, bits, g) in enumerate(shapes)]
+    want = [run_gemm(p) for p in probs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    bufs = []
+    for si in range(2):
+        for p in probs:
+            need = af.workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size)
+            w = None if need == 0 else torch.empty(need, dtype=torch.uint8, device="cuda")
+            if need:
+                af.workspace_init(w)
+            bufs.append(dict(a=to_dev(p.a_bf), b=to_dev(p.b_bytes), s=to_dev(p.s_bf), w=w,
+                             c=torch.full((p.m, p.n), 0x7FC0, dtype=torch.int16, device="cuda")))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i, p in enumerate(probs):
+            for si, st in enumerate(streams):
+                d = bufs[si * len(probs) + i]
+                with torch.cuda.stream(st):
+                    af.gemm(d["c"], d["a"], d["b"], d["s"], p.m, p.n, p.k, weight_bits=p.bits, group_size=p.group_size, workspace=d["w"])
+    torch.cuda.synchronize()
+    for si in range(2):
+        for i in range(len(probs)):
+            assert np.array_equal(from_dev_u16(bufs[si * len(probs) + i]["c"]), want[i]), f"stream {si}, problem {i}"
+
+
 def test_empty_and_minimal_shapes(af):
     import torch
     p = Problem(1, 16, 64, seed=1)       # the smallest shape the library takes
