@@ -1,0 +1,66 @@
+"""Seeded random walk over the library's argument space: shapes, code widths, scale groups, weight orders, variants and
+epilogues drawn together, each case checked against the CPU oracle through the C ABI.  The directed tests cover the
+corners by design; this one covers combinations nobody thought of (it is deterministic: the seed is fixed)."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import Problem, assert_close_gated, assert_close_ulp, run_gemm
+from test_gpu_prepacked import run_prepacked
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def af():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a device"
+    import awesome_fusion_amd as af
+    af.lib()  # raises if the HIP library was not built: no fallback
+    return af
+
+
+def draw_case(rng):
+    bits = int(rng.choice([8, 4]))
+    packed = bool(rng.integers(0, 2))
+    kunit = 128 if (bits == 4 and packed) else 64
+    m = int(rng.choice([rng.integers(1, 9), rng.integers(9, 49), rng.integers(49, 200), rng.integers(200, 700)]))
+    kmax = 8192 if m < 49 else 1024               # long k with few rows: the split-K plans
+    k = kunit * int(rng.integers(1, kmax // kunit + 1))
+    n = 16 * int(rng.integers(1, 70))
+    groups = [g for g in (0, 32, 64, 128, 256) if g == 0 or k % g == 0]
+    group = int(rng.choice(groups))
+    epilogue = str(rng.choice(["none", "none", "none", "bias", "residual", "bias+residual", "gate", "gate+bias+residual"]))
+    if epilogue.startswith("gate") and n % 32:
+        n += 16                                   # the gated output has n/2 columns, itself a multiple of 16
+    variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256"]))
+    if epilogue != "none" and not (packed and epilogue == "bias"):
+        variant = "auto"                          # the fused entry points choose the kernel themselves
+    return dict(m=m, n=n, k=k, bits=bits, group=group, packed=packed, epilogue=epilogue, variant=variant)
+
+
+CASES = [draw_case(np.random.Generator(np.random.PCG64(1000 + i))) for i in range(300)]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "{m}x{n}x{k}-b{bits}-g{group}-{o}-{variant}-{epilogue}".format(o="packed" if c["packed"] else "rowmajor", **c))
+def test_random_case(af, case):
+    m, n, k, bits, group = case["m"], case["n"], case["k"], case["bits"], case["group"]
+    gated = case["epilogue"].startswith("gate")
+    if gated:
+        p = Problem(m, n, k, bits, group, seed=m + n + k, scale_lo=0.002, scale_hi=0.02 if bits == 8 else 0.2)
+    else:
+        p = Problem(m, n, k, bits, group, seed=m + n + k)
+    if "bias" in case["epilogue"]:
+        p.with_bias()
+    if "residual" in case["epilogue"]:
+        if gated:
+            p.residual_bf = oracle.f32_to_bf16_rne(np.random.default_rng(m).uniform(-2, 2, size=(m, n // 2)).astype(np.float32))
+        else:
+            p.with_residual()
+    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[case["variant"]]
+    act = af.ACT_SILU_GATE if gated else af.ACT_NONE
+    c = run_prepacked(af, p, which, activation=act) if case["packed"] else run_gemm(p, which=which, activation=act)
+    if gated:
+        assert_close_gated(p, c, str(case))
+    else:
+        assert_close_ulp(p, c, str(case))
