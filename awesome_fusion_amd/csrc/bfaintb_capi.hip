@@ -4,7 +4,6 @@
 // (gpu_utils.hpp:5-11, print and exit(0)) every failure is returned to the caller.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
 #include <string.h>
 
 #include "bfaintb_device.hpp"
@@ -33,7 +32,6 @@ using bfaintb::kEmptyWord;
 
 constexpr uint32_t kDecodeAutoMaxM = 32;       // AUTO always runs the decode family up to this m
 constexpr uint32_t kDecodeFamilyAutoMaxM = 4096;  // ... and never beyond this one
-constexpr double kFamilyMargin = 1.0;          // AUTO runs the decode family where its estimate, times this, is below the tiled variant's
 constexpr uint32_t kDecodeMaxM = 32768;        // what the decode family accepts when forced
 constexpr uint32_t kDecodeTargetWgs = 480;        // 4-wave workgroups: a little under two per CU on a 256-CU part
 constexpr uint32_t kDecodeTargetWgsNarrow = 256;  // 8-wave workgroups: one per CU
@@ -206,7 +204,7 @@ int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
         if (m <= kDecodeAutoMaxM) return BFAINTB_VARIANT_DECODE;
         if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
         const DecodePlan pl = decode_plan(m, n, k, bits, 0);
-        return decode_family_estimate_us(m, n, k, bits, pl) * kFamilyMargin < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+        return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     }
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
     if (is_prefill(variant)) return variant;
@@ -475,7 +473,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (m <= kPackedSlabMaxM) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = decode_plan(m, n, k, bits, 0);
-    return decode_family_estimate_us(m, n, k, bits, pl) * kFamilyMargin < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
