@@ -4,6 +4,7 @@
 // (gpu_utils.hpp:5-11, print and exit(0)) every failure is returned to the caller.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "bfaintb_device.hpp"
@@ -36,7 +37,7 @@ constexpr uint32_t kDecodeMaxM = 32768;        // what the decode family accepts
 constexpr uint32_t kDecodeTargetWgs = 480;        // 4-wave workgroups: a little under two per CU on a 256-CU part
 constexpr uint32_t kDecodeTargetWgsNarrow = 256;  // 8-wave workgroups: one per CU
 constexpr uint32_t kMaxSplits = 64;
-constexpr uint32_t kPackedSlabMaxM = 48;       // packed weights: the slab-streaming kernel up to this m, the row-blocked family beyond
+constexpr uint32_t kPackedSlabMaxM = 48;       // packed weights: the slab-streaming kernel never runs more rows of A than this
 
 int check_format(uint32_t k, int bits, uint32_t group_size)
 {
@@ -128,33 +129,38 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
     return 4.0 + rounds * (k / 64.0) * 1.33;
 }
 
+// The decode family in row blocks: grid z walks blocks of 16*mb rows.  128 columns x 64 rows (mb = 4, 4 waves: one
+// wave per SIMD, 128 accumulator registers) amortises the dequantisation best; smaller row blocks give more
+// workgroups when columns x row blocks alone do not fill the machine.  Picked by estimate.  (Columns per workgroup
+// are fixed by the code width here: what the kernels over packed weights need.)
+DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
+{
+    DecodePlan best{};
+    double best_t = 0.0;
+    for (uint32_t mb = bits == 8 ? 4u : 2u; mb >= 1u; mb >>= 1) {
+        DecodePlan c;
+        c.cols = bits == 8 ? 128u : 256u;
+        c.waves = (bits == 8 && mb <= 2u) ? 8u : 4u;
+        c.mb = mb;
+        const uint32_t tiles = ((n + c.cols - 1u) / c.cols) * ((m + 16u * mb - 1u) / (16u * mb));
+        for (uint32_t s = 1; s <= 16u; s += (s < 4u ? 1u : s < 8u ? 2u : 4u)) {
+            if (forced_splits && s != 1u) break;
+            set_splits(c, k, bits, forced_splits ? forced_splits : s);
+            if (!forced_splits && c.splits != s && s != 1u) continue;  // k does not divide that way
+            if (!forced_splits && s > 1u && tiles * s > 768u) break;
+            const double t = decode_family_estimate_us(m, n, k, bits, c);
+            if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
+        }
+    }
+    return best;
+}
+
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
 {
+    if (m > 32) return decode_plan_row_blocks(m, n, k, bits, forced_splits);  // more than 32 rows of A
     DecodePlan pl;
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
-    if (m > 32) {
-        // More than 32 rows of A: grid z walks blocks of 16*mb rows.  128 columns x 64 rows (mb = 4, 4 waves: one
-        // wave per SIMD, 128 accumulator registers) amortises the dequantisation best; smaller row blocks give
-        // more workgroups when columns x row blocks alone do not fill the machine.  Pick by estimate.
-        DecodePlan best{};
-        double best_t = 0.0;
-        for (uint32_t mb = bits == 8 ? 4u : 2u; mb >= 1u; mb >>= 1) {
-            DecodePlan c;
-            c.cols = bits == 8 ? 128u : 256u;
-            c.waves = (bits == 8 && mb <= 2u) ? 8u : 4u;
-            c.mb = mb;
-            const uint32_t tiles = ((n + c.cols - 1u) / c.cols) * ((m + 16u * mb - 1u) / (16u * mb));
-            for (uint32_t s = 1; s <= 16u; s += (s < 4u ? 1u : s < 8u ? 2u : 4u)) {
-                if (forced_splits && s != 1u) break;
-                set_splits(c, k, bits, forced_splits ? forced_splits : s);
-                if (!forced_splits && c.splits != s && s != 1u) continue;  // k does not divide that way
-                if (!forced_splits && s > 1u && tiles * s > 768u) break;
-                const double t = decode_family_estimate_us(m, n, k, bits, c);
-                if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
-            }
-        }
-        pl = best;
-    } else {
+    {
         // 8-bit codes, 128 columns x 8 waves ("narrow": a lane loads 8 bytes of a row, 16 lanes one 128-byte line)
         // needs half the splits of 256 columns x 4 waves ("wide") for the same number of waves, so half the
         // partial-sum traffic.  Narrow workgroups run one per CU, so they pay for a ragged last round of 256.
@@ -463,14 +469,45 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
                                               weight_bits == 8 ? ldb : ldb / 2u, weight_bits, static_cast<hipStream_t>(stream));
 }
 
-// Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one up to kPackedSlabMaxM rows of A, the
+// Packed weights, "DECODE": the slab-streaming kernel (one workgroup per 16 columns over all of k, no split, every block
+// of 16 rows of A converts the slab again) or the decode family reading packed slabs (128 or 256 columns per workgroup,
+// split along k).  The slab kernel wins while the rows are few; how few depends on how much there is to convert again.
+// Measured, slab / family in us — 4096 x 4096: m = 16: 7.5 / 12.5, 48: 15.3 / 19.7; 11008 x 4096: m = 24: 21.6 / 22.3,
+// 32: 25.5 / 23.0, 48: 39.5 / 26.3; 8192 x 8192, 4-bit: m = 16: 19.0 / 23.6, 32: 34.1 / 28.9; 28672 x 8192, 4-bit:
+// m = 12: 47.6 / 49.2, 16: 56.7 / 50.0, 32: 105.7 / 58.6.
+static uint32_t packed_slab_max_m(uint32_t n, uint32_t k)
+{
+#ifdef BFAINTB_TUNE
+    if (const char* e = getenv("BFAINTB_SLABMAX")) return (uint32_t)atoi(e);
+#endif
+    const uint64_t weights = (uint64_t)n * k;
+    return weights <= (24ull << 20) ? kPackedSlabMaxM : weights <= (128ull << 20) ? 24u : 12u;
+}
+static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k)
+{
+    return m <= packed_slab_max_m(n, k);
+}
+
+// The family's plan over packed weights.  8-bit codes: the one row-major weights get, as long as it uses the 128 columns
+// per workgroup the packed kernels are built for.  4-bit codes: the row-block plan also below 33 rows of A (measured
+// against the small-m plan: 8192 x 8192, m = 32: 28.9 / 36.4 us; 28672 x 8192, m = 24: 56.9 / 65.6 us).
+static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bits)
+{
+    if (bits == 8) {
+        const DecodePlan pl = decode_plan(m, n, k, bits, 0);
+        if (pl.cols == 128u) return pl;
+    }
+    return decode_plan_row_blocks(m, n, k, bits, 0);
+}
+
+// Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the
 // row-blocked family without a split along k beyond) or the tiled kernel, by the estimates that choose for row-major weights.
 static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
     if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
-    if (m <= kPackedSlabMaxM) return BFAINTB_VARIANT_DECODE;
+    if (packed_uses_slab(m, n, k)) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = decode_plan(m, n, k, bits, 0);
     return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
@@ -487,11 +524,13 @@ int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weigh
     return packed_variant(m, n, k, weight_bits, BFAINTB_VARIANT_AUTO);
 }
 
-// Scratch of the packed path: only the row-blocked decode family (more than kPackedSlabMaxM rows of A) splits along k.
+// Scratch of the packed path: only the decode family (where the slab kernel is not used) splits along k.
 static size_t packed_workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int v)
 {
-    if (v != BFAINTB_VARIANT_DECODE || m <= kPackedSlabMaxM) return 0;
-    return workspace_need(m, n, k, bits, BFAINTB_VARIANT_DECODE, 0);
+    if (v != BFAINTB_VARIANT_DECODE || m == 0 || n == 0 || packed_uses_slab(m, n, k)) return 0;
+    const DecodePlan pl = packed_family_plan(m, n, k, bits);
+    if (pl.splits <= 1) return 0;
+    return (((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u;
 }
 
 size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant)
@@ -547,12 +586,12 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st);
     }
-    if (m > kPackedSlabMaxM) {
+    if (!packed_uses_slab(m, n, k)) {
         // beyond a few dozen rows the row-blocked decode family (A reused across 128 or 256 columns) reads the packed
         // slabs: measured at n = k = 4096 and m = 64, 128, 256: 16, 20, 22 us against 18, 34, 63 us for the slab kernel.
         // Same plan as for row-major weights, split along k and workspace protocol included.
         if (m > kDecodeMaxM) return BFAINTB_ERR_BAD_VARIANT;
-        const DecodePlan pl = decode_plan(m, n, k, weight_bits, 0);
+        const DecodePlan pl = packed_family_plan(m, n, k, weight_bits);
         p.k_per_wg = pl.k_per_wg;
         p.splits = pl.splits;
         p.decode_waves = pl.waves;
