@@ -60,10 +60,10 @@ struct DecodePlan {
 };
 
 // Rows of k per workgroup and the number of splits that results, for `splits` wanted.
-static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits)
+static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bool packed = false)
 {
     // rows one workgroup covers per pipeline step of its waves
-    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16) * pl.waves;
+    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16, packed) * pl.waves;
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
     uint32_t per = (k + splits - 1) / splits;
@@ -133,7 +133,7 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
 // wave per SIMD, 128 accumulator registers) amortises the dequantisation best; smaller row blocks give more
 // workgroups when columns x row blocks alone do not fill the machine.  Picked by estimate.  (Columns per workgroup
 // are fixed by the code width here: what the kernels over packed weights need.)
-DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
+DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
 {
     DecodePlan best{};
     double best_t = 0.0;
@@ -145,7 +145,7 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
         const uint32_t tiles = ((n + c.cols - 1u) / c.cols) * ((m + 16u * mb - 1u) / (16u * mb));
         for (uint32_t s = 1; s <= 16u; s += (s < 4u ? 1u : s < 8u ? 2u : 4u)) {
             if (forced_splits && s != 1u) break;
-            set_splits(c, k, bits, forced_splits ? forced_splits : s);
+            set_splits(c, k, bits, forced_splits ? forced_splits : s, packed);
             if (!forced_splits && c.splits != s && s != 1u) continue;  // k does not divide that way
             if (!forced_splits && s > 1u && tiles * s > 768u) break;
             const double t = decode_family_estimate_us(m, n, k, bits, c);
@@ -497,7 +497,7 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
         const DecodePlan pl = decode_plan(m, n, k, bits, 0);
         if (pl.cols == 128u) return pl;
     }
-    return decode_plan_row_blocks(m, n, k, bits, 0);
+    return decode_plan_row_blocks(m, n, k, bits, 0, true);
 }
 
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the

@@ -129,6 +129,19 @@ __device__ __forceinline__ void load_packed(PackedStep<BITS, CPL>& raw, const ui
     }
 }
 
+// 4-bit codes, two neighbouring K-blocks (the first one even) with one 8-byte load per column block
+template <int CPL>
+__device__ __forceinline__ void load_packed_pair(PackedStep<4, CPL>& first, PackedStep<4, CPL>& second, const uint8_t* const (&slab)[CPL],
+                                                 size_t lane_off)
+{
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const uint2 v = *reinterpret_cast<const uint2*>(slab[c] + lane_off);
+        first.d[c][0] = v.x;
+        second.d[c][0] = v.y;
+    }
+}
+
 template <int BITS, int CPL, int MB>
 __device__ __forceinline__ void mac_step_packed(const PackedStep<BITS, CPL>& raw, const float (&cs)[CPL], const uint4 (&afrag)[MB],
                                                 f32x4_t (&acc)[MB][CPL])
@@ -327,10 +340,12 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 // REF: the reference kernel's arithmetic (p.reference_arith): p.scale holds one fp32 scale per column, W is narrowed by
 // truncation.
 template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED, bool REF>
-__global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256) bfaintb_decode_kernel(const GemmParams p)
+// (packed 4-bit codes always run 4 waves, and their two K-blocks per step want the registers of a 256-thread bound)
+__global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED && BITS == 4)) ? 512 : 256)
+bfaintb_decode_kernel(const GemmParams p)
 {
     static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
-    constexpr int KB = decode_blocks_per_step(BITS, CPL);  // blocks of 32 rows per pipeline step
+    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED);  // blocks of 32 rows per pipeline step
     constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
     constexpr uint32_t kRedStride = kCols + 4u;       // floats per row of a wave's tile in LDS (+4: spreads rows over banks)
     constexpr uint32_t kLaneBytes = CPL * BITS / 8;   // bytes of one row a lane loads
@@ -423,7 +438,14 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1)) ? 512 : 256
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
                 const size_t blk = (size_t)step * KB + q;
-                if constexpr (PACKED) {
+                if constexpr (PACKED && KB == 2) {
+                    // the step's two K-blocks (an even one and its successor) lie side by side in a lane's share of the chunk
+                    if (q == 0) {
+                        const uint32_t kblock = kblock0 + (uint32_t)blk;
+                        load_packed_pair<CPL>(st.raw[0], st.raw[1], slab,
+                                              (size_t)(kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
+                    }
+                } else if constexpr (PACKED) {
                     const uint32_t kblock = kblock0 + (uint32_t)blk;
                     load_packed<BITS, CPL>(st.raw[q], slab, (size_t)(kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
                 } else {
@@ -604,7 +626,7 @@ static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
     constexpr uint32_t kCols = 16u * CPL;
     constexpr uint32_t kRows = 16u * MB;
     const uint32_t waves = p.decode_waves;
-    if (MB > 2 && waves != 4u) return hipErrorInvalidValue;  // MB = 4 needs the register budget of one wave per SIMD
+    if ((MB > 2 || (PACKED && BITS == 4)) && waves != 4u) return hipErrorInvalidValue;  // kernels compiled for 256 threads
     const dim3 grid((p.n + kCols - 1u) / kCols, p.splits, (p.m + kRows - 1u) / kRows);
     if (grid.z > 65535u) return hipErrorInvalidValue;
     const uint32_t pass_rows = 16u * (uint32_t)decode_rows16_per_pass(CPL, MB);

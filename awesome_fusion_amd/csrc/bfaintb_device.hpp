@@ -48,9 +48,10 @@ inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 }
 
 // Decode variant: blocks of 32 rows of k a wave loads per pipeline step (cpl = weights per lane and
-// row).  Two blocks for the 8-byte-per-row layouts measured no faster than one: more bytes in flight
-// per wave, fewer waves per CU.
-__host__ __device__ constexpr int decode_blocks_per_step(int /*bits*/, int /*cpl*/) { return 1; }
+// row).  Row-major weights: one; two blocks for the 8-byte-per-row layouts measured no faster (more bytes in
+// flight per wave, fewer waves per CU).  Packed 4-bit codes: two, so that a lane fetches 8 bytes per column block
+// (half of its 128-row chunk) instead of 4.
+__host__ __device__ constexpr int decode_blocks_per_step(int bits, int /*cpl*/, bool packed) { return (packed && bits == 4) ? 2 : 1; }
 
 struct GemmParams {
     uint16_t* c;
