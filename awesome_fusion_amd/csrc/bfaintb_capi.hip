@@ -157,7 +157,9 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
 
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
 {
-    if (m > 32) return decode_plan_row_blocks(m, n, k, bits, forced_splits);  // more than 32 rows of A
+    // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
+    // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
+    if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits);
     DecodePlan pl;
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     {
@@ -171,6 +173,9 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         // the split-K partial sums (written, read back and cleared as fp32) stay below a quarter of the weight bytes
         uint32_t cap = (uint32_t)(((uint64_t)k * (uint32_t)bits) / (256u * (m ? m : 1u)));
         if (cap < 1) cap = 1;
+        // ... unless the weights are few: such launches are bound by latency, not by traffic, and want workgroups
+        // (n = k = 4096, m = 32: 10.7 us with 8 splits against 12.6 us with 4; 16 splits are slower again)
+        if (few && cap < 8u) cap = 8u;
         // narrow, large matrix: every further split costs traffic and a longer reduction; whole rounds count
         const uint32_t narrow_blocks = (n + 127u) / 128u;
         uint32_t narrow_splits = 1;
