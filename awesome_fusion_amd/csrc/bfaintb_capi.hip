@@ -63,7 +63,7 @@ struct DecodePlan {
 static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bool packed = false)
 {
     // rows one workgroup covers per pipeline step of its waves
-    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16, packed) * pl.waves;
+    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16, packed, (int)pl.mb) * pl.waves;
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
     uint32_t per = (k + splits - 1) / splits;
@@ -173,11 +173,11 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
     return best;
 }
 
-DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
+DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
 {
     // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
     // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
-    if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits);
+    if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed);
     DecodePlan pl;
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     {
@@ -220,7 +220,7 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 if (splits > cap) splits = cap;
             }
         }
-        set_splits(pl, k, bits, splits);
+        set_splits(pl, k, bits, splits, packed);
     }
     return pl;
 }
@@ -517,7 +517,7 @@ static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k)
 static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
     if (bits == 8) {
-        const DecodePlan pl = decode_plan(m, n, k, bits, 0);
+        const DecodePlan pl = decode_plan(m, n, k, bits, 0, true);
         if (pl.cols == 128u) return pl;
     }
     return decode_plan_row_blocks(m, n, k, bits, 0, true);
@@ -532,7 +532,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
     if (packed_uses_slab(m, n, k)) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
-    const DecodePlan pl = decode_plan(m, n, k, bits, 0);
+    const DecodePlan pl = packed_family_plan(m, n, k, bits);
     return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 

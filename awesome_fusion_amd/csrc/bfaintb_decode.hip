@@ -129,16 +129,22 @@ __device__ __forceinline__ void load_packed(PackedStep<BITS, CPL>& raw, const ui
     }
 }
 
-// 4-bit codes, two neighbouring K-blocks (the first one even) with one 8-byte load per column block
-template <int CPL>
-__device__ __forceinline__ void load_packed_pair(PackedStep<4, CPL>& first, PackedStep<4, CPL>& second, const uint8_t* const (&slab)[CPL],
+// Two neighbouring K-blocks (the first one even) with one load per column block: 16 bytes (8-bit codes) or 8 (4-bit)
+template <int BITS, int CPL>
+__device__ __forceinline__ void load_packed_pair(PackedStep<BITS, CPL>& first, PackedStep<BITS, CPL>& second, const uint8_t* const (&slab)[CPL],
                                                  size_t lane_off)
 {
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
-        const uint2 v = *reinterpret_cast<const uint2*>(slab[c] + lane_off);
-        first.d[c][0] = v.x;
-        second.d[c][0] = v.y;
+        if constexpr (BITS == 8) {
+            const uint4 v = *reinterpret_cast<const uint4*>(slab[c] + lane_off);
+            first.d[c][0] = v.x; first.d[c][1] = v.y;
+            second.d[c][0] = v.z; second.d[c][1] = v.w;
+        } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(slab[c] + lane_off);
+            first.d[c][0] = v.x;
+            second.d[c][0] = v.y;
+        }
     }
 }
 
@@ -345,7 +351,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED 
 bfaintb_decode_kernel(const GemmParams p)
 {
     static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
-    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED);  // blocks of 32 rows per pipeline step
+    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED, MB);  // blocks of 32 rows per pipeline step
     constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
     constexpr uint32_t kRedStride = kCols + 4u;       // floats per row of a wave's tile in LDS (+4: spreads rows over banks)
     constexpr uint32_t kLaneBytes = CPL * BITS / 8;   // bytes of one row a lane loads
@@ -442,7 +448,7 @@ bfaintb_decode_kernel(const GemmParams p)
                     // the step's two K-blocks (an even one and its successor) lie side by side in a lane's share of the chunk
                     if (q == 0) {
                         const uint32_t kblock = kblock0 + (uint32_t)blk;
-                        load_packed_pair<CPL>(st.raw[0], st.raw[1], slab,
+                        load_packed_pair<BITS, CPL>(st.raw[0], st.raw[1], slab,
                                               (size_t)(kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
                     }
                 } else if constexpr (PACKED) {

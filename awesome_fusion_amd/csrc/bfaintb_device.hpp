@@ -49,9 +49,15 @@ inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 
 // Decode variant: blocks of 32 rows of k a wave loads per pipeline step (cpl = weights per lane and
 // row).  Row-major weights: one; two blocks for the 8-byte-per-row layouts measured no faster (more bytes in
-// flight per wave, fewer waves per CU).  Packed 4-bit codes: two, so that a lane fetches 8 bytes per column block
-// (half of its 128-row chunk) instead of 4.
-__host__ __device__ constexpr int decode_blocks_per_step(int bits, int /*cpl*/, bool packed) { return (packed && bits == 4) ? 2 : 1; }
+// flight per wave, fewer waves per CU).  Packed weights: two, so that a lane fetches its two neighbouring K-blocks of a
+// column block with one load (16 bytes for 8-bit codes: its whole share of a 64-row chunk; 8 bytes for 4-bit codes:
+// half of its share of a 128-row chunk) instead of two loads of half a sector each.
+// (Not for 8-bit codes with two blocks of 16 rows of A per workgroup: that kernel runs 8 waves on 256 registers each, and the
+// second K-block in flight would spill.)
+__host__ __device__ constexpr int decode_blocks_per_step(int bits, int /*cpl*/, bool packed, int mb)
+{
+    return (packed && !(bits == 8 && mb == 2)) ? 2 : 1;
+}
 
 struct GemmParams {
     uint16_t* c;
