@@ -494,21 +494,24 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
 
 // Packed weights, "DECODE": the slab-streaming kernel (one workgroup per 16 columns over all of k, no split, every block
 // of 16 rows of A converts the slab again) or the decode family reading packed slabs (128 or 256 columns per workgroup,
-// split along k).  The slab kernel wins while the rows are few; how few depends on how much there is to convert again.
-// Measured, slab / family in us — 4096 x 4096: m = 16: 7.5 / 12.5, 48: 15.3 / 19.7; 11008 x 4096: m = 24: 21.6 / 22.3,
-// 32: 25.5 / 23.0, 48: 39.5 / 26.3; 8192 x 8192, 4-bit: m = 16: 19.0 / 23.6, 32: 34.1 / 28.9; 28672 x 8192, 4-bit:
-// m = 12: 47.6 / 49.2, 16: 56.7 / 50.0, 32: 105.7 / 58.6.
-static uint32_t packed_slab_max_m(uint32_t n, uint32_t k)
+// split along k).  The slab kernel wins while the rows are few.  Measured, slab / family in us —
+// 8-bit codes: m = 8 is the slab kernel's everywhere; at m = 12, 16, 32: 4096 x 4096 6.2 / 9.0, 6.9 / 9.5, 10.7 / 12.1
+// (48: 15.6 / 13.6), but 5120 x 5120 14.0 / 10.5, 15.9 / 10.7, 22.8 / 15.8; 32000 x 4096 35.3 / 25.7, 38.3 / 25.1,
+// 63.2 / 35.1; 8192 x 8192 22.5 / 21.4, 22.6 / 21.3, 33.6 / 29.4: beyond 8 rows only the matrix whose 256 slabs make
+// exactly one round of workgroups keeps the slab kernel.
+// 4-bit codes: 8192 x 8192: m = 16: 19.0 / 23.6, 32: 34.1 / 28.9; 28672 x 8192: m = 12: 47.6 / 49.2, 16: 56.7 / 50.0.
+static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
 {
 #ifdef BFAINTB_TUNE
     if (const char* e = getenv("BFAINTB_SLABMAX")) return (uint32_t)atoi(e);
 #endif
     const uint64_t weights = (uint64_t)n * k;
+    if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : 8u;
     return weights <= (24ull << 20) ? kPackedSlabMaxM : weights <= (128ull << 20) ? 24u : 12u;
 }
-static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k)
+static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
-    return m <= packed_slab_max_m(n, k);
+    return m <= packed_slab_max_m(n, k, bits);
 }
 
 // The family's plan over packed weights.  8-bit codes: the one row-major weights get, as long as it uses the 128 columns
@@ -530,7 +533,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
     if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
-    if (packed_uses_slab(m, n, k)) return BFAINTB_VARIANT_DECODE;
+    if (packed_uses_slab(m, n, k, bits)) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
     return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
@@ -550,7 +553,7 @@ int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weigh
 // Scratch of the packed path: only the decode family (where the slab kernel is not used) splits along k.
 static size_t packed_workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int v)
 {
-    if (v != BFAINTB_VARIANT_DECODE || m == 0 || n == 0 || packed_uses_slab(m, n, k)) return 0;
+    if (v != BFAINTB_VARIANT_DECODE || m == 0 || n == 0 || packed_uses_slab(m, n, k, bits)) return 0;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
     if (pl.splits <= 1) return 0;
     return (((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u;
@@ -609,7 +612,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st);
     }
-    if (!packed_uses_slab(m, n, k)) {
+    if (!packed_uses_slab(m, n, k, weight_bits)) {
         // beyond a few dozen rows the row-blocked decode family (A reused across 128 or 256 columns) reads the packed
         // slabs: measured at n = k = 4096 and m = 64, 128, 256: 16, 20, 22 us against 18, 34, 63 us for the slab kernel.
         // Same plan as for row-major weights, split along k and workspace protocol included.

@@ -33,7 +33,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 106 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 107 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -169,8 +169,8 @@ BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, 
  * order of the matrix instruction ("mfma16": column blocks of 16, K-chunks of 64 rows, a lane's two 8-row operands
  * adjacent; bfaintb_packed.hip states it byte by byte); bfaintb_gemm_prepacked multiplies by the packed copy.  A
  * block of 16 columns is then one contiguous slab, n / 16 workgroups stream their slabs linearly and own their
- * outputs, and a few rows of A (up to 48 against 16 Mi weights, up to 12 against more than 128 Mi) need no split
- * along k, no workspace and no second pass.  Successor of the
+ * outputs, and a few rows of A (8 in general; more on small matrices and for 4-bit codes) need no split along k, no workspace
+ * and no second pass.  Successor of the
  * reference's host-side formatter mem_transfer<int8_t, ...> (include/mem_transfer.hpp:23-32), which writes the
  * bytes the device will read; the reference itself keeps B row-major (bfAintBGemm.cc:101-103).
  *   packed    device buffer of bfaintb_prepack_bytes(n, k, weight_bits) bytes (= n * k * weight_bits / 8), 16-byte aligned;
@@ -194,8 +194,8 @@ BFAINTB_API int bfaintb_gemm_prepacked(void* c, const void* a, const void* packe
 BFAINTB_API int bfaintb_gemm_prepacked_fused(void* c, const void* a, const void* packed_b, const void* scale,
                                  const bfaintb_epilogue* epilogue, uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc,
                                  int weight_bits, uint32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
-/* Scratch bfaintb_gemm_prepacked needs: 0 where the slab-streaming kernel runs (m <= 48 while n * k <= 24 Mi, m <= 24 up
- * to 128 Mi, m <= 12 beyond) and for the tiled kernels; in between, what the decode family needs when it splits along k:
+/* Scratch bfaintb_gemm_prepacked needs: 0 where the slab-streaming kernel runs (8-bit codes: m <= 8, m <= 32 when n * k <= 16 Mi and
+ * n >= 4096; 4-bit codes: m <= 48 while n * k <= 24 Mi, m <= 24 up to 128 Mi, m <= 12 beyond) and for the tiled kernels; in between, what the decode family needs when it splits along k:
  * always ask, for the shape at hand.  Same workspace protocol as bfaintb_gemm
  * (bfaintb_workspace_init once; one workspace may serve both entry points). */
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);

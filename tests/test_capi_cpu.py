@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
-    assert af.lib().bfaintb_version() == 106
+    assert af.lib().bfaintb_version() == 107
     assert "bfaintb_gemm_bias" in names
 
 
