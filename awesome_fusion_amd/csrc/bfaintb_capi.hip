@@ -63,7 +63,7 @@ struct DecodePlan {
 static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bool packed = false)
 {
     // rows one workgroup covers per pipeline step of its waves
-    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16, packed, (int)pl.mb) * pl.waves;
+    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16, packed) * pl.waves;
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
     uint32_t per = (k + splits - 1) / splits;

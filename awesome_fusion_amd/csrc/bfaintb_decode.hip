@@ -116,7 +116,7 @@ struct PackedStep {
 
 // lane_off: where this lane's codes of the K-block sit inside a column block's slab; slab[c]: the slab of column block c
 template <int BITS, int CPL>
-__device__ __forceinline__ void load_packed(PackedStep<BITS, CPL>& raw, const uint8_t* const (&slab)[CPL], size_t lane_off)
+__device__ __forceinline__ void load_packed(PackedStep<BITS, CPL>& raw, const uint8_t* const (&slab)[CPL], uint32_t lane_off)
 {
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
@@ -132,7 +132,7 @@ __device__ __forceinline__ void load_packed(PackedStep<BITS, CPL>& raw, const ui
 // Two neighbouring K-blocks (the first one even) with one load per column block: 16 bytes (8-bit codes) or 8 (4-bit)
 template <int BITS, int CPL>
 __device__ __forceinline__ void load_packed_pair(PackedStep<BITS, CPL>& first, PackedStep<BITS, CPL>& second, const uint8_t* const (&slab)[CPL],
-                                                 size_t lane_off)
+                                                 uint32_t lane_off)
 {
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
@@ -351,7 +351,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED 
 bfaintb_decode_kernel(const GemmParams p)
 {
     static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
-    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED, MB);  // blocks of 32 rows per pipeline step
+    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED);  // blocks of 32 rows per pipeline step
     constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
     constexpr uint32_t kRedStride = kCols + 4u;       // floats per row of a wave's tile in LDS (+4: spreads rows over banks)
     constexpr uint32_t kLaneBytes = CPL * BITS / 8;   // bytes of one row a lane loads
@@ -397,7 +397,7 @@ bfaintb_decode_kernel(const GemmParams p)
         for (int c = 0; c < CPL; ++c) {
             uint32_t gb = cb * CPL + (uint32_t)c;
             if (gb >= nblocks) gb = nblocks - 1u;
-            slab[c] = p.b + (size_t)gb * slab_bytes + (size_t)lane * 16u;
+            slab[c] = p.b + (size_t)gb * slab_bytes;  // the same for every lane: scalar registers; the lane's share is in the offset
             pk_col[c] = 16u * gb + (uint32_t)nl;
         }
     }
@@ -449,11 +449,12 @@ bfaintb_decode_kernel(const GemmParams p)
                     if (q == 0) {
                         const uint32_t kblock = kblock0 + (uint32_t)blk;
                         load_packed_pair<BITS, CPL>(st.raw[0], st.raw[1], slab,
-                                              (size_t)(kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
+                                                    (uint32_t)lane * 16u + (kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
                     }
                 } else if constexpr (PACKED) {
                     const uint32_t kblock = kblock0 + (uint32_t)blk;
-                    load_packed<BITS, CPL>(st.raw[q], slab, (size_t)(kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
+                    load_packed<BITS, CPL>(st.raw[q], slab,
+                                           (uint32_t)lane * 16u + (kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
                 } else {
                     load_raw<BITS, CPL>(st.raw[q], bptr + blk * bstep, p.ldb_bytes);
                 }

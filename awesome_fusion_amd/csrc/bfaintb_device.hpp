@@ -52,12 +52,7 @@ inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 // flight per wave, fewer waves per CU).  Packed weights: two, so that a lane fetches its two neighbouring K-blocks of a
 // column block with one load (16 bytes for 8-bit codes: its whole share of a 64-row chunk; 8 bytes for 4-bit codes:
 // half of its share of a 128-row chunk) instead of two loads of half a sector each.
-// (Not for 8-bit codes with two blocks of 16 rows of A per workgroup: that kernel runs 8 waves on 256 registers each, and the
-// second K-block in flight would spill.)
-__host__ __device__ constexpr int decode_blocks_per_step(int bits, int /*cpl*/, bool packed, int mb)
-{
-    return (packed && !(bits == 8 && mb == 2)) ? 2 : 1;
-}
+__host__ __device__ constexpr int decode_blocks_per_step(int /*bits*/, int /*cpl*/, bool packed) { return packed ? 2 : 1; }
 
 struct GemmParams {
     uint16_t* c;
