@@ -499,15 +499,17 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
 // (48: 15.6 / 13.6), but 5120 x 5120 14.0 / 10.5, 15.9 / 10.7, 22.8 / 15.8; 32000 x 4096 35.3 / 25.7, 38.3 / 25.1,
 // 63.2 / 35.1; 8192 x 8192 22.5 / 21.4, 22.6 / 21.3, 33.6 / 29.4: beyond 8 rows only the matrix whose 256 slabs make
 // exactly one round of workgroups keeps the slab kernel.
-// 4-bit codes: 8192 x 8192: m = 16: 19.0 / 23.6, 32: 34.1 / 28.9; 28672 x 8192: m = 12: 47.6 / 49.2, 16: 56.7 / 50.0.
+// 4-bit codes: 48 rows up to 24 Mi weights (4096 x 4096, m = 16: 6.5 us, the family 9 and more), 24 below 64 Mi (4096 x
+// 11008: m = 20: 20.8 / 23.6, 24: 22.3 / 23.5), 16 at 64 Mi (8192 x 8192: m = 20: 26.5 / 25.9), 8 beyond (32000 x 4096:
+// m = 12: 28.0 / 26.4; 28672 x 8192: m = 12: 44.5 / 39.9).
 static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
 {
 #ifdef BFAINTB_TUNE
     if (const char* e = getenv("BFAINTB_SLABMAX")) return (uint32_t)atoi(e);
 #endif
     const uint64_t weights = (uint64_t)n * k;
-    if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : 8u;
-    return weights <= (24ull << 20) ? kPackedSlabMaxM : weights <= (128ull << 20) ? 24u : 12u;
+    if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
+    return weights <= (24ull << 20) ? kPackedSlabMaxM : weights < (64ull << 20) ? 24u : weights == (64ull << 20) ? 16u : 8u;
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
