@@ -2,6 +2,7 @@
 """Benchmark of the bfAintBGemm hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+    python bench.py --scan        (a map of kernel times over shapes and m, not the benchmark)
 
 A step is one GEMM launch through the C ABI on synthetic, seeded inputs already resident in HBM.
 The headline workload is the decode shape the metric is quoted on (bf16 A [1,4096] x int8 B
@@ -302,6 +303,34 @@ def roofline_entry(w, ms, bound, suffix=""):
             "algorithmic_bytes": w.bytes, "flops": w.flops}
 
 
+SCAN_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (8192, 8192), (28672, 8192), (2048, 8192), (32000, 4096)]   # (n, k)
+SCAN_M = [1, 4, 8, 16, 24, 32, 48, 64, 128, 256, 512, 1024, 2048]
+
+
+def scan():
+    """Kernel time of bfaintb_gemm and bfaintb_gemm_prepacked, variant left to the library, over SCAN_SHAPES x {8-bit per
+    channel, 4-bit group 128} x SCAN_M.  Up to 32 rows of A the launches rotate over copies of B that exceed the last-level
+    cache (the decode protocol of the headline figure); beyond, two copies.  Not a roofline statement: a map to read
+    anomalies from (a time that falls as m grows, a weight order that loses to the other)."""
+    import torch
+    import awesome_fusion_amd as af
+    af.lib()
+    for (n, k) in SCAN_SHAPES:
+        for (bits, group) in ((8, 0), (4, 128)):
+            row = {"n": n, "k": k, "weight_bits": bits, "group_size": group, "m": SCAN_M, "row_major_us": [], "prepacked_us": []}
+            for m in SCAN_M:
+                b_bytes = n * k * bits // 8
+                copies = max(2, min(40, (640 << 20) // b_bytes)) if m <= 32 else 2
+                w = Workload(f"scan_m{m}_n{n}_k{k}_b{bits}", m, n, k, bits, group, copies=copies)
+                steps = 100 if m <= 64 else 20
+                for packed in (False, True):
+                    ev_ms, _ = time_graph(af, w, steps, 5, rotate=True, packed=packed)
+                    row["prepacked_us" if packed else "row_major_us"].append(round(ev_ms * 1e3, 2))
+                del w
+                torch.cuda.empty_cache()
+            print(json.dumps(row), flush=True)
+
+
 def cpu_baseline(w, c_gpu_f32, budget_s=12.0):
     """host_ref.hpp's gemm_rrr timed on this machine's cores on the same inputs the GPU consumed:
     the reference's own compiled routine when the wrapper library is present, else the C port."""
@@ -366,6 +395,8 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (decode sweep, int4 group-128)")
+    ap.add_argument("--scan", action="store_true", help="instead of the benchmark: what the library's own choice of kernel takes over a grid of "
+                    "matrix shapes, code widths and m, row-major and pre-packed weights; one JSON line per matrix")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload family: decode | prefill | decode_cold | decode_packed_cold "
                     "(decode_cold: nothing but the headline's cold-B launches, for a kernel trace without the hot and eager variants; "
@@ -375,6 +406,9 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM would shard over the columns "
               "of B with no exchange between GPUs).  Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    if args.scan:
+        scan()
+        return
 
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
