@@ -20,6 +20,35 @@ def af():
     return af
 
 
+def run_strided(af, p, which, act, packed, pad):
+    """The same product with lda = k + pad, ldc = ldr = columns + pad; the padding of C must come back untouched."""
+    import torch
+    from helpers import Workspace, from_dev_u16, to_dev
+    out_n = p.n // 2 if act else p.n
+    a = np.full((p.m, p.k + pad), 0x7FC0, np.uint16)          # NaN in the padding: it must never be read as data
+    a[:, :p.k] = p.a_bf
+    res = None
+    if p.residual_bf is not None:
+        r = np.full((p.m, out_n + pad), 0x7FC0, np.uint16)
+        r[:, :out_n] = p.residual_bf
+        res = to_dev(r)
+    c = torch.full((p.m, out_n + pad), 0x7FC1, dtype=torch.int16, device="cuda")
+    bias = None if p.bias_bf is None else to_dev(p.bias_bf)
+    kw = dict(weight_bits=p.bits, group_size=p.group_size, bias=bias, residual=res, ldr=None if res is None else out_n + pad, activation=act)
+    if packed:
+        pk = torch.zeros(af.prepack_bytes(p.n, p.k, p.bits), dtype=torch.uint8, device="cuda")
+        af.prepack(pk, to_dev(p.b_bytes), p.n, p.k, weight_bits=p.bits)
+        ws = Workspace().get(af.prepacked_workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size, which))
+        af.gemm_prepacked(c, to_dev(a), pk, to_dev(p.s_bf), p.m, p.n, p.k, lda=p.k + pad, ldc=out_n + pad, workspace=ws, which=which, **kw)
+    else:
+        ws = Workspace().get(af.workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size, which))
+        af.gemm(c, to_dev(a), to_dev(p.b_bytes), to_dev(p.s_bf), p.m, p.n, p.k, lda=p.k + pad, ldc=out_n + pad, workspace=ws, which=which, **kw)
+    torch.cuda.synchronize()
+    got = from_dev_u16(c)
+    assert np.all(got[:, out_n:] == 0x7FC1), "padding of C was written"
+    return np.ascontiguousarray(got[:, :out_n])
+
+
 def draw_case(rng):
     bits = int(rng.choice([8, 4]))
     packed = bool(rng.integers(0, 2))
@@ -36,7 +65,8 @@ def draw_case(rng):
     variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256"]))
     if epilogue != "none" and not (packed and epilogue == "bias"):
         variant = "auto"                          # the fused entry points choose the kernel themselves
-    return dict(m=m, n=n, k=k, bits=bits, group=group, packed=packed, epilogue=epilogue, variant=variant)
+    pad = int(rng.choice([0, 0, 8, 24]))           # extra elements per row of A, C (and the residual): strided operands
+    return dict(m=m, n=n, k=k, bits=bits, group=group, packed=packed, epilogue=epilogue, variant=variant, pad=pad)
 
 
 CASES = [draw_case(np.random.Generator(np.random.PCG64(1000 + i))) for i in range(300)]
@@ -59,7 +89,10 @@ def test_random_case(af, case):
             p.with_residual()
     which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[case["variant"]]
     act = af.ACT_SILU_GATE if gated else af.ACT_NONE
-    c = run_prepacked(af, p, which, activation=act) if case["packed"] else run_gemm(p, which=which, activation=act)
+    if case["pad"]:
+        c = run_strided(af, p, which, act, case["packed"], case["pad"])
+    else:
+        c = run_prepacked(af, p, which, activation=act) if case["packed"] else run_gemm(p, which=which, activation=act)
     if gated:
         assert_close_gated(p, c, str(case))
     else:
