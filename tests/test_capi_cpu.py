@@ -27,6 +27,21 @@ def test_library_exports_every_declared_symbol():
     assert "bfaintb_gemm_bias" in names
 
 
+def test_public_header_is_plain_c(tmp_path):
+    """include/bfaintb_gemm.h is the boundary a C caller binds to: it must compile as C99 on its own, and as C++."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "bfaintb_gemm.h"\n'
+                   'int main(void) { bfaintb_epilogue e = {0, 0, 0, BFAINTB_ACT_NONE}; bfaintb_packed_header h; (void)e; (void)h;\n'
+                   '  return bfaintb_gemm_variant(1, 16, 64, 8, 0) == BFAINTB_VARIANT_DECODE ? 0 : 1; }\n')
+    inc = os.path.join(root, "include")
+    for cmd in (["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-I", inc, str(src)],
+                ["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)]):
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+
+
 def test_variant_choice_and_split():
     assert af.variant(1, 4096, 4096) == af.DECODE
     assert af.variant(32, 4096, 4096) == af.DECODE
