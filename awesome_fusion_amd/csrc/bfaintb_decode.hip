@@ -71,10 +71,8 @@ __device__ __forceinline__ void prepare_row(uint32_t (&out)[CPL / 4], const uint
         for (int i = 0; i < CPL / 4; ++i) out[i] = codes8_to_s8(in[i]);
     } else {
         static_assert(BITS == 8 || CPL == 16, "4-bit codes: 16 columns per lane");
-        out[0] = codes4_even_to_s8x16(in[0]);
-        out[1] = codes4_odd_to_s8x16(in[0]);
-        out[2] = codes4_even_to_s8x16(in[1]);
-        out[3] = codes4_odd_to_s8x16(in[1]);
+        codes4_to_s8x16(in[0], out[0], out[1]);
+        codes4_to_s8x16(in[1], out[2], out[3]);
     }
 }
 
@@ -163,7 +161,8 @@ __device__ __forceinline__ void mac_step_packed(const PackedStep<BITS, CPL>& raw
             w.z = pack_bf16_rne(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
             w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
         } else {
-            const uint32_t ev = codes4_even_to_s8x16(raw.d[c][0]), od = codes4_odd_to_s8x16(raw.d[c][0]);
+            uint32_t ev, od;
+            codes4_to_s8x16(raw.d[c][0], ev, od);
             w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
             w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
             w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);

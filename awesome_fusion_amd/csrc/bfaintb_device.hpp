@@ -139,8 +139,15 @@ __device__ __forceinline__ float sbyte_to_f32(uint32_t x)
 //   4-bit: excess-8 nibble c = q + 8; c ^ 8 is q as int4; moved to the HIGH nibble of a byte it reads
 //          as the int8 value 16*q, and the column's scale is pre-divided by 16 (exact: a power of two).
 __device__ __forceinline__ uint32_t codes8_to_s8(uint32_t x) { return x ^ 0x80808080u; }
-__device__ __forceinline__ uint32_t codes4_even_to_s8x16(uint32_t x) { return ((x << 4) & 0xf0f0f0f0u) ^ 0x80808080u; }
-__device__ __forceinline__ uint32_t codes4_odd_to_s8x16(uint32_t x) { return (x & 0xf0f0f0f0u) ^ 0x80808080u; }
+// Both at once for a dword of eight codes: every code's top bit is flipped first (one operation for the dword), then the even
+// codes move up into their bytes' high nibbles and the low nibbles are cleared: 4 operations, where flipping each half
+// after its mask takes 5.
+__device__ __forceinline__ void codes4_to_s8x16(uint32_t x, uint32_t& even, uint32_t& odd)
+{
+    const uint32_t y = x ^ 0x88888888u;
+    even = (y << 4) & 0xf0f0f0f0u;
+    odd = y & 0xf0f0f0f0u;
+}
 
 // 16 bits holding four consecutive 4-bit codes (column j in nibble j) -> dword whose byte j reads as int8(16*q_j).
 // Byte 0 of (x << 4) is code 0 in the high nibble over zeros; byte 0 of x has code 1 in its high nibble, byte 1 of

@@ -256,7 +256,8 @@ __device__ __forceinline__ void decode_packed_body(const GemmParams& p)
                         w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
                     } else {
                         // nibble r of the dword is row r: even rows from the low nibbles, odd rows from the high ones
-                        const uint32_t ev = codes4_even_to_s8x16(wd[h]), od = codes4_odd_to_s8x16(wd[h]);
+                        uint32_t ev, od;
+                        codes4_to_s8x16(wd[h], ev, od);
                         w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
                         w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
                         w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);

@@ -250,8 +250,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
         if constexpr (PACKED && BITS == 4) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {  // dword d = 2 i + h: 8 nibbles = rows 0..7 of one column
-                b_s8[2 * d] = codes4_even_to_s8x16(b_reg[d]);
-                b_s8[2 * d + 1] = codes4_odd_to_s8x16(b_reg[d]);
+                codes4_to_s8x16(b_reg[d], b_s8[2 * d], b_s8[2 * d + 1]);
             }
             return;
         }

@@ -190,7 +190,8 @@ bfaintb_prefill128_kernel(const GemmParams p)
                     w[h].z = pack_bf16<REF>(sbyte_to_f32<0>(hi) * s, sbyte_to_f32<1>(hi) * s);
                     w[h].w = pack_bf16<REF>(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
                 } else {
-                    const uint32_t ev = codes4_even_to_s8x16(b_reg[h]), od = codes4_odd_to_s8x16(b_reg[h]);
+                    uint32_t ev, od;
+                    codes4_to_s8x16(b_reg[h], ev, od);
                     w[h].x = pack_bf16<REF>(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
                     w[h].y = pack_bf16<REF>(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
                     w[h].z = pack_bf16<REF>(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
