@@ -4,7 +4,6 @@
 // (gpu_utils.hpp:5-11, print and exit(0)) every failure is returned to the caller.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
 #include <string.h>
 
 #include "bfaintb_device.hpp"
@@ -504,9 +503,6 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
 // m = 12: 28.0 / 26.4; 28672 x 8192: m = 12: 44.5 / 39.9).
 static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
 {
-#ifdef BFAINTB_TUNE
-    if (const char* e = getenv("BFAINTB_SLABMAX")) return (uint32_t)atoi(e);
-#endif
     const uint64_t weights = (uint64_t)n * k;
     if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
     return weights <= (24ull << 20) ? kPackedSlabMaxM : weights < (64ull << 20) ? 24u : weights == (64ull << 20) ? 16u : 8u;
