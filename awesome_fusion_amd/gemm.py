@@ -63,6 +63,13 @@ def lib():
             raise RuntimeError(
                 f"{_LIB} is missing: build it with `make -C awesome_fusion_amd/csrc` "
                 "(or __graft_entry__.build()); this package has no CPU fallback")
+        # torch ships its own HIP runtime: when a process is going to use torch for device memory (this binding's callers
+        # do), that runtime has to be the one this library binds to, so torch is loaded first.  Loaded the other way round,
+        # the library's launches fail with "no ROCm-capable device" against tensors torch allocated.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(_LIB)
         L.bfaintb_gemm.restype = C.c_int
         L.bfaintb_gemm.argtypes = [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp,
