@@ -223,8 +223,8 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
             const float noise_scale = 2.0f * std::sqrt((float)k) * std::ldexp(1.0f, -24);
             for (auto& v : noise) v *= noise_scale;
             const UlpReport rep = valid_vector_ulp(c_ref.data(), c_dev.data(), (long)m * n, 2.0, 1e-3, 1e-2, noise.data());
-            // outputs that cancel to almost nothing: at most 2 in 10^4 (plus one), each within the noise bound
-            const long allowed = (long)((double)m * n * 2e-4) + 1;
+            // outputs that cancel to almost nothing: at most 2 in 10^4 (plus three), each within the noise bound
+            const long allowed = (long)((double)m * n * 2e-4) + 3;
             std::printf("ulp check: %ld of %ld outside 2 bf16 ULP (or 1e-2 relative below 1e-3), %ld more only within the fp32 summation "
                         "noise (allowed %ld), worst %.3f ULP at %ld\n", rep.failing, (long)m * n, rep.cancelling, allowed, rep.worst_ulp,
                         rep.worst_index);
