@@ -132,11 +132,12 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
 // wave per SIMD, 128 accumulator registers) amortises the dequantisation best; smaller row blocks give more
 // workgroups when columns x row blocks alone do not fill the machine.  Picked by estimate.  (Columns per workgroup
 // are fixed by the code width here: what the kernels over packed weights need.)
-DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
+DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false,
+                                  uint32_t max_mb = 4u)
 {
     DecodePlan best{};
     double best_t = 0.0;
-    for (uint32_t mb = bits == 8 ? 4u : 2u; mb >= 1u; mb >>= 1) {
+    for (uint32_t mb = bits == 8 ? max_mb : (max_mb < 2u ? max_mb : 2u); mb >= 1u; mb >>= 1) {
         DecodePlan c;
         c.cols = bits == 8 ? 128u : 256u;
         c.waves = (bits == 8 && mb <= 2u) ? 8u : 4u;
@@ -179,6 +180,13 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
     if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed);
     DecodePlan pl;
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
+    // 8-bit codes, 17 to 32 rows, a small or narrow matrix: one 32-row block per workgroup cannot fill the machine without
+    // splitting k further than it likes; two blocks of 16 rows with their own workgroups (the second stream hits in cache)
+    // and the split that fills one round do (m = 32, n x k = 1024 x 4096: 7.0 against 8.9 us; 2048 x 8192: 10.9 against
+    // 14.0; 1024 x 16384: 11.7 against 16.3; 4096 x 2048: 7.9 against 9.3; 4096 x 4096: 10.7 against 10.8; beyond 16 MiB
+    // at more than 2048 columns the one block wins: 3072 x 8192: 15.4 against 14.4)
+    if (bits == 8 && m > 16 && forced_splits == 0 && (weight_bytes <= (16ull << 20) || n <= 2048u))
+        return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u);
     {
         // 8-bit codes, 128 columns x 8 waves ("narrow": a lane loads 8 bytes of a row, 16 lanes one 128-byte line)
         // needs half the splits of 256 columns x 4 waves ("wide") for the same number of waves, so half the

@@ -225,6 +225,8 @@ def test_prefill_variant_on_small_m_matches_decode(af):
     (200, 1040, 2048, 8, 128, 3),   # four row blocks, group scales, forced odd split
     (48, 1024, 2048, 4, 128, 0),    # 4-bit codes: row blocks of 32
     (130, 528, 1024, 4, 0, 2),
+    (5000, 256, 256, 8, 0, 0),      # very tall A: thousands of row blocks along grid z
+    (20000, 128, 128, 4, 64, 0),
 ])
 def test_decode_family_with_row_blocks_matches_oracle(af, m, n, k, bits, group, split):
     """The decode kernel forced onto m > 32: grid z walks blocks of rows; each must agree with the oracle and,
