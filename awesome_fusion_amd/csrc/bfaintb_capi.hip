@@ -225,6 +225,14 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
                 splits = ((narrow ? kDecodeTargetWgsNarrow : kDecodeTargetWgs) + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
+                // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each
+                // and whose partial sums the reducing workgroup must collect: beyond 16 splits (32 once k is long enough
+                // for four steps per wave) the launch gets slower again.  Measured at m = 1, 16 splits against what the
+                // target asks for: 4-bit 1024 x 8192 9.6 / 14.5 us, 1024 x 4096 7.7 / 9.0, 4096 x 8192 10.9 / 12.8,
+                // 4096 x 11008 12.7 / 13.9; 8-bit 1024 x 8192 7.9 / 9.3, 256 x 16384 8.6 / 13.6; 32 splits: 4-bit
+                // 1024 x 16384 12.2 (16: 14.0, 64: 15.5), 1024 x 28672 15.5 (16: 19.5, 56: 16.8).
+                const uint32_t most = k >= (bits == 4 ? 16384u : 24576u) ? 32u : 16u;
+                if (splits > most) splits = most;
             }
         }
         set_splits(pl, k, bits, splits, packed);
@@ -512,6 +520,9 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
 static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
 {
     const uint64_t weights = (uint64_t)n * k;
+    // 8-bit codes, a narrow matrix with long columns: n/16 workgroups that each walk all of k alone take 0.75 us per 1024
+    // rows whatever n is; the family splits k instead (1024 x 16384, m = 1: 12.7 us the slab kernel, 10.2 the split)
+    if (bits == 8 && n < 2048u && k >= 12288u) return 0u;
     if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
     return weights <= (24ull << 20) ? kPackedSlabMaxM : weights < (64ull << 20) ? 24u : weights == (64ull << 20) ? 16u : 8u;
 }

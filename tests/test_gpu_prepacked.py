@@ -95,7 +95,9 @@ def test_pack_honours_the_row_stride(af):
     (33, 96, 1152, 4, 128), (70, 64, 1600, 8, 32), (1, 32, 8256, 8, 0), (40, 128, 4096, 8, 128), (5, 1024, 2048, 4, 128),
     # every launch form: one batch per wave (k = 4096 / 2048 for 8-bit with 1 / 2 row blocks, 4096 for 4-bit), pipelined
     # (long k, per-channel scales), with one and two row blocks
-    (20, 48, 2048, 8, 0), (3, 32, 4096, 4, 128), (2, 32, 8192, 4, 0), (40, 32, 8256, 8, 0), (24, 32, 8192, 4, 0), (9, 64, 4096, 8, 0)])
+    (20, 48, 2048, 8, 0), (3, 32, 4096, 4, 128), (2, 32, 8192, 4, 0), (40, 32, 8256, 8, 0), (24, 32, 8192, 4, 0), (9, 64, 4096, 8, 0),
+    # 8-bit codes, narrow with long columns: the split family instead of the slab kernel, also for a few rows
+    (1, 1024, 12288, 8, 0), (4, 272, 12288, 8, 64), (8, 512, 16384, 8, 0)])
 def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
     p = Problem(m, n, k, bits, group, seed=m + n + k)
     assert_close_ulp(p, run_prepacked(af, p, af.DECODE), f"packed decode {m}x{n}x{k} b{bits} g{group}")
