@@ -133,14 +133,14 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
 // workgroups when columns x row blocks alone do not fill the machine.  Picked by estimate.  (Columns per workgroup
 // are fixed by the code width here: what the kernels over packed weights need.)
 DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false,
-                                  uint32_t max_mb = 4u)
+                                  uint32_t max_mb = 4u, bool wide8 = false)
 {
     DecodePlan best{};
     double best_t = 0.0;
     for (uint32_t mb = bits == 8 ? max_mb : (max_mb < 2u ? max_mb : 2u); mb >= 1u; mb >>= 1) {
         DecodePlan c;
         c.cols = bits == 8 ? 128u : 256u;
-        c.waves = (bits == 8 && mb <= 2u) ? 8u : 4u;
+        c.waves = ((bits == 8 && mb <= 2u) || (wide8 && mb == 1u)) ? 8u : 4u;  // wide8: 4-bit codes, 256 columns x 8 waves
         c.mb = mb;
         const uint32_t tiles = ((n + c.cols - 1u) / c.cols) * ((m + 16u * mb - 1u) / (16u * mb));
         // 8-bit codes: split along k until the workgroups fill one round of the 256 CUs, not beyond: measured at m = 40 and 64 over
@@ -175,11 +175,16 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
 
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
 {
+    const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
+    // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built for 4 waves): the two
+    // 16-row blocks run 8 waves each (m = 32, 1024 x 4096: 10.5 against 13.7 us, 17 rows: 10.6 / 17.2; 2048 x 8192:
+    // 15.3 / 18.4; 4096 x 4096: 14.3 / 16.6; larger matrices lose: 4096 x 11008: 26.5 / 21.8)
+    if (bits == 4 && m > 16 && m <= 32 && forced_splits == 0 && !packed && (weight_bytes <= (8ull << 20) || n <= 2048u))
+        return decode_plan_row_blocks(m, n, k, bits, 0, false, 1u, true);
     // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
     // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
     if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed);
     DecodePlan pl;
-    const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     // 8-bit codes, 17 to 32 rows, a small or narrow matrix: one 32-row block per workgroup cannot fill the machine without
     // splitting k further than it likes; two blocks of 16 rows with their own workgroups (the second stream hits in cache)
     // and the split that fills one round do (m = 32, n x k = 1024 x 4096: 7.0 against 8.9 us; 2048 x 8192: 10.9 against
@@ -214,16 +219,23 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         const bool fills_rounds = narrow_wgs * 20u >= ((narrow_wgs + 255u) / 256u) * 256u * 19u;  // >= 95 % of whole rounds
         const bool narrow = bits == 8 && (few || m >= 8 || fills_rounds);
         pl.cols = narrow ? 128u : 256u;
-        pl.waves = narrow ? 8u : 4u;
+        // 4-bit codes, 8 to 16 rows: the same 256 columns with 8 waves (twice the waves to hide the activation loads and
+        // the matrix instructions behind; n = k = 4096, m = 16: 11.6 against 14.7 us, 1024 x 8192: 14.1 / 17.4,
+        // 8192 x 8192: 17.2 / 19.2, 28672 x 8192: 36.2 / 37.5; m = 8: 10.1 / 11.2, 10.2 / 12.7, 15.7 / 17.8, 35.1 / 35.3;
+        // no difference at m = 1).  The kernels over packed 4-bit codes are built for 4 waves.
+        const bool wide8 = bits == 4 && m >= 8u && !packed;
+        pl.waves = (narrow || wide8) ? 8u : 4u;
         pl.mb = m <= 16 ? 1u : 2u;
         uint32_t splits = forced_splits;
         if (splits == 0) {
             if (narrow && !few) {
                 splits = narrow_splits;
             } else {
-                // about 256 narrow or 480 wide workgroups: enough waves on every CU to keep the memory system busy
+                // about 256 workgroups of 8 waves or 480 of 4: enough waves on every CU to keep the memory system busy
                 const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
-                splits = ((narrow ? kDecodeTargetWgsNarrow : kDecodeTargetWgs) + col_blocks / 2) / col_blocks;
+                // (8 waves: one workgroup per CU, so never a few workgroups past a whole round - 4-bit codes, m = 8,
+                // 11008 x 4096: 13.4 us with 5 splits = 215 workgroups, 16.7 with 6 = 258; 22016 x 4096: 20.5 / 28.9)
+                splits = pl.waves == 8u ? kDecodeTargetWgsNarrow / col_blocks : (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
                 // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each
                 // and whose partial sums the reducing workgroup must collect: beyond 16 splits (32 once k is long enough
