@@ -235,7 +235,11 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 const uint32_t col_blocks = (n + pl.cols - 1) / pl.cols;
                 // (8 waves: one workgroup per CU, so never a few workgroups past a whole round - 4-bit codes, m = 8,
                 // 11008 x 4096: 13.4 us with 5 splits = 215 workgroups, 16.7 with 6 = 258; 22016 x 4096: 20.5 / 28.9)
-                splits = pl.waves == 8u ? kDecodeTargetWgsNarrow / col_blocks : (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
+                // 4-bit codes with 4 waves like one round as well while the column blocks are few (m = 1: 8192 x 8192
+                // 14.1 us with 256 workgroups, 15.7 with 416; 5120 x 5120 9.7 / 11.7; 8192 x 4096 10.6 / 11.8; from 100
+                // column blocks on the 480 are as good or a little better: 28672 x 8192 35.0 against 36.0)
+                const bool one_round = pl.waves == 8u || (bits == 4 && col_blocks <= 64u);
+                splits = one_round ? kDecodeTargetWgsNarrow / col_blocks : (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
                 // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each
                 // and whose partial sums the reducing workgroup must collect: beyond 16 splits (32 once k is long enough
