@@ -148,8 +148,11 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
         // workgroups that still fit one round (4096 x 4096, m = 40, 32-row blocks: 19.3 / 14.4 / 11.2 / 15.7 us with
         // 64 / 128 / 256 / 512 workgroups; 11008 x 4096: 21.2 us with 172, 25.4 us with 344).
         if (bits == 8 && forced_splits == 0) {
+            // (at most 16 splits, 8 while k is short: 512 x 4096, m = 48: 11.0 us with 16 splits, 7.0 with 8; 1024 x 8192, m = 32:
+            // 9.1 with 16, 10.1 with 8)
             uint32_t s = 256u / tiles;
-            if (s > 16u) s = 16u;
+            const uint32_t most = k >= 8192u ? 16u : k / 512u > 8u ? k / 512u : 8u;
+            if (s > most) s = most;
             for (; s > 1u; --s) {
                 set_splits(c, k, bits, s, packed);
                 if (c.splits == s) break;  // k divides that way
@@ -183,6 +186,12 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         return decode_plan_row_blocks(m, n, k, bits, 0, false, 1u, true);
     // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
     // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
+    // 8-bit codes, more than 32 rows, but so few columns that even 16-row blocks make at most 40 workgroups per split: only
+    // those (the 32- and 64-row kernels spend longer in their reductions than such a launch has; 768 x 5120, m = 48: 7.5
+    // against 10.8 us; 1536 x 8960: 10.8 / 14.3; 256 x 7168, m = 128: 7.8 / 11.7; with more blocks the larger ones win:
+    // 2048 x 8192, m = 128: 20.2 / 16.3)
+    if (bits == 8 && m > 32 && forced_splits == 0 && (uint64_t)((n + 127u) / 128u) * ((m + 15u) / 16u) <= 40u)
+        return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u);
     if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed);
     DecodePlan pl;
     // 8-bit codes, 17 to 32 rows, a small or narrow matrix: one 32-row block per workgroup cannot fill the machine without
