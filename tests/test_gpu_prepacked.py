@@ -106,6 +106,25 @@ def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
 
 
 @pytest.mark.parametrize("m,n,k,bits,group", [
+    (24, 1024, 4096, 8, 0),      # 8-bit, 17..32 rows, small matrix: two 16-row blocks that split k to fill one round
+    (32, 528, 8192, 8, 64),
+    (48, 768, 5120, 8, 0),       # so few columns that only 16-row blocks are used beyond 32 rows too
+    (128, 256, 7168, 8, 128),
+    (12, 528, 2048, 4, 64),      # 4-bit, 8..16 rows: 256 columns x 8 waves (row-major), ragged last column block
+    (16, 4096, 4096, 4, 128),
+    (24, 1040, 4096, 4, 0),      # 4-bit, 17..32 rows, narrow: two 8-wave blocks of 16 rows
+    (1, 1024, 8192, 4, 128),     # narrow with long columns: the split factor stops at 16
+    (8, 11008, 4096, 4, 128),    # 8-wave workgroups: the split stays within one round of workgroups
+    (4, 1024, 12288, 8, 0),      # packed 8-bit, narrow and long: the split family instead of the slab kernel
+])
+def test_plan_corners_both_weight_orders(af, m, n, k, bits, group):
+    """Shapes on either side of the launch-plan rules for small, narrow and long matrices, kernel left to the library."""
+    p = Problem(m, n, k, bits, group, seed=m * 3 + n + k)
+    assert_close_ulp(p, run_gemm(p), f"row-major {m}x{n}x{k} b{bits} g{group}")
+    assert_close_ulp(p, run_prepacked(af, p), f"packed {m}x{n}x{k} b{bits} g{group}")
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [
     (49, 128, 512, 8, 0), (64, 4096, 1024, 8, 0), (100, 272, 448, 8, 64), (130, 48, 1024, 8, 32), (200, 1040, 256, 8, 0), (300, 144, 2048, 8, 128),
     (64, 256, 512, 4, 0), (97, 528, 1024, 4, 128), (150, 80, 640, 4, 32), (260, 1296, 384, 4, 128),
     # shapes whose plan splits along k (few column groups, long k): partial sums meet in the workspace
