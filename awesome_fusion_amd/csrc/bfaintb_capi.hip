@@ -131,7 +131,8 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
 // The decode family in row blocks: grid z walks blocks of 16*mb rows.  128 columns x 64 rows (mb = 4, 4 waves: one
 // wave per SIMD, 128 accumulator registers) amortises the dequantisation best; smaller row blocks give more
 // workgroups when columns x row blocks alone do not fill the machine.  Picked by estimate.  (Columns per workgroup
-// are fixed by the code width here: what the kernels over packed weights need.)
+// are fixed by the code width here: what the kernels over packed weights need.)  max_mb: the largest row block to
+// consider, in units of 16 rows; wide8: blocks of 16 rows of 4-bit codes run 8 waves instead of 4.
 DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false,
                                   uint32_t max_mb = 4u, bool wide8 = false)
 {
@@ -179,19 +180,19 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
 {
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
-    // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built for 4 waves): the two
-    // 16-row blocks run 8 waves each (m = 32, 1024 x 4096: 10.5 against 13.7 us, 17 rows: 10.6 / 17.2; 2048 x 8192:
+    // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built
+    // for 4 waves): the two 16-row blocks run 8 waves each (m = 32, 1024 x 4096: 10.5 against 13.7 us, 17 rows: 10.6 / 17.2; 2048 x 8192:
     // 15.3 / 18.4; 4096 x 4096: 14.3 / 16.6; larger matrices lose: 4096 x 11008: 26.5 / 21.8)
     if (bits == 4 && m > 16 && m <= 32 && forced_splits == 0 && !packed && (weight_bytes <= (8ull << 20) || n <= 2048u))
         return decode_plan_row_blocks(m, n, k, bits, 0, false, 1u, true);
-    // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
-    // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
     // 8-bit codes, more than 32 rows, but so few columns that even 16-row blocks make at most 40 workgroups per split: only
     // those (the 32- and 64-row kernels spend longer in their reductions than such a launch has; 768 x 5120, m = 48: 7.5
     // against 10.8 us; 1536 x 8960: 10.8 / 14.3; 256 x 7168, m = 128: 7.8 / 11.7; with more blocks the larger ones win:
     // 2048 x 8192, m = 128: 20.2 / 16.3)
     if (bits == 8 && m > 32 && forced_splits == 0 && (uint64_t)((n + 127u) / 128u) * ((m + 15u) / 16u) <= 40u)
         return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u);
+    // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
+    // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
     if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed);
     DecodePlan pl;
     // 8-bit codes, 17 to 32 rows, a small or narrow matrix: one 32-row block per workgroup cannot fill the machine without
