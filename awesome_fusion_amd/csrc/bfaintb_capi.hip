@@ -549,6 +549,9 @@ static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
     // 8-bit codes, a narrow matrix with long columns: n/16 workgroups that each walk all of k alone take 0.75 us per 1024
     // rows whatever n is; the family splits k instead (1024 x 16384, m = 1: 12.7 us the slab kernel, 10.2 the split)
     if (bits == 8 && n < 2048u && k >= 12288u) return 0u;
+    // 4-bit codes in that corner: up to 20 rows (1024 x 16384, slab / family: m = 17: 22.4 / 24.5 us, 24: 31.4 / 24.8,
+    // 32: 35.8 / 25.1; 512 x 12288, m = 24: 22.4 / 21.5; with k = 8192 the slab kernel stays ahead up to its 48 rows)
+    if (bits == 4 && n < 2048u && k >= 12288u) return 20u;
     if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
     return weights <= (24ull << 20) ? kPackedSlabMaxM : weights < (64ull << 20) ? 24u : weights == (64ull << 20) ? 16u : 8u;
 }

@@ -2,7 +2,7 @@
 """Benchmark of the bfAintBGemm hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
-    python bench.py --scan        (a map of kernel times over shapes and m, not the benchmark)
+    python bench.py --scan [narrow]   (a map of kernel times over shapes and m, not the benchmark)
 
 A step is one GEMM launch through the C ABI on synthetic, seeded inputs already resident in HBM.
 The headline workload is the decode shape the metric is quoted on (bf16 A [1,4096] x int8 B
@@ -304,18 +304,19 @@ def roofline_entry(w, ms, bound, suffix=""):
 
 
 SCAN_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (8192, 8192), (28672, 8192), (2048, 8192), (32000, 4096)]   # (n, k)
+SCAN_SHAPES_NARROW = [(1024, 4096), (1024, 8192), (512, 4096), (2048, 4096), (1536, 8960), (256, 7168), (1024, 16384)]
 SCAN_M = [1, 4, 8, 16, 24, 32, 48, 64, 128, 256, 512, 1024, 2048]
 
 
-def scan():
-    """Kernel time of bfaintb_gemm and bfaintb_gemm_prepacked, variant left to the library, over SCAN_SHAPES x {8-bit per
+def scan(shapes=None):
+    """Kernel time of bfaintb_gemm and bfaintb_gemm_prepacked, variant left to the library, over shapes x {8-bit per
     channel, 4-bit group 128} x SCAN_M.  Up to 32 rows of A the launches rotate over copies of B that exceed the last-level
     cache (the decode protocol of the headline figure); beyond, two copies.  Not a roofline statement: a map to read
     anomalies from (a time that falls as m grows, a weight order that loses to the other)."""
     import torch
     import awesome_fusion_amd as af
     af.lib()
-    for (n, k) in SCAN_SHAPES:
+    for (n, k) in (SCAN_SHAPES if shapes is None else shapes):
         for (bits, group) in ((8, 0), (4, 128)):
             row = {"n": n, "k": k, "weight_bits": bits, "group_size": group, "m": SCAN_M, "row_major_us": [], "prepacked_us": []}
             for m in SCAN_M:
@@ -395,8 +396,11 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (decode sweep, int4 group-128)")
-    ap.add_argument("--scan", action="store_true", help="instead of the benchmark: what the library's own choice of kernel takes over a grid of "
-                    "matrix shapes, code widths and m, row-major and pre-packed weights; one JSON line per matrix")
+    ap.add_argument("--scan", nargs="?", const="llm", default="", choices=["llm", "narrow"],
+                    help="instead of the benchmark: what the library's own choice of kernel takes over a grid of "
+                    "matrix shapes, code widths and m, row-major and pre-packed weights; one JSON line per matrix "
+                    "(llm: projection and MLP shapes of 7B..70B models; narrow: 256..2048 columns, the key/value "
+                    "projections of grouped-query attention)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload family: decode | prefill | decode_cold | decode_packed_cold "
                     "(decode_cold: nothing but the headline's cold-B launches, for a kernel trace without the hot and eager variants; "
@@ -407,7 +411,7 @@ def main():
               "of B with no exchange between GPUs).  Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if args.scan:
-        scan()
+        scan(SCAN_SHAPES_NARROW if args.scan == "narrow" else SCAN_SHAPES)
         return
 
     import torch
