@@ -227,7 +227,13 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         }
         const uint32_t narrow_wgs = narrow_blocks * narrow_splits;
         const bool fills_rounds = narrow_wgs * 20u >= ((narrow_wgs + 255u) / 256u) * 256u * 19u;  // >= 95 % of whole rounds
-        const bool narrow = bits == 8 && (few || m >= 8 || fills_rounds);
+        // m >= 8 on a wide matrix: once 256-column blocks fill their one round with at most 3 splits (more than 64 of
+        // them) their partial sums no longer outweigh the better stream (m = 8 / 16 / 32, wide against narrow:
+        // 22016 x 4096 20.9 / 22.7 / 28.2 against 21.9 / 23.4 / 31.6 us; 28672 x 8192 46.2 / 48.3 / 54.2 against 49.8 / 53.1 /
+        // 61.5; 18944 x 3584 16.9 / 18.3 / 24.0 against 18.0 / 19.9 / 25.1; with fewer blocks narrow stays ahead:
+        // 11008 x 4096 13.9 / 14.9 / 17.9 against 13.8 / 16.5 / 22.1; 14336 x 4096 17.2 / 18.5 / 21.4 against 17.6 / 19.0 / 25.1)
+        const bool many_wide_blocks = (n + 255u) / 256u > 64u;
+        const bool narrow = bits == 8 && (few || fills_rounds || (m >= 8 && (!many_wide_blocks || packed)));  // packed weights: the kernels are built for 128 columns
         pl.cols = narrow ? 128u : 256u;
         // 4-bit codes, 8 to 16 rows: the same 256 columns with 8 waves (twice the waves to hide the activation loads and
         // the matrix instructions behind; n = k = 4096, m = 16: 11.6 against 14.7 us, 1024 x 8192: 14.1 / 17.4,
@@ -248,7 +254,10 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 // 4-bit codes with 4 waves like one round as well while the column blocks are few (m = 1: 8192 x 8192
                 // 14.1 us with 256 workgroups, 15.7 with 416; 5120 x 5120 9.7 / 11.7; 8192 x 4096 10.6 / 11.8; from 100
                 // column blocks on the 480 are as good or a little better: 28672 x 8192 35.0 against 36.0)
-                const bool one_round = pl.waves == 8u || (bits == 4 && col_blocks <= 64u);
+                // 8-bit codes with 4 waves: one round on every shape measured (m = 1: 11008 x 4096 12.7 us with 215 workgroups,
+                // 13.2 with 473; 9216 x 4096 11.7 / 13.1; 5120 x 8192 12.8 / 15.7; 18944 x 3584 15.8 / 17.4; 22016 x 4096
+                // 19.6 / 21.8; 28672 x 8192 43.8 / 44.8; a few workgroups past the round are the worst case: 258 -> 15.3 us)
+                const bool one_round = pl.waves == 8u || bits == 8 || (bits == 4 && col_blocks <= 64u);
                 splits = one_round ? kDecodeTargetWgsNarrow / col_blocks : (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
                 // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each

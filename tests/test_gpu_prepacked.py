@@ -116,6 +116,9 @@ def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
     (1, 1024, 8192, 4, 128),     # narrow with long columns: the split factor stops at 16
     (8, 11008, 4096, 4, 128),    # 8-wave workgroups: the split stays within one round of workgroups
     (4, 1024, 12288, 8, 0),      # packed 8-bit, narrow and long: the split family instead of the slab kernel
+    (2, 9216, 4096, 8, 0),       # 8-bit, 256 columns x 4 waves on a large matrix: the split that fills one round (7 x 36 workgroups)
+    (16, 16640, 2048, 8, 0),     # 8 rows and more, over 64 blocks of 256 columns: those blocks (row-major) instead of 128-column ones
+    (24, 16640, 2048, 8, 64),    # the same with two 16-row accumulators per wave
 ])
 def test_plan_corners_both_weight_orders(af, m, n, k, bits, group):
     """Shapes on either side of the launch-plan rules for small, narrow and long matrices, kernel left to the library."""
