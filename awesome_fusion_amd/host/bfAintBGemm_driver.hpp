@@ -15,8 +15,9 @@
 //             on the device (:27,101), bfaintb_gemm_reference (truncating kernel arithmetic); 8-bit codes, per column only.
 //             With data = 0 the validation is the reference's, operand for operand (:198-214).
 // Metrics are the reference's (:186-195) in decimal units with the scale bytes counted.
-// Validation needs a host GEMM to compare with; it is supplied by the caller of driver_main (the
-// test build passes one); the plain binary has none and refuses `validation`.
+// Validation compares with a host GEMM supplied by the caller of driver_main: the shipped binary passes the
+// harness's own gemm_rrr (host_ref.hpp), the test build the CPU checker's.  Return code: 0, 1 when a launch
+// or the validation failed, 2 for a bad command line.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -81,8 +82,7 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
     const int warm_ups = 10;
     if (m <= 0 || n <= 0 || k <= 0 || total_loop <= 0) { std::printf("bad sizes\n"); return 2; }
     if (validation && (checker == nullptr || checker->gemm_rrr == nullptr)) {
-        std::printf("validation requested, but this binary was built without a host GEMM to compare with "
-                    "(the test build of the driver links one)\n");
+        std::printf("validation requested, but driver_main was given no host GEMM to compare with\n");
         return 2;
     }
     const int groups = group_size ? k / group_size : 1;
@@ -158,10 +158,15 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
     GPU_CHECK_ERROR(hipEventCreate(&evt_11));
     GPU_CHECK_ERROR(hipDeviceSynchronize());
     GPU_CHECK_ERROR(hipEventRecord(evt_00, nullptr));
-    for (int i = 0; i < total_loop; i++) (void)launch();
+    int timed_rc = 0;  // the first non-zero return code of the timed launches
+    for (int i = 0; i < total_loop; i++) {
+        const int r = launch();
+        if (r && !timed_rc) timed_rc = r;
+    }
     GPU_CHECK_ERROR(hipEventRecord(evt_11, nullptr));
     GPU_CHECK_ERROR(hipEventSynchronize(evt_11));
     GPU_CHECK_ERROR(hipDeviceSynchronize());
+    if (timed_rc) { std::printf("bfaintb_gemm failed in the timed loop: [%d] %s\n", timed_rc, bfaintb_error_string(timed_rc)); return 1; }
     float elapsed_ms = 0.f;
     GPU_CHECK_ERROR(hipEventElapsedTime(&elapsed_ms, evt_00, evt_11));
     GPU_CHECK_ERROR(hipEventDestroy(evt_00));
