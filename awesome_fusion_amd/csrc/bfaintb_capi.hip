@@ -6,6 +6,9 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "bfaintb_device.hpp"
 #include "../../include/bfaintb_gemm.h"
 
@@ -23,6 +26,7 @@ hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t strea
 hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t decode_prepare_device();
 }  // namespace bfaintb
 
 namespace {
@@ -295,11 +299,65 @@ size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant,
     if (variant != BFAINTB_VARIANT_DECODE || m == 0 || n == 0) return 0;
     const DecodePlan pl = decode_plan(m, n, k, bits, forced_split);
     if (pl.splits <= 1) return 0;
-    // one fp32 word per (split but the last, row, column), rounded up to 256 bytes
-    return (((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u;
+    // the header, then one fp32 word per (split but the last, row, column), rounded up to 256 bytes
+    return bfaintb::kWorkspaceHeaderBytes + ((((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u);
 }
 
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+// ---- per-device set-up: kernel attributes ----
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    std::atomic<int> ready{0};      // kernel attributes set on this device
+};
+DeviceState g_devices[kMaxDevices];
+std::mutex g_setup_mutex;
+std::atomic<uint32_t> g_split_wait_limit{bfaintb::kDefaultSplitWaitLimit};
+std::atomic<uint32_t> g_debug_flags{0};
+
+bool stream_is_capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
+// The current device's state, its kernels prepared.  The set-up makes runtime calls that are not stream operations, so
+// it must not run for the first time under stream capture: such a call is refused (BFAINTB_ERR_NOT_INITIALISED) and
+// bfaintb_init is the way to run it beforehand.
+int device_state(hipStream_t stream, DeviceState** out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return BFAINTB_ERR_UNSUPPORTED;
+    DeviceState& st = g_devices[dev];
+    if (!st.ready.load(std::memory_order_acquire)) {
+        if (stream_is_capturing(stream)) return BFAINTB_ERR_NOT_INITIALISED;
+        std::lock_guard<std::mutex> lock(g_setup_mutex);
+        if (!st.ready.load(std::memory_order_relaxed)) {
+            e = bfaintb::decode_prepare_device();
+            if (e != hipSuccess) return (int)e;
+            st.ready.store(1, std::memory_order_release);
+        }
+    }
+    *out = &st;
+    return BFAINTB_OK;
+}
+
+int init_workspace_on(void* workspace, size_t workspace_bytes, hipStream_t stream)
+{
+    if (workspace_bytes % 4 != 0 || workspace_bytes / 4 >= (1ull << 32) || workspace_bytes < bfaintb::kWorkspaceHeaderBytes)
+        return BFAINTB_ERR_WORKSPACE;
+    // every word becomes "no partial sum here" (and "no failure" in the header), then the header gets its mark; fill
+    // kernels rather than hipMemsetAsync, so that the call may be recorded into a HIP graph
+    hipError_t e = bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)(workspace_bytes / 4), kEmptyWord, stream);
+    if (e == hipSuccess) e = bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace) + 1, 1u, bfaintb::kWorkspaceMagic, stream);
+    return (int)e;
+}
 
 }  // namespace
 
@@ -318,6 +376,8 @@ const char* bfaintb_error_string(int code)
         case BFAINTB_ERR_UNSUPPORTED: return "unsupported format: weight_bits must be 8 or 4; group_size 0 or a multiple of 32 that divides k";
         case BFAINTB_ERR_WORKSPACE: return "workspace missing or smaller than bfaintb_gemm_workspace_bytes reports";
         case BFAINTB_ERR_BAD_VARIANT: return "unknown kernel variant, or variant cannot run this shape";
+        case BFAINTB_ERR_NOT_INITIALISED: return "first call on this device made under stream capture: call bfaintb_init() beforehand";
+        case BFAINTB_ERR_WORKSPACE_POISONED: return "a split-K wait gave up on this workspace (results of that call hold NaNs): initialise it again";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -357,11 +417,40 @@ int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream
 {
     if (workspace == nullptr || workspace_bytes == 0) return BFAINTB_OK;
     if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
-    if (workspace_bytes % 4 != 0 || workspace_bytes / 4 >= (1ull << 32)) return BFAINTB_ERR_WORKSPACE;
-    // every word becomes "no partial sum here"; a fill kernel rather than hipMemsetAsync, so that the
-    // call may be recorded into a HIP graph
-    return (int)bfaintb::launch_fill_u32(static_cast<uint32_t*>(workspace), (uint32_t)(workspace_bytes / 4), kEmptyWord,
-                                         static_cast<hipStream_t>(stream));
+    return init_workspace_on(workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int bfaintb_workspace_status(const void* workspace, void* stream)
+{
+    if (workspace == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    uint32_t header[2] = {0, 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemcpyAsync(header, workspace, sizeof(header), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return (int)e;
+    if (header[1] != bfaintb::kWorkspaceMagic) return BFAINTB_ERR_WORKSPACE;
+    return header[0] == kEmptyWord ? BFAINTB_OK : BFAINTB_ERR_WORKSPACE_POISONED;
+}
+
+int bfaintb_init(void* stream)
+{
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DeviceState* dev = nullptr;
+    return device_state(st, &dev);
+}
+
+int bfaintb_debug_control(uint32_t what, uint32_t value)
+{
+    switch (what) {
+        case BFAINTB_DEBUG_SPLIT_WAIT_LIMIT:
+            g_split_wait_limit.store(value ? value : bfaintb::kDefaultSplitWaitLimit);
+            return BFAINTB_OK;
+        case BFAINTB_DEBUG_WITHHOLD_PARTIALS:
+            if (value) g_debug_flags.fetch_or(bfaintb::kDebugWithholdPartials);
+            else g_debug_flags.fetch_and(~bfaintb::kDebugWithholdPartials);
+            return BFAINTB_OK;
+        default: return BFAINTB_ERR_UNSUPPORTED;
+    }
 }
 
 // what the epilogue descriptor asks for, checked: bias and residual pointers (either may be null) and the residual's row stride
@@ -385,6 +474,20 @@ static int read_epilogue(Epilogue& out, const bfaintb_epilogue* ep, uint32_t n)
     out.ldr = ep->ldr;
     out.activation = ep->activation;
     if (ep->residual != nullptr && (ep->ldr < out.out_cols(n) || ep->ldr % 8u != 0)) return BFAINTB_ERR_BAD_LD;
+    return BFAINTB_OK;
+}
+
+// points the kernel at a split-K workspace: header first, partial sums behind it
+static int attach_workspace(GemmParams& p, void* workspace, size_t workspace_bytes, size_t need)
+{
+    if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
+    if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
+    if (need >= (1ull << 31)) return BFAINTB_ERR_BAD_VARIANT;  // the kernel addresses the workspace with 32-bit offsets
+    p.ws_header = static_cast<uint32_t*>(workspace);
+    p.partials = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + bfaintb::kWorkspaceHeaderBytes);
+    p.partial_bytes = (uint32_t)(need - bfaintb::kWorkspaceHeaderBytes);
+    p.split_wait_limit = g_split_wait_limit.load(std::memory_order_relaxed);
+    p.debug_flags = g_debug_flags.load(std::memory_order_relaxed);
     return BFAINTB_OK;
 }
 
@@ -443,14 +546,15 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.decode_waves = pl.waves;
     p.decode_cols = pl.cols;
     p.decode_mb = pl.mb;
+    // (every argument check comes before the first runtime call)
+    const size_t need = p.splits > 1 ? workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) : 0;
     if (p.splits > 1) {
-        const size_t need = workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k);
-        if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
-        if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
-        if (need >= (1ull << 31)) return BFAINTB_ERR_BAD_VARIANT;  // the kernel addresses the workspace with 32-bit offsets
-        p.partials = static_cast<unsigned long long*>(workspace);
-        p.partial_bytes = (uint32_t)need;
+        e = attach_workspace(p, workspace, workspace_bytes, need);
+        if (e) return e;
     }
+    DeviceState* dev = nullptr;
+    e = device_state(st, &dev);
+    if (e) return e;
 #ifdef BFAINTB_TRACE
     // timestamp sink: behind the split-K area (instrumented callers pass a larger workspace)
     p.trace = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + ((workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) + 255) & ~(size_t)255));
@@ -611,7 +715,7 @@ static size_t packed_workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits
     if (v != BFAINTB_VARIANT_DECODE || m == 0 || n == 0 || packed_uses_slab(m, n, k, bits)) return 0;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
     if (pl.splits <= 1) return 0;
-    return (((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u;
+    return bfaintb::kWorkspaceHeaderBytes + ((((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u);
 }
 
 size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant)
@@ -679,13 +783,12 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
         p.decode_cols = pl.cols;
         p.decode_mb = pl.mb;
         if (p.splits > 1) {
-            const size_t need = packed_workspace_need(m, n, k, weight_bits, v);
-            if (workspace == nullptr || workspace_bytes < need) return BFAINTB_ERR_WORKSPACE;
-            if (misaligned16(workspace)) return BFAINTB_ERR_ALIGNMENT;
-            if (need >= (1ull << 31)) return BFAINTB_ERR_BAD_VARIANT;
-            p.partials = static_cast<unsigned long long*>(workspace);
-            p.partial_bytes = (uint32_t)need;
+            e = attach_workspace(p, workspace, workspace_bytes, packed_workspace_need(m, n, k, weight_bits, v));
+            if (e) return e;
         }
+        DeviceState* dev = nullptr;
+        e = device_state(st, &dev);
+        if (e) return e;
         return (int)bfaintb::launch_decode_family_packed(p, weight_bits, st);
     }
     return (int)bfaintb::launch_decode_packed(p, weight_bits, st);

@@ -41,6 +41,17 @@ __device__ __forceinline__ float silu_gate(float g, float u)
 // bf16 inputs have zero low bits).
 constexpr uint32_t kEmptyWord = 0xffffffffu;
 
+// The first 256 bytes of a split-K workspace are its header; the partial sums follow.
+//   word 0  sticky failure mark: kEmptyWord while all is well, kWorkspaceGaveUp once a reducing workgroup has given up
+//           waiting for a partial sum (the workspace may then hold words at rest that are not empty: initialise it again)
+//   word 1  kWorkspaceMagic, written by the initialisation: tells an initialised workspace from arbitrary memory
+// The GEMM kernels never read the header; bfaintb_workspace_status does, on the host.
+constexpr uint32_t kWorkspaceHeaderBytes = 256;
+constexpr uint32_t kWorkspaceGaveUp = 0x0bad0badu;
+constexpr uint32_t kWorkspaceMagic = 0x42464157u;  // "BFAW"
+constexpr uint32_t kDefaultSplitWaitLimit = 1u << 18;  // re-reads of a split-K word before giving up (each a memory round trip)
+constexpr uint32_t kDebugWithholdPartials = 1u;        // GemmParams.debug_flags: producers keep their sums to themselves
+
 template <typename Tuple, size_t... I>
 inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 {
@@ -82,6 +93,9 @@ struct GemmParams {
     uint32_t splits;     // workgroups along k
     unsigned long long* partials;  // [splits - 1][m][n] fp32 partial sums; kEmptyWord wherever none is waiting
     uint32_t partial_bytes;        // size of that area (below 2^31)
+    uint32_t* ws_header;           // the workspace's header (see kWorkspaceHeaderBytes), or null without split-K
+    uint32_t split_wait_limit;     // fetch attempts of the reducing workgroup before it gives up
+    uint32_t debug_flags;          // kDebug* (test hooks; zero in normal operation)
 #ifdef BFAINTB_TRACE
     unsigned long long* trace;  // timestamp sink (instrumented builds only)
 #endif

@@ -2,7 +2,7 @@
 // decode kernel that streams that order.
 //
 // The reference ships B to the device exactly as the host wrote it, row-major K x N
-// (/root/reference/bfAintBGemm/include/mem_transfer.hpp:23-32, bfAintBGemm.cc:101-103), and its kernel re-reads
+// (/root/reference/bfAintBGemm/mem_transfer.hpp:23-32, bfAintBGemm.cc:101-103), and its kernel re-reads
 // it with a row stride (bf16gemm_kernel_gfx90a.s:239-262).  Row-major B forces a decode workgroup to own at
 // least 128 columns (whole 128-byte lines per row), so n = 4096 yields 32 column blocks and the other CUs have
 // to be filled by splitting K, with a second pass over partial sums.  In the packed order a block of 16 columns
@@ -224,7 +224,9 @@ __device__ __forceinline__ void decode_packed_body(const GemmParams& p)
         for (int i = 0; i < kBatch; ++i) {
             uint32_t c = base + (uint32_t)i * kPackedWaves;
             if (c >= chunks) c = chunks - 1u;
-            b.w[i] = *reinterpret_cast<const uint4*>(slab + (size_t)c * 1024u);
+            // (non-temporal: read once, streamed past the caches' other contents)
+            const u32x4_t wv = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(slab + (size_t)c * 1024u));
+            b.w[i] = make_uint4(wv[0], wv[1], wv[2], wv[3]);
 #pragma unroll
             for (uint32_t h = 0; h < kBlocks; ++h)
 #pragma unroll

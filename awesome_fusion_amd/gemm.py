@@ -130,6 +130,12 @@ def lib():
         L.bfaintb_error_string.restype = C.c_char_p
         L.bfaintb_error_string.argtypes = [C.c_int]
         L.bfaintb_version.restype = C.c_int
+        L.bfaintb_workspace_status.restype = C.c_int
+        L.bfaintb_workspace_status.argtypes = [_vp, _vp]
+        L.bfaintb_init.restype = C.c_int
+        L.bfaintb_init.argtypes = [_vp]
+        L.bfaintb_debug_control.restype = C.c_int
+        L.bfaintb_debug_control.argtypes = [_u32, _u32]
         _lib = L
     return _lib
 
@@ -182,6 +188,28 @@ def workspace_init(workspace, nbytes=None, stream=None):
     rc = lib().bfaintb_workspace_init(_ptr(workspace), nbytes, _stream_handle(stream))
     if rc:
         raise BfaintbError(rc, "bfaintb_workspace_init")
+
+
+def workspace_status(workspace, stream=None):
+    """bfaintb_workspace_status: 0, or a negative BFAINTB_ERR_* (never initialised / a split-K wait gave up)."""
+    return lib().bfaintb_workspace_status(_ptr(workspace), _stream_handle(stream))
+
+
+def init(stream=None):
+    """bfaintb_init on the current device (kernel attributes); needed only before a first call under capture."""
+    rc = lib().bfaintb_init(_stream_handle(stream))
+    if rc:
+        raise BfaintbError(rc, "bfaintb_init")
+
+
+DEBUG_SPLIT_WAIT_LIMIT, DEBUG_WITHHOLD_PARTIALS = 1, 2
+ERR_WORKSPACE, ERR_NOT_INITIALISED, ERR_WORKSPACE_POISONED = -6, -8, -9
+
+
+def debug_control(what, value):
+    rc = lib().bfaintb_debug_control(what, value)
+    if rc:
+        raise BfaintbError(rc, "bfaintb_debug_control")
 
 
 def _epilogue(bias, residual, ldr, n, activation=ACT_NONE):

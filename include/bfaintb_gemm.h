@@ -14,8 +14,12 @@
  *
  * All pointers are DEVICE pointers owned by the caller.  Calls are asynchronous and ordered on
  * `stream` (a hipStream_t passed as void*; NULL is the default stream, which is what the reference
- * launches on).  No call allocates, frees or synchronises.  Return value: 0 on success, a negative
- * BFAINTB_ERR_* for a rejected argument (nothing was launched), or a positive hipError_t.
+ * launches on).  No call allocates or frees; only bfaintb_init and bfaintb_workspace_status wait for the
+ * device.  Return value: 0 on success, a negative BFAINTB_ERR_* for a rejected argument (nothing was
+ * launched), or a positive hipError_t.
+ *
+ * The first GEMM call on a device prepares the library's kernels there (a few runtime calls that are not
+ * stream operations).  A caller whose first call would come under stream capture runs bfaintb_init before.
  */
 #ifndef BFAINTB_GEMM_H
 #define BFAINTB_GEMM_H
@@ -33,7 +37,7 @@ extern "C" {
 #define BFAINTB_API
 #endif
 
-#define BFAINTB_VERSION 107 /* major*10000 + minor*100 + patch */
+#define BFAINTB_VERSION 200 /* major*10000 + minor*100 + patch */
 
 enum {
     BFAINTB_OK = 0,
@@ -43,7 +47,9 @@ enum {
     BFAINTB_ERR_ALIGNMENT = -4,     /* a pointer is not 16-byte aligned */
     BFAINTB_ERR_UNSUPPORTED = -5,   /* weight_bits not 8 or 4; group_size not 0 or a multiple of 32 dividing k */
     BFAINTB_ERR_WORKSPACE = -6,     /* workspace NULL/too small for this shape (see bfaintb_gemm_workspace_bytes) */
-    BFAINTB_ERR_BAD_VARIANT = -7    /* unknown variant, or a variant that cannot run this shape */
+    BFAINTB_ERR_BAD_VARIANT = -7,   /* unknown variant, or a variant that cannot run this shape */
+    BFAINTB_ERR_NOT_INITIALISED = -8,     /* the first call on a device came under stream capture: call bfaintb_init before */
+    BFAINTB_ERR_WORKSPACE_POISONED = -9   /* bfaintb_workspace_status: a split-K wait gave up on this workspace */
 };
 
 /* Which kernel family runs a shape. */
@@ -79,7 +85,7 @@ enum {
  *   group_size    0: one scale per output channel (the reference's only mode);
  *                 otherwise rows per scale group along k (multiple of 32, divides k)
  *   workspace     device scratch of at least bfaintb_gemm_workspace_bytes(...) bytes that has been
- *                 passed through bfaintb_workspace_init once (equivalently: every byte is 0xff).
+ *                 passed through bfaintb_workspace_init once.
  *                 The call leaves it in that state again, ready for the next call of any shape.
  *                 Two calls that may run concurrently must not share a workspace.  May be NULL
  *                 when the required size is 0.
@@ -153,16 +159,46 @@ BFAINTB_API int bfaintb_gemm_reference_ex(void* c, const void* a, const void* b,
                               uint32_t lda, uint32_t ldb, uint32_t ldc, void* workspace, size_t workspace_bytes, void* stream,
                               int variant, uint32_t split_k);
 
-/* Scratch the GEMM needs for a shape: one fp32 word per (split but the last, row, column) of the
- * split-K partial sums, rounded up to 256 bytes; 0 when the shape runs without split-K.  Depends only
+/* Scratch the GEMM needs for a shape: a 256-byte header, then one fp32 word per (split but the last, row,
+ * column) of the split-K partial sums, rounded up to 256 bytes; 0 when the shape runs without split-K.  Depends only
  * on its arguments.  The reference kernel has no scratch (no split-K, bfAintBGemm.cc:107-109). */
 BFAINTB_API size_t bfaintb_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 BFAINTB_API size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
                                        int variant, uint32_t split_k);
 
-/* Prepares a freshly allocated workspace: marks every word "no partial sum here" (all bits set).
- * Stream-ordered, graph-capturable; workspace_bytes must be a multiple of 4. */
+/* Prepares a freshly allocated workspace: marks every word "no partial sum here" (all bits set) and writes the
+ * 256-byte header the sizes above include.  Stream-ordered, graph-capturable; workspace_bytes a multiple of 4, at least 256. */
 BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Health of a workspace, read back from its header (waits for `stream`): BFAINTB_OK; BFAINTB_ERR_WORKSPACE when the
+ * memory was never passed through bfaintb_workspace_init; BFAINTB_ERR_WORKSPACE_POISONED when a reducing workgroup
+ * gave up waiting for a partial sum (after 2^18 fetch attempts, about a tenth of a second: the workgroups it waits
+ * for wait for nothing themselves, so this means a launch was lost or two overlapping calls shared the workspace).
+ * The output of that call holds NaNs where the sums were incomplete, and the workspace may hold stray partial sums:
+ * initialise it again before further use.  The mark is sticky until then.  No counterpart in the reference (no
+ * split-K there, bfAintBGemm.cc:107-109).
+ */
+BFAINTB_API int bfaintb_workspace_status(const void* workspace, void* stream);
+
+/*
+ * Prepares the library on the current device (kernel attributes).  Optional: the first GEMM call on a device does the same by
+ * itself, except under stream capture, where it returns BFAINTB_ERR_NOT_INITIALISED instead.  Call it outside any
+ * capture, once per device (further calls return at once).  Stands where the reference's main() loads its code object
+ * (bfAintBGemm.cc:63-66: hipSetDevice, hipModuleLoad, hipModuleGetFunction).
+ */
+BFAINTB_API int bfaintb_init(void* stream);
+
+/*
+ * Test hooks (no effect on results in normal operation; process-wide, read by each following launch):
+ *   BFAINTB_DEBUG_SPLIT_WAIT_LIMIT   value = fetch attempts a reducing workgroup makes before it gives up (0 restores 2^18)
+ *   BFAINTB_DEBUG_WITHHOLD_PARTIALS  value != 0: the workgroups of all splits but the last compute and then keep their
+ *                                    sums to themselves, so the reducer's wait runs out — the way to exercise the
+ *                                    give-up path with every kernel exiting normally
+ */
+#define BFAINTB_DEBUG_SPLIT_WAIT_LIMIT 1u
+#define BFAINTB_DEBUG_WITHHOLD_PARTIALS 2u
+BFAINTB_API int bfaintb_debug_control(uint32_t what, uint32_t value);
 
 /*
  * Pre-packed weights.  bfaintb_prepack reorders a row-major B (the layout above) once, offline, into the operand
@@ -171,7 +207,7 @@ BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, 
  * block of 16 columns is then one contiguous slab, n / 16 workgroups stream their slabs linearly and own their
  * outputs, and a few rows of A (8 in general; more on small matrices and for 4-bit codes) need no split along k, no workspace
  * and no second pass.  Successor of the
- * reference's host-side formatter mem_transfer<int8_t, ...> (include/mem_transfer.hpp:23-32), which writes the
+ * reference's host-side formatter mem_transfer<int8_t, ...> (mem_transfer.hpp:23-32), which writes the
  * bytes the device will read; the reference itself keeps B row-major (bfAintBGemm.cc:101-103).
  *   packed    device buffer of bfaintb_prepack_bytes(n, k, weight_bits) bytes (= n * k * weight_bits / 8), 16-byte aligned;
  *             4-bit codes need k % 128 == 0 in this format (bfaintb_prepack_bytes returns 0 otherwise)

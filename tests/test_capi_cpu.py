@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(af.library_path())
     for name in names:
         assert hasattr(lib, name), name
-    assert af.lib().bfaintb_version() == 107
+    assert af.lib().bfaintb_version() == 200
     assert "bfaintb_gemm_bias" in names
 
 
@@ -63,7 +63,7 @@ def test_variant_choice_and_split():
     s = af.split_k(1, 4096, 4096)
     assert 1 < s <= 64 and 4096 % s == 0
     # none for the prefill variant or without split-K
-    assert af.workspace_bytes(1, 4096, 4096) == (s - 1) * 1 * 4096 * 4   # one fp32 word per (split but the last, row, column)
+    assert af.workspace_bytes(1, 4096, 4096) == 256 + (s - 1) * 1 * 4096 * 4   # the header, then one fp32 word per (split but the last, row, column)
     assert af.workspace_bytes(4096, 4096, 4096) == 0
     assert af.workspace_bytes(8, 4096, 4096, force_split_k=1) == 0
     assert af.kernel_name(1) == "bfaintb_decode_kernel" and af.kernel_name(4096) == "bfaintb_prefill_kernel"

@@ -208,8 +208,47 @@ def test_workspace_is_left_ready_for_the_next_call(af):
     for i, (m, n, k) in enumerate(shapes):
         p = Problem(m, n, k, seed=i)
         assert_close_ulp(p, run_gemm(p), f"call {i}")
-        # every word of the workspace is back to "no partial sum here" (all bits set)
-        assert bool((helpers._ws.t == 0xFF).all()), f"workspace not restored after call {i}"
+        # every word behind the 256-byte header is back to "no partial sum here" (all bits set); the header says "healthy"
+        assert bool((helpers._ws.t[256:] == 0xFF).all()), f"workspace not restored after call {i}"
+        assert af.workspace_status(helpers._ws.t) == 0
+
+
+def test_workspace_status_and_the_give_up_path(af):
+    """The reducer's bounded wait, driven from the host so that every kernel exits normally: the producing workgroups are
+    told to keep their sums (a test hook), the reducer's attempts are capped at a few, so it gives up: the output holds
+    NaNs, the workspace's header records it until the workspace is initialised again, and then everything works."""
+    import torch
+    p = Problem(4, 1024, 4096, seed=5)
+    need = af.workspace_bytes(p.m, p.n, p.k)
+    assert need > 256 and af.split_k(p.m, p.n, p.k) > 1
+    raw = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    assert af.workspace_status(raw) == af.ERR_WORKSPACE            # arbitrary memory: never initialised
+    af.workspace_init(raw)
+    assert af.workspace_status(raw) == 0
+    a, b, s = to_dev(p.a_bf), to_dev(p.b_bytes), to_dev(p.s_bf)
+    c = torch.zeros((p.m, p.n), dtype=torch.int16, device="cuda")
+    af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=raw)
+    torch.cuda.synchronize()
+    good = from_dev_u16(c).copy()
+    assert_close_ulp(p, good, "before")
+    assert af.workspace_status(raw) == 0
+    try:
+        af.debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 3)
+        af.debug_control(af.DEBUG_WITHHOLD_PARTIALS, 1)
+        af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=raw)
+        torch.cuda.synchronize()
+    finally:
+        af.debug_control(af.DEBUG_WITHHOLD_PARTIALS, 0)
+        af.debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 0)
+    bad = from_dev_u16(c)
+    assert np.isnan(widen(bad)).all(), "every output misses partial sums: all NaN"
+    assert af.workspace_status(raw) == af.ERR_WORKSPACE_POISONED
+    assert af.workspace_status(raw) == af.ERR_WORKSPACE_POISONED   # sticky
+    af.workspace_init(raw)
+    assert af.workspace_status(raw) == 0
+    af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=raw)
+    torch.cuda.synchronize()
+    assert np.array_equal(from_dev_u16(c), good)
 
 
 def test_prefill_variant_on_small_m_matches_decode(af):
@@ -449,3 +488,45 @@ def test_empty_and_minimal_shapes(af):
     assert af.gemm(a, a, a, a, 0, 16, 64) == 0     # m = 0: nothing to do, nothing launched
     assert af.gemm(a, a, a, a, 4, 0, 64) == 0      # n = 0
     torch.cuda.synchronize()
+
+
+def test_first_call_under_capture_is_refused_until_init():
+    """A fresh process whose first library call comes under stream capture: the call is refused (the per-device set-up
+    makes runtime calls that are not stream operations) and nothing is recorded; after bfaintb_init the same capture
+    works and replays correctly."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r'''
+import sys
+sys.path.insert(0, %r); sys.path.insert(0, %r)
+import numpy as np, torch
+import awesome_fusion_amd as af
+from helpers import Problem, to_dev, from_dev_u16, assert_close_ulp
+p = Problem(4, 1024, 4096, seed=3)
+a, b, s = to_dev(p.a_bf), to_dev(p.b_bytes), to_dev(p.s_bf)
+c = torch.zeros((p.m, p.n), dtype=torch.int16, device="cuda")
+ws = torch.empty(af.workspace_bytes(p.m, p.n, p.k), dtype=torch.uint8, device="cuda")
+torch.cuda.synchronize()
+g = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g):
+    rc_ws = af.lib().bfaintb_workspace_init(ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    rc = af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=ws, check=False)
+assert rc_ws == 0 and rc == af.ERR_NOT_INITIALISED, (rc_ws, rc)
+g.replay()   # what was recorded: the workspace's initialisation (fill kernels), nothing of the refused calls
+torch.cuda.synchronize()
+assert af.workspace_status(ws) == 0
+af.init()
+g2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g2):
+    af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=ws)
+for rep in range(3):
+    c.zero_()
+    g2.replay()
+    torch.cuda.synchronize()
+    assert_close_ulp(p, from_dev_u16(c), "replay %%d" %% rep)
+print("capture-first ok")
+''' % (root, os.path.join(root, "tests"))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "capture-first ok" in r.stdout, r.stdout[-2000:] + r.stderr[-3000:]
