@@ -29,6 +29,12 @@ hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_
 hipError_t decode_prepare_device();
 }  // namespace bfaintb
 
+// Split-K scratch of bfaintb_gemm_static: one array per GPU the library runs on, held until the process ends.  In host
+// code this name is only a handle for hipGetSymbolAddress; device_state() resolves it once per device and everything
+// else uses the resolved pointer.
+#define BFAINTB_STATIC_SCRATCH_BYTES (8u << 20)
+static __device__ __align__(256) unsigned char scratch[BFAINTB_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 using bfaintb::GemmParams;
@@ -305,10 +311,12 @@ size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant,
 
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
 
-// ---- per-device set-up: kernel attributes ----
+// ---- per-device set-up: kernel attributes, and the address and first filling of the static scratch ----
 constexpr int kMaxDevices = 64;
 struct DeviceState {
     std::atomic<int> ready{0};      // kernel attributes set on this device
+    std::atomic<int> scratch_ready{0};  // static scratch resolved and filled with the empty pattern
+    void* scratch_ptr = nullptr;
 };
 DeviceState g_devices[kMaxDevices];
 std::mutex g_setup_mutex;
@@ -359,6 +367,29 @@ int init_workspace_on(void* workspace, size_t workspace_bytes, hipStream_t strea
     return (int)e;
 }
 
+// The device's static scratch, resolved and (the first time, outside any capture) filled with the empty pattern.
+int static_scratch(DeviceState& st, hipStream_t stream, void** out)
+{
+    if (!st.scratch_ready.load(std::memory_order_acquire)) {
+        if (stream_is_capturing(stream)) return BFAINTB_ERR_NOT_INITIALISED;
+        std::lock_guard<std::mutex> lock(g_setup_mutex);
+        if (!st.scratch_ready.load(std::memory_order_relaxed)) {
+            void* ptr = nullptr;
+            hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            if (ptr == nullptr) return BFAINTB_ERR_WORKSPACE;
+            const int rc = init_workspace_on(ptr, BFAINTB_STATIC_SCRATCH_BYTES, stream);
+            if (rc) return rc;
+            e = hipStreamSynchronize(stream);  // once per device: every stream may use the scratch from here on
+            if (e != hipSuccess) return (int)e;
+            st.scratch_ptr = ptr;
+            st.scratch_ready.store(1, std::memory_order_release);
+        }
+    }
+    *out = st.scratch_ptr;
+    return BFAINTB_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -378,6 +409,7 @@ const char* bfaintb_error_string(int code)
         case BFAINTB_ERR_BAD_VARIANT: return "unknown kernel variant, or variant cannot run this shape";
         case BFAINTB_ERR_NOT_INITIALISED: return "first call on this device made under stream capture: call bfaintb_init() beforehand";
         case BFAINTB_ERR_WORKSPACE_POISONED: return "a split-K wait gave up on this workspace (results of that call hold NaNs): initialise it again";
+        case BFAINTB_ERR_STATIC_SCRATCH: return "shape needs more split-K scratch than bfaintb_gemm_static holds (8 MiB): use bfaintb_gemm with a workspace";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -436,7 +468,10 @@ int bfaintb_init(void* stream)
 {
     hipStream_t st = static_cast<hipStream_t>(stream);
     DeviceState* dev = nullptr;
-    return device_state(st, &dev);
+    int rc = device_state(st, &dev);
+    if (rc) return rc;
+    void* ptr = nullptr;
+    return static_scratch(*dev, st, &ptr);
 }
 
 int bfaintb_debug_control(uint32_t what, uint32_t value)
@@ -493,7 +528,7 @@ static int attach_workspace(GemmParams& p, void* workspace, size_t workspace_byt
 
 static int gemm_impl(void* c, const void* a, const void* b, const void* scale, const Epilogue& ep, uint32_t m, uint32_t n, uint32_t k,
                      uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
-                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k)
+                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k, bool use_static_scratch = false)
 {
     const void* bias = ep.bias;
     int e = check_format(k, weight_bits, group_size);
@@ -548,13 +583,20 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.decode_mb = pl.mb;
     // (every argument check comes before the first runtime call)
     const size_t need = p.splits > 1 ? workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) : 0;
-    if (p.splits > 1) {
+    if (p.splits > 1 && !use_static_scratch) {
         e = attach_workspace(p, workspace, workspace_bytes, need);
         if (e) return e;
     }
+    if (use_static_scratch && need > BFAINTB_STATIC_SCRATCH_BYTES) return BFAINTB_ERR_STATIC_SCRATCH;
     DeviceState* dev = nullptr;
     e = device_state(st, &dev);
     if (e) return e;
+    if (p.splits > 1 && use_static_scratch) {
+        e = static_scratch(*dev, st, &workspace);
+        if (e) return e;
+        e = attach_workspace(p, workspace, BFAINTB_STATIC_SCRATCH_BYTES, need);
+        if (e) return e;
+    }
 #ifdef BFAINTB_TRACE
     // timestamp sink: behind the split-K area (instrumented callers pass a larger workspace)
     p.trace = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(workspace) + ((workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) + 255) & ~(size_t)255));
@@ -873,6 +915,15 @@ int bfaintb_gemm(void* c, const void* a, const void* b, const void* scale, uint3
     return bfaintb_gemm_ex(c, a, b, scale, m, n, k, lda, ldb, ldc, weight_bits, group_size, workspace, workspace_bytes,
                            stream, BFAINTB_VARIANT_AUTO, 0);
 }
+
+int bfaintb_gemm_static(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k, uint32_t lda,
+                        uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* stream)
+{
+    return gemm_impl(c, a, b, scale, Epilogue{}, m, n, k, lda, ldb, ldc, weight_bits, group_size, nullptr, 0, stream, BFAINTB_VARIANT_AUTO,
+                     0, true);
+}
+
+size_t bfaintb_gemm_static_scratch_bytes(void) { return BFAINTB_STATIC_SCRATCH_BYTES; }
 
 int bfaintb_dequant(void* w, const void* b, const void* scale, uint32_t n, uint32_t k, uint32_t ldb, uint32_t ldw,
                     int weight_bits, uint32_t group_size, void* stream)

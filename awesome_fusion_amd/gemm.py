@@ -134,6 +134,10 @@ def lib():
         L.bfaintb_workspace_status.argtypes = [_vp, _vp]
         L.bfaintb_init.restype = C.c_int
         L.bfaintb_init.argtypes = [_vp]
+        L.bfaintb_gemm_static.restype = C.c_int
+        L.bfaintb_gemm_static.argtypes = [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, C.c_int, _u32, _vp]
+        L.bfaintb_gemm_static_scratch_bytes.restype = C.c_size_t
+        L.bfaintb_gemm_static_scratch_bytes.argtypes = []
         L.bfaintb_debug_control.restype = C.c_int
         L.bfaintb_debug_control.argtypes = [_u32, _u32]
         _lib = L
@@ -196,14 +200,23 @@ def workspace_status(workspace, stream=None):
 
 
 def init(stream=None):
-    """bfaintb_init on the current device (kernel attributes); needed only before a first call under capture."""
+    """bfaintb_init on the current device (kernel attributes, static scratch); needed only before a first call under capture."""
     rc = lib().bfaintb_init(_stream_handle(stream))
     if rc:
         raise BfaintbError(rc, "bfaintb_init")
 
 
+def gemm_static(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bits=8, group_size=0, stream=None, check=True):
+    """bfaintb_gemm_static: the GEMM on the library's own per-GPU scratch; allocates nothing."""
+    rc = lib().bfaintb_gemm_static(_ptr(c), _ptr(a), _ptr(b), _ptr(scale), m, n, k, k if lda is None else lda,
+                                   n if ldb is None else ldb, n if ldc is None else ldc, weight_bits, group_size, _stream_handle(stream))
+    if rc and check:
+        raise BfaintbError(rc, "bfaintb_gemm_static")
+    return rc
+
+
 DEBUG_SPLIT_WAIT_LIMIT, DEBUG_WITHHOLD_PARTIALS = 1, 2
-ERR_WORKSPACE, ERR_NOT_INITIALISED, ERR_WORKSPACE_POISONED = -6, -8, -9
+ERR_WORKSPACE, ERR_NOT_INITIALISED, ERR_WORKSPACE_POISONED, ERR_STATIC_SCRATCH = -6, -8, -9, -10
 
 
 def debug_control(what, value):

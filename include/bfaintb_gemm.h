@@ -49,7 +49,8 @@ enum {
     BFAINTB_ERR_WORKSPACE = -6,     /* workspace NULL/too small for this shape (see bfaintb_gemm_workspace_bytes) */
     BFAINTB_ERR_BAD_VARIANT = -7,   /* unknown variant, or a variant that cannot run this shape */
     BFAINTB_ERR_NOT_INITIALISED = -8,     /* the first call on a device came under stream capture: call bfaintb_init before */
-    BFAINTB_ERR_WORKSPACE_POISONED = -9   /* bfaintb_workspace_status: a split-K wait gave up on this workspace */
+    BFAINTB_ERR_WORKSPACE_POISONED = -9,  /* bfaintb_workspace_status: a split-K wait gave up on this workspace */
+    BFAINTB_ERR_STATIC_SCRATCH = -10      /* bfaintb_gemm_static: the shape needs more scratch than the library holds */
 };
 
 /* Which kernel family runs a shape. */
@@ -182,12 +183,28 @@ BFAINTB_API int bfaintb_workspace_init(void* workspace, size_t workspace_bytes, 
 BFAINTB_API int bfaintb_workspace_status(const void* workspace, void* stream);
 
 /*
- * Prepares the library on the current device (kernel attributes).  Optional: the first GEMM call on a device does the same by
+ * Prepares the library on the current device — kernel attributes, and the scratch of bfaintb_gemm_static filled with
+ * its at-rest pattern on `stream` — and waits for that.  Optional: the first GEMM call on a device does the same by
  * itself, except under stream capture, where it returns BFAINTB_ERR_NOT_INITIALISED instead.  Call it outside any
  * capture, once per device (further calls return at once).  Stands where the reference's main() loads its code object
  * (bfAintBGemm.cc:63-66: hipSetDevice, hipModuleLoad, hipModuleGetFunction).
  */
 BFAINTB_API int bfaintb_init(void* stream);
+
+/*
+ * The GEMM for callers that cannot allocate or carry a workspace — code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  bfaintb_gemm without the workspace arguments: the split-K partial sums go to a
+ * scratch array the library holds in device memory, one per GPU, 8 MiB (bfaintb_gemm_static_scratch_bytes), kept
+ * until the process ends.  Same kernels, same variant choice and bit-for-bit the results of bfaintb_gemm.  A shape
+ * whose bfaintb_gemm_workspace_bytes exceeds the scratch is refused with BFAINTB_ERR_STATIC_SCRATCH (nothing launched).
+ * Every call on a GPU shares that GPU's scratch (each call leaves it in its at-rest state for the next): calls that may
+ * overlap on one GPU — different streams, different host threads — race on it and must use bfaintb_gemm with
+ * workspaces of their own.  Allocates nothing, on any call.  No counterpart in the reference, whose kernel needs no
+ * scratch (no split-K).
+ */
+BFAINTB_API int bfaintb_gemm_static(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
+                        uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* stream);
+BFAINTB_API size_t bfaintb_gemm_static_scratch_bytes(void);
 
 /*
  * Test hooks (no effect on results in normal operation; process-wide, read by each following launch):

@@ -513,7 +513,8 @@ g = torch.cuda.CUDAGraph()
 with torch.cuda.graph(g):
     rc_ws = af.lib().bfaintb_workspace_init(ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
     rc = af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=ws, check=False)
-assert rc_ws == 0 and rc == af.ERR_NOT_INITIALISED, (rc_ws, rc)
+    rc_static = af.gemm_static(c, a, b, s, p.m, p.n, p.k, check=False)
+assert rc_ws == 0 and rc == af.ERR_NOT_INITIALISED and rc_static == af.ERR_NOT_INITIALISED, (rc_ws, rc, rc_static)
 g.replay()   # what was recorded: the workspace's initialisation (fill kernels), nothing of the refused calls
 torch.cuda.synchronize()
 assert af.workspace_status(ws) == 0
