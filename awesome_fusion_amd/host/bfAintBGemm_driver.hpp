@@ -220,13 +220,18 @@ inline int driver_main(int argc, char** argv, const HostChecker* checker, Driver
             // the reference's own criterion (exact small-integer data)
             res = valid_vector<CDataType>(c_ref.data(), c_dev.data(), m * n);
         } else {
-            // sum_k |a*w| per output, from the same host routine, bounds the rounding noise of either side's fp32 sum
+            // sum_k |a*w| per output, from the same host routine: 12 * 2^-24 of it covers the rounding error of an fp32 sum of those
+            // terms on both sides (measured worst: 4.4 such units for the sequential host sum, 1.3 for the device); only outputs
+            // that cancel to almost nothing (below an eighth of the rms of C) may lean on it
             std::vector<float> noise((std::size_t)m * n);
             for (auto& v : a_seen) v = std::fabs(v);
             for (auto& v : w_seen) v = std::fabs(v);
             checker->gemm_rrr(noise.data(), a_seen.data(), w_seen.data(), ones.data(), m, n, k, lda, n, n);
-            const float noise_scale = 2.0f * std::sqrt((float)k) * std::ldexp(1.0f, -24);
-            for (auto& v : noise) v *= noise_scale;
+            double sq = 0.0;
+            for (const float v : c_ref) sq += (double)v * v;
+            const float near_zero = 0.125f * (float)std::sqrt(sq / ((double)m * n));
+            const float noise_scale = 12.0f * std::ldexp(1.0f, -24);
+            for (std::size_t i = 0; i < noise.size(); ++i) noise[i] = std::fabs(c_ref[i]) < near_zero ? noise[i] * noise_scale : 0.0f;
             const UlpReport rep = valid_vector_ulp(c_ref.data(), c_dev.data(), (long)m * n, 2.0, 1e-3, 1e-2, noise.data());
             // outputs that cancel to almost nothing: at most 2 in 10^4 (plus three), each within the noise bound
             const long allowed = (long)((double)m * n * 2e-4) + 3;

@@ -49,9 +49,9 @@ struct UlpReport {
 };
 
 // `noise`, if given, is a per-element bound on what the rounding of an fp32 sum may contribute on either
-// side (the caller passes 2 * sqrt(k) * 2^-24 * sum_k |a*w|): an output that cancels to almost nothing can
-// differ from the reference by more than two of ITS ULPs whatever order the device adds in.  Such elements
-// are counted separately; the caller decides how many it tolerates.
+// side (the caller passes a few times 2^-24 * sum_k |a*w| for outputs near zero, and 0 elsewhere): an output
+// that cancels to almost nothing can differ from the reference by more than two of ITS ULPs whatever order
+// the device adds in.  Such elements are counted separately; the caller decides how many it tolerates.
 inline UlpReport valid_vector_ulp(const float* ref, const bfloat16* pred, long n, double max_ulp = 2.0, double small_abs = 1e-3,
                                   double small_rel = 1e-2, const float* noise = nullptr)
 {

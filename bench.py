@@ -1,23 +1,26 @@
 #!/usr/bin/env python3
 """Benchmark of the bfAintBGemm hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
-    python bench.py --scan [narrow]   (a map of kernel times over shapes and m, not the benchmark)
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu] [--only WORKLOAD]
 
 A step is one GEMM launch through the C ABI on synthetic, seeded inputs already resident in HBM.
 The headline workload is the decode shape the metric is quoted on (bf16 A [1,4096] x int8 B
-[4096,4096], per-channel bf16 scales); the prefill shape (M = 4096) is measured in the same run and
-reported under "extra".  The metric definitions follow the reference driver's printout
-(/root/reference/bfAintBGemm/bfAintBGemm.cc:186-195: flops = 2mnk, bytes = 2(mk+mn) + nk) with two
-corrections stated in the output: decimal units, and the scale bytes are counted.
+[4096,4096], per-channel bf16 scales); the prefill shape (M = 4096), the decode sweep over the MLP
+up-projection shape (N = 11008, M = 1, 16, 32) and the 4-bit group-128 shape (28672 x 8192, M = 1, 16, 2048)
+are measured in the same run and reported under "extra".  The metric definitions follow the reference
+driver's printout (/root/reference/bfAintBGemm/bfAintBGemm.cc:186-195: flops = 2mnk, bytes = 2(mk+mn) + nk)
+with two corrections stated in the output: decimal units, and the scale bytes are counted.
 
-Timing: W untimed warm-up launches, then exactly K launches recorded into one HIP graph; the graph is
-replayed five times, each replay between its own pair of events on the launch stream (and a host
-clock, after/before a device synchronize), and the median replay is reported.  The graph keeps host launch overhead out of a microsecond-scale kernel's
-measurement; the reference's own protocol is the same minus the graph (10 launches in one event pair,
-bfAintBGemm.cc:171-186).  For the decode shape consecutive launches read DIFFERENT copies of B
-(enough copies to exceed the 256 MB last-level cache), so the figure is an HBM figure; the
-same-buffer ("hot") figure is reported beside it.
+Timing: W untimed warm-up launches, then HIP graphs of exactly K launches each.  Consecutive launches read
+DIFFERENT copies of B, and the rotation carries on from one graph to the next (ceil(copies / K) graphs, replayed
+in turn), so that whatever K is every copy is re-read only after all the others — more than twice the 256 MB
+last-level cache — have passed: the decode figures are HBM figures (the same-buffer "hot" figure is reported
+beside the headline).  An event pair on the launch stream (and a host clock, after/before a device
+synchronize) brackets enough back-to-back replays to hold at least 400 launches, so the graph-launch latency is
+amortised the same way for K = 20 as for K = 400; five such measurements, the median is reported; a step is
+one launch, ms_per_step = elapsed / launches.  The graph keeps host launch overhead out of a microsecond-scale
+kernel's measurement; the reference's own protocol is the same minus the graph (10 launches in one event pair,
+bfAintBGemm.cc:171-186).
 """
 import argparse
 import json
@@ -33,19 +36,23 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 LLC_BYTES = 256 << 20
-REPLAYS = 5                   # timed replays of the K-launch graph; the median one is reported
+REPLAYS = 5                   # timed measurements; the median one is reported
+MIN_LAUNCHES = 400            # launches inside one event pair (several replays of the K-launch graphs)
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
-# scaled by the same counters on a copy kernel of known size); see profiles/*.txt for the runs.
-MEASURED_TRAFFIC_BYTES = {
-    # fetch 8392.5 KiB x 1.997 + write 232.0 KiB (plain launches; profiles/bench_pmc_fetch_size.txt, bench_pmc_write_size.txt)
-    "decode_m1_n4096_k4096_int8_perchannel": 17398385,
-    # fetch 65698.5 KiB x 1.997 + write 32768.0 KiB (plain launches)
-    "prefill_m4096_n4096_k4096_int8_perchannel": 167893415,
-    # the same shapes through bfaintb_gemm_prepacked: fetch 8273.0 KiB x 1.997 + write 8.0 KiB; fetch 65712.0 KiB x 1.997 + write 32768.0 KiB
-    "decode_m1_n4096_k4096_int8_perchannel_prepacked": 16924658,
-    "prefill_m4096_n4096_k4096_int8_perchannel_prepacked": 167921020,
+# HBM bytes per launch RECORDED from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file's own --only commands
+# (KiB per dispatch, each scaled by what the same counter reads for a copy kernel of known size: fetch x 1.997,
+# write x 1.000); the files under profiles/ hold the runs.  Not measured by a plain run of this file: the output
+# names the source beside the figure.
+RECORDED_TRAFFIC = {
+    # name: (bytes, source)
+    "decode_m1_n4096_k4096_int8_perchannel": (17398385, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
+    "prefill_m4096_n4096_k4096_int8_perchannel": (167893415, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
+    "decode_m1_n4096_k4096_int8_perchannel_prepacked": (16924658, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
+    "prefill_m4096_n4096_k4096_int8_perchannel_prepacked": (167921020, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
 }
+
+C3_ROWS = (1, 16, 32)        # BASELINE config 3 (M in {1,4,8,16,32}): the rows the default line carries; --sweep has all five
+C5_ROWS = (1, 16, 2048)      # BASELINE config 5: 4-bit codes, scale groups of 128 rows
 
 
 def algorithmic_bytes(m, n, k, bits, group):
@@ -78,6 +85,16 @@ class Workload:
         self.bytes = algorithmic_bytes(m, n, k, bits, group)
         self.flops = 2 * m * n * k
 
+    def rows(self, m, name):
+        """The same weights against the first m rows of A (a view: nothing is copied)."""
+        import copy
+        w = copy.copy(self)
+        w.name, w.m = name, m
+        w.a, w.c = self.a[:m], self.c[:m]
+        w.bytes = algorithmic_bytes(m, self.n, self.k, self.bits, self.group)
+        w.flops = 2 * m * self.n * self.k
+        return w
+
     def workspace(self, af):
         import torch
         need = af.workspace_bytes(self.m, self.n, self.k, self.bits, self.group)
@@ -88,7 +105,45 @@ class Workload:
         return ws
 
 
-def time_graph(af, w, steps, warmup, rotate, packed=False):
+def time_launches(launch, nb, steps, warmup):
+    """launch(i) issues the i-th launch of a rotation over nb buffers.  Returns (event_ms_per_launch, wall_ms_per_launch,
+    info): graphs of `steps` launches each that together walk the whole rotation, replayed in turn, enough replays
+    per event pair to hold MIN_LAUNCHES launches."""
+    import torch
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    ngraphs = max(1, -(-nb // steps))
+    graphs = []
+    for j in range(ngraphs):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(steps):
+                launch(j * steps + i)
+        graphs.append(g)
+    for g in graphs:  # untimed: the first replay pays the graph's upload
+        g.replay()
+    torch.cuda.synchronize()
+    per_pair = max(ngraphs, -(-MIN_LAUNCHES // steps))
+    per_pair = -(-per_pair // ngraphs) * ngraphs  # whole turns of the rotation
+    ev, wall = [], []
+    for _ in range(REPLAYS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for r in range(per_pair):
+            graphs[r % ngraphs].replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ev.append(e0.elapsed_time(e1) / (per_pair * steps))
+        wall.append((t1 - t0) * 1e3 / (per_pair * steps))
+    mid = sorted(range(REPLAYS), key=lambda i: ev[i])[REPLAYS // 2]
+    return ev[mid], wall[mid], {"graphs": ngraphs, "replays_per_event_pair": per_pair, "launches_per_event_pair": per_pair * steps}
+
+
+def time_graph(af, w, steps, warmup, rotate, packed=False, info=None):
     """Returns (event_ms_per_step, wall_ms_per_step).  packed: every copy of B is reordered once (untimed, as a model
     loader would) and the launches go through bfaintb_gemm_prepacked."""
     import torch
@@ -112,29 +167,10 @@ def time_graph(af, w, steps, warmup, rotate, packed=False):
         else:
             af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
 
-    for i in range(warmup):
-        launch(i)
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for i in range(steps):
-            launch(i)
-    g.replay()  # untimed: first replay pays graph upload
-    torch.cuda.synchronize()
-    ev, wall = [], []
-    for _ in range(REPLAYS):  # each replay is exactly `steps` launches inside one event pair; the median replay is reported
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record()
-        g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        ev.append(e0.elapsed_time(e1) / steps)
-        wall.append((t1 - t0) * 1e3 / steps)
-    mid = sorted(range(REPLAYS), key=lambda i: ev[i])[REPLAYS // 2]
-    return ev[mid], wall[mid]
+    ev, wall, inf = time_launches(launch, nb, steps, warmup)
+    if info is not None:
+        info.update(inf)
+    return ev, wall
 
 
 def time_fused_epilogue(af, w, steps, warmup):
@@ -144,35 +180,16 @@ def time_fused_epilogue(af, w, steps, warmup):
     ws = w.workspace(af)
     bias = torch.randn(w.n, device="cuda").to(torch.bfloat16)
     res = torch.randn((w.m, w.n), device="cuda").to(torch.bfloat16)
+    nb = len(w.b)
 
     def fused(i):
-        af.gemm(w.c, w.a, w.b[i % len(w.b)], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws, bias=bias, residual=res)
+        af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws, bias=bias, residual=res)
 
     def unfused(i):
-        af.gemm(w.c, w.a, w.b[i % len(w.b)], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
+        af.gemm(w.c, w.a, w.b[i % nb], w.s, w.m, w.n, w.k, weight_bits=w.bits, group_size=w.group, workspace=ws)
         w.c.add_(bias).add_(res)
 
-    out = []
-    for launch in (fused, unfused):
-        for i in range(warmup):
-            launch(i)
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for i in range(steps):
-                launch(i)
-        g.replay()
-        torch.cuda.synchronize()
-        ev = []
-        for _ in range(REPLAYS):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            g.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            ev.append(e0.elapsed_time(e1) / steps)
-        out.append(sorted(ev)[REPLAYS // 2])
-    return out[0], out[1]
+    return time_launches(fused, nb, steps, warmup)[0], time_launches(unfused, nb, steps, warmup)[0]
 
 
 def time_gated(af, w, steps, warmup, packed):
@@ -189,7 +206,7 @@ def time_gated(af, w, steps, warmup, packed):
             af.prepack(pk, w.b[i], w.n, w.k, weight_bits=w.bits)
             pks.append(pk)
         need = af.prepacked_workspace_bytes(w.m, w.n, w.k, w.bits, w.group)
-        pws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        pws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
         af.workspace_init(pws)
 
     def plain(i, c, act):
@@ -205,48 +222,13 @@ def time_gated(af, w, steps, warmup, packed):
         plain(i, w.c, af.ACT_NONE)
         torch.mul(torch.nn.functional.silu(w.c[:, 0::2]), w.c[:, 1::2], out=out)
 
-    res = []
-    for launch in (fused, unfused):
-        for i in range(warmup):
-            launch(i)
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for i in range(steps):
-                launch(i)
-        g.replay()
-        torch.cuda.synchronize()
-        ev = []
-        for _ in range(REPLAYS):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            g.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            ev.append(e0.elapsed_time(e1) / steps)
-        res.append(sorted(ev)[REPLAYS // 2])
-    return res[0], res[1]
+    return time_launches(fused, nb, steps, warmup)[0], time_launches(unfused, nb, steps, warmup)[0]
 
 
 def time_read_ceiling(af, w, steps, warmup):
     """The same rotation of B copies through a kernel that only fetches the bytes."""
-    import torch
     nb = len(w.b)
-    for i in range(warmup):
-        af.probe_read(w.b[i % nb])
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for i in range(steps):
-            af.probe_read(w.b[i % nb])
-    g.replay()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps
+    return time_launches(lambda i: af.probe_read(w.b[i % nb]), nb, steps, warmup)[0]
 
 
 def time_vendor_bf16_gemm(w, steps, warmup):
@@ -258,21 +240,7 @@ def time_vendor_bf16_gemm(w, steps, warmup):
     wb = (wq * w.s.float()[0][None, :]).to(torch.bfloat16)
     del wq
     out = torch.empty((w.m, w.n), dtype=torch.bfloat16, device="cuda")
-    for _ in range(warmup):
-        torch.matmul(w.a, wb, out=out)
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for _ in range(steps):
-            torch.matmul(w.a, wb, out=out)
-    g.replay()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps
+    return time_launches(lambda i: torch.matmul(w.a, wb, out=out), 1, steps, warmup)[0]
 
 
 def time_eager(af, w, steps, warmup):
@@ -298,47 +266,20 @@ def roofline_entry(w, ms, bound, suffix=""):
     else:
         achieved = w.flops / (ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
-    return {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name + suffix), "kernel_us": round(ms * 1e3, 3),
-            "algorithmic_bytes": w.bytes, "flops": w.flops}
+    traffic, source = RECORDED_TRAFFIC.get(w.name + suffix, (None, None))
+    out = {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+           "traffic": traffic, "kernel_us": round(ms * 1e3, 3), "algorithmic_bytes": w.bytes, "flops": w.flops}
+    if traffic is not None:
+        out["traffic_source"] = "recorded rocprofv3 --pmc run, not measured by this run: " + source
+    return out
 
 
-SCAN_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (8192, 8192), (28672, 8192), (2048, 8192), (32000, 4096)]   # (n, k)
-SCAN_SHAPES_NARROW = [(1024, 4096), (1024, 8192), (512, 4096), (2048, 4096), (1536, 8960), (256, 7168), (1024, 16384)]
-SCAN_M = [1, 4, 8, 16, 24, 32, 48, 64, 128, 256, 512, 1024, 2048]
-
-
-def scan(shapes=None):
-    """Kernel time of bfaintb_gemm and bfaintb_gemm_prepacked, variant left to the library, over shapes x {8-bit per
-    channel, 4-bit group 128} x SCAN_M.  Up to 32 rows of A the launches rotate over copies of B that exceed the last-level
-    cache (the decode protocol of the headline figure); beyond, two copies.  Not a roofline statement: a map to read
-    anomalies from (a time that falls as m grows, a weight order that loses to the other)."""
-    import torch
-    import awesome_fusion_amd as af
-    af.lib()
-    for (n, k) in (SCAN_SHAPES if shapes is None else shapes):
-        for (bits, group) in ((8, 0), (4, 128)):
-            row = {"n": n, "k": k, "weight_bits": bits, "group_size": group, "m": SCAN_M, "row_major_us": [], "prepacked_us": []}
-            for m in SCAN_M:
-                b_bytes = n * k * bits // 8
-                copies = max(2, min(40, (640 << 20) // b_bytes)) if m <= 32 else 2
-                w = Workload(f"scan_m{m}_n{n}_k{k}_b{bits}", m, n, k, bits, group, copies=copies)
-                steps = 100 if m <= 64 else 20
-                for packed in (False, True):
-                    ev_ms, _ = time_graph(af, w, steps, 5, rotate=True, packed=packed)
-                    row["prepacked_us" if packed else "row_major_us"].append(round(ev_ms * 1e3, 2))
-                del w
-                torch.cuda.empty_cache()
-            print(json.dumps(row), flush=True)
-
-
-def cpu_baseline(w, c_gpu_f32, budget_s=12.0):
+def cpu_baseline(w, c_gpu_f32, budget_s=8.0):
     """host_ref.hpp's gemm_rrr timed on this machine's cores on the same inputs the GPU consumed:
     the reference's own compiled routine when the wrapper library is present, else the C port."""
     import ctypes as C
     from concurrent.futures import ThreadPoolExecutor
     import oracle
-    import torch
     fp = C.POINTER(C.c_float)
     a = w.a.float().cpu().numpy()                       # the bf16 activations, widened
     s = w.s.float().cpu().numpy()[0].copy()             # the bf16 scales, widened (per-channel workloads)
@@ -373,21 +314,34 @@ def cpu_baseline(w, c_gpu_f32, budget_s=12.0):
         while True:
             list(ex.map(lambda j: call(*j), jobs))
             reps2 += 1
-            el = time.perf_counter() - t0
-            if el > budget_s * 0.4 or reps2 >= 200:
+            el2 = time.perf_counter() - t0
+            if el2 > budget_s * 0.4 or reps2 >= 200:
                 break
-    tn = el / reps2
+    tn = el2 / reps2
     assert np.array_equal(c.view(np.uint32), c_single.view(np.uint32)), "threaded CPU baseline changed the result"
     d = c_gpu_f32 - c
     nrms = float(np.sqrt((d.astype(np.float64) ** 2).sum() / (2.0 * (c.astype(np.float64) ** 2).sum())))
     unit_val = lambda t: w.bytes / t / 1e9
     return ({"value": round(unit_val(t1), 4), "unit": "GB/s", "cores": 1, "kind": kind,
-             "sample": f"full {w.name} problem x{reps} repetitions ({el and t1 * reps:.1f} s), gemm_rrr on float inputs",
+             "sample": f"full {w.name} problem x{reps} repetitions ({t1 * reps:.1f} s), gemm_rrr on float inputs",
              "gflops": round(w.flops / t1 / 1e9, 3), "ms_per_step": round(t1 * 1e3, 3)},
             {"value": round(unit_val(tn), 4), "unit": "GB/s", "cores": cores, "kind": kind,
-             "sample": f"full {w.name} problem x{reps2} repetitions, columns split over {cores} threads",
+             "sample": f"full {w.name} problem x{reps2} repetitions ({tn * reps2:.1f} s), columns split over {cores} threads",
              "gflops": round(w.flops / tn / 1e9, 3), "ms_per_step": round(tn * 1e3, 3)},
             nrms)
+
+
+def config3_workload(m_max=32):
+    return Workload(f"decode_m{m_max}_n11008_k4096_int8_perchannel", m_max, 11008, 4096, copies=14)   # 14 x 43 MiB = 602 MiB
+
+
+def config5_workload(m_max):
+    # 6 x 112 MiB = 672 MiB of rotating weights for the decode rows; the tiled kernel re-reads its panels from cache anyway
+    return Workload(f"m{m_max}_n28672_k8192_int4_group128", m_max, 28672, 8192, bits=4, group=128, copies=6 if m_max <= 32 else 1)
+
+
+def compact(entry):
+    return {k: entry[k] for k in ("workload", "bound", "kernel_us", "achieved", "unit", "frac", "algorithmic_bytes", "flops", "steps") if k in entry}
 
 
 def main():
@@ -395,24 +349,17 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (decode sweep, int4 group-128)")
-    ap.add_argument("--scan", nargs="?", const="llm", default="", choices=["llm", "narrow"],
-                    help="instead of the benchmark: what the library's own choice of kernel takes over a grid of "
-                    "matrix shapes, code widths and m, row-major and pre-packed weights; one JSON line per matrix "
-                    "(llm: projection and MLP shapes of 7B..70B models; narrow: 256..2048 columns, the key/value "
-                    "projections of grouped-query attention)")
+    ap.add_argument("--sweep", action="store_true", help="also time the secondary shapes (all five rows of the decode sweep, "
+                    "pre-packed forms, the rows between decode and prefill, the gated MLP)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="time only this workload family: decode | prefill | decode_cold | decode_packed_cold "
-                    "(decode_cold: nothing but the headline's cold-B launches, for a kernel trace without the hot and eager variants; "
-                    "decode_packed_cold: the same launches over pre-packed weights)")
+    ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
+                    "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
+                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM would shard over the columns "
               "of B with no exchange between GPUs).  Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
-    if args.scan:
-        scan(SCAN_SHAPES_NARROW if args.scan == "narrow" else SCAN_SHAPES)
-        return
 
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -423,31 +370,54 @@ def main():
     K, W = args.steps, args.warmup
     out_extra = {}
 
-    # ---- headline: decode M=1, N=K=4096, int8 per-channel; cold B (rotating copies > last-level cache)
+    # ---- one secondary workload alone (profiling runs)
+    if args.only.startswith(("c3_m", "c5_m", "mid_m")):
+        m = int(args.only.split("_m")[1])
+        if args.only.startswith("c3_"):
+            w = config3_workload(m)
+        elif args.only.startswith("c5_"):
+            w = config5_workload(m)
+        else:
+            w = Workload(f"mid_m{m}_n4096_k4096_int8_perchannel", m, 4096, 4096, copies=4)
+        steps = min(K, 200) if m <= 32 else 10
+        ev_ms, wall_ms = time_graph(af, w, steps, min(W, 10), rotate=True)
+        bound = "hbm" if m <= 32 else "mfma"
+        print(json.dumps({"metric": f"bfAintBGemm {w.name}", "value": roofline_entry(w, wall_ms, bound)["achieved"],
+                          "unit": "GB/s" if bound == "hbm" else "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": min(W, 10),
+                          "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                          "dtype": "bf16", "data": "synthetic", "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, bound)}))
+        return
+
+    # ---- headline: decode M=1, N=K=4096, int8 per-channel; cold B (rotating copies > 2 x last-level cache)
     res = None
     cold_only = args.only in ("decode_cold", "decode_packed_cold")
     if args.only in ("", "decode", "decode_cold", "decode_packed_cold"):
         copies = LLC_BYTES * 2 // (4096 * 4096) + 8  # 40 copies = 640 MiB
         w = Workload("decode_m1_n4096_k4096_int8_perchannel", 1, 4096, 4096, copies=copies)
-        ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True, packed=args.only == "decode_packed_cold")
+        info = {}
+        ev_ms, wall_ms = time_graph(af, w, K, W, rotate=True, packed=args.only == "decode_packed_cold", info=info)
         if args.only == "decode_packed_cold":
             w.name += "_prepacked"
         hot_ms, _ = (ev_ms, wall_ms) if cold_only else time_graph(af, w, K, W, rotate=False)
         eager_ms = ev_ms if cold_only else time_eager(af, w, K, W)
         read_ms = ev_ms if cold_only else time_read_ceiling(af, w, K, W)
         c_gpu = w.c.float().cpu().numpy()
+        b_bytes = w.b[0].numel()
         res = {
             "metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=1: effective HBM bandwidth (algorithmic bytes / time per launch, B cold)",
             "value": round(w.bytes / (wall_ms * 1e-3) / 1e9, 3), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
             "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16", "data": "synthetic",
             "config": {"workload": w.name, "m": 1, "n": 4096, "k": 4096, "weight_bits": 8, "group_size": 0,
-                       "b_copies_rotated": copies, "split_k": af.split_k(1, 4096, 4096), "launch": "hip graph of K launches, median of 5 replays",
+                       "b_copies_rotated": copies, "bytes_between_rereads_of_a_copy": (copies - 1) * b_bytes,
+                       "last_level_cache_bytes": LLC_BYTES, "split_k": af.split_k(1, 4096, 4096),
+                       "launch": f"{info['graphs']} HIP graphs of K = {K} launches that together walk all {copies} copies, replayed in turn; "
+                                 f"{info['replays_per_event_pair']} replays ({info['launches_per_event_pair']} launches) inside one event pair; "
+                                 f"median of {REPLAYS} pairs; a step is one launch",
                        "units": "decimal; scale bytes counted"},
             "roofline": roofline_entry(w, ev_ms, "hbm"),
         }
         res["tflops"] = round(w.flops / (wall_ms * 1e-3) / 1e12, 4)
-        b_bytes = w.b[0].numel()
         if not cold_only:
             res["roofline"]["fetch_only_kernel_us"] = round(read_ms * 1e3, 3)
             res["roofline"]["fetch_only_GBps"] = round(b_bytes / read_ms / 1e6, 1)
@@ -486,11 +456,12 @@ def main():
                                                     "note": "torch.matmul bf16 x bf16 on pre-dequantised weights (no dequantisation work): context, not a baseline"}
         except Exception as exc:  # context only
             entry["vendor_bf16_gemm_same_shape"] = {"error": str(exc)[:200]}
-        f_ms, u_ms = time_fused_epilogue(af, w, pk, max(5, W // 4))
-        entry["bias_residual"] = {"fused_kernel_us": round(f_ms * 1e3, 3), "gemm_then_two_elementwise_us": round(u_ms * 1e3, 3),
-                                  "note": "C = A.W + bias + residual: one bfaintb_gemm_fused launch against bfaintb_gemm + torch add_ x2"}
-        pk_ms, _ = time_graph(af, w, pk, max(5, W // 4), rotate=True, packed=True)
-        entry["prepacked"] = {**roofline_entry(w, pk_ms, "mfma", "_prepacked"), "note": "bfaintb_gemm_prepacked, same shape"}
+        if args.only == "":
+            f_ms, u_ms = time_fused_epilogue(af, w, pk, max(5, W // 4))
+            entry["bias_residual"] = {"fused_kernel_us": round(f_ms * 1e3, 3), "gemm_then_two_elementwise_us": round(u_ms * 1e3, 3),
+                                      "note": "C = A.W + bias + residual: one bfaintb_gemm_fused launch against bfaintb_gemm + torch add_ x2"}
+            pk_ms, _ = time_graph(af, w, pk, max(5, W // 4), rotate=True, packed=True)
+            entry["prepacked"] = {**roofline_entry(w, pk_ms, "mfma", "_prepacked"), "note": "bfaintb_gemm_prepacked, same shape"}
         out_extra["prefill_m4096"] = entry
         if res is None:
             res = {"metric": "bfAintBGemm bf16 x int8 GEMM, N=K=4096, M=4096: TFLOP/s", "value": entry["value"], "unit": "TFLOP/s",
@@ -500,27 +471,44 @@ def main():
         del w
         torch.cuda.empty_cache()
 
+    # ---- BASELINE's decode sweep (N = 11008) and 4-bit group-128 shape (28672 x 8192): compact roofline rows
+    if args.only == "":
+        rows = []
+        w32 = config3_workload(32)
+        for m in ((1, 4, 8, 16, 32) if args.sweep else C3_ROWS):
+            w = w32.rows(m, f"decode_m{m}_n11008_k4096_int8_perchannel")
+            steps = min(K, 200)
+            ev_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True)
+            rows.append(compact({"workload": w.name, "steps": steps, **roofline_entry(w, ev_ms, "hbm")}))
+            if args.sweep and m <= 8:
+                pk_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True, packed=True)
+                rows.append(compact({"workload": w.name + "_prepacked", "steps": steps, **roofline_entry(w, pk_ms, "hbm")}))
+        out_extra["config3_decode_sweep_n11008_k4096_int8"] = rows
+        del w32, w
+        torch.cuda.empty_cache()
+        rows = []
+        w16 = config5_workload(16)
+        for m in C5_ROWS:
+            if m <= 16:
+                w = w16.rows(m, f"m{m}_n28672_k8192_int4_group128")
+                steps = min(K, 100)
+            else:
+                del w16, w
+                torch.cuda.empty_cache()
+                w = config5_workload(m)
+                steps = 10
+            ev_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True)
+            rows.append(compact({"workload": w.name, "steps": steps, **roofline_entry(w, ev_ms, "hbm" if m <= 32 else "mfma")}))
+            if args.sweep and m == 1:
+                pk_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True, packed=True)
+                rows.append(compact({"workload": w.name + "_prepacked", "steps": steps, **roofline_entry(w, pk_ms, "hbm")}))
+        out_extra["config5_int4_group128_n28672_k8192"] = rows
+        del w
+        torch.cuda.empty_cache()
+
     if args.sweep:
         sweep = []
-        for m in (1, 4, 8, 16, 32):
-            w = Workload(f"decode_m{m}_n11008_k4096_int8_perchannel", m, 11008, 4096, copies=14)
-            ev_ms, _ = time_graph(af, w, min(K, 200), W, rotate=True)
-            sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "hbm")})
-            if m <= 8:
-                pk_ms, _ = time_graph(af, w, min(K, 200), W, rotate=True, packed=True)
-                sweep.append({"workload": w.name + "_prepacked", **roofline_entry(w, pk_ms, "hbm")})
-            del w
-            torch.cuda.empty_cache()
-        for m in (1, 16, 2048):
-            w = Workload(f"m{m}_n28672_k8192_int4_group128", m, 28672, 8192, bits=4, group=128, copies=6 if m <= 32 else 1)
-            ev_ms, _ = time_graph(af, w, min(K, 100) if m <= 32 else 10, min(W, 10), rotate=True)
-            sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "hbm" if m <= 32 else "mfma")})
-            if m == 1:
-                pk_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True, packed=True)
-                sweep.append({"workload": w.name + "_prepacked", **roofline_entry(w, pk_ms, "hbm")})
-            del w
-            torch.cuda.empty_cache()
-        # between decode and prefill: what AUTO picks for a few hundred rows of A (row-blocked decode family, then 128x128 tiles)
+        # between decode and prefill: what AUTO picks for a few hundred rows of A (row-blocked decode family, then the tiled kernels)
         for m in (64, 256, 640, 1024):
             w = Workload(f"mid_m{m}_n4096_k4096_int8_perchannel", m, 4096, 4096, copies=4)
             ev_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True)

@@ -15,3 +15,21 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def golden_dir():
     return os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """After a GPU session: what the acceptance checks found (outputs outside the 2-ULP bound per call), for the report."""
+    import json
+    try:
+        import helpers
+    except ImportError:
+        return
+    if not helpers.ACCEPTANCE_LOG:
+        return
+    out = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "acceptance_counts.json"), "w") as f:
+            json.dump(helpers.ACCEPTANCE_LOG, f, indent=0)
+    except OSError:
+        pass

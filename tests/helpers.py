@@ -128,15 +128,25 @@ def ulp_violations(c_ref, c_bits, max_ulp=2.0, small_abs=1e-3, small_rel=1e-2):
     return np.nonzero(~ok)[0], err / ulp
 
 
+# what every assert_close_ulp call found, for the acceptance report (tests/conftest.py writes it out at the end of a GPU session)
+ACCEPTANCE_LOG = []
+NOISE_FACTOR = 8.0   # the escape below: this many times 2^-24 * sum_k |a_k w_k| on top of 2 ULP
+NEAR_ZERO = 0.125    # ... and only for outputs below this fraction of rms(C)
+
+
 def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
     """The acceptance bound of this build: every output within 2 bf16 ULP of the fp32
     sequential-K oracle, or within 1e-2 relative where |ref| < 1e-3.
 
     No summation order other than the oracle's own can meet that bound for outputs that cancel to
     (almost) nothing: there a bf16 ULP is smaller than the fp32 rounding noise of the K-term sum on
-    EITHER side.  Such outputs are rare (counted, capped at max_frac of the outputs), and each must lie
-    within 2 ULP plus the standard estimate of an fp32 sum's rounding error, sqrt(K) * 2^-24 * sum_k
-    |a_k w_k|, of the fp64-accumulated value.  Returns (worst error in ULP, number of such outputs)."""
+    EITHER side.  Such outputs are rare (counted, capped at max_frac of the outputs, and recorded in
+    ACCEPTANCE_LOG); each must be small (|ref| < rms(C) / 8: an output of ordinary size has no such excuse)
+    and must lie within 2 ULP + 8 * 2^-24 * sum_k |a_k w_k| of the fp64-accumulated value.  The second
+    term is a few times the rounding error an fp32 sum of those terms makes in any order (measured worst
+    over the BASELINE shapes: 1.3 of these units for the device, 4.4 for the sequential oracle); one
+    dropped or doubled term of ordinary size is a thousand of them.
+    Returns (worst error in ULP among the outputs inside the bound, number of outputs that took the escape)."""
     a = p.a_bf if rows is None else p.a_bf[rows]
     c_ref = oracle.gemm_bf16_rows(a, p.w_bf, threads=threads)
     bias = None if p.bias_bf is None else widen(p.bias_bf)
@@ -151,20 +161,30 @@ def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
     # (a handful is always allowed: over 4000 random problems of a few thousand outputs each, six had 2 or 3 such outputs)
     assert len(bad) <= max(3, int(max_frac * c_ref.size)), \
         f"{what}: {len(bad)} of {c_ref.size} outputs outside 2 ULP (worst {ulps.max():.2f} ULP)"
+    worst_units = 0.0
     if len(bad):
         n = c_ref.shape[1]
+        rms = float(np.sqrt(np.mean(c_ref.astype(np.float64) ** 2)))
         af_, wf_ = widen(a).astype(np.float64), widen(p.w_bf).astype(np.float64)
         got = widen(np.asarray(c_bits, np.uint16).ravel()[bad]).astype(np.float64)
         for flat, g in zip(bad, got):
             i, j = divmod(int(flat), n)
+            assert abs(float(c_ref[i, j])) < NEAR_ZERO * rms, \
+                f"{what}: output ({i},{j}) = {g!r} is outside 2 ULP of {c_ref[i, j]!r} and not near zero (rms of C {rms:.3g})"
             terms = af_[i] * wf_[:, j]
             exact = terms.sum() + (0.0 if bias is None else float(bias[j])) + (0.0 if res is None else float(res[i, j]))
             _, e = np.frexp(abs(exact))
-            tol = 2.0 * np.ldexp(1.0, max(int(e) - 1, -126) - 7) + np.sqrt(p.k) * 2.0 ** -24 * np.abs(terms).sum()
+            unit = 2.0 ** -24 * np.abs(terms).sum()
+            tol = 2.0 * np.ldexp(1.0, max(int(e) - 1, -126) - 7) + NOISE_FACTOR * unit
+            worst_units = max(worst_units, abs(g - exact) / unit)
             assert abs(g - exact) <= tol, f"{what}: output ({i},{j}) = {g!r}, exact {exact!r}, fp32 oracle " \
                                           f"{c_ref[i, j]!r}: off by {abs(g - exact):.3e} > {tol:.3e}"
     ok_ulps = np.delete(ulps, bad)
-    return (float(ok_ulps.max()) if ok_ulps.size else 0.0), len(bad)
+    worst = float(ok_ulps.max()) if ok_ulps.size else 0.0
+    ACCEPTANCE_LOG.append({"what": what, "m": int(c_ref.shape[0]), "n": p.n, "k": p.k, "weight_bits": p.bits, "group_size": p.group_size,
+                           "outputs": int(c_ref.size), "outside_2ulp": int(len(bad)), "worst_ulp_inside": round(worst, 3),
+                           "worst_outside_vs_fp64_in_units_of_2^-24_sum_abs": round(float(worst_units), 3)})
+    return worst, len(bad)
 
 
 def gated_reference(p, rows=None, threads=8):
