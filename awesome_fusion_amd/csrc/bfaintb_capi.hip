@@ -55,9 +55,12 @@ int check_format(uint32_t k, int bits, uint32_t group_size)
     return BFAINTB_OK;
 }
 
-int check_shape(uint32_t m, uint32_t n, uint32_t k)
+// Row-major weights: n a multiple of 8 (of 16 for 4-bit codes: a lane reads 16 of them per row), k a multiple of 8 (one
+// 16-byte chunk of activations).  The kernels run a partial last step for the rest of k (the reference kernel needs
+// n % 64 == 0 and k % 64 == 0: bf16gemm_kernel_gfx90a.s:341-343, :402-408).
+int check_shape(uint32_t m, uint32_t n, uint32_t k, int bits = 8)
 {
-    if (k == 0 || n % 16u != 0 || k % 64u != 0) return BFAINTB_ERR_BAD_SHAPE;
+    if (k == 0 || n % (bits == 4 ? 16u : 8u) != 0 || k % 8u != 0) return BFAINTB_ERR_BAD_SHAPE;
     if (m >= (1u << 31) || n >= (1u << 31) || k >= (1u << 31)) return BFAINTB_ERR_BAD_SHAPE;
     return BFAINTB_OK;
 }
@@ -243,7 +246,8 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         // 61.5; 18944 x 3584 16.9 / 18.3 / 24.0 against 18.0 / 19.9 / 25.1; with fewer blocks narrow stays ahead:
         // 11008 x 4096 13.9 / 14.9 / 17.9 against 13.8 / 16.5 / 22.1; 14336 x 4096 17.2 / 18.5 / 21.4 against 17.6 / 19.0 / 25.1)
         const bool many_wide_blocks = (n + 255u) / 256u > 64u;
-        const bool narrow = bits == 8 && (few || fills_rounds || (m >= 8 && (!many_wide_blocks || packed)));  // packed weights: the kernels are built for 128 columns
+        // (n not a multiple of 16: only the 8-codes-per-lane shape can read the last columns)
+        const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 || (m >= 8 && (!many_wide_blocks || packed)));  // packed weights: the kernels are built for 128 columns
         pl.cols = narrow ? 128u : 256u;
         // 4-bit codes, 8 to 16 rows: the same 256 columns with 8 waves (twice the waves to hide the activation loads and
         // the matrix instructions behind; n = k = 4096, m = 16: 11.6 against 14.7 us, 1024 x 8192: 14.1 / 17.4,
@@ -401,7 +405,7 @@ const char* bfaintb_error_string(int code)
     switch (code) {
         case BFAINTB_OK: return "success";
         case BFAINTB_ERR_NULL_POINTER: return "null device pointer";
-        case BFAINTB_ERR_BAD_SHAPE: return "unsupported shape: need n % 16 == 0, k % 64 == 0, k > 0, sizes below 2^31";
+        case BFAINTB_ERR_BAD_SHAPE: return "unsupported shape: need n % 8 == 0 (4-bit codes: n % 16 == 0), k % 8 == 0, k > 0, sizes below 2^31; pre-packed weights: n % 16 == 0, k % 64 == 0 (4-bit: k % 128 == 0)";
         case BFAINTB_ERR_BAD_LD: return "bad leading dimension: need lda >= k, ldb >= n, ldc >= n, lda % 8 == 0, ldb % 16 == 0, ldc % 8 == 0";
         case BFAINTB_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
         case BFAINTB_ERR_UNSUPPORTED: return "unsupported format: weight_bits must be 8 or 4; group_size 0 or a multiple of 32 that divides k";
@@ -420,7 +424,7 @@ int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, ui
 {
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
-    e = check_shape(m, n, k);
+    e = check_shape(m, n, k, weight_bits);
     if (e) return e;
     return resolve_variant(m, n, k, weight_bits, BFAINTB_VARIANT_AUTO);
 }
@@ -434,7 +438,7 @@ uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bit
 size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant,
                                        uint32_t split_k)
 {
-    if (check_format(k, weight_bits, group_size) || check_shape(m, n, k)) return 0;
+    if (check_format(k, weight_bits, group_size) || check_shape(m, n, k, weight_bits)) return 0;
     const int v = resolve_variant(m, n, k, weight_bits, variant);
     if (v < 0) return 0;
     return workspace_need(m, n, k, weight_bits, v, split_k);
@@ -509,6 +513,7 @@ static int read_epilogue(Epilogue& out, const bfaintb_epilogue* ep, uint32_t n)
     out.ldr = ep->ldr;
     out.activation = ep->activation;
     if (ep->residual != nullptr && (ep->ldr < out.out_cols(n) || ep->ldr % 8u != 0)) return BFAINTB_ERR_BAD_LD;
+    if (ep->activation == BFAINTB_ACT_SILU_GATE && n % 16u != 0) return BFAINTB_ERR_BAD_SHAPE;  // n / 2 output columns, stored 8 at a time
     return BFAINTB_OK;
 }
 
@@ -534,7 +539,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
     if (ep.reference_arith && (weight_bits != 8 || group_size != 0)) return BFAINTB_ERR_UNSUPPORTED;
-    e = check_shape(m, n, k);
+    e = check_shape(m, n, k, weight_bits);
     if (e) return e;
     if (lda < k || ldb < n || ldc < ep.out_cols(n) || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
     const int v = resolve_variant(m, n, k, weight_bits, variant);
@@ -609,7 +614,7 @@ static int check_packed_shape(uint32_t n, uint32_t k, int weight_bits)
 {
     const int e = check_shape(1, n, k);
     if (e) return e;
-    return (weight_bits == 4 && k % 128u != 0) ? BFAINTB_ERR_BAD_SHAPE : BFAINTB_OK;
+    return (n % 16u != 0 || k % (weight_bits == 4 ? 128u : 64u) != 0) ? BFAINTB_ERR_BAD_SHAPE : BFAINTB_OK;
 }
 
 size_t bfaintb_prepack_bytes(uint32_t n, uint32_t k, int weight_bits)
@@ -930,7 +935,7 @@ int bfaintb_dequant(void* w, const void* b, const void* scale, uint32_t n, uint3
 {
     int e = check_format(k, weight_bits, group_size);
     if (e) return e;
-    if (k == 0 || n % 16u != 0 || k % 2u != 0) return BFAINTB_ERR_BAD_SHAPE;
+    if (k == 0 || n % (weight_bits == 4 ? 16u : 8u) != 0 || k % 2u != 0) return BFAINTB_ERR_BAD_SHAPE;
     if (ldb < n || ldw < n || ldb % 16u != 0 || ldw % 8u != 0) return BFAINTB_ERR_BAD_LD;
     if (n == 0) return BFAINTB_OK;
     if (w == nullptr || b == nullptr || scale == nullptr) return BFAINTB_ERR_NULL_POINTER;

@@ -394,7 +394,10 @@ bfaintb_decode_kernel(const GemmParams p)
     const uint32_t kb = ks * p.k_per_wg + (uint32_t)wave * k_per_wave;
     uint32_t ke = kb + k_per_wave;
     if (ke > p.k) ke = p.k;
-    const int nsteps = kb < ke ? (int)((ke - kb) / (32u * KB)) : 0;  // k_per_wave and k are multiples of 32*KB
+    const int nsteps = kb < ke ? (int)((ke - kb) / (32u * KB)) : 0;
+    // Row-major weights, k not a multiple of 32 (it is one of 8): the wave that holds the end of k runs one more, partial
+    // step.  (Packed weights come in whole K-chunks; scale groups are multiples of 32 rows that divide k.)
+    const uint32_t tail_rows = (PACKED || GROUPED || kb >= ke) ? 0u : (ke - kb) % 32u;
 
     const uint8_t* bptr = p.b + (size_t)(kb + 8u * kg) * p.ldb_bytes + (size_t)n_ld * BITS / 8;
     const size_t bstep = (size_t)32 * p.ldb_bytes;
@@ -440,7 +443,7 @@ bfaintb_decode_kernel(const GemmParams p)
 #pragma unroll
         for (int c = 0; c < CPL; ++c) acc[mb][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    if (nsteps > 0) {
+    if (nsteps > 0 || tail_rows != 0u) {
         // Two register stages, used alternately: the loads of step s+1 are issued before step s is
         // computed.  A step is KB blocks of 32 rows, so that a lane has 128 bytes of B in flight per
         // stage whatever CPL is.  Every load is unconditional and sits in straight-line code (the
@@ -519,33 +522,58 @@ bfaintb_decode_kernel(const GemmParams p)
                 else mac_step<BITS, CPL, MB, REF>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
             }
         };
-        Stage s0, s1;
-        if constexpr (REF) {
-            const float4* sf = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.scale) + n_ld);
+        auto request_scales = [&](Stage& st) {  // one scale per column: requested once, before the first weights
+            if constexpr (REF) {
+                const float4* sf = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.scale) + n_ld);
 #pragma unroll
-            for (int i = 0; i < CPL / 4; ++i) {
-                const float4 v = sf[i];
-                cs[4 * i] = v.x; cs[4 * i + 1] = v.y; cs[4 * i + 2] = v.z; cs[4 * i + 3] = v.w;
+                for (int i = 0; i < CPL / 4; ++i) {
+                    const float4 v = sf[i];
+                    cs[4 * i] = v.x; cs[4 * i + 1] = v.y; cs[4 * i + 2] = v.z; cs[4 * i + 3] = v.w;
+                }
+            } else if constexpr (!GROUPED) {
+                if constexpr (PACKED) load_scales_packed<CPL>(st.sraw[0], sptr, pk_col);
+                else load_scales<CPL>(st.sraw[0], sptr);
             }
-        } else if constexpr (!GROUPED) {
-            if constexpr (PACKED) load_scales_packed<CPL>(s0.sraw[0], sptr, pk_col);
-            else load_scales<CPL>(s0.sraw[0], sptr);
+        };
+        if (nsteps > 0) {
+            Stage s0, s1;
+            request_scales(s0);
+            load_stage(s0, 0);
+            if constexpr (!GROUPED && !REF) apply_scales<BITS, CPL>(cs, s0.sraw[0]);
+            int s = 0;
+            for (; s + 2 < nsteps; s += 2) {
+                load_stage(s1, s + 1);
+                compute_stage(s0);
+                load_stage(s0, s + 2);
+                compute_stage(s1);
+            }
+            if (nsteps - s == 2) {
+                load_stage(s1, s + 1);
+                compute_stage(s0);
+                compute_stage(s1);
+            } else {
+                compute_stage(s0);
+            }
         }
-        load_stage(s0, 0);
-        if constexpr (!GROUPED && !REF) apply_scales<BITS, CPL>(cs, s0.sraw[0]);
-        int s = 0;
-        for (; s + 2 < nsteps; s += 2) {
-            load_stage(s1, s + 1);
-            compute_stage(s0);
-            load_stage(s0, s + 2);
-            compute_stage(s1);
-        }
-        if (nsteps - s == 2) {
-            load_stage(s1, s + 1);
-            compute_stage(s0);
-            compute_stage(s1);
-        } else {
-            compute_stage(s0);
+        if constexpr (!PACKED && !GROUPED) {
+            if (tail_rows != 0u) {
+                // the partial step: groups of 8 rows past the end of k get zero activations (and re-read the last 8 rows
+                // of B, whose products with zero vanish)
+                Stage st;
+                if (nsteps == 0) {
+                    request_scales(st);
+                    if constexpr (!REF) apply_scales<BITS, CPL>(cs, st.sraw[0]);
+                }
+                const uint32_t krow = kb + 32u * (uint32_t)nsteps + 8u * (uint32_t)kg;
+                const bool live = krow < p.k;
+                load_raw<BITS, CPL>(st.raw[0], p.b + (size_t)(live ? krow : p.k - 8u) * p.ldb_bytes + (size_t)n_ld * BITS / 8, p.ldb_bytes);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    st.af[0][mb] = make_uint4(0u, 0u, 0u, 0u);
+                    if (live) st.af[0][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + (size_t)nsteps * 32);
+                }
+                compute_stage(st);
+            }
         }
     }
     TRACE_MARK(2);

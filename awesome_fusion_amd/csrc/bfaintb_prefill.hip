@@ -116,11 +116,19 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     // so the lane fetches the chunk that the swizzle puts there: chunk (l%8) ^ ((row >> 1) & 7).
     // (arrays below keep the 256-row tile's extent whatever MT is: with array bounds that depend on MT this compiler's host
     // pass stops emitting the kernel's launch stub; the unused elements cost nothing)
-    uint32_t a_voff[4];
+    // The last K-step may be partial (k a multiple of 8, not of 64): there the chunks of 8 k past the end are fetched
+    // from beyond the buffer's extent, which reads as zero; B's rows past k read as zero codes — finite weights — and
+    // their products with those zeros vanish.
+    const uint32_t ksteps = (p.k + (uint32_t)kBK - 1u) / (uint32_t)kBK;
+    const uint32_t last_chunks = (p.k - (ksteps - 1u) * (uint32_t)kBK) / 8u;  // valid 16-byte chunks per row in the last step: 1..8
+    const uint32_t a_extent = ((rows_valid - 1u) * p.lda + p.k) * 2u;
+    uint32_t a_voff[4], a_voff_last[4];
 #pragma unroll
     for (uint32_t j = 0; j < MT; ++j) {
         const uint32_t row = 8u * MT * wave + 8u * j + (lane >> 3);
-        a_voff[j] = (row * p.lda + (((lane & 7u) ^ ((row >> 1) & 7u)) * 8u)) * 2u;
+        const uint32_t chunk = (lane & 7u) ^ ((row >> 1) & 7u);
+        a_voff[j] = (row * p.lda + chunk * 8u) * 2u;
+        a_voff_last[j] = chunk < last_chunks ? a_voff[j] : a_extent;
     }
     // W, row-major: k-group = wave (rows 8*wave..+7 of the step), 4 columns per lane
     const uint32_t b_voff = BITS == 8 ? 4u * lane : 2u * lane;
@@ -184,7 +192,6 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     if constexpr (!GROUPED) fetch_scales(0);
 
     uint32_t b_reg[8];
-    const uint32_t ksteps = p.k / kBK;
 
     // A tile of K-step `kt` -> LDS stage (asynchronous; counted by vmcnt like any other load)
     auto dma_a = [&](auto stage_c, uint32_t kt) {
@@ -192,7 +199,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 #pragma unroll
         for (uint32_t j = 0; j < MT; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
-                                                     a_voff[j], kt * (uint32_t)kBK * 2u, 0, 0);
+                                                     kt + 1u == ksteps ? a_voff_last[j] : a_voff[j], kt * (uint32_t)kBK * 2u, 0, 0);
     };
     // raw W codes of K-step `kt` -> registers (kt is clamped by the callers, so every load is in range)
     auto gload = [&](uint32_t kt) {
@@ -259,7 +266,9 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     };
     auto update_scales = [&](uint32_t kt) {
         if constexpr (GROUPED) {
-            const uint32_t g = (kt * (uint32_t)kBK + (PACKED ? 0u : 8u * wave)) / p.group_size;
+            uint32_t g = (kt * (uint32_t)kBK + (PACKED ? 0u : 8u * wave)) / p.group_size;
+            const uint32_t groups = p.k / p.group_size;
+            if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do, their products vanish
             if (g != cur_group) {
                 cur_group = g;
                 fetch_scales(g);

@@ -88,11 +88,18 @@ bfaintb_prefill128_kernel(const GemmParams p)
                                                    kBufferFlags);
 
     // A: instruction j of wave w fills rows 16w + 8j .. +7; lane l fetches the chunk the swizzle places at its position
-    uint32_t a_voff[2];
+    // (a partial last K-step — k a multiple of 8, not of 64 — fetches its chunks past the end of k from beyond the
+    // buffer's extent, which reads as zero; B's rows past k read as zero codes, finite weights, and the products vanish)
+    const uint32_t ksteps = (p.k + 63u) / 64u;
+    const uint32_t last_chunks = (p.k - (ksteps - 1u) * 64u) / 8u;
+    const uint32_t a_extent = ((rows_valid - 1u) * p.lda + p.k) * 2u;
+    uint32_t a_voff[2], a_voff_last[2];
 #pragma unroll
     for (uint32_t j = 0; j < 2; ++j) {
         const uint32_t row = 16u * wave + 8u * j + (lane >> 3);
-        a_voff[j] = (row * p.lda + (((lane & 7u) ^ ((row >> 1) & 7u)) * 8u)) * 2u;
+        const uint32_t chunk = (lane & 7u) ^ ((row >> 1) & 7u);
+        a_voff[j] = (row * p.lda + chunk * 8u) * 2u;
+        a_voff_last[j] = chunk < last_chunks ? a_voff[j] : a_extent;
     }
     // W addressing (see the header)
     const uint32_t b_voff = PACKED ? wave * slab_bytes + lane * 16u : (BITS == 8 ? 2u * lane : lane);
@@ -139,7 +146,9 @@ bfaintb_prefill128_kernel(const GemmParams p)
     if constexpr (!GROUPED) fetch_scales(0);
     auto update_scales = [&](uint32_t kt) {
         if constexpr (GROUPED) {
-            const uint32_t g = (kt * 64u + (PACKED ? 0u : 8u * wave)) / p.group_size;
+            uint32_t g = (kt * 64u + (PACKED ? 0u : 8u * wave)) / p.group_size;
+            const uint32_t groups = p.k / p.group_size;
+            if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do, their products vanish
             if (g != cur_group) {
                 cur_group = g;
                 fetch_scales(g);
@@ -147,15 +156,14 @@ bfaintb_prefill128_kernel(const GemmParams p)
         }
     };
 
-    const uint32_t ksteps = p.k / 64u;
     uint32_t b_reg[8];  // row-major: one (16-bit or 8-bit) load per row; packed: 4 (8-bit codes) or 2 dwords
 
     auto dma_a = [&](auto stage_c, uint32_t kt) {
         uint8_t* base = a_tile(stage_c) + wave * 2048u;
 #pragma unroll
         for (uint32_t j = 0; j < 2; ++j)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16, a_voff[j],
-                                                     kt * 128u, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
+                                                     kt + 1u == ksteps ? a_voff_last[j] : a_voff[j], kt * 128u, 0, 0);
     };
     auto gload = [&](uint32_t kt) {
         if constexpr (PACKED) {

@@ -210,8 +210,8 @@ class QuantLinear(torch.nn.Module):
 
     def __init__(self, in_features, out_features, weight_bits=8, group_size=0, bias=False, device=None):
         super().__init__()
-        if out_features % 16 or in_features % 64:
-            raise ValueError("QuantLinear: the kernels need out_features % 16 == 0 and in_features % 64 == 0")
+        if out_features % 16 or in_features % 8:
+            raise ValueError("QuantLinear: the kernels need out_features % 16 == 0 (rows of B stay 16-byte aligned) and in_features % 8 == 0")
         groups = in_features // group_size if group_size else 1
         self.in_features, self.out_features = in_features, out_features
         self.weight_bits, self.group_size = weight_bits, group_size

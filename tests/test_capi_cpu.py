@@ -75,13 +75,24 @@ def rc(**kw):
     return af.gemm(d.pop("c"), d.pop("a"), d.pop("b"), d.pop("scale"), d.pop("m"), d.pop("n"), d.pop("k"), **d)
 
 
+def test_ragged_shapes_are_accepted_by_the_host_side_queries():
+    # n % 8 == 0 and k % 8 == 0 for 8-bit codes (the reference kernel needs multiples of 64), n % 16 == 0 for 4-bit codes
+    assert af.variant(1, 4104, 4072) == af.DECODE and af.variant(33, 1000, 1000) in (af.DECODE, af.PREFILL)
+    assert af.variant(300, 1000, 1000) in (af.DECODE, af.PREFILL) and af.variant(16, 1008, 1000, 4, 0) == af.DECODE
+    assert af.variant(1, 4100, 4072) == -2 and af.variant(1, 4104, 4071) == -2 and af.variant(1, 1000, 1000, 4, 0) == -2
+    assert af.workspace_bytes(1, 4104, 4072) > 256          # split along k: the partial last step belongs to the last split
+    # the packed order keeps whole chunks and column blocks
+    assert af.prepack_bytes(4104, 4096) == 0 and af.prepack_bytes(4096, 4072) == 0 and af.prepacked_variant(1, 4104, 4096) == -2
+
+
 def test_rejects_bad_arguments_without_launching():
     L = af.lib()
     assert rc(weight_bits=5) == -5
     assert rc(group_size=48) == -5            # not a multiple of 32
     assert rc(group_size=96) == -5            # does not divide k = 256
-    assert rc(n=100) == -2                    # n % 16
-    assert rc(k=100) == -2                    # k % 64 (the reference kernel has the same limit, asm main loop)
+    assert rc(n=100) == -2                    # n % 8
+    assert rc(n=104, weight_bits=4, ldb=112, ldc=104) == -2   # 4-bit codes: n % 16
+    assert rc(k=100) == -2                    # k % 8 (the reference kernel needs k % 64: asm main loop)
     assert rc(k=0) == -2
     assert rc(lda=128) == -3                  # lda < k
     assert rc(ldb=64) == -3
@@ -112,7 +123,7 @@ def test_rejects_bad_arguments_without_launching():
         d = dict(c=P, a=P, b=P, scale=P, m=64, n=128, k=256, stream=0, check=False)
         d.update(kw)
         return af.gemm_reference(d.pop("c"), d.pop("a"), d.pop("b"), d.pop("scale"), d.pop("m"), d.pop("n"), d.pop("k"), **d)
-    assert ref_rc(n=100) == -2 and ref_rc(k=96) == -2 and ref_rc(ldb=64) == -3 and ref_rc(ldc=120) == -3
+    assert ref_rc(n=100) == -2 and ref_rc(k=100) == -2 and ref_rc(ldb=64) == -3 and ref_rc(ldc=120) == -3
     assert ref_rc(scale=None) == -1 and ref_rc(scale=P + 4) == -4 and ref_rc(which=9) == -7 and ref_rc(m=0) == 0
     assert ref_rc(m=8, k=1024, which=af.DECODE, force_split_k=2) == -6
     # dequant entry point

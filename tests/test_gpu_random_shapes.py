@@ -97,3 +97,81 @@ def test_random_case(af, case):
         assert_close_gated(p, c, str(case))
     else:
         assert_close_ulp(p, c, str(case))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Ragged shapes: n a multiple of 8 (16 for 4-bit codes), k a multiple of 8 — the tails the reference kernel never handled
+# (its N-tail flag compares the wrong index, bf16gemm_kernel_gfx90a.s:341-343; its K dispatch knows multiples of 64 only,
+# :402-408).  Row-major weights (the packed order keeps whole chunks).  A, B and C carry padding filled with NaNs / a
+# sentinel: nothing of it may be read as data or written.
+
+def run_ragged(af, p, which, act=0, pad=0):
+    import torch
+    from helpers import Workspace, from_dev_u16, to_dev
+    out_n = p.n // 2 if act else p.n
+    lda, ldc = p.k + pad, (out_n + 7) // 8 * 8 + pad
+    ldb = (p.n + 15) // 16 * 16                                  # rows of B stay 16-byte aligned
+    a = np.full((p.m, lda), 0x7FC0, np.uint16)
+    a[:, :p.k] = p.a_bf
+    b = np.full((p.k, ldb * p.bits // 8), 0x55, np.uint8)
+    b[:, :p.n * p.bits // 8] = p.b_bytes
+    res = None
+    if p.residual_bf is not None:
+        r = np.full((p.m, ldc), 0x7FC0, np.uint16)
+        r[:, :out_n] = p.residual_bf
+        res = to_dev(r)
+    c = torch.full((p.m, ldc), 0x7FC1, dtype=torch.int16, device="cuda")
+    bias = None if p.bias_bf is None else to_dev(p.bias_bf)
+    ws = Workspace().get(af.workspace_bytes(p.m, p.n, p.k, p.bits, p.group_size, which))
+    af.gemm(c, to_dev(a), to_dev(b), to_dev(p.s_bf), p.m, p.n, p.k, lda=lda, ldb=ldb, ldc=ldc, workspace=ws, which=which,
+            weight_bits=p.bits, group_size=p.group_size, bias=bias, residual=res, ldr=None if res is None else ldc, activation=act)
+    torch.cuda.synchronize()
+    got = from_dev_u16(c)
+    assert np.all(got[:, out_n:] == 0x7FC1), "padding of C was written"
+    return np.ascontiguousarray(got[:, :out_n])
+
+
+@pytest.mark.parametrize("m,n,k,bits,group,variant", [
+    (33, 1000, 1000, 8, 0, "auto"), (33, 1000, 1000, 8, 0, "decode"), (33, 1000, 1000, 8, 0, "prefill_128"), (33, 1000, 1000, 8, 0, "prefill_256"),
+    (1, 4104, 4072, 8, 0, "auto"), (16, 4104, 4072, 8, 0, "auto"), (32, 520, 1048, 8, 0, "auto"),
+    (1, 8, 8, 8, 0, "auto"), (5, 24, 16, 8, 0, "decode"), (5, 24, 24, 8, 0, "prefill_128"), (70, 40, 8, 8, 0, "prefill_256"),
+    (300, 1000, 1000, 8, 0, "auto"), (700, 1000, 1000, 8, 0, "prefill_256"), (130, 264, 72, 8, 0, "decode"),
+    (16, 1008, 1000, 4, 0, "auto"), (1, 4112, 4072, 4, 0, "auto"), (300, 1008, 1000, 4, 0, "prefill_128"), (300, 1008, 1000, 4, 0, "prefill_256"),
+    (48, 1000, 992, 8, 32, "auto"), (300, 1000, 992, 8, 32, "prefill_128"), (300, 1000, 96, 8, 32, "prefill_256"), (8, 1008, 96, 4, 32, "auto"),
+])
+def test_ragged_shapes(af, m, n, k, bits, group, variant):
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[variant]
+    assert_close_ulp(p, run_ragged(af, p, which, pad=8), f"ragged {m}x{n}x{k} int{bits} g{group} {variant}")
+
+
+def draw_ragged(rng):
+    bits = int(rng.choice([8, 8, 4]))
+    m = int(rng.choice([rng.integers(1, 9), rng.integers(9, 49), rng.integers(49, 200), rng.integers(200, 500)]))
+    group = int(rng.choice([0, 0, 0, 32, 128]))
+    kunit = group if group else 8
+    kmax = 6144 if m < 49 else 1024
+    k = kunit * int(rng.integers(1, kmax // kunit + 1))
+    n = (16 if bits == 4 else 8) * int(rng.integers(1, 140 if bits == 8 else 70))
+    epilogue = str(rng.choice(["none", "none", "bias", "bias+residual", "gate"]))
+    if epilogue == "gate":
+        n = (n + 15) // 16 * 16
+    variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256"])) if epilogue == "none" else "auto"
+    return dict(m=m, n=n, k=k, bits=bits, group=group, epilogue=epilogue, variant=variant, pad=int(rng.choice([0, 8, 24])))
+
+
+RAGGED = [draw_ragged(np.random.Generator(np.random.PCG64(5000 + i))) for i in range(150)]
+
+
+@pytest.mark.parametrize("case", RAGGED, ids=lambda c: "{m}x{n}x{k}-b{bits}-g{group}-{variant}-{epilogue}".format(**c))
+def test_random_ragged_case(af, case):
+    m, n, k, bits, group = case["m"], case["n"], case["k"], case["bits"], case["group"]
+    gated = case["epilogue"] == "gate"
+    p = Problem(m, n, k, bits, group, seed=m + n + k, **(dict(scale_lo=0.002, scale_hi=0.02 if bits == 8 else 0.2) if gated else {}))
+    if "bias" in case["epilogue"]:
+        p.with_bias()
+    if "residual" in case["epilogue"]:
+        p.with_residual()
+    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[case["variant"]]
+    c = run_ragged(af, p, which, af.ACT_SILU_GATE if gated else af.ACT_NONE, case["pad"])
+    (assert_close_gated if gated else assert_close_ulp)(p, c, str(case))
