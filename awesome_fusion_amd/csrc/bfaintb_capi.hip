@@ -14,7 +14,7 @@
 
 namespace bfaintb {
 hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream);
-hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream, bool wreg);
 hipError_t launch_dequant(uint16_t* w, const uint8_t* b, const uint16_t* scale, uint32_t n, uint32_t k, uint32_t ldb_bytes,
                           uint32_t ldw, int bits, uint32_t group_size, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* dst, uint32_t count, uint32_t value, hipStream_t stream);
@@ -119,7 +119,8 @@ static bool prefill_small_tiles(uint32_t m, uint32_t n)
 
 static bool is_prefill(int v)
 {
-    return v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256 || v == BFAINTB_VARIANT_PREFILL_128;
+    return v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256 || v == BFAINTB_VARIANT_PREFILL_128 ||
+           v == BFAINTB_VARIANT_PREFILL_256_LDS;
 }
 
 // tile size of a tiled-variant launch: forced, or by shape
@@ -577,7 +578,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
 #else
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
 #endif
-        return (int)bfaintb::launch_prefill(p, weight_bits, st);
+        return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
 
     const DecodePlan pl = decode_plan(m, n, k, weight_bits, split_k);

@@ -1,0 +1,391 @@
+// Tiled variant, 256x256 tiles, weights kept in registers: the form of the prefill kernel for row-major B.
+//
+// Same job and the same reference kernel replaced as bfaintb_prefill_kernel
+// (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:184-630).  That kernel stages both operands in LDS and is bound
+// by LDS traffic as much as by the matrix pipe (per K-step a CU reads 192 KiB and writes 64 KiB of LDS).  Here only A
+// goes through LDS:
+//   256 threads = 4 waves side by side along n; a wave owns ALL 256 rows x 64 columns of the tile, i.e. 16 x 4
+//   accumulators of v_mfma_f32_16x16x32_bf16 (256 accumulator registers: one wave per SIMD, the whole register file).
+//   Because a wave owns its 64 columns outright, it converts exactly the weights it multiplies by, straight into the
+//   matrix instruction's operand registers: no W tile in LDS, no duplicate conversion, no LDS writes by the waves at all.
+//   Lane (c16 = lane % 16, kq = lane / 16) loads, per block of 32 k and for each of the 8 rows k0 + 8 kq + r, one dword =
+//   the codes of columns 4 c16 .. 4 c16 + 3 of the wave's 64 (16-bit loads for 4-bit codes): byte j of those 8 dwords is
+//   the 8-element operand of column 4 c16 + j, rows 8 kq .. 8 kq + 7 — the layout v_mfma_f32_16x16x32_bf16 wants.
+//   A: global -> LDS directly (buffer_load ... lds), two stages of 256 rows x 64 k (32 KiB each), rows of 128 bytes in 8
+//   chunks of 16, chunk c of row r at position c ^ ((r >> 1) & 7); a fragment read is one ds_read_b128 (16 rows x 32 k).
+//   Per K-step a CU reads 128 KiB of LDS and the copy engine writes 32 KiB.
+// Pipeline per K-step of 64 (registers: operands of this step; raw codes of the next, loaded one step ago): request the
+//   A tile of step+1 into the other stage and the raw codes of step+2; convert the raw codes of step+1 into the second
+//   operand set between the matrix instructions; 128 matrix instructions (2 blocks of 32 k x 16 row blocks x 4 columns),
+//   A fragments fetched a few ahead; wait for the A copy; one barrier.
+// Accumulator (mt, j), register r of lane (c16, q = lane / 16): row 16 mt + 4 q + r, column 64 w + 4 c16 + j of the tile.
+// Epilogue: bias, rounding to bf16, staging through LDS in [m][n] order, 16-byte row-contiguous stores.
+#include <utility>
+#include "bfaintb_device.hpp"
+
+namespace bfaintb {
+
+namespace {
+constexpr uint32_t kWrTile = 256, kWrK = 64;
+constexpr uint32_t kWrStageBytes = 256 * 128;  // one A stage
+constexpr uint32_t kWrCRowBytes = 256 * 2;     // epilogue staging row
+
+__device__ __forceinline__ uint32_t wr_swz(uint32_t row, uint32_t chunk) { return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4); }
+
+// acc += a x b with the accumulator pinned to the accumulation registers and updated in place.  Written as assembly
+// because the compiler, given 256 accumulator registers, keeps part of them in ordinary registers and shuttles them
+// back and forth around every matrix instruction (measured on this kernel's first form: 1772 copies for 384 matrix
+// instructions).  What the compiler's hazard bookkeeping cannot see behind the assembly is kept safe by construction:
+// the operands a and b are written (LDS reads, conversions) long before, under wait counts the compiler does insert
+// for assembly operands; the accumulators are read by ordinary instructions only in the epilogue, behind explicit idle
+// cycles (wreg_settle) that cover a matrix instruction's write latency.
+__device__ __forceinline__ void mfma16(f32x4_t& acc, const bf16x8_t& a, const bf16x8_t& b)
+{
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void wreg_settle()
+{
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+}
+}  // namespace
+
+template <int BITS, bool GROUPED>
+__global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmParams p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kWrStageBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kWrStageBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_c0[kWrStageBytes];  // epilogue staging only
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_c1[kWrStageBytes];
+    auto a_tile = [&](auto stage_c) -> uint8_t* { return decltype(stage_c)::value == 0 ? lds_a0 : lds_a1; };
+
+    using C0 = std::integral_constant<uint32_t, 0>;
+    using C1 = std::integral_constant<uint32_t, 1>;
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..3: the wave's 64 columns
+    const uint32_t c16 = lane & 15u, kq = lane >> 4;
+
+    // ---- tile of this workgroup: ids that share an XCD (id mod 8) cover consecutive logical ids, which walk groups of
+    //      4 tile-rows column by column (as in bfaintb_prefill_kernel)
+    const uint32_t tiles_m = (p.m + kWrTile - 1) / kWrTile, tiles_n = (p.n + kWrTile - 1) / kWrTile;
+    const uint32_t wgs = p.tile_count;
+    const uint32_t per_xcd = (wgs + 7u) / 8u;
+    const uint32_t local = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if (local >= wgs) return;
+    const uint32_t logical = p.tile_first + local;
+    const uint32_t group = logical / (4u * tiles_n);
+    const uint32_t first_m = group * 4u;
+    const uint32_t group_rows = tiles_m - first_m < 4u ? tiles_m - first_m : 4u;
+    const uint32_t in_group = logical - group * 4u * tiles_n;
+    const uint32_t tm = first_m + in_group % group_rows;
+    const uint32_t tn = in_group / group_rows;
+    const uint32_t m0 = tm * kWrTile, n0 = tn * kWrTile;
+
+    const uint32_t rows_valid = p.m - m0 < kWrTile ? p.m - m0 : kWrTile;
+    const uint32_t a_extent = ((rows_valid - 1u) * p.lda + p.k) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)a_extent, kBufferFlags);
+    const uint32_t cols_valid = p.n - n0 < kWrTile ? p.n - n0 : kWrTile;
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
+        kBufferFlags);
+
+    const uint32_t ksteps = (p.k + kWrK - 1u) / kWrK;
+    const uint32_t last_chunks = (p.k - (ksteps - 1u) * kWrK) / 8u;  // valid 16-byte chunks per row of A in the last step
+
+    // A copy: instruction j of wave w fills rows 64 w + 8 j .. + 7; lane l lands at row + l / 8, chunk position l % 8, so it
+    // fetches chunk (l % 8) ^ ((row >> 1) & 7) = (l % 8) ^ (l / 16) for even j and that ^ 4 for odd j: two lane offsets, the
+    // row advance of j (and the K advance) in the scalar offset.
+    const uint32_t a_row = 64u * wave + (lane >> 3);
+    const uint32_t chunk_e = (lane & 7u) ^ ((lane >> 4) & 7u), chunk_o = chunk_e ^ 4u;
+    const uint32_t a_voff_e = (a_row * p.lda + chunk_e * 8u) * 2u, a_voff_o = (a_row * p.lda + chunk_o * 8u) * 2u;
+    // a chunk past the end of k (partial last step) is fetched from beyond the extent: it reads as zero
+    const uint32_t a_last_e = chunk_e < last_chunks ? a_voff_e : a_extent, a_last_o = chunk_o < last_chunks ? a_voff_o : a_extent;
+    auto dma_a = [&](auto stage_c, uint32_t kt) {
+        uint8_t* base = a_tile(stage_c) + wave * 8192u;
+        const bool last = kt + 1u == ksteps;
+        const uint32_t ve = last ? a_last_e : a_voff_e, vo = last ? a_last_o : a_voff_o;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
+                                                     (j & 1u) ? vo : ve, kt * kWrK * 2u + j * 16u * p.lda, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);  // the copy's requests stay ahead of the loads that follow: the wait below counts on it
+    };
+
+    // W: this lane's 4 columns, rows 8 kq .. 8 kq + 7 of a block of 32 k
+    const uint32_t wcol = 64u * wave + 4u * c16;                 // within the tile
+    const uint32_t b_voff = 8u * kq * p.ldb_bytes + (BITS == 8 ? wcol : wcol / 2u);
+    const bool w_ok = n0 + wcol < p.n;
+    struct Raw {
+        uint32_t d[2][8];   // [block of 32 k][row]
+        uint32_t s[2][2];   // grouped scales of the two blocks: 4 bf16 each
+    };
+    auto gload = [&](Raw& raw, uint32_t kt) {
+#pragma unroll
+        for (uint32_t blk = 0; blk < 2; ++blk) {
+            const uint32_t row0 = (kt * kWrK + 32u * blk) * p.ldb_bytes;
+#pragma unroll
+            for (uint32_t r = 0; r < 8; ++r) {
+                if constexpr (BITS == 8) raw.d[blk][r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
+                else raw.d[blk][r] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
+            }
+            if constexpr (GROUPED) {
+                uint32_t g = (kt * kWrK + 32u * blk) / p.group_size;
+                const uint32_t groups = p.k / p.group_size;
+                if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do
+                uint2 sr = make_uint2(0, 0);
+                if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + n0 + wcol);
+                raw.s[blk][0] = sr.x;
+                raw.s[blk][1] = sr.y;
+            }
+        }
+    };
+    float cs[4];
+    if constexpr (!GROUPED) {
+        uint2 sr = make_uint2(0, 0);
+        if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + n0 + wcol);
+        cs[0] = make_col_scale<BITS>(sr.x & 0xffffu);
+        cs[1] = make_col_scale<BITS>(sr.x >> 16);
+        cs[2] = make_col_scale<BITS>(sr.y & 0xffffu);
+        cs[3] = make_col_scale<BITS>(sr.y >> 16);
+    }
+    struct Ops {
+        bf16x8_t w[2][4];  // [block of 32 k][column j]
+    };
+    // one column of one block: 8 weights -> operand
+    auto convert_col = [&](Ops& ops, const uint32_t (&s8)[8], const float (&sc)[4], auto blk_c, auto j_c) {
+        constexpr int BLK = decltype(blk_c)::value, J = decltype(j_c)::value;
+        uint4 w;
+        w.x = pack_bf16_rne(sbyte_to_f32<J>(s8[0]) * sc[J], sbyte_to_f32<J>(s8[1]) * sc[J]);
+        w.y = pack_bf16_rne(sbyte_to_f32<J>(s8[2]) * sc[J], sbyte_to_f32<J>(s8[3]) * sc[J]);
+        w.z = pack_bf16_rne(sbyte_to_f32<J>(s8[4]) * sc[J], sbyte_to_f32<J>(s8[5]) * sc[J]);
+        w.w = pack_bf16_rne(sbyte_to_f32<J>(s8[6]) * sc[J], sbyte_to_f32<J>(s8[7]) * sc[J]);
+        ops.w[BLK][J] = __builtin_bit_cast(bf16x8_t, w);
+    };
+    // the raw rows of one block -> signed bytes, and the block's four column scales
+    auto prepare_block = [&](uint32_t (&s8)[8], float (&sc)[4], const Raw& raw, auto blk_c) {
+        constexpr int BLK = decltype(blk_c)::value;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) s8[r] = BITS == 8 ? codes8_to_s8(raw.d[BLK][r]) : codes4_quad_to_s8x16(raw.d[BLK][r]);
+        if constexpr (GROUPED) {
+            sc[0] = make_col_scale<BITS>(raw.s[BLK][0] & 0xffffu);
+            sc[1] = make_col_scale<BITS>(raw.s[BLK][0] >> 16);
+            sc[2] = make_col_scale<BITS>(raw.s[BLK][1] & 0xffffu);
+            sc[3] = make_col_scale<BITS>(raw.s[BLK][1] >> 16);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sc[j] = cs[j];
+        }
+    };
+    auto convert_block = [&](Ops& ops, const Raw& raw, auto blk_c) {
+        uint32_t s8[8];
+        float sc[4];
+        prepare_block(s8, sc, raw, blk_c);
+        convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 0>{});
+        convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 1>{});
+        convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 2>{});
+        convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 3>{});
+    };
+
+    // byte `col` (a compile-time value at every call site) of a dword of signed bytes, as fp32
+    auto sbyte_sel = [&](uint32_t x, uint32_t col) -> float {
+        return col == 0 ? sbyte_to_f32<0>(x) : col == 1 ? sbyte_to_f32<1>(x) : col == 2 ? sbyte_to_f32<2>(x) : sbyte_to_f32<3>(x);
+    };
+    auto load_group_scales = [&](Raw& raw, uint32_t kt, uint32_t blk) {
+        uint32_t g = (kt * kWrK + 32u * blk) / p.group_size;
+        const uint32_t groups = p.k / p.group_size;
+        if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do
+        uint2 sr = make_uint2(0, 0);
+        if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + n0 + wcol);
+        raw.s[blk][0] = sr.x;
+        raw.s[blk][1] = sr.y;
+    };
+    auto block_scales = [&](float (&sc)[4], const Raw& raw, auto blk_c) {
+        constexpr int BLK = decltype(blk_c)::value;
+        sc[0] = make_col_scale<BITS>(raw.s[BLK][0] & 0xffffu);
+        sc[1] = make_col_scale<BITS>(raw.s[BLK][0] >> 16);
+        sc[2] = make_col_scale<BITS>(raw.s[BLK][1] & 0xffffu);
+        sc[3] = make_col_scale<BITS>(raw.s[BLK][1] >> 16);
+    };
+
+    f32x4_t acc[16][4];
+#pragma unroll
+    for (int mt = 0; mt < 16; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // fragment (mt, blk): row 16 mt + c16 of the tile, chunk 4 blk + kq
+    uint32_t a_rd[2];
+#pragma unroll
+    for (uint32_t blk = 0; blk < 2; ++blk) a_rd[blk] = wr_swz(c16, 4u * blk + kq);  // + mt * 2048 (16 rows; the swizzle repeats every 16 rows)
+    auto read_frag = [&](auto stage_c, uint32_t blk, uint32_t mt) -> bf16x8_t {
+        return *reinterpret_cast<const bf16x8_t*>(a_tile(stage_c) + a_rd[blk] + mt * 2048u);
+    };
+
+    // One K-step: stage S and `cur` hold this step; `nxt` receives the operands of step kt + 1 from `raw1` (loaded one
+    // step ago); `raw2` receives the codes of step kt + 2.
+    // With one wave per SIMD nothing overlaps by itself: the wave issues in order, and the matrix pipe idles whenever the
+    // wave is busy issuing something else for longer than a matrix instruction runs (16 cycles).  So the step is written
+    // as 128 slots of one matrix instruction plus at most a few other instructions, fenced so the compiler keeps them
+    // that way: slot (g, i, j) — group g of 16 (block of 32 k = g / 4, row blocks 4 (g % 4) .. + 3), row block i, column j:
+    //   j = 0  fetch the A fragment (g + 1, i) of the next group
+    //   j = 1  a quarter of a column's conversion: column g % 4 of block g / 4 of the NEXT step's weights, rows 2 i, 2 i + 1
+    //          of the lane's 8 (five instructions)
+    //   j = 2  one request to memory: the 8 A copies in groups 0-1, the 16 raw-code loads in groups 2-5, the scales in group 6
+    //   j = 3  in group 3: two rows of the next block's codes made signed
+    auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const Raw& raw1, Raw& raw2) {
+        constexpr uint32_t S = decltype(stage_c)::value;
+        using Other = std::integral_constant<uint32_t, S ^ 1u>;
+        bf16x8_t af[2][4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) af[0][i] = read_frag(stage_c, 0, i);
+        const uint32_t kt1 = kt + 1 < ksteps ? kt + 1 : kt, kt2 = kt + 2 < ksteps ? kt + 2 : ksteps - 1;
+        const bool last = kt1 + 1u == ksteps;
+        const uint32_t a_ve = last ? a_last_e : a_voff_e, a_vo = last ? a_last_o : a_voff_o;
+        uint8_t* const a_dst = a_tile(Other{}) + wave * 8192u;
+        uint32_t s8[8];
+        float sc[4];
+        uint32_t wq[2][4][4];  // the next step's operands as they are built: [block][column][dword]
+        prepare_block(s8, sc, raw1, B0{});
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t g = 0; g < 8; ++g) {
+            const uint32_t blk = g >> 2, mt0 = 4u * (g & 3u);
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    mfma16(acc[mt0 + i][j], af[g & 1][i], cur.w[blk][j]);
+                    if (j == 0 && g + 1 < 8) af[(g + 1) & 1][i] = read_frag(stage_c, (g + 1) >> 2, 4u * ((g + 1) & 3u) + i);
+                    if (j == 1) {
+                        const uint32_t col = g & 3u;
+                        wq[blk][col][i] = pack_bf16_rne(sbyte_sel(s8[2 * i], col) * sc[col], sbyte_sel(s8[2 * i + 1], col) * sc[col]);
+                    }
+                    if (j == 2) {
+                        const uint32_t q = 4u * g + i;  // 0..31
+                        if (q < 8) {
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16,
+                                                                     (q & 1u) ? a_vo : a_ve, kt1 * kWrK * 2u + q * 16u * p.lda, 0, 0);
+                        } else if (q < 24) {
+                            const uint32_t lb = (q - 8u) >> 3, r = (q - 8u) & 7u;
+                            const uint32_t soff = (kt2 * kWrK + 32u * lb + r) * p.ldb_bytes;
+                            if constexpr (BITS == 8) raw2.d[lb][r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, b_voff, soff, 0);
+                            else raw2.d[lb][r] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_b, b_voff, soff, 0);
+                        } else if (GROUPED && q < 26) {
+                            load_group_scales(raw2, kt2, q - 24u);
+                        }
+                    }
+                    if (j == 3 && g == 3) {
+                        // block 1's codes made signed, two rows per slot, into the half of s8 whose conversion is done
+                        // (rows 2 i, 2 i + 1 of block 0 were last used by slot (3, i, 1))
+                        s8[2 * i] = BITS == 8 ? codes8_to_s8(raw1.d[1][2 * i]) : codes4_quad_to_s8x16(raw1.d[1][2 * i]);
+                        s8[2 * i + 1] = BITS == 8 ? codes8_to_s8(raw1.d[1][2 * i + 1]) : codes4_quad_to_s8x16(raw1.d[1][2 * i + 1]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if (g == 3) {
+                if constexpr (GROUPED) block_scales(sc, raw1, B1{});
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int b2 = 0; b2 < 2; ++b2)
+#pragma unroll
+            for (int c2 = 0; c2 < 4; ++c2)
+                nxt.w[b2][c2] = __builtin_bit_cast(bf16x8_t, make_uint4(wq[b2][c2][0], wq[b2][c2][1], wq[b2][c2][2], wq[b2][c2][3]));
+        // this wave's part of the next A tile has landed in LDS (the loads of raw codes and scales issued after it may still fly)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GROUPED ? 18 : 16) : "memory");
+        __syncthreads();
+    };
+
+    // ---- prologue: A tile 0 -> stage 0; operands of step 0; raw codes of step 1
+    Ops ops0, ops1;
+    Raw rawa, rawb;
+    dma_a(C0{}, 0);
+    gload(rawa, 0);
+    convert_block(ops0, rawa, B0{});
+    convert_block(ops0, rawa, B1{});
+    gload(rawa, ksteps > 1 ? 1 : 0);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GROUPED ? 18 : 16) : "memory");
+    __syncthreads();
+
+    uint32_t kt = 0;
+    for (; kt + 1 < ksteps; kt += 2) {
+        step(C0{}, kt, ops0, ops1, rawa, rawb);
+        step(C1{}, kt + 1, ops1, ops0, rawb, rawa);
+    }
+    if (kt < ksteps) step(C0{}, kt, ops0, ops1, rawa, rawb);
+
+    // ---- epilogue: bf16 tile through LDS (rows 64 q .. 64 q + 63 in the q-th array), then 16-byte row-contiguous stores
+    wreg_settle();  // the last matrix instructions have written their accumulators
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
+    __syncthreads();
+    auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_c0 : lds_c1; };
+    {
+        float bias[4] = {0.f, 0.f, 0.f, 0.f};
+        const bool has_bias = p.bias != nullptr;
+        if (has_bias && w_ok) {
+            const uint2 raw = *reinterpret_cast<const uint2*>(p.bias + n0 + wcol);
+            bias[0] = bf16_bits_to_f32(raw.x & 0xffffu);
+            bias[1] = bf16_bits_to_f32(raw.x >> 16);
+            bias[2] = bf16_bits_to_f32(raw.y & 0xffffu);
+            bias[3] = bf16_bits_to_f32(raw.y >> 16);
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < 16; ++mt) {
+            uint8_t* base = c_rows(mt >> 2);
+#pragma unroll
+            for (uint32_t r = 0; r < 4; ++r) {
+                const uint32_t row = 16u * (mt & 3u) + 4u * kq + r;  // within the 64 rows of this array
+                uint2 o;
+                // without a bias the sums are stored as they are (adding +0 would turn a -0 sum into +0)
+                if (has_bias) {
+                    o.x = pack_bf16_rne(acc[mt][0][r] + bias[0], acc[mt][1][r] + bias[1]);
+                    o.y = pack_bf16_rne(acc[mt][2][r] + bias[2], acc[mt][3][r] + bias[3]);
+                } else {
+                    o.x = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
+                    o.y = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
+                }
+                *reinterpret_cast<uint2*>(base + row * kWrCRowBytes + wcol * 2u) = o;
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (uint32_t pass = 0; pass < 32u; ++pass) {
+        const uint32_t row = pass * 8u + (tid >> 5);
+        const uint32_t ch = tid & 31u;
+        const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
+        if (gm < p.m && gn < p.n) {
+            const uint4 v = *reinterpret_cast<const uint4*>(c_rows(row >> 6) + (row & 63u) * kWrCRowBytes + ch * 16u);
+            *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) = v;
+        }
+    }
+}
+
+// Runs `tile_count` whole 256x256 tiles from `tile_first` on (the caller splits off a last, thin round for the half-tile kernel).
+template <int BITS, bool GROUPED>
+static hipError_t launch_wreg_t(const GemmParams& p, hipStream_t stream)
+{
+    const uint32_t grid = (p.tile_count + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
+    void (*kernel)(const GemmParams) = bfaintb_prefill_wreg_kernel<BITS, GROUPED>;
+    return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
+}
+
+// Whether this kernel can serve a launch: row-major weights, this library's arithmetic, no residual or gate.
+bool prefill_wreg_serves(const GemmParams& p)
+{
+    return !p.reference_arith && p.residual == nullptr && p.activation == kActNone;
+}
+
+hipError_t launch_prefill_wreg(const GemmParams& p, int bits, hipStream_t stream)
+{
+    const bool grouped = p.group_size != 0;
+    if (bits == 8) return grouped ? launch_wreg_t<8, true>(p, stream) : launch_wreg_t<8, false>(p, stream);
+    return grouped ? launch_wreg_t<4, true>(p, stream) : launch_wreg_t<4, false>(p, stream);
+}
+
+}  // namespace bfaintb

@@ -62,7 +62,7 @@ def draw_case(rng):
     epilogue = str(rng.choice(["none", "none", "none", "bias", "residual", "bias+residual", "gate", "gate+bias+residual"]))
     if epilogue.startswith("gate") and n % 32:
         n += 16                                   # the gated output has n/2 columns, itself a multiple of 16
-    variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256"]))
+    variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256", "prefill_256_lds"]))
     if epilogue != "none" and not (packed and epilogue == "bias"):
         variant = "auto"                          # the fused entry points choose the kernel themselves
     pad = int(rng.choice([0, 0, 8, 24]))           # extra elements per row of A, C (and the residual): strided operands
@@ -87,7 +87,8 @@ def test_random_case(af, case):
             p.residual_bf = oracle.f32_to_bf16_rne(np.random.default_rng(m).uniform(-2, 2, size=(m, n // 2)).astype(np.float32))
         else:
             p.with_residual()
-    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[case["variant"]]
+    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256,
+             "prefill_256_lds": af.PREFILL_256_LDS}[case["variant"]]
     act = af.ACT_SILU_GATE if gated else af.ACT_NONE
     if case["pad"]:
         c = run_strided(af, p, which, act, case["packed"], case["pad"])
@@ -135,13 +136,14 @@ def run_ragged(af, p, which, act=0, pad=0):
     (33, 1000, 1000, 8, 0, "auto"), (33, 1000, 1000, 8, 0, "decode"), (33, 1000, 1000, 8, 0, "prefill_128"), (33, 1000, 1000, 8, 0, "prefill_256"),
     (1, 4104, 4072, 8, 0, "auto"), (16, 4104, 4072, 8, 0, "auto"), (32, 520, 1048, 8, 0, "auto"),
     (1, 8, 8, 8, 0, "auto"), (5, 24, 16, 8, 0, "decode"), (5, 24, 24, 8, 0, "prefill_128"), (70, 40, 8, 8, 0, "prefill_256"),
-    (300, 1000, 1000, 8, 0, "auto"), (700, 1000, 1000, 8, 0, "prefill_256"), (130, 264, 72, 8, 0, "decode"),
+    (300, 1000, 1000, 8, 0, "auto"), (700, 1000, 1000, 8, 0, "prefill_256"), (700, 1000, 1000, 8, 0, "prefill_256_lds"), (130, 264, 72, 8, 0, "decode"),
+    (33000, 264, 72, 8, 0, "prefill_256"), (33000, 272, 72, 4, 0, "prefill_256"), (33000, 264, 96, 8, 32, "prefill_256"),   # whole rounds of 256x256 tiles
     (16, 1008, 1000, 4, 0, "auto"), (1, 4112, 4072, 4, 0, "auto"), (300, 1008, 1000, 4, 0, "prefill_128"), (300, 1008, 1000, 4, 0, "prefill_256"),
     (48, 1000, 992, 8, 32, "auto"), (300, 1000, 992, 8, 32, "prefill_128"), (300, 1000, 96, 8, 32, "prefill_256"), (8, 1008, 96, 4, 32, "auto"),
 ])
 def test_ragged_shapes(af, m, n, k, bits, group, variant):
     p = Problem(m, n, k, bits, group, seed=m + n + k)
-    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[variant]
+    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256, "prefill_256_lds": af.PREFILL_256_LDS}[variant]
     assert_close_ulp(p, run_ragged(af, p, which, pad=8), f"ragged {m}x{n}x{k} int{bits} g{group} {variant}")
 
 
@@ -156,7 +158,7 @@ def draw_ragged(rng):
     epilogue = str(rng.choice(["none", "none", "bias", "bias+residual", "gate"]))
     if epilogue == "gate":
         n = (n + 15) // 16 * 16
-    variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256"])) if epilogue == "none" else "auto"
+    variant = str(rng.choice(["auto", "decode", "prefill_128", "prefill_256", "prefill_256_lds"])) if epilogue == "none" else "auto"
     return dict(m=m, n=n, k=k, bits=bits, group=group, epilogue=epilogue, variant=variant, pad=int(rng.choice([0, 8, 24])))
 
 
@@ -172,6 +174,7 @@ def test_random_ragged_case(af, case):
         p.with_bias()
     if "residual" in case["epilogue"]:
         p.with_residual()
-    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256}[case["variant"]]
+    which = {"auto": af.AUTO, "decode": af.DECODE, "prefill_128": af.PREFILL_128, "prefill_256": af.PREFILL_256,
+             "prefill_256_lds": af.PREFILL_256_LDS}[case["variant"]]
     c = run_ragged(af, p, which, af.ACT_SILU_GATE if gated else af.ACT_NONE, case["pad"])
     (assert_close_gated if gated else assert_close_ulp)(p, c, str(case))
