@@ -11,13 +11,14 @@
 //   Lane (c16 = lane % 16, kq = lane / 16) loads, per block of 32 k and for each of the 8 rows k0 + 8 kq + r, one dword =
 //   the codes of columns 4 c16 .. 4 c16 + 3 of the wave's 64 (16-bit loads for 4-bit codes): byte j of those 8 dwords is
 //   the 8-element operand of column 4 c16 + j, rows 8 kq .. 8 kq + 7 — the layout v_mfma_f32_16x16x32_bf16 wants.
-//   A: global -> LDS directly (buffer_load ... lds), two stages of 256 rows x 64 k (32 KiB each), rows of 128 bytes in 8
+//   A: global -> LDS directly (buffer_load ... lds), four stages of 256 rows x 64 k (32 KiB each), rows of 128 bytes in 8
 //   chunks of 16, chunk c of row r at position c ^ ((r >> 1) & 7); a fragment read is one ds_read_b128 (16 rows x 32 k).
 //   Per K-step a CU reads 128 KiB of LDS and the copy engine writes 32 KiB.
 // Pipeline per K-step of 64 (registers: operands of this step; raw codes of the next, loaded one step ago): request the
-//   A tile of step+1 into the other stage and the raw codes of step+2; convert the raw codes of step+1 into the second
-//   operand set between the matrix instructions; 128 matrix instructions (2 blocks of 32 k x 16 row blocks x 4 columns),
-//   A fragments fetched a few ahead; wait for the A copy; one barrier.
+//   A tile of step+2 into the stage read two steps ago and the raw codes of step+2; convert the raw codes of step+1 into
+//   the second operand set between the matrix instructions; 128 matrix instructions (2 blocks of 32 k x 16 row blocks x
+//   4 columns), A fragments fetched one group of 16 ahead — the last group fetches the next step's first fragments, so no
+//   step starts by waiting for LDS; one barrier, in the middle of the step.
 // Accumulator (mt, j), register r of lane (c16, q = lane / 16): row 16 mt + 4 q + r, column 64 w + 4 c16 + j of the tile.
 // Epilogue: bias, rounding to bf16, staging through LDS in [m][n] order, 16-byte row-contiguous stores.
 #include <utility>
@@ -54,9 +55,14 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
 {
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kWrStageBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kWrStageBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_c0[kWrStageBytes];  // epilogue staging only
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_c1[kWrStageBytes];
-    auto a_tile = [&](auto stage_c) -> uint8_t* { return decltype(stage_c)::value == 0 ? lds_a0 : lds_a1; };
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a2[kWrStageBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a3[kWrStageBytes];
+    // (four separate arrays rather than one block: the compiler then knows that fragment reads of one stage cannot alias
+    // the asynchronous copies into another, and does not make them wait for those)
+    auto a_tile = [&](auto stage_c) -> uint8_t* {
+        constexpr uint32_t St = decltype(stage_c)::value;
+        return St == 0 ? lds_a0 : St == 1 ? lds_a1 : St == 2 ? lds_a2 : lds_a3;
+    };
 
     using C0 = std::integral_constant<uint32_t, 0>;
     using C1 = std::integral_constant<uint32_t, 1>;
@@ -231,23 +237,23 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
     // as 128 slots of one matrix instruction plus at most a few other instructions, fenced so the compiler keeps them
     // that way: slot (g, i, j) — group g of 16 (block of 32 k = g / 4, row blocks 4 (g % 4) .. + 3), row block i, column j:
     //   j = 0  fetch the A fragment (g + 1, i) of the next group
-    //   j = 1  a quarter of a column's conversion: column g % 4 of block g / 4 of the NEXT step's weights, rows 2 i, 2 i + 1
-    //          of the lane's 8 (five instructions)
+    //   j = 1, 3  a quarter of a column's conversion: column g % 4 of block g / 4 of the NEXT step's weights, rows 2 i,
+    //          2 i + 1 of the lane's 8 (five instructions, three in slot 1 and two in slot 3)
     //   j = 2  one request to memory: the 8 A copies in groups 0-1, the 16 raw-code loads in groups 2-5, the scales in group 6
-    //   j = 3  in group 3: two rows of the next block's codes made signed
+    //   j = 3  also, in group 3: two rows of the next block's codes made signed
+    bf16x8_t af[2][4];  // A fragments of the group being multiplied and of the next one; af[0] carries over from step to step
     auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const Raw& raw1, Raw& raw2) {
         constexpr uint32_t S = decltype(stage_c)::value;
-        using Other = std::integral_constant<uint32_t, S ^ 1u>;
-        bf16x8_t af[2][4];
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) af[0][i] = read_frag(stage_c, 0, i);
-        const uint32_t kt1 = kt + 1 < ksteps ? kt + 1 : kt, kt2 = kt + 2 < ksteps ? kt + 2 : ksteps - 1;
-        const bool last = kt1 + 1u == ksteps;
+        using Next = std::integral_constant<uint32_t, (S + 1u) & 3u>;
+        using Target = std::integral_constant<uint32_t, (S + 2u) & 3u>;
+        const uint32_t kt2 = kt + 2 < ksteps ? kt + 2 : ksteps - 1;
+        const bool last = kt2 + 1u == ksteps;
         const uint32_t a_ve = last ? a_last_e : a_voff_e, a_vo = last ? a_last_o : a_voff_o;
-        uint8_t* const a_dst = a_tile(Other{}) + wave * 8192u;
+        uint8_t* const a_dst = a_tile(Target{}) + wave * 8192u;
         uint32_t s8[8];
         float sc[4];
         uint32_t wq[2][4][4];  // the next step's operands as they are built: [block][column][dword]
+        float f_lo = 0.f, f_hi = 0.f;
         prepare_block(s8, sc, raw1, B0{});
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -258,16 +264,20 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
 #pragma unroll
                 for (uint32_t j = 0; j < 4; ++j) {
                     mfma16(acc[mt0 + i][j], af[g & 1][i], cur.w[blk][j]);
-                    if (j == 0 && g + 1 < 8) af[(g + 1) & 1][i] = read_frag(stage_c, (g + 1) >> 2, 4u * ((g + 1) & 3u) + i);
-                    if (j == 1) {
+                    if (j == 0) {
+                        if (g + 1 < 8) af[(g + 1) & 1][i] = read_frag(stage_c, (g + 1) >> 2, 4u * ((g + 1) & 3u) + i);
+                        else af[0][i] = read_frag(Next{}, 0, i);  // the next step's first group (its stage is complete: see the barrier)
+                    }
+                    if (j == 1) {  // (the five instructions of a quarter column are split 3 + 2 over slots j = 1 and j = 3)
                         const uint32_t col = g & 3u;
-                        wq[blk][col][i] = pack_bf16_rne(sbyte_sel(s8[2 * i], col) * sc[col], sbyte_sel(s8[2 * i + 1], col) * sc[col]);
+                        f_lo = sbyte_sel(s8[2 * i], col) * sc[col];
+                        f_hi = sbyte_sel(s8[2 * i + 1], col);
                     }
                     if (j == 2) {
                         const uint32_t q = 4u * g + i;  // 0..31
                         if (q < 8) {
                             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16,
-                                                                     (q & 1u) ? a_vo : a_ve, kt1 * kWrK * 2u + q * 16u * p.lda, 0, 0);
+                                                                     (q & 1u) ? a_vo : a_ve, kt2 * kWrK * 2u + q * 16u * p.lda, 0, 0);
                         } else if (q < 24) {
                             const uint32_t lb = (q - 8u) >> 3, r = (q - 8u) & 7u;
                             const uint32_t soff = (kt2 * kWrK + 32u * lb + r) * p.ldb_bytes;
@@ -277,6 +287,7 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                             load_group_scales(raw2, kt2, q - 24u);
                         }
                     }
+                    if (j == 3) wq[blk][g & 3u][i] = pack_bf16_rne(f_lo, f_hi * sc[g & 3u]);
                     if (j == 3 && g == 3) {
                         // block 1's codes made signed, two rows per slot, into the half of s8 whose conversion is done
                         // (rows 2 i, 2 i + 1 of block 0 were last used by slot (3, i, 1))
@@ -288,6 +299,14 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
             }
             if (g == 3) {
                 if constexpr (GROUPED) block_scales(sc, raw1, B1{});
+                // The step's one barrier, in the middle.  Before it the wave makes sure that its part of the A tile of step
+                // kt + 1 has landed (requested during step kt - 1; since then it has requested the rest of that step's codes and
+                // scales, this step's A copy and 8 loads of codes: at most that many requests may still be in flight).  Behind
+                // it every wave's part has: the next step's first fragments can be fetched at the end of this one, and the
+                // copy this step started (into the stage read two steps ago) overwrites nothing a wave still reads — every
+                // wave that reaches this barrier has passed the previous one, i.e. finished the step before it.
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((GROUPED ? 18 : 16) + 16) : "memory");
+                __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -296,34 +315,40 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
 #pragma unroll
             for (int c2 = 0; c2 < 4; ++c2)
                 nxt.w[b2][c2] = __builtin_bit_cast(bf16x8_t, make_uint4(wq[b2][c2][0], wq[b2][c2][1], wq[b2][c2][2], wq[b2][c2][3]));
-        // this wave's part of the next A tile has landed in LDS (the loads of raw codes and scales issued after it may still fly)
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GROUPED ? 18 : 16) : "memory");
-        __syncthreads();
     };
 
-    // ---- prologue: A tile 0 -> stage 0; operands of step 0; raw codes of step 1
+    // ---- prologue: A tiles 0 and 1 -> stages 0 and 1; operands of step 0; raw codes of step 1; the first fragments
     Ops ops0, ops1;
     Raw rawa, rawb;
     dma_a(C0{}, 0);
+    dma_a(C1{}, ksteps > 1 ? 1 : 0);
     gload(rawa, 0);
     convert_block(ops0, rawa, B0{});
     convert_block(ops0, rawa, B1{});
     gload(rawa, ksteps > 1 ? 1 : 0);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GROUPED ? 18 : 16) : "memory");
     __syncthreads();
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) af[0][i] = read_frag(C0{}, 0, i);
 
+    using C2 = std::integral_constant<uint32_t, 2>;
+    using C3 = std::integral_constant<uint32_t, 3>;
     uint32_t kt = 0;
-    for (; kt + 1 < ksteps; kt += 2) {
+    for (; kt + 3 < ksteps; kt += 4) {
         step(C0{}, kt, ops0, ops1, rawa, rawb);
         step(C1{}, kt + 1, ops1, ops0, rawb, rawa);
+        step(C2{}, kt + 2, ops0, ops1, rawa, rawb);
+        step(C3{}, kt + 3, ops1, ops0, rawb, rawa);
     }
     if (kt < ksteps) step(C0{}, kt, ops0, ops1, rawa, rawb);
+    if (kt + 1 < ksteps) step(C1{}, kt + 1, ops1, ops0, rawb, rawa);
+    if (kt + 2 < ksteps) step(C2{}, kt + 2, ops0, ops1, rawa, rawb);
 
     // ---- epilogue: bf16 tile through LDS (rows 64 q .. 64 q + 63 in the q-th array), then 16-byte row-contiguous stores
     wreg_settle();  // the last matrix instructions have written their accumulators
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
     __syncthreads();
-    auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_c0 : lds_c1; };
+    auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_a2 : lds_a3; };
     {
         float bias[4] = {0.f, 0.f, 0.f, 0.f};
         const bool has_bias = p.bias != nullptr;
