@@ -407,7 +407,7 @@ const char* bfaintb_error_string(int code)
         case BFAINTB_OK: return "success";
         case BFAINTB_ERR_NULL_POINTER: return "null device pointer";
         case BFAINTB_ERR_BAD_SHAPE: return "unsupported shape: need n % 8 == 0 (4-bit codes: n % 16 == 0), k % 8 == 0, k > 0, sizes below 2^31; pre-packed weights: n % 16 == 0, k % 64 == 0 (4-bit: k % 128 == 0)";
-        case BFAINTB_ERR_BAD_LD: return "bad leading dimension: need lda >= k, ldb >= n, ldc >= n, lda % 8 == 0, ldb % 16 == 0, ldc % 8 == 0";
+        case BFAINTB_ERR_BAD_LD: return "bad leading dimension: need lda >= k, n <= ldb < 2^27, ldc >= n, lda % 8 == 0, ldb % 16 == 0, ldc % 8 == 0";
         case BFAINTB_ERR_ALIGNMENT: return "pointer not 16-byte aligned";
         case BFAINTB_ERR_UNSUPPORTED: return "unsupported format: weight_bits must be 8 or 4; group_size 0 or a multiple of 32 that divides k";
         case BFAINTB_ERR_WORKSPACE: return "workspace missing or smaller than bfaintb_gemm_workspace_bytes reports";
@@ -543,6 +543,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     e = check_shape(m, n, k, weight_bits);
     if (e) return e;
     if (lda < k || ldb < n || ldc < ep.out_cols(n) || lda % 8u != 0 || ldb % 16u != 0 || ldc % 8u != 0) return BFAINTB_ERR_BAD_LD;
+    if (ldb >= (1u << 27)) return BFAINTB_ERR_BAD_LD;  // a lane's offset within 32 rows of B is kept in 32 bits
     const int v = resolve_variant(m, n, k, weight_bits, variant);
     if (v < 0) return v;
     if (m == 0 || n == 0) return BFAINTB_OK;

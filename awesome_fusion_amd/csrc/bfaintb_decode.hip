@@ -34,7 +34,7 @@ struct RawStep {
     uint32_t d[8][kDwords];  // 8 rows x CPL codes
 };
 
-// Signed value of column C (0..CPL-1) of one prepared row, as fp32 (x16 for 4-bit codes).
+// Signed value of column C (0..CPL-1) of one prepared row, as fp32 (divided by 16 for 4-bit codes).
 template <int BITS, int C, int PD>
 __device__ __forceinline__ float value_f32(const uint32_t (&row)[PD])
 {
@@ -43,23 +43,26 @@ __device__ __forceinline__ float value_f32(const uint32_t (&row)[PD])
     } else {
         // prepared 4-bit row: dwords {even columns of raw dword 0, odd of 0, even of 1, odd of 1};
         // column C sits in raw dword C/8, byte (C%8)/2
-        return sbyte_to_f32<(C % 8) / 2>(row[2 * (C / 8) + (C % 2)]);
+        return nibble_to_f32_sixteenth<(C % 8) / 2>(row[2 * (C / 8) + (C % 2)]);
     }
 }
 
 // Non-temporal loads: the weights are read once, and marked so they stream through the caches without displacing the
 // activations, the scales, the workspace and the kernel's own code (measured on the fetch alone: 16 MiB in 3.9 us
 // against 4.3 us with plain loads; 43 MiB in 7.9 against 8.7 us).
+// `rows` is the same for every lane of the wave (it stays in scalar registers and advances there); `lane_off` is the
+// lane's place within the 8 x CPL block, 32 bits wide.
 template <int BITS, int CPL>
-__device__ __forceinline__ void load_raw(RawStep<BITS, CPL>& raw, const uint8_t* rowptr, uint32_t ldb_bytes)
+__device__ __forceinline__ void load_raw(RawStep<BITS, CPL>& raw, const uint8_t* rows, uint32_t lane_off, uint32_t ldb_bytes)
 {
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
+        const uint8_t* src = rows + (size_t)r * ldb_bytes + lane_off;
         if constexpr (RawStep<BITS, CPL>::kDwords == 4) {
-            const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(rowptr + (size_t)r * ldb_bytes));
+            const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
             raw.d[r][0] = v[0]; raw.d[r][1] = v[1]; raw.d[r][2] = v[2]; raw.d[r][3] = v[3];
         } else {
-            const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(rowptr + (size_t)r * ldb_bytes));
+            const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(src));
             raw.d[r][0] = v[0]; raw.d[r][1] = v[1];
         }
     }
@@ -74,8 +77,8 @@ __device__ __forceinline__ void prepare_row(uint32_t (&out)[CPL / 4], const uint
         for (int i = 0; i < CPL / 4; ++i) out[i] = codes8_to_s8(in[i]);
     } else {
         static_assert(BITS == 8 || CPL == 16, "4-bit codes: 16 columns per lane");
-        codes4_to_s8x16(in[0], out[0], out[1]);
-        codes4_to_s8x16(in[1], out[2], out[3]);
+        codes4_to_nibbles(in[0], out[0], out[1]);
+        codes4_to_nibbles(in[1], out[2], out[3]);
     }
 }
 
@@ -165,11 +168,11 @@ __device__ __forceinline__ void mac_step_packed(const PackedStep<BITS, CPL>& raw
             w.w = pack_bf16_rne(sbyte_to_f32<2>(hi) * s, sbyte_to_f32<3>(hi) * s);
         } else {
             uint32_t ev, od;
-            codes4_to_s8x16(raw.d[c][0], ev, od);
-            w.x = pack_bf16_rne(sbyte_to_f32<0>(ev) * s, sbyte_to_f32<0>(od) * s);
-            w.y = pack_bf16_rne(sbyte_to_f32<1>(ev) * s, sbyte_to_f32<1>(od) * s);
-            w.z = pack_bf16_rne(sbyte_to_f32<2>(ev) * s, sbyte_to_f32<2>(od) * s);
-            w.w = pack_bf16_rne(sbyte_to_f32<3>(ev) * s, sbyte_to_f32<3>(od) * s);
+            codes4_to_nibbles(raw.d[c][0], ev, od);
+            w.x = pack_bf16_rne(nibble_to_f32_sixteenth<0>(ev) * s, nibble_to_f32_sixteenth<0>(od) * s);
+            w.y = pack_bf16_rne(nibble_to_f32_sixteenth<1>(ev) * s, nibble_to_f32_sixteenth<1>(od) * s);
+            w.z = pack_bf16_rne(nibble_to_f32_sixteenth<2>(ev) * s, nibble_to_f32_sixteenth<2>(od) * s);
+            w.w = pack_bf16_rne(nibble_to_f32_sixteenth<3>(ev) * s, nibble_to_f32_sixteenth<3>(od) * s);
         }
         const bf16x8_t wf = __builtin_bit_cast(bf16x8_t, w);
 #pragma unroll
@@ -190,11 +193,13 @@ __device__ __forceinline__ void load_scales_packed(uint4 (&sraw)[CPL / 8], const
     for (int i = 0; i < CPL / 8; ++i) sraw[i] = make_uint4(d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3]);
 }
 
+// `srow`: a row of scales, the same for every lane; `first_col`: the lane's first column
 template <int CPL>
-__device__ __forceinline__ void load_scales(uint4 (&sraw)[CPL / 8], const uint16_t* sptr)
+__device__ __forceinline__ void load_scales(uint4 (&sraw)[CPL / 8], const uint16_t* srow, uint32_t first_col)
 {
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(srow) + first_col * 2u;
 #pragma unroll
-    for (int i = 0; i < CPL / 8; ++i) sraw[i] = *reinterpret_cast<const uint4*>(sptr + 8 * i);
+    for (int i = 0; i < CPL / 8; ++i) sraw[i] = *reinterpret_cast<const uint4*>(src + 16 * i);
 }
 
 template <int BITS, int CPL>
@@ -207,8 +212,8 @@ __device__ __forceinline__ void apply_scales(float (&cs)[CPL], const uint4 (&sra
     }
 #pragma unroll
     for (int i = 0; i < CPL / 2; ++i) {
-        cs[2 * i] = make_col_scale<BITS>(d[i] & 0xffffu);
-        cs[2 * i + 1] = make_col_scale<BITS>(d[i] >> 16);
+        cs[2 * i] = make_col_scale_nibble<BITS>(d[i] & 0xffffu);
+        cs[2 * i + 1] = make_col_scale_nibble<BITS>(d[i] >> 16);
     }
 }
 
@@ -374,7 +379,7 @@ bfaintb_decode_kernel(const GemmParams p)
 
     TRACE_MARK(0);
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same for the wave's lanes: what follows from it stays scalar
     const int nl = lane & 15;
     const int kg = lane >> 4;
     const uint32_t cb = blockIdx.x;
@@ -399,7 +404,10 @@ bfaintb_decode_kernel(const GemmParams p)
     // step.  (Packed weights come in whole K-chunks; scale groups are multiples of 32 rows that divide k.)
     const uint32_t tail_rows = (PACKED || GROUPED || kb >= ke) ? 0u : (ke - kb) % 32u;
 
-    const uint8_t* bptr = p.b + (size_t)(kb + 8u * kg) * p.ldb_bytes + (size_t)n_ld * BITS / 8;
+    // the wave's first row of B (scalar) and this lane's place in a block of 32 rows (the host has checked that 32 rows'
+    // worth of bytes fit 32 bits)
+    const uint8_t* bptr = p.b + (size_t)kb * p.ldb_bytes;
+    const uint32_t b_lane = 8u * (uint32_t)kg * p.ldb_bytes + n_ld * BITS / 8u;
     const size_t bstep = (size_t)32 * p.ldb_bytes;
     // packed: K-chunks of 64 (8-bit) or 128 (4-bit) rows, 1024 bytes each, hold 2 or 4 K-blocks of 32 rows; a lane's 16
     // bytes of a chunk are its K-blocks in order
@@ -456,7 +464,7 @@ bfaintb_decode_kernel(const GemmParams p)
             uint4 sraw[KB][CPL / 8];
         };
         float cs[CPL];
-        const uint16_t* sptr = p.scale + (PACKED ? 0u : n_ld);
+        const uint16_t* sptr = p.scale;
         // packed weights with grouped scales: the wave's transposition table in LDS, behind the reduction area, and
         // the columns whose scales this lane fetches (kept inside the scale row)
         uint16_t* sc_table = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(red) + p.decode_scale_lds) + (uint32_t)wave * 16u * CPL;
@@ -478,7 +486,7 @@ bfaintb_decode_kernel(const GemmParams p)
                     load_packed<BITS, CPL>(st.raw[q], slab,
                                            (kUniformSlabs ? (uint32_t)lane * 16u : 0u) + (kblock / kBlocksPerChunk) * 1024u + (kblock % kBlocksPerChunk) * kBlockBytes);
                 } else {
-                    load_raw<BITS, CPL>(st.raw[q], bptr + blk * bstep, p.ldb_bytes);
+                    load_raw<BITS, CPL>(st.raw[q], bptr + blk * bstep, b_lane, p.ldb_bytes);
                 }
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) st.af[q][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + blk * 32);
@@ -491,12 +499,20 @@ bfaintb_decode_kernel(const GemmParams p)
                         st.sraw[q][0].x = v.x;
                         st.sraw[q][0].y = v.y;
                     } else {
-                        load_scales<CPL>(st.sraw[q], srow);
+                        load_scales<CPL>(st.sraw[q], srow, n_ld);
                     }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic that follows
         };
+        // row-major weights with grouped scales: blocks of 32 rows until the next group begins (0: the block at hand opens
+        // one — so does the wave's first, wherever in a group it lies), and how many the group after that spans
+        uint32_t blocks_to_group = 0u;
+        uint32_t next_group_blocks = 0u;
+        if constexpr (GROUPED && !PACKED) {
+            const uint32_t kb_uniform = __builtin_amdgcn_readfirstlane(kb);
+            next_group_blocks = (p.group_size - kb_uniform % p.group_size) / 32u;
+        }
         auto compute_stage = [&](Stage& st) {
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
@@ -516,7 +532,13 @@ bfaintb_decode_kernel(const GemmParams p)
                     for (int i = 0; i < CPL / 8; ++i) mine[i] = *reinterpret_cast<const uint4*>(sc_table + (uint32_t)nl * CPL + 8u * i);
                     apply_scales<BITS, CPL>(cs, mine);
                 } else if constexpr (GROUPED) {
-                    apply_scales<BITS, CPL>(cs, st.sraw[q]);
+                    // the scales change only where a group of rows begins: widen them there, not for every block
+                    if (blocks_to_group == 0u) {
+                        apply_scales<BITS, CPL>(cs, st.sraw[q]);
+                        blocks_to_group = next_group_blocks;
+                        next_group_blocks = p.group_size / 32u;
+                    }
+                    --blocks_to_group;
                 }
                 if constexpr (PACKED) mac_step_packed<BITS, CPL, MB>(st.raw[q], cs, st.af[q], acc);
                 else mac_step<BITS, CPL, MB, REF>(st.raw[q], cs, st.af[q], acc, std::make_integer_sequence<int, CPL>{});
@@ -532,7 +554,7 @@ bfaintb_decode_kernel(const GemmParams p)
                 }
             } else if constexpr (!GROUPED) {
                 if constexpr (PACKED) load_scales_packed<CPL>(st.sraw[0], sptr, pk_col);
-                else load_scales<CPL>(st.sraw[0], sptr);
+                else load_scales<CPL>(st.sraw[0], sptr, n_ld);
             }
         };
         if (nsteps > 0) {
@@ -566,7 +588,7 @@ bfaintb_decode_kernel(const GemmParams p)
                 }
                 const uint32_t krow = kb + 32u * (uint32_t)nsteps + 8u * (uint32_t)kg;
                 const bool live = krow < p.k;
-                load_raw<BITS, CPL>(st.raw[0], p.b + (size_t)(live ? krow : p.k - 8u) * p.ldb_bytes + (size_t)n_ld * BITS / 8, p.ldb_bytes);
+                load_raw<BITS, CPL>(st.raw[0], p.b + (size_t)(live ? krow : p.k - 8u) * p.ldb_bytes, n_ld * BITS / 8u, p.ldb_bytes);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     st.af[0][mb] = make_uint4(0u, 0u, 0u, 0u);

@@ -153,14 +153,37 @@ __device__ __forceinline__ float sbyte_to_f32(uint32_t x)
 //   4-bit: excess-8 nibble c = q + 8; c ^ 8 is q as int4; moved to the HIGH nibble of a byte it reads
 //          as the int8 value 16*q, and the column's scale is pre-divided by 16 (exact: a power of two).
 __device__ __forceinline__ uint32_t codes8_to_s8(uint32_t x) { return x ^ 0x80808080u; }
-// Both at once for a dword of eight codes: every code's top bit is flipped first (one operation for the dword), then the even
-// codes move up into their bytes' high nibbles and the low nibbles are cleared: 4 operations, where flipping each half
-// after its mask takes 5.
+// Both halves of a dword of eight codes: the even codes move up into their bytes' high nibbles; each half is then one
+// three-input bit operation (mask the high nibbles, flip every code's top bit): 3 operations for the dword.
 __device__ __forceinline__ void codes4_to_s8x16(uint32_t x, uint32_t& even, uint32_t& odd)
 {
-    const uint32_t y = x ^ 0x88888888u;
-    even = (y << 4) & 0xf0f0f0f0u;
-    odd = y & 0xf0f0f0f0u;
+    even = ((x << 4) & 0xf0f0f0f0u) ^ 0x80808080u;
+    odd = (x & 0xf0f0f0f0u) ^ 0x80808080u;
+}
+
+// The same eight codes for the conversion instruction that reads a nibble directly (v_cvt_off_f32_i4: bits 3:0 of its
+// source as a two's-complement value, divided by 16 — exact): flip every code's top bit, and shift the odd codes down to
+// the low nibbles of their bytes.  2 operations for the dword; the bits above a nibble are ignored by the instruction.
+__device__ __forceinline__ void codes4_to_nibbles(uint32_t x, uint32_t& even, uint32_t& odd)
+{
+    even = x ^ 0x88888888u;
+    odd = even >> 4;
+    asm("" : "+v"(odd));  // keep the shifted dword: its bytes are then picked by the conversion's own byte select
+}
+// q / 16 of the code in the low nibble of byte I
+template <int I>
+__device__ __forceinline__ float nibble_to_f32_sixteenth(uint32_t x)
+{
+    if constexpr (I == 0) return __builtin_amdgcn_cvt_off_f32_i4((int)x);
+    return __builtin_amdgcn_cvt_off_f32_i4((int)((x >> (8 * I)) & 0xffu));
+}
+// The multiplier that goes with it: 16 x scale (exact; a scale of 2^124 or more would overflow here, one that small
+// that scale / 16 is not exact would lose bits in make_col_scale below: neither occurs in quantised weights).
+template <int BITS>
+__device__ __forceinline__ float make_col_scale_nibble(uint32_t scale_bf16_bits)
+{
+    const float s = bf16_bits_to_f32(scale_bf16_bits);
+    return BITS == 8 ? s : s * 16.0f;
 }
 
 // 16 bits holding four consecutive 4-bit codes (column j in nibble j) -> dword whose byte j reads as int8(16*q_j).

@@ -43,7 +43,7 @@ enum {
     BFAINTB_OK = 0,
     BFAINTB_ERR_NULL_POINTER = -1,  /* c, a, b or scale is NULL (with m,n,k all non-zero) */
     BFAINTB_ERR_BAD_SHAPE = -2,     /* n not a multiple of 16, k not a multiple of 64, or sizes overflow 2^31 */
-    BFAINTB_ERR_BAD_LD = -3,        /* lda < k, ldb < n, ldc < n, or a leading dimension that breaks 16-byte rows */
+    BFAINTB_ERR_BAD_LD = -3,        /* lda < k, ldb < n, ldb >= 2^27, ldc < n, or a leading dimension that breaks 16-byte rows */
     BFAINTB_ERR_ALIGNMENT = -4,     /* a pointer is not 16-byte aligned */
     BFAINTB_ERR_UNSUPPORTED = -5,   /* weight_bits not 8 or 4; group_size not 0 or a multiple of 32 dividing k */
     BFAINTB_ERR_WORKSPACE = -6,     /* workspace NULL/too small for this shape (see bfaintb_gemm_workspace_bytes) */
