@@ -40,15 +40,22 @@ REPLAYS = 5                   # timed measurements; the median one is reported
 MIN_LAUNCHES = 400            # launches inside one event pair (several replays of the K-launch graphs)
 
 # HBM bytes per launch RECORDED from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file's own --only commands
-# (KiB per dispatch, each scaled by what the same counter reads for a copy kernel of known size: fetch x 1.997,
-# write x 1.000); the files under profiles/ hold the runs.  Not measured by a plain run of this file: the output
-# names the source beside the figure.
+# (KiB per dispatch, each scaled by what the same counter reads for a 16 MiB device-to-device copy: fetch x 1.997,
+# write x 1.000); the files under profiles/ hold the runs and their commands.  Not measured by a plain run of this
+# file: the output names the source beside the figure.
 RECORDED_TRAFFIC = {
     # name: (bytes, source)
-    "decode_m1_n4096_k4096_int8_perchannel": (17398385, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
-    "prefill_m4096_n4096_k4096_int8_perchannel": (167893415, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
-    "decode_m1_n4096_k4096_int8_perchannel_prepacked": (16924658, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
-    "prefill_m4096_n4096_k4096_int8_perchannel_prepacked": (167921020, "profiles/bench_pmc_fetch_size.txt, profiles/bench_pmc_write_size.txt"),
+    "decode_m1_n4096_k4096_int8_perchannel": (17422124, "profiles/decode_m1_n4096_k4096_int8.txt"),
+    "decode_m1_n4096_k4096_int8_perchannel_prepacked": (16929572, "profiles/decode_m1_n4096_k4096_int8_prepacked.txt"),
+    "prefill_m4096_n4096_k4096_int8_perchannel": (169307846, "profiles/prefill_m4096_n4096_k4096_int8.txt"),
+    "decode_m1_n11008_k4096_int8_perchannel": (46267304, "profiles/decode_m1_n11008_k4096_int8.txt"),
+    "decode_m16_n11008_k4096_int8_perchannel": (49015179, "profiles/decode_m16_n11008_k4096_int8.txt"),
+    "decode_m32_n11008_k4096_int8_perchannel": (52631370, "profiles/decode_m32_n11008_k4096_int8.txt"),
+    "m1_n28672_k8192_int4_group128": (122577159, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
+    "m16_n28672_k8192_int4_group128": (130157043, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
+    "m2048_n28672_k8192_int4_group128": (896485920, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
+    "mid_m256_n4096_k4096_int8_perchannel": (35861389, "profiles/mid_m256_n4096_k4096_int8.txt"),
+    "mid_m1024_n4096_k4096_int8_perchannel": (92276733, "profiles/mid_m1024_n4096_k4096_int8.txt"),
 }
 
 C3_ROWS = (1, 16, 32)        # BASELINE config 3 (M in {1,4,8,16,32}): the rows the default line carries; --sweep has all five
