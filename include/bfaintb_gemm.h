@@ -42,7 +42,7 @@ extern "C" {
 enum {
     BFAINTB_OK = 0,
     BFAINTB_ERR_NULL_POINTER = -1,  /* c, a, b or scale is NULL (with m,n,k all non-zero) */
-    BFAINTB_ERR_BAD_SHAPE = -2,     /* n not a multiple of 16, k not a multiple of 64, or sizes overflow 2^31 */
+    BFAINTB_ERR_BAD_SHAPE = -2,     /* n not a multiple of 8 (16 for 4-bit codes), k not a multiple of 8, or sizes overflow 2^31 */
     BFAINTB_ERR_BAD_LD = -3,        /* lda < k, ldb < n, ldb >= 2^27, ldc < n, or a leading dimension that breaks 16-byte rows */
     BFAINTB_ERR_ALIGNMENT = -4,     /* a pointer is not 16-byte aligned */
     BFAINTB_ERR_UNSUPPORTED = -5,   /* weight_bits not 8 or 4; group_size not 0 or a multiple of 32 dividing k */
@@ -79,8 +79,10 @@ enum {
  *          (The reference stores fp32 scales, bfAintBGemm.cc:27; this build's contract is bf16,
  *          which makes q*scale exact in fp32 and the dequantised weight a single rounding.)
  *   c      bf16 [m, ldc].
- * Requirements: n % 16 == 0, k % 64 == 0, lda % 8 == 0, ldb % 16 == 0, ldc % 8 == 0, all four
- * pointers 16-byte aligned, |scale| finite and below 2^120.
+ * Requirements: n % 8 == 0 (n % 16 == 0 for 4-bit codes), k % 8 == 0 (the reference kernel needs n % 64 == 0 and
+ * k % 64 == 0, bf16gemm_kernel_gfx90a.s:341-343, :402-408), lda % 8 == 0, ldb % 16 == 0, ldb < 2^27, ldc % 8 == 0,
+ * all four pointers 16-byte aligned, |scale| finite and below 2^120.  Pre-packed weights (below) keep whole chunks:
+ * n % 16 == 0 and k % 64 == 0 (k % 128 == 0 for 4-bit codes).
  */
 
 /*

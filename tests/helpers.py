@@ -130,7 +130,7 @@ def ulp_violations(c_ref, c_bits, max_ulp=2.0, small_abs=1e-3, small_rel=1e-2):
 
 # what every assert_close_ulp call found, for the acceptance report (tests/conftest.py writes it out at the end of a GPU session)
 ACCEPTANCE_LOG = []
-NOISE_FACTOR = 8.0   # the escape below: this many times 2^-24 * sum_k |a_k w_k| on top of 2 ULP
+NOISE_FACTOR = 2.0   # the escape below: this many times 2^-24 * sum_k |a_k w_k| on top of 2 ULP (worst seen over the GPU suite: 0.61)
 NEAR_ZERO = 0.125    # ... and only for outputs below this fraction of rms(C)
 
 
