@@ -65,6 +65,9 @@ int check_shape(uint32_t m, uint32_t n, uint32_t k, int bits = 8)
     return BFAINTB_OK;
 }
 
+// tuning hook (bfaintb_debug_control): the only row-block size, in units of 16 rows, decode_plan_row_blocks may pick; 0 = free
+std::atomic<uint32_t> g_force_row_block{0};
+
 // Launch shape of the decode variant: columns and waves per workgroup, blocks of 16 rows of A per workgroup,
 // rows of k per workgroup, workgroups along k.
 struct DecodePlan {
@@ -97,13 +100,19 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
     const double col_blocks = (double)((n + pl.cols - 1u) / pl.cols);
     const double waves = row_blocks * col_blocks * pl.splits * pl.waves;
     const double busy = waves >= 1024.0 ? 1.0 : waves / 1024.0;
-    const double cycles_per_weight = 10.0 + 6.25 * pl.mb;
+    // 8-bit codes, refitted to a scan over row-block size x split factor at m = 40 .. 512 on 4096 x 4096, 11008 x 4096,
+    // 4096 x 11008 and 2048 x 8192 (the choice of row block then lands within 0.5 % of the best on all 27 points; the
+    // constants before it picked 16-row blocks where 32-row blocks with twice the splits run 6-24 % faster): larger row
+    // blocks cost a little less per weight than first fitted, every further row block re-streams half of B from beyond
+    // the caches, and the stream slows with idle CUs, not with idle wave slots.
+    const double cycles_per_weight = bits == 8 ? 10.0 + 5.0 * pl.mb : 10.0 + 6.25 * pl.mb;
     // workgroups beyond one per CU share a CU's arithmetic: the last, partly filled round costs a whole one
     // (measured at n = k = 4096, 64-row blocks: m = 512 -> 256 workgroups, 35 us; m = 640 -> 320 workgroups, 61 us)
     const double wgs = row_blocks * col_blocks * pl.splits;
     const double ragged = wgs > 256.0 ? (double)(uint64_t)((wgs + 255.0) / 256.0) * 256.0 / wgs : 1.0;
     const double compute = row_blocks * weights * cycles_per_weight / 65536.0 / 2000.0 / busy * ragged;
-    const double stream = weights * bits / 8.0 * (1.0 + 0.3 * (row_blocks - 1.0)) / 3.5e6 / busy;
+    const double stream_busy = bits == 8 ? (wgs >= 256.0 ? 1.0 : wgs / 256.0) : busy;
+    const double stream = weights * bits / 8.0 * (1.0 + (bits == 8 ? 0.5 : 0.3) * (row_blocks - 1.0)) / 3.5e6 / stream_busy;
     const double partial = pl.splits > 1 ? 3.0 + 12.0 * (pl.splits - 1.0) * m * n / 1.5e6 : 0.0;
     return 5.0 + (compute > stream ? compute : stream) + partial;
 }
@@ -152,7 +161,9 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
 {
     DecodePlan best{};
     double best_t = 0.0;
+    const uint32_t only_mb = g_force_row_block.load(std::memory_order_relaxed);
     for (uint32_t mb = bits == 8 ? max_mb : (max_mb < 2u ? max_mb : 2u); mb >= 1u; mb >>= 1) {
+        if (only_mb != 0u && mb != only_mb && only_mb <= (bits == 8 ? max_mb : 2u)) continue;
         DecodePlan c;
         c.cols = bits == 8 ? 128u : 256u;
         c.waves = ((bits == 8 && mb <= 2u) || (wide8 && mb == 1u)) ? 8u : 4u;  // wide8: 4-bit codes, 256 columns x 8 waves
@@ -488,6 +499,10 @@ int bfaintb_debug_control(uint32_t what, uint32_t value)
         case BFAINTB_DEBUG_WITHHOLD_PARTIALS:
             if (value) g_debug_flags.fetch_or(bfaintb::kDebugWithholdPartials);
             else g_debug_flags.fetch_and(~bfaintb::kDebugWithholdPartials);
+            return BFAINTB_OK;
+        case BFAINTB_DEBUG_FORCE_ROW_BLOCK:
+            if (value != 0u && value != 1u && value != 2u && value != 4u) return BFAINTB_ERR_UNSUPPORTED;
+            g_force_row_block.store(value);
             return BFAINTB_OK;
         default: return BFAINTB_ERR_UNSUPPORTED;
     }

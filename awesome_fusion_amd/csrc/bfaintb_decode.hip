@@ -218,7 +218,7 @@ __device__ __forceinline__ void apply_scales(float (&cs)[CPL], const uint4 (&sra
 }
 
 #ifdef BFAINTB_TRACE
-#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) p.trace[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
+#define TRACE_MARK(i) do { if ((threadIdx.x & 63) == 0) p.trace[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); } while (0)
 #else
 #define TRACE_MARK(i) do { } while (0)
 #endif

@@ -216,7 +216,7 @@ def gemm_static(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bi
     return rc
 
 
-DEBUG_SPLIT_WAIT_LIMIT, DEBUG_WITHHOLD_PARTIALS = 1, 2
+DEBUG_SPLIT_WAIT_LIMIT, DEBUG_WITHHOLD_PARTIALS, DEBUG_FORCE_ROW_BLOCK = 1, 2, 3
 ERR_WORKSPACE, ERR_NOT_INITIALISED, ERR_WORKSPACE_POISONED, ERR_STATIC_SCRATCH = -6, -8, -9, -10
 
 

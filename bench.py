@@ -58,13 +58,13 @@ RECORDED_TRAFFIC = {
     "mid_m1024_n4096_k4096_int8_perchannel": (92276733, "profiles/mid_m1024_n4096_k4096_int8.txt"),
 }
 
-# Parity counts RECORDED from the GPU test suite (tests/helpers.py: assert_close_ulp logs every check; the session writes
-# gpurun_out/acceptance_counts.json): per BASELINE config, outputs checked against the fp32 sequential-K oracle, how
+# Parity counts RECORDED from the GPU test suite (tests/helpers.py: assert_close_ulp logs every check; tests/conftest.py
+# writes them out as acceptance_counts.json when the session ends): per BASELINE config, outputs checked against the fp32 sequential-K oracle, how
 # many missed the bound (2 bf16 ULP, or 1e-2 relative below 1e-3) and were accepted as near-zero outputs within
 # 2 ULP + 2 * 2^-24 * sum|a w| of the fp64 sum, the worst accepted distance in ULP and the worst such excess in units
 # of 2^-24 * sum|a w|.  Not measured by a run of this file.
 RECORDED_ACCEPTANCE = {
-    "source": "tests (-m gpu) via tests/conftest.py -> gpurun_out/acceptance_counts.json; not measured by this run",
+    "source": "tests (-m gpu): tests/conftest.py writes acceptance_counts.json at session end; not measured by this run",
     "C1_m32_n64_k64": "bit-exact against the golden fixture: no tolerance",
     "C2_decode_m1_n4096_k4096": {"checks": 11, "outputs": 45056, "outside_bound": 0, "worst_ulp": 1.20, "worst_excess_units": 0.0},
     "C3_n11008_k4096_m1_4_8_16_32": {"checks": 5, "outputs": 671488, "outside_bound": 12, "worst_ulp": 1.81, "worst_excess_units": 0.08},

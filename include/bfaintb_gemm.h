@@ -217,9 +217,12 @@ BFAINTB_API size_t bfaintb_gemm_static_scratch_bytes(void);
  *   BFAINTB_DEBUG_WITHHOLD_PARTIALS  value != 0: the workgroups of all splits but the last compute and then keep their
  *                                    sums to themselves, so the reducer's wait runs out — the way to exercise the
  *                                    give-up path with every kernel exiting normally
+ *   BFAINTB_DEBUG_FORCE_ROW_BLOCK    value = 1, 2 or 4: beyond 32 rows of A the decode family runs blocks of 16 x value rows
+ *                                    whatever its estimates say (tuning; results do not depend on it); 0 restores the choice
  */
 #define BFAINTB_DEBUG_SPLIT_WAIT_LIMIT 1u
 #define BFAINTB_DEBUG_WITHHOLD_PARTIALS 2u
+#define BFAINTB_DEBUG_FORCE_ROW_BLOCK 3u
 BFAINTB_API int bfaintb_debug_control(uint32_t what, uint32_t value);
 
 /*
