@@ -25,6 +25,8 @@ hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k,
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
+hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, hipStream_t stream);
+bool prefill128_wreg_serves(const GemmParams& p);
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t decode_prepare_device();
 }  // namespace bfaintb
@@ -129,22 +131,23 @@ static bool prefill_small_tiles(uint32_t m, uint32_t n)
 static bool is_prefill(int v)
 {
     return v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256 || v == BFAINTB_VARIANT_PREFILL_128 ||
-           v == BFAINTB_VARIANT_PREFILL_256_LDS;
+           v == BFAINTB_VARIANT_PREFILL_256_LDS || v == BFAINTB_VARIANT_PREFILL_128_LDS;
 }
 
 // tile size of a tiled-variant launch: forced, or by shape
 static bool use_small_tiles(int v, uint32_t m, uint32_t n)
 {
-    return v == BFAINTB_VARIANT_PREFILL_128 || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n));
+    return v == BFAINTB_VARIANT_PREFILL_128 || v == BFAINTB_VARIANT_PREFILL_128_LDS || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n));
 }
 
 // Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
-// k.  Small tiles: a K-step takes 0.7 us on an empty machine and 0.9 us with a workgroup on every CU.
-static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k)
+// k.  Small tiles: a K-step takes 0.65 us on an empty machine and 0.70 us with a workgroup on every CU with row-major
+// weights (the kernel that keeps them in registers), 0.70 and 0.90 us with packed weights (both operands through LDS).
+static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, bool packed = false)
 {
     if (prefill_small_tiles(m, n)) {
         const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
-        return 4.0 + (k / 64.0) * (0.70 + 0.0008 * tiles);
+        return 4.0 + (k / 64.0) * (packed ? 0.70 + 0.0008 * tiles : 0.65 + 0.0002 * tiles);
     }
     const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
     const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
@@ -592,7 +595,11 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
 #ifdef BFAINTB_TRACE
         p.trace = static_cast<unsigned long long*>(workspace);  // per-quarter cycle totals, 8 words per wave
 #else
-        if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
+        if (use_small_tiles(v, m, n)) {
+            // row-major weights: the form that keeps them in registers, unless the other one is asked for by name
+            if (v != BFAINTB_VARIANT_PREFILL_128_LDS && bfaintb::prefill128_wreg_serves(p)) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, st);
+            return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
+        }
 #endif
         return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
@@ -759,7 +766,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (packed_uses_slab(m, n, k, bits)) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
-    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, true) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
@@ -978,8 +985,11 @@ const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_siz
     int v = variant;
     if (v == BFAINTB_VARIANT_AUTO) v = m <= kDecodeAutoMaxM ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     if (v == BFAINTB_VARIANT_DECODE) return "bfaintb_decode_kernel";
-    if (v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256) return "bfaintb_prefill_kernel";
-    if (v == BFAINTB_VARIANT_PREFILL_128) return "bfaintb_prefill128_kernel";
+    // (row-major weights, plain or bias epilogue; the forms with both operands in LDS serve the rest)
+    if (v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256) return "bfaintb_prefill_wreg_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL_256_LDS) return "bfaintb_prefill_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL_128) return "bfaintb_prefill128_wreg_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL_128_LDS) return "bfaintb_prefill128_kernel";
     (void)weight_bits;
     (void)group_size;
     return "";

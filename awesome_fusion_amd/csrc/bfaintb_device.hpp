@@ -207,4 +207,17 @@ __device__ __forceinline__ float make_col_scale(uint32_t scale_bf16_bits)
     return BITS == 8 ? s : s * 0.0625f;
 }
 
+// A workgroup barrier without the memory fence that __syncthreads() carries.  That fence makes the compiler wait, before
+// the barrier, for EVERY asynchronous global -> LDS copy issued so far — also the ones meant to land steps later — which
+// turns a pipeline of several stages into one of a single stage.  The caller states what must have completed with
+// explicit wait counts (its own part of the stage the others are about to read: s_waitcnt vmcnt; its LDS reads of the
+// stage about to be overwritten were consumed by matrix instructions it has already issued); the empty assembly
+// statements keep the compiler from moving memory operations across the barrier.
+__device__ __forceinline__ void barrier_no_fence()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 }  // namespace bfaintb

@@ -1,0 +1,448 @@
+// Tiled variant, 128x128 tiles, weights kept in registers: the form of the small-tile kernel for row-major B.
+//
+// Same job and the same reference kernel replaced as bfaintb_prefill128_kernel
+// (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:184-630; the reference's own tile is 32 x 64,
+// /root/reference/bfAintBGemm/bfAintBGemm.cc:105-109).  That kernel converts W into LDS and every wave reads both
+// operands back: a K-step takes 0.75 us whatever the load on the machine, three times its matrix-instruction time.
+// Here, as in bfaintb_prefill_wreg_kernel, only A goes through LDS:
+//   256 threads = 4 waves side by side along n; a wave owns ALL 128 rows x 32 columns of the tile = 8 x 2 accumulators
+//   of v_mfma_f32_16x16x32_bf16, converts exactly the weights it multiplies by, straight into the instruction's
+//   operand registers, and each weight of the tile is converted once.
+//   The vector-memory path takes about 20 cycles per instruction of a wave whatever it moves (measured: with the codes
+//   fetched by 16 two-byte loads per wave and step, 80 instructions per CU and step took 1600 cycles and the kernel was
+//   no faster than its predecessor; without them a step took 0.48 us instead of 0.80).  So the codes, too, come in by the
+//   asynchronous copy — 16 bytes per lane, 8 KiB (4 for 4-bit codes) per step in 2 (1) instructions per wave — into
+//   four LDS stages of their own, kept as stored (rows of the tile's 128 codes), and each lane picks its codes out of
+//   LDS: lane (c16 = lane % 16, kq = lane / 16) reads, per block of 32 k and for each of the 8 rows k0 + 8 kq + r, the
+//   codes of columns 2 c16, 2 c16 + 1 of the wave's 32 (one ds_read_u16; u8 for 4-bit codes): code j of those 8 reads
+//   is the 8-element operand of column 2 c16 + j, rows 8 kq .. 8 kq + 7.  The 16-byte chunks of a row are rotated by
+//   twice (once) the row's block of 8, so the four kq groups of a wave read from different banks.
+//   A: global -> LDS directly, four stages of 128 rows x 64 k (16 KiB each), same chunk swizzle as the other tiled
+//   kernels; the copies of step kt + 3 (A and codes) start at step kt, behind the step's one barrier (which also says
+//   every wave is done reading the stages they overwrite).  96 KiB of LDS in all.
+//   Per K-step a CU reads 64 KiB of A fragments and 8 KiB of codes from LDS and the copy engine writes 24.
+// Each of the step's 16 (block of 32 k, row block) pairs runs two matrix instructions and carries one sixteenth of
+// the conversion of the next step's weights (two weights: five instructions), so conversion and matrix work
+// alternate finely without hand-placed fences.
+// Accumulator (mt, j), register r of lane (c16, q = lane / 16): row 16 mt + 4 q + r, column 32 w + 2 c16 + j of the tile.
+// Epilogue: as bfaintb_prefill128_kernel — fp32 sums staged in LDS in [m][n] order, each thread finishes 8 neighbouring
+// columns of a row (bias, SiLU gate, residual, the one rounding) and stores them with one 16-byte write.
+#include <utility>
+#include "bfaintb_device.hpp"
+
+namespace bfaintb {
+
+namespace {
+constexpr uint32_t kTw = 128, kTwK = 64;
+constexpr uint32_t kTwStage = 128 * 128;  // bytes of one A stage
+constexpr uint32_t kTwCodeStage = 64 * 128;  // bytes of one stage of codes (8-bit; half of it used by 4-bit codes)
+
+__device__ __forceinline__ uint32_t tw_swz(uint32_t row, uint32_t chunk) { return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4); }
+}  // namespace
+
+template <int BITS, bool GROUPED>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) bfaintb_prefill128_wreg_kernel(const GemmParams p)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kTwStage];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kTwStage];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a2[kTwStage];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a3[kTwStage];
+    constexpr uint32_t kRowBytes = 128u * BITS / 8u;  // a tile row of codes
+    // (the codes of one K-step: 64 rows; the arrays keep the 8-bit extent for both code widths — an extent that depends
+    // on a template parameter, in an array the lambdas below capture, makes the host pass drop the kernel's launch
+    // stub without a diagnostic)
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_w0[kTwCodeStage];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_w1[kTwCodeStage];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_w2[kTwCodeStage];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_w3[kTwCodeStage];
+    auto w_tile = [&](auto stage_c) -> uint8_t* {
+        constexpr uint32_t St = decltype(stage_c)::value;
+        return St == 0 ? lds_w0 : St == 1 ? lds_w1 : St == 2 ? lds_w2 : lds_w3;
+    };
+    auto a_tile = [&](auto stage_c) -> uint8_t* {
+        constexpr uint32_t St = decltype(stage_c)::value;
+        return St == 0 ? lds_a0 : St == 1 ? lds_a1 : St == 2 ? lds_a2 : lds_a3;
+    };
+    using C0 = std::integral_constant<uint32_t, 0>;
+    using C1 = std::integral_constant<uint32_t, 1>;
+    using C2 = std::integral_constant<uint32_t, 2>;
+    using C3 = std::integral_constant<uint32_t, 3>;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..3: the wave's 32 columns
+    const uint32_t c16 = lane & 15u, kq = lane >> 4;
+
+    // ---- tile of this workgroup (the order of bfaintb_prefill128_kernel: the ids an XCD receives cover consecutive
+    //      logical ids, which walk groups of 8 tile-rows column by column)
+    const uint32_t tiles_m = (p.m + kTw - 1) / kTw, tiles_n = (p.n + kTw - 1) / kTw;
+    const uint32_t wgs = tiles_m * tiles_n;
+    const uint32_t per_xcd = (wgs + 7u) / 8u;
+    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= wgs) return;
+    const uint32_t group = logical / (8u * tiles_n);
+    const uint32_t first_m = group * 8u;
+    const uint32_t group_rows = tiles_m - first_m < 8u ? tiles_m - first_m : 8u;
+    const uint32_t in_group = logical - group * 8u * tiles_n;
+    const uint32_t tm = first_m + in_group % group_rows;
+    const uint32_t tn = in_group / group_rows;
+    const uint32_t m0 = tm * kTw, n0 = tn * kTw;
+
+    const uint32_t rows_valid = p.m - m0 < kTw ? p.m - m0 : kTw;
+    const uint32_t a_extent = ((rows_valid - 1u) * p.lda + p.k) * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)a_extent, kBufferFlags);
+    const uint32_t cols_valid = p.n - n0 < kTw ? p.n - n0 : kTw;
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
+        kBufferFlags);
+
+    const uint32_t ksteps = (p.k + kTwK - 1u) / kTwK;
+    const uint32_t last_chunks = (p.k - (ksteps - 1u) * kTwK) / 8u;  // valid 16-byte chunks per row of A in the last step
+    auto clamp = [&](uint32_t t) { return t < ksteps ? t : ksteps - 1u; };
+
+    // A copy: instruction j of wave w fills rows 32 w + 8 j .. + 7; lane l lands at row + l / 8, chunk position l % 8, so
+    // it fetches chunk (l % 8) ^ ((row >> 1) & 7) = (l % 8) ^ (l / 16) for even j and that ^ 4 for odd j; the row advance
+    // of j and the K advance sit in the scalar offset.  A chunk past the end of k (partial last step) is fetched from
+    // beyond the extent and reads as zero; rows of B past k read as zero codes, finite weights, and multiply those zeros.
+    const uint32_t a_row = 32u * wave + (lane >> 3);
+    const uint32_t chunk_e = (lane & 7u) ^ ((lane >> 4) & 7u), chunk_o = chunk_e ^ 4u;
+    const uint32_t a_voff_e = (a_row * p.lda + chunk_e * 8u) * 2u, a_voff_o = (a_row * p.lda + chunk_o * 8u) * 2u;
+    const uint32_t a_last_e = chunk_e < last_chunks ? a_voff_e : a_extent, a_last_o = chunk_o < last_chunks ? a_voff_o : a_extent;
+    auto dma_a = [&](auto stage_c, uint32_t kt) {
+        uint8_t* base = a_tile(stage_c) + wave * 4096u;
+        const bool last = kt + 1u == ksteps;
+        const uint32_t ve = last ? a_last_e : a_voff_e, vo = last ? a_last_o : a_voff_o;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
+                                                     (j & 1u) ? vo : ve, kt * kTwK * 2u + j * 16u * p.lda, 0, 0);
+    };
+
+    // W codes.  Copy: a 16-byte-per-lane instruction fills 1024 bytes = kRowsPerCopy rows of the stage; the step's 64
+    // rows take kCopies instructions, kCopiesPerWave for each wave.  Lane l lands at row l / kChunks of its block, chunk
+    // position l % kChunks, and fetches the chunk the rotation puts there: position = chunk + kRot * (row / 8 % 4).
+    constexpr uint32_t kChunks = kRowBytes / 16u;        // 8 or 4 chunks per row
+    constexpr uint32_t kRowsPerCopy = 1024u / kRowBytes; // 8 or 16
+    constexpr uint32_t kCopiesPerWave = 64u / kRowsPerCopy / 4u;  // 2 or 1
+    constexpr uint32_t kRot = BITS == 8 ? 2u : 1u;       // a wave's 16 lanes of one kq cover 32 (16) bytes of a row
+    uint32_t w_voff[2];  // (fixed extent: see the note on the arrays above)
+#pragma unroll
+    for (uint32_t j = 0; j < kCopiesPerWave; ++j) {
+        const uint32_t row = (kCopiesPerWave * wave + j) * kRowsPerCopy + lane / kChunks;  // within the step
+        const uint32_t chunk = ((lane % kChunks) - kRot * ((row >> 3) & 3u)) & (kChunks - 1u);
+        w_voff[j] = row * p.ldb_bytes + chunk * 16u;
+    }
+    auto dma_w = [&](auto stage_c, uint32_t kt) {
+        uint8_t* base = w_tile(stage_c) + kCopiesPerWave * wave * 1024u;
+#pragma unroll
+        for (uint32_t j = 0; j < kCopiesPerWave; ++j)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16, w_voff[j],
+                                                     kt * kTwK * p.ldb_bytes, 0, 0);
+    };
+    // Pick: this lane's 2 columns (byte offset wbyte of a row), rows 8 kq .. 8 kq + 7 of block blk of 32 k: row
+    // 32 blk + 8 kq + r, whose block of 8 is 4 blk + kq, rotation kRot * kq
+    const uint32_t wcol = 32u * wave + 2u * c16;  // within the tile
+    const uint32_t wbyte = wcol * BITS / 8u;
+    const uint32_t w_rd = (8u * kq) * kRowBytes + ((((wbyte >> 4) + kRot * kq) & (kChunks - 1u)) << 4) + (wbyte & 15u);  // + 32 blk rows + r rows
+    struct Raw {
+        uint32_t d[2][8];  // [block of 32 k][row]: two codes
+    };
+    auto pick = [&](Raw& raw, auto stage_c) {
+        const uint8_t* tile = w_tile(stage_c) + w_rd;
+#pragma unroll
+        for (uint32_t blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (uint32_t r = 0; r < 8; ++r) {
+                if constexpr (BITS == 8) raw.d[blk][r] = *reinterpret_cast<const uint16_t*>(tile + (32u * blk + r) * kRowBytes);
+                else raw.d[blk][r] = *(tile + (32u * blk + r) * kRowBytes);
+            }
+    };
+    // Scales go through a buffer resource so that the load is issued whatever the lane's column (the wait counts
+    // below count requests): columns past n read other columns' scales, or zero beyond the array; their results are
+    // never stored.
+    const uint32_t scale_rows = GROUPED ? p.k / p.group_size : 1u;
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.scale), 0, (int)(((scale_rows - 1u) * p.lds + p.n) * 2u), kBufferFlags);
+    const uint32_t s_voff = (n0 + wcol) * 2u;
+    auto group_scales = [&](uint32_t (&sr)[2], uint32_t kt) {
+#pragma unroll
+        for (uint32_t blk = 0; blk < 2; ++blk) {
+            uint32_t g = (kt * kTwK + 32u * blk) / p.group_size;
+            if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
+            sr[blk] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, g * p.lds * 2u, 0);
+        }
+    };
+    float cs[2] = {0.f, 0.f};  // one scale per column: fixed
+    if constexpr (!GROUPED) {
+        const uint32_t sr = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, 0, 0);
+        cs[0] = make_col_scale_nibble<BITS>(sr & 0xffffu);
+        cs[1] = make_col_scale_nibble<BITS>(sr >> 16);
+    }
+    struct Ops {
+        uint32_t w[2][2][4];  // [block of 32 k][column j][dword]: the 8-element operand as 4 packed pairs
+    };
+    // the two codes of a load, ready for the conversion: signed bytes (8-bit codes); two's-complement nibbles, the second
+    // shifted down to a low nibble (4-bit codes)
+    auto prepare = [&](uint32_t x, uint32_t& c0, uint32_t& c1) {
+        if constexpr (BITS == 8) {
+            c0 = x ^ 0x8080u;
+            c1 = c0;
+        } else {
+            c0 = x ^ 0x88u;
+            c1 = c0 >> 4;
+        }
+    };
+    auto value = [&](uint32_t c, uint32_t j) -> float {
+        if constexpr (BITS == 8) return j == 0 ? sbyte_to_f32<0>(c) : sbyte_to_f32<1>(c);
+        else return nibble_to_f32_sixteenth<0>(c);
+    };
+    // one sixteenth of a step's conversion: rows 2 pr, 2 pr + 1 of column j of block blk
+    auto convert_pair = [&](Ops& ops, const Raw& raw, uint32_t (&pre)[2][8][2], const float (&sc)[2][2], uint32_t blk, uint32_t j, uint32_t pr) {
+        if (j == 0) {
+            prepare(raw.d[blk][2 * pr], pre[blk][2 * pr][0], pre[blk][2 * pr][1]);
+            prepare(raw.d[blk][2 * pr + 1], pre[blk][2 * pr + 1][0], pre[blk][2 * pr + 1][1]);
+        }
+        ops.w[blk][j][pr] = pack_bf16_rne(value(pre[blk][2 * pr][j], j) * sc[blk][j], value(pre[blk][2 * pr + 1][j], j) * sc[blk][j]);
+    };
+    auto block_scales = [&](float (&sc)[2][2], const uint32_t (&sr)[2]) {
+#pragma unroll
+        for (uint32_t blk = 0; blk < 2; ++blk) {
+            if constexpr (GROUPED) {
+                sc[blk][0] = make_col_scale_nibble<BITS>(sr[blk] & 0xffffu);
+                sc[blk][1] = make_col_scale_nibble<BITS>(sr[blk] >> 16);
+            } else {
+                sc[blk][0] = cs[0];
+                sc[blk][1] = cs[1];
+            }
+        }
+    };
+    auto convert_all = [&](Ops& ops, const Raw& raw, const uint32_t (&sr)[2]) {
+        uint32_t pre[2][8][2];
+        float sc[2][2];
+        block_scales(sc, sr);
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u) convert_pair(ops, raw, pre, sc, u >> 3, (u >> 2) & 1u, u & 3u);
+    };
+
+    f32x4_t acc[8][2];
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[mt][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // fragment (mt, blk): row 16 mt + c16 of the tile, chunk 4 blk + kq (the swizzle repeats every 16 rows)
+    bf16x8_t af[4];  // the fragments of the next few units, carried from step to step
+    uint32_t a_rd[2];
+#pragma unroll
+    for (uint32_t blk = 0; blk < 2; ++blk) a_rd[blk] = tw_swz(c16, 4u * blk + kq);
+
+    // One K-step.  `cur`: the operands of this step; `nxt` receives those of step kt + 1, converted from the codes in stage
+    // S + 1; stage S holds this step's A; the copies of step kt + 3 go into stage S + 3 = S - 1, which every wave finished
+    // reading (A during step kt - 1, the codes during step kt - 2) before the barrier at the top.  `s1`: the group scales
+    // of step kt + 1 (requested one step ago), `s2` receives those of step kt + 2.
+    // With one wave per SIMD the wave issues in order and the matrix pipe idles whenever something else takes longer to
+    // issue than a matrix instruction runs, so the step is written as 32 fenced slots of one matrix instruction plus a
+    // few other instructions: unit u = (block of 32 k, row block) has two slots (the wave's two columns groups);
+    //   slot 0 of unit u: the A fragment of unit u + kAhead (the last kAhead units fetch the next step's first
+    //          fragments: its stage is complete, see the wait below); the two code reads that conversion pair u + 4 needs;
+    //          the first half of conversion pair u (two weights: sign flips, two conversions)
+    //   slot 1 of unit u: one memory request (units 0 .. 5: the copies; 6, 7: the group scales); the second half of
+    //          pair u (two multiplications, the rounding pack)
+    constexpr uint32_t kAhead = 4;
+    auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const uint32_t (&s1)[2], uint32_t (&s2)[2]) {
+        constexpr uint32_t S = decltype(stage_c)::value;
+        using Next = std::integral_constant<uint32_t, (S + 1u) & 3u>;
+        using Target = std::integral_constant<uint32_t, (S + 3u) & 3u>;
+        // At most the requests of the step before this one may still be in flight: then this wave's part of this step's
+        // AND the next step's A (requested three and two steps ago) and of the next step's codes (two steps ago) has
+        // landed.  Behind the barrier every wave's has.
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + kCopiesPerWave + (GROUPED ? 2 : 0)) : "memory");
+        barrier_no_fence();  // (a fenced barrier would also wait for the copies of the steps ahead)
+        const uint32_t kt3 = clamp(kt + 3), kt2 = clamp(kt + 2);
+        const bool last3 = kt3 + 1u == ksteps;
+        const uint32_t ve = last3 ? a_last_e : a_voff_e, vo = last3 ? a_last_o : a_voff_o;
+        uint8_t* const a_dst = a_tile(Target{}) + wave * 4096u;
+        uint8_t* const w_dst = w_tile(Target{}) + kCopiesPerWave * wave * 1024u;
+        const uint8_t* const a_src = a_tile(stage_c);
+        const uint8_t* const a_nxt = a_tile(Next{});
+        const uint8_t* const w_src = w_tile(Next{}) + w_rd;
+        uint32_t code[2][8];   // the codes of step kt + 1 as read: [block][row], two codes each
+        uint32_t pre[2][8][2];
+        float sc[2][2];
+        float f0 = 0.f, f1 = 0.f;
+        block_scales(sc, s1);
+        // pair v = (block v / 8, rows 2 (v / 2 % 4), + 1, column v % 2): its two rows are read by the pair with column 0
+        auto read_codes = [&](uint32_t v) {
+            const uint32_t blk = v >> 3, pr = (v >> 1) & 3u;
+#pragma unroll
+            for (uint32_t h = 0; h < 2; ++h) {
+                const uint32_t r = 2u * pr + h;
+                if constexpr (BITS == 8) code[blk][r] = *reinterpret_cast<const uint16_t*>(w_src + (32u * blk + r) * kRowBytes);
+                else code[blk][r] = *(w_src + (32u * blk + r) * kRowBytes);
+            }
+        };
+        read_codes(0);
+        read_codes(2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u) {
+            const uint32_t blk = u >> 3, mt = u & 7u;
+            const uint32_t cblk = u >> 3, cpr = (u >> 1) & 3u, cj = u & 1u;  // conversion pair u
+            const bf16x8_t a_now = af[u % kAhead];
+            const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][0][0], cur.w[blk][0][1], cur.w[blk][0][2], cur.w[blk][0][3]));
+            const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][1][0], cur.w[blk][1][1], cur.w[blk][1][2], cur.w[blk][1][3]));
+            // ---- slot 0
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_now, wf0, acc[mt][0], 0, 0, 0);
+            if (u + kAhead < 16) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
+            else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - 16u) * 2048u);
+            if (cj == 0 && u + 4 < 16) read_codes(u + 4);
+            if (cj == 0) {
+                prepare(code[cblk][2 * cpr], pre[cblk][2 * cpr][0], pre[cblk][2 * cpr][1]);
+                prepare(code[cblk][2 * cpr + 1], pre[cblk][2 * cpr + 1][0], pre[cblk][2 * cpr + 1][1]);
+            }
+            f0 = value(pre[cblk][2 * cpr][cj], cj);
+            f1 = value(pre[cblk][2 * cpr + 1][cj], cj);
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- slot 1
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_now, wf1, acc[mt][1], 0, 0, 0);
+            if (u < 4) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + u * 1024u), 16, (u & 1u) ? vo : ve,
+                                                         kt3 * kTwK * 2u + u * 16u * p.lda, 0, 0);
+            } else if (u < 4 + kCopiesPerWave) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + (u - 4u) * 1024u), 16, w_voff[u - 4u],
+                                                         kt3 * kTwK * p.ldb_bytes, 0, 0);
+            } else if (GROUPED && u == 6) {
+                group_scales(s2, kt2);
+            }
+            nxt.w[cblk][cj][cpr] = pack_bf16_rne(f0 * sc[cblk][cj], f1 * sc[cblk][cj]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // ---- prologue: A tiles and codes of steps 0, 1, 2 -> stages 0, 1, 2; operands of step 0
+    Ops ops0, ops1;
+    uint32_t sa[2] = {0u, 0u}, sb[2] = {0u, 0u};  // group scales, alternating: sb = step 0 (then 2, ...), sa = step 1 (then 3, ...)
+    dma_w(C0{}, 0);
+    dma_a(C0{}, 0);
+    dma_w(C1{}, clamp(1));
+    dma_a(C1{}, clamp(1));
+    dma_w(C2{}, clamp(2));
+    dma_a(C2{}, clamp(2));
+    if constexpr (GROUPED) {
+        group_scales(sb, 0);
+        group_scales(sa, clamp(1));
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    barrier_no_fence();
+    {
+        Raw raw;
+        pick(raw, C0{});
+        convert_all(ops0, raw, sb);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kAhead; ++u) af[u] = *reinterpret_cast<const bf16x8_t*>(a_tile(C0{}) + a_rd[0] + u * 2048u);
+
+    uint32_t kt = 0;
+    for (; kt + 3 < ksteps; kt += 4) {
+        step(C0{}, kt, ops0, ops1, sa, sb);
+        step(C1{}, kt + 1, ops1, ops0, sb, sa);
+        step(C2{}, kt + 2, ops0, ops1, sa, sb);
+        step(C3{}, kt + 3, ops1, ops0, sb, sa);
+    }
+    if (kt < ksteps) step(C0{}, kt, ops0, ops1, sa, sb);
+    if (kt + 1 < ksteps) step(C1{}, kt + 1, ops1, ops0, sb, sa);
+    if (kt + 2 < ksteps) step(C2{}, kt + 2, ops0, ops1, sa, sb);
+
+    // ---- epilogue: fp32 sums -> LDS in [m][n] order (rows 32 q .. 32 q + 31 in the q-th array), then finish row-wise
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
+    __syncthreads();                                   // ... and every wave is done reading the stages
+    auto c_rows = [&](uint32_t q) -> float* {
+        return reinterpret_cast<float*>(q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_a2 : lds_a3);
+    };
+#pragma unroll
+    for (uint32_t mt = 0; mt < 8; ++mt) {
+        float* base = c_rows(mt >> 1);
+#pragma unroll
+        for (uint32_t r = 0; r < 4; ++r) {
+            const uint32_t row = 16u * (mt & 1u) + 4u * kq + r;  // within the 32 rows of this array
+            *reinterpret_cast<float2*>(base + row * kTw + wcol) = make_float2(acc[mt][0][r], acc[mt][1][r]);
+        }
+    }
+    __syncthreads();
+    const bool gated = p.activation == kActSiluGate;
+    const uint32_t ch = tid & 15u;  // 8 columns: 8 ch .. 8 ch + 7 of the tile
+    const uint32_t gn = n0 + 8u * ch;
+    float bias[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bias[i] = 0.f;
+    if (p.bias != nullptr && gn < p.n) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p.bias + gn);
+        const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bias[2 * i] = bf16_bits_to_f32(d[i] & 0xffffu);
+            bias[2 * i + 1] = bf16_bits_to_f32(d[i] >> 16);
+        }
+    }
+    const bool plain = p.bias == nullptr && p.residual == nullptr && !gated;  // the bare sums keep a -0 as it is
+#pragma unroll
+    for (uint32_t pass = 0; pass < 8; ++pass) {
+        const uint32_t row = 16u * pass + (tid >> 4);
+        const uint32_t gm = m0 + row;
+        if (gm >= p.m || gn >= p.n) continue;
+        const float* src = c_rows(row >> 5) + (row & 31u) * kTw + 8u * ch;
+        const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+        float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if (!plain) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += bias[i];
+        }
+        if (gated) {
+            float o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] = silu_gate(v[2 * i], v[2 * i + 1]);
+            if (p.residual != nullptr) {
+                const uint2 r = *reinterpret_cast<const uint2*>(p.residual + (size_t)gm * p.ldr + gn / 2u);
+                o[0] += bf16_bits_to_f32(r.x & 0xffffu);
+                o[1] += bf16_bits_to_f32(r.x >> 16);
+                o[2] += bf16_bits_to_f32(r.y & 0xffffu);
+                o[3] += bf16_bits_to_f32(r.y >> 16);
+            }
+            *reinterpret_cast<uint2*>(p.c + (size_t)gm * p.ldc + gn / 2u) = make_uint2(pack_bf16_rne(o[0], o[1]), pack_bf16_rne(o[2], o[3]));
+        } else {
+            if (p.residual != nullptr) {
+                const uint4 r = *reinterpret_cast<const uint4*>(p.residual + (size_t)gm * p.ldr + gn);
+                const uint32_t d[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    v[2 * i] += bf16_bits_to_f32(d[i] & 0xffffu);
+                    v[2 * i + 1] += bf16_bits_to_f32(d[i] >> 16);
+                }
+            }
+            *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) =
+                make_uint4(pack_bf16_rne(v[0], v[1]), pack_bf16_rne(v[2], v[3]), pack_bf16_rne(v[4], v[5]), pack_bf16_rne(v[6], v[7]));
+        }
+    }
+}
+
+template <int BITS, bool GROUPED>
+static hipError_t launch_prefill128_wreg_t(const GemmParams& p, hipStream_t stream)
+{
+    const uint32_t tiles = ((p.m + kTw - 1) / kTw) * ((p.n + kTw - 1) / kTw);
+    const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
+    void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED>;
+    return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
+}
+
+// Whether this kernel can serve a launch: row-major weights (the caller's business), this library's own arithmetic.
+bool prefill128_wreg_serves(const GemmParams& p) { return !p.reference_arith; }
+
+hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, hipStream_t stream)
+{
+    const bool grouped = p.group_size != 0;
+    if (bits == 8) return grouped ? launch_prefill128_wreg_t<8, true>(p, stream) : launch_prefill128_wreg_t<8, false>(p, stream);
+    return grouped ? launch_prefill128_wreg_t<4, true>(p, stream) : launch_prefill128_wreg_t<4, false>(p, stream);
+}
+
+}  // namespace bfaintb

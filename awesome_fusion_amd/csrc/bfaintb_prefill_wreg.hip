@@ -306,7 +306,7 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                 // copy this step started (into the stage read two steps ago) overwrites nothing a wave still reads — every
                 // wave that reaches this barrier has passed the previous one, i.e. finished the step before it.
                 asm volatile("s_waitcnt vmcnt(%0)" ::"n"((GROUPED ? 18 : 16) + 16) : "memory");
-                __syncthreads();
+                barrier_no_fence();  // (a fenced barrier would also wait for the copy this step has just started)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }

@@ -14,6 +14,7 @@ _LIB = os.path.join(_HERE, "libbfaintb_gemm.so")
 AUTO, DECODE, PREFILL = 0, 1, 2
 PREFILL_256, PREFILL_128 = 3, 4  # the tiled variant with its tile size forced (tests, tuning)
 PREFILL_256_LDS = 5               # ... and its form with both operands in LDS forced
+PREFILL_128_LDS = 6               # the same for the 128-tile kernel
 ACT_NONE, ACT_SILU_GATE = 0, 1
 
 

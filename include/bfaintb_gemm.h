@@ -61,9 +61,12 @@ enum {
                                   * holds at most 256 of those (the large tiles would leave most CUs idle) */
     BFAINTB_VARIANT_PREFILL_256 = 3, /* the tiled kernel with 256x256 tiles, whatever the shape (tests, tuning) */
     BFAINTB_VARIANT_PREFILL_128 = 4, /* the tiled kernel with 128x128 tiles, whatever the shape (tests, tuning) */
-    BFAINTB_VARIANT_PREFILL_256_LDS = 5 /* 256x256 tiles with both operands staged in LDS — the form pre-packed weights,
+    BFAINTB_VARIANT_PREFILL_256_LDS = 5, /* 256x256 tiles with both operands staged in LDS — the form pre-packed weights,
                                           * residuals and the gate epilogue use; row-major weights otherwise run the form
                                           * that keeps the weights in registers (tests, tuning) */
+    BFAINTB_VARIANT_PREFILL_128_LDS = 6  /* 128x128 tiles with both operands staged in LDS — the form pre-packed weights
+                                          * use; row-major weights otherwise run the form that keeps the weights in
+                                          * registers (tests, tuning) */
 };
 
 /*

@@ -57,8 +57,10 @@ def test_variant_choice_and_split():
     assert af.prefill_tile(1024, 4096) == 128 and af.prefill_tile(1025, 4096) == 256
     assert af.prefill_tile(128, 28672) == 128 and af.prefill_tile(4096, 4096) == 256 and af.prefill_tile(1, 16) == 128
     assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128) == 0 == af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_256)
-    assert af.kernel_name(64, which=af.PREFILL_128) == "bfaintb_prefill128_kernel"
-    assert af.kernel_name(64, which=af.PREFILL_256) == af.kernel_name(64, which=af.PREFILL) == "bfaintb_prefill_kernel"
+    assert af.kernel_name(64, which=af.PREFILL_128) == "bfaintb_prefill128_wreg_kernel"
+    assert af.kernel_name(64, which=af.PREFILL_128_LDS) == "bfaintb_prefill128_kernel"
+    assert af.kernel_name(64, which=af.PREFILL_256) == af.kernel_name(64, which=af.PREFILL) == "bfaintb_prefill_wreg_kernel"
+    assert af.kernel_name(64, which=af.PREFILL_256_LDS) == "bfaintb_prefill_kernel"
     assert af.split_k(4096, 4096, 4096) == 1
     s = af.split_k(1, 4096, 4096)
     assert 1 < s <= 64 and 4096 % s == 0
@@ -66,7 +68,7 @@ def test_variant_choice_and_split():
     assert af.workspace_bytes(1, 4096, 4096) == 256 + (s - 1) * 1 * 4096 * 4   # the header, then one fp32 word per (split but the last, row, column)
     assert af.workspace_bytes(4096, 4096, 4096) == 0
     assert af.workspace_bytes(8, 4096, 4096, force_split_k=1) == 0
-    assert af.kernel_name(1) == "bfaintb_decode_kernel" and af.kernel_name(4096) == "bfaintb_prefill_kernel"
+    assert af.kernel_name(1) == "bfaintb_decode_kernel" and af.kernel_name(4096) == "bfaintb_prefill_wreg_kernel"
 
 
 def rc(**kw):

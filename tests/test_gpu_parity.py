@@ -167,6 +167,18 @@ def test_tile_sizes_agree_bit_for_bit(af, m, n, k, bits, group):
     assert np.array_equal(run_gemm(p, which=af.PREFILL_128), run_gemm(p, which=af.PREFILL_256))
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [(130, 272, 72, 8, 0), (700, 1008, 1000, 8, 0), (300, 528, 512, 8, 64), (1000, 1008, 384, 4, 0),
+                                              (130, 4112, 256, 4, 128), (1024, 4096, 1088, 8, 0), (257, 272, 8, 4, 0)])
+def test_small_tile_forms_agree_bit_for_bit(af, m, n, k, bits, group):
+    """The 128x128-tile kernel that keeps the weights in registers (row-major weights: what PREFILL_128 runs) against the
+    one that stages both operands in LDS: same products, same order of addition, so the same bits — partial tiles in m
+    and n, K-steps that are not whole, one to seventeen steps, both code widths, grouped scales."""
+    p = Problem(m, n, k, bits, group, seed=m + 2 * n + k)
+    c = run_gemm(p, which=af.PREFILL_128)
+    assert_close_ulp(p, c, f"128-tile, weights in registers: {m}x{n}x{k} bits={bits} g={group}")
+    assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128_LDS))
+
+
 def test_tiled_variant_picks_its_tile_size_by_shape(af):
     """PREFILL runs 128x128 tiles while m x n holds at most 256 of them, 256x256 tiles beyond; either way the result
     meets the oracle and is the forced form's, bit for bit."""
