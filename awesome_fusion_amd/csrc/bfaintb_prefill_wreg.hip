@@ -20,7 +20,8 @@
 //   4 columns), A fragments fetched one group of 16 ahead — the last group fetches the next step's first fragments, so no
 //   step starts by waiting for LDS; one barrier, in the middle of the step.
 // Accumulator (mt, j), register r of lane (c16, q = lane / 16): row 16 mt + 4 q + r, column 64 w + 4 c16 + j of the tile.
-// Epilogue: bias, rounding to bf16, staging through LDS in [m][n] order, 16-byte row-contiguous stores.
+// Epilogue: bias, rounding to bf16, staging through LDS in [m][n] order, 16-byte row-contiguous stores; with a residual or
+// the SiLU gate the fp32 sums are staged instead, 128 rows at a time, and finished 8 columns per thread.
 #include <utility>
 #include "bfaintb_device.hpp"
 
@@ -349,7 +350,9 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
     __syncthreads();
     auto c_rows = [&](uint32_t q) -> uint8_t* { return q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_a2 : lds_a3; };
-    {
+    const bool gated = p.activation == kActSiluGate;
+    if (p.residual == nullptr && !gated) {
+        // the bare sums, or sums + bias: rounded in registers, staged as bf16 (rows 64 q .. 64 q + 63 in the q-th array)
         float bias[4] = {0.f, 0.f, 0.f, 0.f};
         const bool has_bias = p.bias != nullptr;
         if (has_bias && w_ok) {
@@ -377,17 +380,84 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                 *reinterpret_cast<uint2*>(base + row * kWrCRowBytes + wcol * 2u) = o;
             }
         }
-    }
-    __syncthreads();
+        __syncthreads();
 #pragma unroll 4
-    for (uint32_t pass = 0; pass < 32u; ++pass) {
-        const uint32_t row = pass * 8u + (tid >> 5);
-        const uint32_t ch = tid & 31u;
-        const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
-        if (gm < p.m && gn < p.n) {
-            const uint4 v = *reinterpret_cast<const uint4*>(c_rows(row >> 6) + (row & 63u) * kWrCRowBytes + ch * 16u);
-            *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) = v;
+        for (uint32_t pass = 0; pass < 32u; ++pass) {
+            const uint32_t row = pass * 8u + (tid >> 5);
+            const uint32_t ch = tid & 31u;
+            const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
+            if (gm < p.m && gn < p.n) {
+                const uint4 v = *reinterpret_cast<const uint4*>(c_rows(row >> 6) + (row & 63u) * kWrCRowBytes + ch * 16u);
+                *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) = v;
+            }
         }
+        return;
+    }
+    // Residual and / or the SiLU gate: the fp32 sums are staged in [m][n] order, 128 rows at a time (128 x 256 x 4 bytes
+    // = the four arrays, rows 32 q .. 32 q + 31 of the half in the q-th), and each thread finishes 8 neighbouring columns
+    // of a row — bias, gate, residual, the one rounding — as the small-tile kernels do.
+    const uint32_t ch = tid & 31u;  // 8 columns: 8 ch .. 8 ch + 7 of the tile
+    const uint32_t gn = n0 + 8u * ch;
+    float bias8[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bias8[i] = 0.f;
+    if (p.bias != nullptr && gn < p.n) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(p.bias + gn);
+        const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bias8[2 * i] = bf16_bits_to_f32(d[i] & 0xffffu);
+            bias8[2 * i + 1] = bf16_bits_to_f32(d[i] >> 16);
+        }
+    }
+#pragma unroll
+    for (uint32_t half = 0; half < 2; ++half) {
+#pragma unroll
+        for (uint32_t mh = 0; mh < 8; ++mh) {
+            const uint32_t mt = 8u * half + mh;
+            float* base = reinterpret_cast<float*>(c_rows(mh >> 1));
+#pragma unroll
+            for (uint32_t r = 0; r < 4; ++r) {
+                const uint32_t row = 16u * (mh & 1u) + 4u * kq + r;  // within the 32 rows of this array
+                *reinterpret_cast<float4*>(base + row * kWrTile + wcol) = make_float4(acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]);
+            }
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (uint32_t pass = 0; pass < 16u; ++pass) {
+            const uint32_t row = pass * 8u + (tid >> 5);  // within the half
+            const uint32_t gm = m0 + 128u * half + row;
+            if (gm >= p.m || gn >= p.n) continue;
+            const float* src = reinterpret_cast<const float*>(c_rows(row >> 5)) + (row & 31u) * kWrTile + 8u * ch;
+            const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+            float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += bias8[i];
+            if (gated) {
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = silu_gate(v[2 * i], v[2 * i + 1]);
+                if (p.residual != nullptr) {
+                    const uint2 r = *reinterpret_cast<const uint2*>(p.residual + (size_t)gm * p.ldr + gn / 2u);
+                    o[0] += bf16_bits_to_f32(r.x & 0xffffu);
+                    o[1] += bf16_bits_to_f32(r.x >> 16);
+                    o[2] += bf16_bits_to_f32(r.y & 0xffffu);
+                    o[3] += bf16_bits_to_f32(r.y >> 16);
+                }
+                *reinterpret_cast<uint2*>(p.c + (size_t)gm * p.ldc + gn / 2u) = make_uint2(pack_bf16_rne(o[0], o[1]), pack_bf16_rne(o[2], o[3]));
+            } else {
+                const uint4 r = *reinterpret_cast<const uint4*>(p.residual + (size_t)gm * p.ldr + gn);
+                const uint32_t d[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    v[2 * i] += bf16_bits_to_f32(d[i] & 0xffffu);
+                    v[2 * i + 1] += bf16_bits_to_f32(d[i] >> 16);
+                }
+                *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) =
+                    make_uint4(pack_bf16_rne(v[0], v[1]), pack_bf16_rne(v[2], v[3]), pack_bf16_rne(v[4], v[5]), pack_bf16_rne(v[6], v[7]));
+            }
+        }
+        __syncthreads();  // the second half overwrites the staging area
     }
 }
 
@@ -400,11 +470,8 @@ static hipError_t launch_wreg_t(const GemmParams& p, hipStream_t stream)
     return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
 }
 
-// Whether this kernel can serve a launch: row-major weights, this library's arithmetic, no residual or gate.
-bool prefill_wreg_serves(const GemmParams& p)
-{
-    return !p.reference_arith && p.residual == nullptr && p.activation == kActNone;
-}
+// Whether this kernel can serve a launch: row-major weights (the caller's business), this library's own arithmetic.
+bool prefill_wreg_serves(const GemmParams& p) { return !p.reference_arith; }
 
 hipError_t launch_prefill_wreg(const GemmParams& p, int bits, hipStream_t stream)
 {
