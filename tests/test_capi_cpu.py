@@ -99,6 +99,7 @@ def test_rejects_bad_arguments_without_launching():
     assert rc(lda=128) == -3                  # lda < k
     assert rc(ldb=64) == -3
     assert rc(ldc=64) == -3
+    assert rc(ldb=1 << 27) == -3              # a lane's offset within 32 rows of B is kept in 32 bits
     assert rc(lda=260) == -3                  # rows of A would lose 16-byte alignment
     assert rc(a=None) == -1
     assert rc(c=0) == -1
@@ -134,6 +135,9 @@ def test_rejects_bad_arguments_without_launching():
     assert af.dequant(P, P, None, 128, 256, stream=0, check=False) == -1
     assert L.bfaintb_workspace_init(P, 66, None) == -6   # not a whole number of words
     assert L.bfaintb_workspace_init(None, 0, None) == 0
+    # tuning and test hooks: values outside their ranges are refused, valid ones change no result (GPU tests)
+    assert L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 3) == -5 and L.bfaintb_debug_control(99, 0) == -5
+    assert L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 2) == 0 and L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 0) == 0
 
 
 def test_prepacked_entry_points_validate_before_launching():

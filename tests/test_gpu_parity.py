@@ -190,6 +190,20 @@ def test_tiled_variant_picks_its_tile_size_by_shape(af):
         assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128 if tile == 128 else af.PREFILL_256)), f"{m}x{n}"
 
 
+def test_forced_row_block_changes_the_plan_not_the_contract(af):
+    """The tuning hook that pins the decode family's row-block size: every size meets the oracle, and the hook's 0 restores
+    the library's own choice (same bits as before)."""
+    p = Problem(100, 1040, 512, 8, 0, seed=11)
+    own = run_gemm(p, which=af.DECODE)
+    try:
+        for mb in (1, 2, 4):
+            af.debug_control(af.DEBUG_FORCE_ROW_BLOCK, mb)
+            assert_close_ulp(p, run_gemm(p, which=af.DECODE), f"row blocks of {16 * mb}")
+    finally:
+        af.debug_control(af.DEBUG_FORCE_ROW_BLOCK, 0)
+    assert np.array_equal(own, run_gemm(p, which=af.DECODE))
+
+
 @pytest.mark.parametrize("m", [5, 80])
 def test_leading_dimensions_and_untouched_padding(af, m):
     import torch
