@@ -34,7 +34,7 @@ hipError_t decode_prepare_device();
 // Split-K scratch of bfaintb_gemm_static: one array per GPU the library runs on, held until the process ends.  In host
 // code this name is only a handle for hipGetSymbolAddress; device_state() resolves it once per device and everything
 // else uses the resolved pointer.
-#define BFAINTB_STATIC_SCRATCH_BYTES (8u << 20)
+#define BFAINTB_STATIC_SCRATCH_BYTES (16u << 20)
 static __device__ __align__(256) unsigned char scratch[BFAINTB_STATIC_SCRATCH_BYTES];
 
 namespace {
@@ -143,11 +143,61 @@ static bool use_small_tiles(int v, uint32_t m, uint32_t n)
 // Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
 // k.  Small tiles: a K-step takes 0.65 us on an empty machine and 0.70 us with a workgroup on every CU with row-major
 // weights (the kernel that keeps them in registers), 0.70 and 0.90 us with packed weights (both operands through LDS).
+// The small-tile kernel over row-major weights may split k: grid y walks the splits, each workgroup runs its share of
+// the K-steps and the workgroup of the last split adds the others' sums (same workspace and protocol as the decode
+// family).  Worth it while tiles x splits still fit one workgroup per CU.
+struct TilePlan {
+    uint32_t k_per_wg, splits;
+    double us;
+};
+constexpr uint32_t kMaxTileSplits = 16;
+
+static size_t split_workspace_bytes(uint32_t splits, uint32_t m, uint32_t n)
+{
+    if (splits <= 1) return 0;
+    // the header, then one fp32 word per (split but the last, row, column), rounded up to 256 bytes
+    return bfaintb::kWorkspaceHeaderBytes + ((((size_t)(splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u);
+}
+
+static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, uint32_t forced_splits)
+{
+    const uint32_t ksteps = (k + 63u) / 64u;
+    const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
+    auto shape = [&](uint32_t want) {
+        TilePlan t;
+        if (want > kMaxTileSplits) want = kMaxTileSplits;
+        if (want < 1u) want = 1u;
+        const uint32_t per = (ksteps + want - 1u) / want;
+        t.k_per_wg = per * 64u;
+        t.splits = (ksteps + per - 1u) / per;
+        // the hand-over: the producers' device-scope stores have to arrive (some 6 us after the last K-step), then the
+        // reducing workgroup fetches a tile's worth of sums per split through its one CU, slower the more CUs do so at once
+        // (8-bit, n = k = 4096, us with 1 / 2 / 3 / 4 splits: m = 128: 43.4 / 32.7 / 26.2 / 28.3; m = 256: 43.9 / 34.0 /
+        // 27.2 / 31.1; m = 512: 44.3 / 36.4 / 44.1 / 42.3; 8192 x 8192, m = 256: 83.2 / 55.8 / 69.9 / 62.5)
+        const double hand_over = t.splits > 1u ? 4.5 + (t.splits - 1.0) * (2.0 + 0.04 * tiles) : 0.0;
+        t.us = 4.0 + per * (0.65 + 0.0002 * tiles * t.splits) + hand_over;
+        return t;
+    };
+    if (forced_splits) return shape(forced_splits);
+    TilePlan best = shape(1);
+    static const uint32_t kCandidates[] = {2, 3, 4, 6, 8};
+    for (uint32_t s : kCandidates) {
+        if (tiles * s > 256.0) break;
+        const TilePlan t = shape(s);
+        if (t.splits != s) continue;  // k does not divide that way
+        // (at most 256 tiles' worth of sums in all, 14 MiB: within the 32-bit offsets of the kernel and within the scratch of
+        // the entry point that brings its own)
+        if (t.us < best.us) best = t;
+    }
+    return best;
+}
+
 static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, bool packed = false)
 {
     if (prefill_small_tiles(m, n)) {
         const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
-        return 4.0 + (k / 64.0) * (packed ? 0.70 + 0.0008 * tiles : 0.65 + 0.0002 * tiles);
+        if (!packed) return tile128_plan(m, n, k, 0).us;
+        return 4.0 + (k / 64.0) * (0.70 + 0.0008 * tiles);
     }
     const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
     const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
@@ -319,13 +369,15 @@ int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
     return BFAINTB_ERR_BAD_VARIANT;
 }
 
+// whether a tiled-variant launch over row-major weights goes to the small-tile kernel that can split k
+static bool tiled_may_split(int v, uint32_t m, uint32_t n) { return use_small_tiles(v, m, n) && v != BFAINTB_VARIANT_PREFILL_128_LDS; }
+
 size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant, uint32_t forced_split)
 {
-    if (variant != BFAINTB_VARIANT_DECODE || m == 0 || n == 0) return 0;
-    const DecodePlan pl = decode_plan(m, n, k, bits, forced_split);
-    if (pl.splits <= 1) return 0;
-    // the header, then one fp32 word per (split but the last, row, column), rounded up to 256 bytes
-    return bfaintb::kWorkspaceHeaderBytes + ((((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u);
+    if (m == 0 || n == 0) return 0;
+    if (variant == BFAINTB_VARIANT_DECODE) return split_workspace_bytes(decode_plan(m, n, k, bits, forced_split).splits, m, n);
+    if (is_prefill(variant) && tiled_may_split(variant, m, n)) return split_workspace_bytes(tile128_plan(m, n, k, forced_split).splits, m, n);
+    return 0;
 }
 
 inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
@@ -428,7 +480,7 @@ const char* bfaintb_error_string(int code)
         case BFAINTB_ERR_BAD_VARIANT: return "unknown kernel variant, or variant cannot run this shape";
         case BFAINTB_ERR_NOT_INITIALISED: return "first call on this device made under stream capture: call bfaintb_init() beforehand";
         case BFAINTB_ERR_WORKSPACE_POISONED: return "a split-K wait gave up on this workspace (results of that call hold NaNs): initialise it again";
-        case BFAINTB_ERR_STATIC_SCRATCH: return "shape needs more split-K scratch than bfaintb_gemm_static holds (8 MiB): use bfaintb_gemm with a workspace";
+        case BFAINTB_ERR_STATIC_SCRATCH: return "shape needs more split-K scratch than bfaintb_gemm_static holds (16 MiB): use bfaintb_gemm with a workspace";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -446,8 +498,10 @@ int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, ui
 
 uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
 {
-    if (bfaintb_gemm_variant(m, n, k, weight_bits, group_size) != BFAINTB_VARIANT_DECODE) return 1;
-    return decode_plan(m, n, k, weight_bits, 0).splits;
+    const int v = bfaintb_gemm_variant(m, n, k, weight_bits, group_size);
+    if (v == BFAINTB_VARIANT_DECODE) return decode_plan(m, n, k, weight_bits, 0).splits;
+    if (v == BFAINTB_VARIANT_PREFILL && tiled_may_split(v, m, n)) return tile128_plan(m, n, k, 0).splits;
+    return 1;
 }
 
 size_t bfaintb_gemm_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int variant,
@@ -589,42 +643,52 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.splits = 1;
     hipStream_t st = static_cast<hipStream_t>(stream);
 
-    if (is_prefill(v)) {
+    const bool tiled = is_prefill(v);
+    bool small_wreg = false;  // the small-tile kernel that keeps row-major weights in registers (and may split k)
+    if (tiled) {
         // the prefill kernel addresses B and a 256-row panel of A through 32-bit buffer extents
         if ((uint64_t)k * p.ldb_bytes >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
 #ifdef BFAINTB_TRACE
         p.trace = static_cast<unsigned long long*>(workspace);  // per-quarter cycle totals, 8 words per wave
-#else
-        if (use_small_tiles(v, m, n)) {
-            // row-major weights: the form that keeps them in registers, unless the other one is asked for by name
-            if (v != BFAINTB_VARIANT_PREFILL_128_LDS && bfaintb::prefill128_wreg_serves(p)) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, st);
-            return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
-        }
-#endif
         return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
+#endif
+        // row-major weights on small tiles: that form, unless the other one is asked for by name
+        small_wreg = tiled_may_split(v, m, n) && bfaintb::prefill128_wreg_serves(p);
+        if (small_wreg) {
+            const TilePlan tp = tile128_plan(m, n, k, split_k);
+            p.k_per_wg = tp.k_per_wg;
+            p.splits = tp.splits;
+        }
+    } else {
+        const DecodePlan pl = decode_plan(m, n, k, weight_bits, split_k);
+        p.k_per_wg = pl.k_per_wg;
+        p.splits = pl.splits;
+        p.decode_waves = pl.waves;
+        p.decode_cols = pl.cols;
+        p.decode_mb = pl.mb;
     }
-
-    const DecodePlan pl = decode_plan(m, n, k, weight_bits, split_k);
-    p.k_per_wg = pl.k_per_wg;
-    p.splits = pl.splits;
-    p.decode_waves = pl.waves;
-    p.decode_cols = pl.cols;
-    p.decode_mb = pl.mb;
     // (every argument check comes before the first runtime call)
-    const size_t need = p.splits > 1 ? workspace_need(m, n, k, weight_bits, BFAINTB_VARIANT_DECODE, split_k) : 0;
+    const size_t need = split_workspace_bytes(p.splits, m, n);
     if (p.splits > 1 && !use_static_scratch) {
         e = attach_workspace(p, workspace, workspace_bytes, need);
         if (e) return e;
     }
     if (use_static_scratch && need > BFAINTB_STATIC_SCRATCH_BYTES) return BFAINTB_ERR_STATIC_SCRATCH;
     DeviceState* dev = nullptr;
-    e = device_state(st, &dev);
-    if (e) return e;
+    if (!tiled || (p.splits > 1 && use_static_scratch)) {
+        e = device_state(st, &dev);
+        if (e) return e;
+    }
     if (p.splits > 1 && use_static_scratch) {
         e = static_scratch(*dev, st, &workspace);
         if (e) return e;
         e = attach_workspace(p, workspace, BFAINTB_STATIC_SCRATCH_BYTES, need);
         if (e) return e;
+    }
+    if (tiled) {
+        if (small_wreg) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, st);
+        if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
+        return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
 #ifdef BFAINTB_TRACE
     // timestamp sink: behind the split-K area (instrumented callers pass a larger workspace)

@@ -97,8 +97,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
         kBufferFlags);
 
-    const uint32_t ksteps = (p.k + kTwK - 1u) / kTwK;
-    const uint32_t last_chunks = (p.k - (ksteps - 1u) * kTwK) / 8u;  // valid 16-byte chunks per row of A in the last step
+    // K-steps of this workgroup: all of them, or the share of split blockIdx.y (p.k_per_wg rows each; the host makes sure
+    // every split has at least one).  kt below counts within the share; kbase + kt is the step of the whole matrix.
+    const uint32_t ksteps_all = (p.k + kTwK - 1u) / kTwK;
+    const uint32_t ks = blockIdx.y;
+    const uint32_t kbase = ks * (p.k_per_wg / kTwK);
+    const uint32_t ksteps = p.k_per_wg / kTwK < ksteps_all - kbase ? p.k_per_wg / kTwK : ksteps_all - kbase;
+    const uint32_t last_chunks = (p.k - (ksteps_all - 1u) * kTwK) / 8u;  // valid 16-byte chunks per row of A in the last step
     auto clamp = [&](uint32_t t) { return t < ksteps ? t : ksteps - 1u; };
 
     // A copy: instruction j of wave w fills rows 32 w + 8 j .. + 7; lane l lands at row + l / 8, chunk position l % 8, so
@@ -111,12 +116,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t a_last_e = chunk_e < last_chunks ? a_voff_e : a_extent, a_last_o = chunk_o < last_chunks ? a_voff_o : a_extent;
     auto dma_a = [&](auto stage_c, uint32_t kt) {
         uint8_t* base = a_tile(stage_c) + wave * 4096u;
-        const bool last = kt + 1u == ksteps;
+        const bool last = kbase + kt + 1u == ksteps_all;
         const uint32_t ve = last ? a_last_e : a_voff_e, vo = last ? a_last_o : a_voff_o;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
-                                                     (j & 1u) ? vo : ve, kt * kTwK * 2u + j * 16u * p.lda, 0, 0);
+                                                     (j & 1u) ? vo : ve, (kbase + kt) * kTwK * 2u + j * 16u * p.lda, 0, 0);
     };
 
     // W codes.  Copy: a 16-byte-per-lane instruction fills 1024 bytes = kRowsPerCopy rows of the stage; the step's 64
@@ -138,7 +143,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
         for (uint32_t j = 0; j < kCopiesPerWave; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16, w_voff[j],
-                                                     kt * kTwK * p.ldb_bytes, 0, 0);
+                                                     (kbase + kt) * kTwK * p.ldb_bytes, 0, 0);
     };
     // Pick: this lane's 2 columns (byte offset wbyte of a row), rows 8 kq .. 8 kq + 7 of block blk of 32 k: row
     // 32 blk + 8 kq + r, whose block of 8 is 4 blk + kq, rotation kRot * kq
@@ -168,7 +173,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     auto group_scales = [&](uint32_t (&sr)[2], uint32_t kt) {
 #pragma unroll
         for (uint32_t blk = 0; blk < 2; ++blk) {
-            uint32_t g = (kt * kTwK + 32u * blk) / p.group_size;
+            uint32_t g = ((kbase + kt) * kTwK + 32u * blk) / p.group_size;
             if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
             sr[blk] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, g * p.lds * 2u, 0);
         }
@@ -260,7 +265,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + kCopiesPerWave + (GROUPED ? 2 : 0)) : "memory");
         barrier_no_fence();  // (a fenced barrier would also wait for the copies of the steps ahead)
         const uint32_t kt3 = clamp(kt + 3), kt2 = clamp(kt + 2);
-        const bool last3 = kt3 + 1u == ksteps;
+        const bool last3 = kbase + kt3 + 1u == ksteps_all;
         const uint32_t ve = last3 ? a_last_e : a_voff_e, vo = last3 ? a_last_o : a_voff_o;
         uint8_t* const a_dst = a_tile(Target{}) + wave * 4096u;
         uint8_t* const w_dst = w_tile(Target{}) + kCopiesPerWave * wave * 1024u;
@@ -308,10 +313,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_now, wf1, acc[mt][1], 0, 0, 0);
             if (u < 4) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + u * 1024u), 16, (u & 1u) ? vo : ve,
-                                                         kt3 * kTwK * 2u + u * 16u * p.lda, 0, 0);
+                                                         (kbase + kt3) * kTwK * 2u + u * 16u * p.lda, 0, 0);
             } else if (u < 4 + kCopiesPerWave) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + (u - 4u) * 1024u), 16, w_voff[u - 4u],
-                                                         kt3 * kTwK * p.ldb_bytes, 0, 0);
+                                                         (kbase + kt3) * kTwK * p.ldb_bytes, 0, 0);
             } else if (GROUPED && u == 6) {
                 group_scales(s2, kt2);
             }
@@ -386,14 +391,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         }
     }
     const bool plain = p.bias == nullptr && p.residual == nullptr && !gated;  // the bare sums keep a -0 as it is
-#pragma unroll
-    for (uint32_t pass = 0; pass < 8; ++pass) {
-        const uint32_t row = 16u * pass + (tid >> 4);
-        const uint32_t gm = m0 + row;
-        if (gm >= p.m || gn >= p.n) continue;
+    // the thread's 8 sums of tile row `row`, as staged
+    auto staged = [&](uint32_t row, float (&v)[8]) {
         const float* src = c_rows(row >> 5) + (row & 31u) * kTw + 8u * ch;
         const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
-        float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    };
+    // bias, gate, residual, rounding and the store of 8 finished sums of global row gm
+    auto finish = [&](uint32_t gm, float (&v)[8]) {
         if (!plain) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] += bias[i];
@@ -423,6 +428,102 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) =
                 make_uint4(pack_bf16_rne(v[0], v[1]), pack_bf16_rne(v[2], v[3]), pack_bf16_rne(v[4], v[5]), pack_bf16_rne(v[6], v[7]));
         }
+    };
+    auto finish_tile = [&]() {
+#pragma unroll
+        for (uint32_t pass = 0; pass < 8; ++pass) {
+            const uint32_t row = 16u * pass + (tid >> 4);
+            if (m0 + row >= p.m || gn >= p.n) continue;
+            float v[8];
+            staged(row, v);
+            finish(m0 + row, v);
+        }
+    };
+    if (p.splits == 1u) {
+        finish_tile();
+        return;
+    }
+    // ---- split-K: the protocol of the decode kernels.  The workspace holds one fp32 word per (split but the last, row,
+    // column), kEmptyWord at rest.  Producers write their sums with device-scope stores and are done; the workgroup of the
+    // last split (dispatched after them: blockIdx.y is the slow index) fetches them, again while any word is still empty,
+    // adds them in split order with its own sums last, finishes the outputs and leaves the words empty.  Only it waits, and
+    // only on workgroups that wait for nothing; the wait is bounded all the same.
+    // Who moves what: thread t has the four columns 4 (t % 32) .. + 3 of tile rows t / 32 + 8 i, i = 0 .. 15, so that one
+    // instruction of a wave covers two whole rows of the tile (512 contiguous bytes each): whole cache lines go out and come
+    // in.  What the hand-over costs all the same is the reducing workgroup's fetch: 64 KiB per split through one CU, which
+    // draws some 15-20 GB/s from beyond its L2 (3-5 us per split; measured with the fetch, the producers' stores and the
+    // emptying switched off in turn), plus about 6 us for the producers' stores to arrive.
+    const __amdgpu_buffer_rsrc_t ws = __builtin_amdgcn_make_buffer_rsrc(p.partials, 0, (int)p.partial_bytes, kBufferFlags);
+    const uint32_t split_bytes = p.m * p.n * 4u;
+    const uint32_t hrow = tid >> 5, hcol = 4u * (tid & 31u);
+    const uint32_t rows_here = p.m - m0 < kTw ? p.m - m0 : kTw;  // rows of this tile that exist
+    const uint32_t mine = (n0 + hcol < p.n && hrow < rows_here) ? (rows_here - hrow + 7u) / 8u : 0u;  // of the thread's 16 rows
+    auto word_off = [&](uint32_t i) { return ((m0 + hrow + 8u * i) * p.n + n0 + hcol) * 4u; };
+    auto held = [&](uint32_t i) -> float4* {
+        const uint32_t row = hrow + 8u * i;
+        return reinterpret_cast<float4*>(c_rows(row >> 5) + (row & 31u) * kTw + hcol);
+    };
+    if (ks != p.splits - 1u) {
+        if (p.debug_flags & kDebugWithholdPartials) return;  // test hook: lets the reducer's wait run out
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i) {
+            if (i >= mine) continue;
+            const float4 v = *held(i);
+            const u32x4_t w4 = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+            __builtin_amdgcn_raw_buffer_store_b128(w4, ws, (int)word_off(i), (int)(ks * split_bytes), kAuxDeviceScope);
+        }
+        return;
+    }
+    float4 total[16];
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t sp = 0; sp + 1u < p.splits; ++sp) {
+        // a split's words of all the thread's rows are fetched together, and fetched again together while any is empty: one
+        // memory round trip per attempt
+        u32x4_t w[16];
+        bool complete = mine == 0u;
+        for (uint32_t tries = 0; !complete && tries < p.split_wait_limit; ++tries) {
+            if (tries) __builtin_amdgcn_s_sleep(2);
+            asm volatile("" ::: "memory");  // other workgroups write these words: every attempt really loads
+#pragma unroll
+            for (uint32_t i = 0; i < 16; ++i)
+                if (i < mine) w[i] = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)word_off(i), (int)(sp * split_bytes), kAuxDeviceScope);
+            complete = true;
+#pragma unroll
+            for (uint32_t i = 0; i < 16; ++i)
+                if (i < mine)
+#pragma unroll
+                    for (int h = 0; h < 4; ++h)
+                        if (w[i][h] == kEmptyWord) complete = false;
+        }
+        // a word that never arrived is still the empty pattern, a NaN, and turns its sum into one; the workspace's header
+        // remembers that it happened
+        if (!complete) __hip_atomic_store(p.ws_header, kWorkspaceGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i) {
+            if (i >= mine) continue;
+            total[i].x += __uint_as_float(w[i][0]);
+            total[i].y += __uint_as_float(w[i][1]);
+            total[i].z += __uint_as_float(w[i][2]);
+            total[i].w += __uint_as_float(w[i][3]);
+        }
+    }
+    // the other splits' sums plus this workgroup's own, back where the finishing pass takes them from
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) {
+        if (i >= mine) continue;
+        float4* own = held(i);
+        const float4 o = *own;
+        *own = make_float4(total[i].x + o.x, total[i].y + o.y, total[i].z + o.z, total[i].w + o.w);
+    }
+    __syncthreads();
+    finish_tile();
+    // the words this workgroup consumed are empty again for the next launch (last: nothing waits for these stores)
+    const u32x4_t empty4 = {kEmptyWord, kEmptyWord, kEmptyWord, kEmptyWord};
+    for (uint32_t sp = 0; sp + 1u < p.splits; ++sp) {
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i)
+            if (i < mine) __builtin_amdgcn_raw_buffer_store_b128(empty4, ws, (int)word_off(i), (int)(sp * split_bytes), kAuxDeviceScope);
     }
 }
 
@@ -432,7 +533,7 @@ static hipError_t launch_prefill128_wreg_t(const GemmParams& p, hipStream_t stre
     const uint32_t tiles = ((p.m + kTw - 1) / kTw) * ((p.n + kTw - 1) / kTw);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
     void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED>;
-    return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
+    return launch_kernel(kernel, dim3(grid, p.splits, 1), dim3(256, 1, 1), 0, stream, p);
 }
 
 // Whether this kernel can serve a launch: row-major weights (the caller's business), this library's own arithmetic.

@@ -58,7 +58,9 @@ enum {
     BFAINTB_VARIANT_AUTO = 0,   /* decode up to m = 32; beyond, whichever the library estimates faster for (m, n, k) */
     BFAINTB_VARIANT_DECODE = 1, /* split-K weight-streaming kernel (HBM-bound); m > 32 in row blocks; accepts m <= 32768 */
     BFAINTB_VARIANT_PREFILL = 2, /* LDS-tiled MFMA kernels (MFMA-bound): 256x256 tiles, or 128x128 tiles while m x n
-                                  * holds at most 256 of those (the large tiles would leave most CUs idle) */
+                                  * holds at most 256 of those (the large tiles would leave most CUs idle); while even
+                                  * the small tiles leave CUs idle, the kernel over row-major weights splits k between
+                                  * workgroups (same workspace and hand-over as the decode family's split-K) */
     BFAINTB_VARIANT_PREFILL_256 = 3, /* the tiled kernel with 256x256 tiles, whatever the shape (tests, tuning) */
     BFAINTB_VARIANT_PREFILL_128 = 4, /* the tiled kernel with 128x128 tiles, whatever the shape (tests, tuning) */
     BFAINTB_VARIANT_PREFILL_256_LDS = 5, /* 256x256 tiles with both operands staged in LDS — the form pre-packed weights,
@@ -103,8 +105,10 @@ BFAINTB_API int bfaintb_gemm(void* c, const void* a, const void* b, const void* 
                  uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                  size_t workspace_bytes, void* stream);
 
-/* Same, with the kernel family and the split-K factor forced (0 = choose).  For benchmarks and
- * tests; split_k is ignored by the prefill variant. */
+/* Same, with the kernel family and the split-K factor forced (0 = choose, 1 = none).  For benchmarks and tests.
+ * split_k applies to the decode family and to the 128x128-tile kernel over row-major weights (at most 16 splits there,
+ * each of whole 64-row steps of k); the 256x256 tiles, the forms with both operands in LDS and the reference
+ * arithmetic run unsplit whatever it says. */
 BFAINTB_API int bfaintb_gemm_ex(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
                     uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* workspace,
                     size_t workspace_bytes, void* stream, int variant, uint32_t split_k);
@@ -202,7 +206,7 @@ BFAINTB_API int bfaintb_init(void* stream);
 /*
  * The GEMM for callers that cannot allocate or carry a workspace — code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  bfaintb_gemm without the workspace arguments: the split-K partial sums go to a
- * scratch array the library holds in device memory, one per GPU, 8 MiB (bfaintb_gemm_static_scratch_bytes), kept
+ * scratch array the library holds in device memory, one per GPU, 16 MiB (bfaintb_gemm_static_scratch_bytes), kept
  * until the process ends.  Same kernels, same variant choice and bit-for-bit the results of bfaintb_gemm.  A shape
  * whose bfaintb_gemm_workspace_bytes exceeds the scratch is refused with BFAINTB_ERR_STATIC_SCRATCH (nothing launched).
  * Every call on a GPU shares that GPU's scratch (each call leaves it in its at-rest state for the next): calls that may

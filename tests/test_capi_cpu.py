@@ -53,10 +53,23 @@ def test_variant_choice_and_split():
     assert af.variant(1, 28672, 8192, 4, 128) == af.DECODE
     # the tiled variant where the row-blocked family's last round would be mostly empty (320 workgroups on 256 CUs)
     assert af.variant(512, 4096, 4096) == af.DECODE and af.variant(640, 4096, 4096) == af.PREFILL
-    # 128x128 tiles up to one per CU, 256x256 beyond; forced forms are accepted as variants and need no workspace
+    # 128x128 tiles up to one per CU, 256x256 beyond; forced forms are accepted as variants
     assert af.prefill_tile(1024, 4096) == 128 and af.prefill_tile(1025, 4096) == 256
     assert af.prefill_tile(128, 28672) == 128 and af.prefill_tile(4096, 4096) == 256 and af.prefill_tile(1, 16) == 128
-    assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128) == 0 == af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_256)
+    # the small tiles over row-major weights split k while tiles x splits fit one workgroup per CU: same workspace layout as
+    # the decode family's; the large tiles, the both-operands-in-LDS form and an unsplit launch need none
+    assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128, force_split_k=3) == 256 + 2 * 64 * 4096 * 4
+    assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128, force_split_k=1) == 0
+    assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128, force_split_k=1000) == 256 + 15 * 64 * 4096 * 4   # at most 16
+    assert af.workspace_bytes(64, 4096, 64, which=af.PREFILL_128, force_split_k=4) == 0                               # one K-step: nothing to split
+    auto = af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128)
+    assert auto > 0 and (auto - 256) % (64 * 4096 * 4) == 0 and ((auto - 256) // (64 * 4096 * 4) + 1) * 32 <= 256
+    assert af.workspace_bytes(1024, 4096, 4096, which=af.PREFILL_128) == 0   # a tile on every CU already
+    assert af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_128_LDS, force_split_k=4) == 0 == af.workspace_bytes(64, 4096, 4096, which=af.PREFILL_256)
+    # AUTO: tiles with k split where the plan says so, reported by split_k and workspace_bytes alike
+    assert af.variant(384, 2048, 8192) == af.PREFILL and af.split_k(384, 2048, 8192) > 1
+    assert af.workspace_bytes(384, 2048, 8192) == 256 + (af.split_k(384, 2048, 8192) - 1) * 384 * 2048 * 4
+    assert af.workspace_bytes(384, 2048, 8192) <= af.lib().bfaintb_gemm_static_scratch_bytes() == 16 << 20
     assert af.kernel_name(64, which=af.PREFILL_128) == "bfaintb_prefill128_wreg_kernel"
     assert af.kernel_name(64, which=af.PREFILL_128_LDS) == "bfaintb_prefill128_kernel"
     assert af.kernel_name(64, which=af.PREFILL_256) == af.kernel_name(64, which=af.PREFILL) == "bfaintb_prefill_wreg_kernel"

@@ -164,17 +164,17 @@ def test_tile_sizes_agree_bit_for_bit(af, m, n, k, bits, group):
     instructions per 64 rows of k), so they must agree in every bit, near-cancelling outputs included: an indexing
     slip in either one shows here even where it would stay inside the 2-ULP bound."""
     p = Problem(m, n, k, bits, group, seed=m + n + k)
-    assert np.array_equal(run_gemm(p, which=af.PREFILL_128), run_gemm(p, which=af.PREFILL_256))
+    assert np.array_equal(run_gemm(p, which=af.PREFILL_128, force_split_k=1), run_gemm(p, which=af.PREFILL_256))
 
 
 @pytest.mark.parametrize("m,n,k,bits,group", [(130, 272, 72, 8, 0), (700, 1008, 1000, 8, 0), (300, 528, 512, 8, 64), (1000, 1008, 384, 4, 0),
                                               (130, 4112, 256, 4, 128), (1024, 4096, 1088, 8, 0), (257, 272, 8, 4, 0)])
 def test_small_tile_forms_agree_bit_for_bit(af, m, n, k, bits, group):
     """The 128x128-tile kernel that keeps the weights in registers (row-major weights: what PREFILL_128 runs) against the
-    one that stages both operands in LDS: same products, same order of addition, so the same bits — partial tiles in m
-    and n, K-steps that are not whole, one to seventeen steps, both code widths, grouped scales."""
+    one that stages both operands in LDS: same products, same order of addition (k unsplit), so the same bits — partial
+    tiles in m and n, K-steps that are not whole, one to seventeen steps, both code widths, grouped scales."""
     p = Problem(m, n, k, bits, group, seed=m + 2 * n + k)
-    c = run_gemm(p, which=af.PREFILL_128)
+    c = run_gemm(p, which=af.PREFILL_128, force_split_k=1)
     assert_close_ulp(p, c, f"128-tile, weights in registers: {m}x{n}x{k} bits={bits} g={group}")
     assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128_LDS))
 
@@ -188,6 +188,76 @@ def test_tiled_variant_picks_its_tile_size_by_shape(af):
         c = run_gemm(p, which=af.PREFILL)
         assert_close_ulp(p, c, f"{m}x{n}")
         assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128 if tile == 128 else af.PREFILL_256)), f"{m}x{n}"
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [(130, 272, 1000, 8, 0), (256, 1040, 2048, 8, 64), (100, 528, 4096, 4, 128), (300, 272, 1088, 4, 0),
+                                              (64, 4096, 4096, 8, 0)])
+def test_tiled_split_k_matches_oracle_and_is_deterministic(af, m, n, k, bits, group):
+    """The 128x128-tile kernel with k split between workgroups: every split factor meets the oracle (shares of whole
+    64-row steps; a last step that is not whole; as many splits as steps; more splits asked for than steps exist), the
+    same factor gives the same bits every time, whatever order the workgroups arrived in, and the workspace is left at
+    rest."""
+    import helpers
+    p = Problem(m, n, k, bits, group, seed=m + n + k + 1)
+    steps = (k + 63) // 64
+    for split in (2, 3, 5, 16):
+        need = af.workspace_bytes(m, n, k, bits, group, af.PREFILL_128, split)
+        per = -(-steps // min(split, 16))
+        runs = -(-steps // per)  # splits that really run
+        assert need == (256 + (((runs - 1) * m * n * 4 + 255) & ~255) if runs > 1 else 0)
+        c = run_gemm(p, which=af.PREFILL_128, force_split_k=split)
+        assert_close_ulp(p, c, f"128-tile split_k={split}: {m}x{n}x{k} bits={bits} g={group}")
+        for _ in range(2):
+            assert np.array_equal(run_gemm(p, which=af.PREFILL_128, force_split_k=split), c), f"split_k={split} not reproducible"
+        assert bool((helpers._ws.t[256:] == 0xFF).all()), f"workspace not at rest after split_k={split}"
+        assert af.workspace_status(helpers._ws.t) == 0
+
+
+def test_tiled_split_k_is_what_auto_runs_and_takes_the_epilogues(af):
+    """A shape whose plan is the small tiles with k split (long k, few tiles): AUTO gives the forced form's bits, and the
+    bias / residual / gate epilogues run on the reduced sums."""
+    m, n, k = 384, 2048, 8192
+    assert af.variant(m, n, k) == af.PREFILL and af.prefill_tile(m, n) == 128
+    split = af.split_k(m, n, k)
+    assert split > 1 and af.workspace_bytes(m, n, k) == 256 + (split - 1) * m * n * 4
+    p = Problem(m, n, k, seed=61)
+    c = run_gemm(p)
+    assert_close_ulp(p, c, "auto")
+    assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128, force_split_k=split))
+    assert not np.array_equal(c, run_gemm(p, which=af.PREFILL_128, force_split_k=1)), "the split changes the order of addition"
+    p.with_bias().with_residual()
+    assert_close_ulp(p, run_gemm(p), "auto, bias + residual")
+    g = gated_problem(m, n, k, 8, 0, seed=62).with_bias()
+    assert_close_gated(g, run_gemm(g, activation=af.ACT_SILU_GATE), "auto, gated")
+
+
+def test_tiled_split_k_gives_up_like_the_decode_family(af):
+    """The bounded wait of the tiled kernel's reducing workgroups, driven from the host as in the decode family's test:
+    producers keep their sums, the attempts are capped: NaNs, a poisoned header, and all well after initialisation."""
+    import torch
+    p = Problem(130, 272, 1024, seed=63)
+    need = af.workspace_bytes(p.m, p.n, p.k, which=af.PREFILL_128, force_split_k=4)
+    raw = torch.empty(need, dtype=torch.uint8, device="cuda")
+    af.workspace_init(raw)
+    a, b, s = to_dev(p.a_bf), to_dev(p.b_bytes), to_dev(p.s_bf)
+    c = torch.zeros((p.m, p.n), dtype=torch.int16, device="cuda")
+    run = lambda: (af.gemm(c, a, b, s, p.m, p.n, p.k, workspace=raw, which=af.PREFILL_128, force_split_k=4), torch.cuda.synchronize())
+    run()
+    good = from_dev_u16(c).copy()
+    assert_close_ulp(p, good, "before")
+    try:
+        af.debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 3)
+        af.debug_control(af.DEBUG_WITHHOLD_PARTIALS, 1)
+        run()
+    finally:
+        af.debug_control(af.DEBUG_WITHHOLD_PARTIALS, 0)
+        af.debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 0)
+    assert np.isnan(widen(from_dev_u16(c))).all(), "every output misses partial sums: all NaN"
+    assert af.workspace_status(raw) == af.ERR_WORKSPACE_POISONED
+    af.workspace_init(raw)
+    run()
+    assert af.workspace_status(raw) == 0
+    assert np.array_equal(from_dev_u16(c), good)
 
 
 def test_forced_row_block_changes_the_plan_not_the_contract(af):

@@ -42,8 +42,10 @@ def _both(af, p):
 
 def test_static_scratch_matches_caller_workspace_on_calls_in_a_row(af):
     # the second input is smaller than the first (it finds the scratch as the first call left it), the third larger
-    # again and 4-bit with group scales, the fourth runs without split-K (the tiled kernel: the scratch is not touched)
-    shapes = [(16, 4096, 4096, 8, 0), (1, 1024, 2048, 8, 0), (4, 4096, 8192, 4, 128), (300, 512, 256, 8, 0), (1, 4096, 4096, 8, 0)]
+    # again and 4-bit with group scales, the fourth runs without split-K (the tiled kernel: the scratch is not touched),
+    # the fifth is the tiled kernel with k split (its partial sums go through the scratch as well)
+    shapes = [(16, 4096, 4096, 8, 0), (1, 1024, 2048, 8, 0), (4, 4096, 8192, 4, 128), (300, 512, 256, 8, 0), (384, 2048, 8192, 8, 0),
+              (1, 4096, 4096, 8, 0)]
     used_split = 0
     for i, (m, n, k, bits, group) in enumerate(shapes):
         p = Problem(m, n, k, bits, group, seed=40 + i)
@@ -51,15 +53,15 @@ def test_static_scratch_matches_caller_workspace_on_calls_in_a_row(af):
         used_split += need > 0
         assert np.array_equal(c_static, c_plain), f"call {i}: {shapes[i]}"
         assert not np.isnan(c_plain.view(np.uint16).astype(np.uint32) << 16).any()
-    assert used_split >= 4  # the comparison did exercise the scratch
+    assert used_split >= 5  # the comparison did exercise the scratch
 
 
 def test_static_scratch_refuses_what_does_not_fit(af):
     L = af.lib()
-    # 32 rows x 11008 columns, k long enough for 8 splits: 9 MiB of partial sums
-    m, n, k = 32, 11008, 28672
+    # 32 rows x 28672 columns, k long enough for 8 splits: 24.5 MiB of partial sums
+    m, n, k = 32, 28672, 28672
     need = L.bfaintb_gemm_workspace_bytes(m, n, k, 8, 0)
-    assert need > L.bfaintb_gemm_static_scratch_bytes() == 8 << 20
+    assert need > L.bfaintb_gemm_static_scratch_bytes() == 16 << 20
     P = 1 << 20  # never dereferenced: the call is refused before any launch
     assert L.bfaintb_gemm_static(P, P, P, P, m, n, k, k, n, n, 8, 0, None) == af.ERR_STATIC_SCRATCH
     assert "bfaintb_gemm" in af.error_string(af.ERR_STATIC_SCRATCH)
