@@ -56,6 +56,7 @@ RECORDED_TRAFFIC = {
     "m2048_n28672_k8192_int4_group128": (896485920, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
     "mid_m256_n4096_k4096_int8_perchannel": (35861798, "profiles/mid_m256_n4096_k4096_int8.txt"),
     "mid_m1024_n4096_k4096_int8_perchannel": (92417830, "profiles/mid_m1024_n4096_k4096_int8.txt"),
+    "mid_m256_n8192_k8192_int8_perchannel": (132209707, "profiles/mid_m256_n8192_k8192_int8.txt"),
 }
 
 # Parity counts RECORDED from the GPU test suite (tests/helpers.py: assert_close_ulp logs every check; tests/conftest.py
@@ -376,7 +377,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
-                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024")
+                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m256_n8192_k8192")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM would shard over the columns "
@@ -394,13 +395,17 @@ def main():
 
     # ---- one secondary workload alone (profiling runs)
     if args.only.startswith(("c3_m", "c5_m", "mid_m")):
-        m = int(args.only.split("_m")[1])
+        import re
+        parsed = re.fullmatch(r"(c3|c5|mid)_m(\d+)(?:_n(\d+)_k(\d+))?", args.only)
+        assert parsed, f"--only {args.only}: not a workload name"
+        m = int(parsed.group(2))
         if args.only.startswith("c3_"):
             w = config3_workload(m)
         elif args.only.startswith("c5_"):
             w = config5_workload(m)
         else:
-            w = Workload(f"mid_m{m}_n4096_k4096_int8_perchannel", m, 4096, 4096, copies=4)
+            n, k = (int(parsed.group(3)), int(parsed.group(4))) if parsed.group(3) else (4096, 4096)
+            w = Workload(f"mid_m{m}_n{n}_k{k}_int8_perchannel", m, n, k, copies=4 if n * k <= 4096 * 4096 else 2)
         steps = min(K, 200) if m <= 32 else 10
         ev_ms, wall_ms = time_graph(af, w, steps, min(W, 10), rotate=True)
         bound = "hbm" if m <= 32 else "mfma"
