@@ -512,7 +512,8 @@ def test_hip_graph_replays_match_eager(af):
     import torch
     from helpers import Workspace
     shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (16, 768, 1024, 8, 0), (96, 512, 512, 8, 0),
-              (4200, 272, 256, 8, 0), (4200, 1040, 128, 4, 64)]   # the tiled kernels: 128x128 tiles, 256x256 tiles (two launches)
+              (4200, 272, 256, 8, 0), (4200, 1040, 128, 4, 64),   # the tiled kernels: 128x128 tiles, 256x256 tiles (two launches)
+              (384, 2048, 8192, 8, 0)]                            # 128x128 tiles with k split (partial sums through the workspace)
     probs = [Problem(m, n, k, bits, g, seed=90 + i) for i, (m, n, k, bits, g) in enumerate(shapes)]
     eager = [run_gemm(p) for p in probs]
     ws = Workspace()
@@ -550,7 +551,10 @@ def test_two_streams_with_their_own_workspaces(af):
     """Launches are stream-ordered and keep no state outside their arguments: GEMMs issued alternately on two streams,
     each stream with its own workspace and output, give the single-stream results."""
     import torch
-    shapes = [(1, 4096, 4096, 8, 0), (8, 1040, 4096, 4, 128), (200, 528, 1024, 8, 0), (4200, 272, 256, 8, 0)]
+    # (the last shape runs the small tiles with k split: 192 workgroups of one per CU, so two launches in flight compete
+    # for CUs while their reducing workgroups wait — for workgroups that wait for nothing, hence never for long)
+    shapes = [(1, 4096, 4096, 8, 0), (8, 1040, 4096, 4, 128), (200, 528, 1024, 8, 0), (4200, 272, 256, 8, 0), (384, 2048, 8192, 8, 0)]
+    assert af.variant(384, 2048, 8192) == af.PREFILL and af.split_k(384, 2048, 8192) > 1
     probs = [Problem(m, n, k, bits, g, seed=300 + i) for i, (m, n, k, bits, g) in enumerate(shapes)]
     want = [run_gemm(p) for p in probs]
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
