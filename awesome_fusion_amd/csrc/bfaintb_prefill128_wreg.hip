@@ -477,36 +477,62 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     float4 total[16];
 #pragma unroll
     for (uint32_t i = 0; i < 16; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (uint32_t sp = 0; sp + 1u < p.splits; ++sp) {
-        // a split's words of all the thread's rows are fetched together, and fetched again together while any is empty: one
-        // memory round trip per attempt
-        u32x4_t w[16];
-        bool complete = mine == 0u;
-        for (uint32_t tries = 0; !complete && tries < p.split_wait_limit; ++tries) {
+    // First wait, at the price of one word per thread and split, until the producers' last stores show: a fetch of whole
+    // tiles that comes too early moves 64 KiB per split of nothing through this CU.  (What a thread stored last is not
+    // bound to arrive last: the fetch below checks every word on its own.)
+    if (mine != 0u) {
+        bool there = false;
+        for (uint32_t tries = 0; !there && tries < p.split_wait_limit; ++tries) {
+            if (tries) __builtin_amdgcn_s_sleep(2);
+            asm volatile("" ::: "memory");
+            there = true;
+            for (uint32_t sp = 0; sp + 1u < p.splits; ++sp) {
+                const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)word_off(mine - 1u), (int)(sp * split_bytes), kAuxDeviceScope);
+                if (v[3] == kEmptyWord) there = false;
+            }
+        }
+    }
+    for (uint32_t sp = 0; sp + 1u < p.splits; sp += 2u) {
+        // two splits' words of all the thread's rows are fetched together (more bytes in flight per CU, fewer round trips),
+        // and fetched again together while any is empty
+        const bool pair = sp + 2u < p.splits;  // the same for every thread
+        u32x4_t w[2][16];
+        // bit 16 j + i: words (j, i) are wanted and have not been seen complete yet; only those are fetched again
+        uint32_t missing = 0u;
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i)
+            if (i < mine) missing |= (1u << i) | (pair ? 1u << (16u + i) : 0u);
+        for (uint32_t tries = 0; missing != 0u && tries < p.split_wait_limit; ++tries) {
             if (tries) __builtin_amdgcn_s_sleep(2);
             asm volatile("" ::: "memory");  // other workgroups write these words: every attempt really loads
 #pragma unroll
-            for (uint32_t i = 0; i < 16; ++i)
-                if (i < mine) w[i] = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)word_off(i), (int)(sp * split_bytes), kAuxDeviceScope);
-            complete = true;
+            for (uint32_t j = 0; j < 2; ++j)
 #pragma unroll
-            for (uint32_t i = 0; i < 16; ++i)
-                if (i < mine)
+                for (uint32_t i = 0; i < 16; ++i)
+                    if (missing & (1u << (16u * j + i)))
+                        w[j][i] = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)word_off(i), (int)((sp + j) * split_bytes), kAuxDeviceScope);
 #pragma unroll
-                    for (int h = 0; h < 4; ++h)
-                        if (w[i][h] == kEmptyWord) complete = false;
+            for (uint32_t j = 0; j < 2; ++j)
+#pragma unroll
+                for (uint32_t i = 0; i < 16; ++i)
+                    if ((missing & (1u << (16u * j + i))) && w[j][i][0] != kEmptyWord && w[j][i][1] != kEmptyWord && w[j][i][2] != kEmptyWord &&
+                        w[j][i][3] != kEmptyWord)
+                        missing &= ~(1u << (16u * j + i));
         }
+        const bool complete = missing == 0u;
         // a word that never arrived is still the empty pattern, a NaN, and turns its sum into one; the workspace's header
         // remembers that it happened
         if (!complete) __hip_atomic_store(p.ws_header, kWorkspaceGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-        for (uint32_t i = 0; i < 16; ++i) {
-            if (i >= mine) continue;
-            total[i].x += __uint_as_float(w[i][0]);
-            total[i].y += __uint_as_float(w[i][1]);
-            total[i].z += __uint_as_float(w[i][2]);
-            total[i].w += __uint_as_float(w[i][3]);
-        }
+        for (uint32_t j = 0; j < 2; ++j)  // in split order
+#pragma unroll
+            for (uint32_t i = 0; i < 16; ++i) {
+                if (i >= mine || (j == 1u && !pair)) continue;
+                total[i].x += __uint_as_float(w[j][i][0]);
+                total[i].y += __uint_as_float(w[j][i][1]);
+                total[i].z += __uint_as_float(w[j][i][2]);
+                total[i].w += __uint_as_float(w[j][i][3]);
+            }
     }
     // the other splits' sums plus this workgroup's own, back where the finishing pass takes them from
 #pragma unroll
