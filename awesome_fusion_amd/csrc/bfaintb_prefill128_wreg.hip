@@ -480,6 +480,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // First wait, at the price of one word per thread and split, until the producers' last stores show: a fetch of whole
     // tiles that comes too early moves 64 KiB per split of nothing through this CU.  (What a thread stored last is not
     // bound to arrive last: the fetch below checks every word on its own.)
+    uint32_t fetch_limit = p.split_wait_limit;
     if (mine != 0u) {
         bool there = false;
         for (uint32_t tries = 0; !there && tries < p.split_wait_limit; ++tries) {
@@ -491,6 +492,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
                 if (v[3] == kEmptyWord) there = false;
             }
         }
+        if (!there) fetch_limit = 1u;  // the wait has run out: one fetch of what there is, no second wait of that length
     }
     for (uint32_t sp = 0; sp + 1u < p.splits; sp += 2u) {
         // two splits' words of all the thread's rows are fetched together (more bytes in flight per CU, fewer round trips),
@@ -502,7 +504,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
         for (uint32_t i = 0; i < 16; ++i)
             if (i < mine) missing |= (1u << i) | (pair ? 1u << (16u + i) : 0u);
-        for (uint32_t tries = 0; missing != 0u && tries < p.split_wait_limit; ++tries) {
+        for (uint32_t tries = 0; missing != 0u && tries < fetch_limit; ++tries) {
             if (tries) __builtin_amdgcn_s_sleep(2);
             asm volatile("" ::: "memory");  // other workgroups write these words: every attempt really loads
 #pragma unroll
