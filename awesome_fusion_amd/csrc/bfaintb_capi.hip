@@ -141,8 +141,9 @@ static bool use_small_tiles(int v, uint32_t m, uint32_t n)
 }
 
 // Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
-// k.  Small tiles: a K-step takes 0.65 us on an empty machine and 0.70 us with a workgroup on every CU with row-major
-// weights (the kernel that keeps them in registers), 0.70 and 0.90 us with packed weights (both operands through LDS).
+// k.  Small tiles: a K-step takes 0.62 us on an empty machine and 0.65 us with a workgroup on every CU with row-major
+// weights (the kernel that keeps them in registers; 0.74 and 0.75 us with 4-bit codes), 0.70 and 0.90 us with packed
+// weights (both operands through LDS).
 // The small-tile kernel over row-major weights may split k: grid y walks the splits, each workgroup runs its share of
 // the K-steps and the workgroup of the last split adds the others' sums (same workspace and protocol as the decode
 // family).  Worth it while tiles x splits still fit one workgroup per CU.
@@ -159,7 +160,7 @@ static size_t split_workspace_bytes(uint32_t splits, uint32_t m, uint32_t n)
     return bfaintb::kWorkspaceHeaderBytes + ((((size_t)(splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u);
 }
 
-static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, uint32_t forced_splits)
+static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits)
 {
     const uint32_t ksteps = (k + 63u) / 64u;
     const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
@@ -172,10 +173,11 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, uint32_t forced
         t.splits = (ksteps + per - 1u) / per;
         // the hand-over: the producers' device-scope stores have to arrive (some 6 us after the last K-step), then the
         // reducing workgroup fetches a tile's worth of sums per split through its one CU, slower the more CUs do so at once
-        // (8-bit, n = k = 4096, us with 1 / 2 / 3 / 4 splits: m = 128: 43.4 / 32.7 / 26.2 / 28.3; m = 256: 43.9 / 34.0 /
-        // 27.2 / 31.1; m = 512: 44.3 / 36.4 / 44.1 / 42.3; 8192 x 8192, m = 256: 83.2 / 55.8 / 69.9 / 62.5)
-        const double hand_over = t.splits > 1u ? 4.5 + (t.splits - 1.0) * (2.0 + 0.04 * tiles) : 0.0;
-        t.us = 4.0 + per * (0.65 + 0.0002 * tiles * t.splits) + hand_over;
+        // (8-bit, n = k = 4096, us with 1 / 2 / 3 / 4 splits: m = 128: 43.4 / 31.1 / 27.5 / 28.3; m = 256: 43.9 / 31.7 /
+        // 28.5 / 29.4; m = 512: 44.3 / 32.9 / 44.1 / 42.3; 8192 x 8192, m = 256: 83.2 / 55.8 / 69.9 / 62.5)
+        const double hand_over = t.splits > 1u ? 2.0 + (t.splits - 1.0) * (3.6 + 0.007 * tiles) : 0.0;
+        // a K-step: 0.62 us (4-bit codes 0.74) on an empty machine, 0.65 (0.75) with a workgroup on every CU
+        t.us = 4.0 + per * ((bits == 4 ? 0.74 : 0.615) + 0.00013 * tiles * t.splits) + hand_over;
         return t;
     };
     if (forced_splits) return shape(forced_splits);
@@ -192,11 +194,11 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, uint32_t forced
     return best;
 }
 
-static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, bool packed = false)
+static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits, bool packed = false)
 {
     if (prefill_small_tiles(m, n)) {
         const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
-        if (!packed) return tile128_plan(m, n, k, 0).us;
+        if (!packed) return tile128_plan(m, n, k, bits, 0).us;
         return 4.0 + (k / 64.0) * (0.70 + 0.0008 * tiles);
     }
     const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
@@ -359,10 +361,16 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
 int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
     if (variant == BFAINTB_VARIANT_AUTO) {
-        if (m <= kDecodeAutoMaxM) return BFAINTB_VARIANT_DECODE;
+        // (up to 64 rows one block of rows streams B once at full matrix-instruction height, while tiles of 128 rows run half
+        // empty: the family wins on every shape measured — 11008 x 4096, m = 64: 24.6 against 29.6 us, 8192 x 8192: 29.8
+        // against 35.0, 4-bit 31.2 against 39.0 — whatever the estimates, which are not that fine, say)
+        if (m <= kDecodeAutoMaxM || m <= 64u) return BFAINTB_VARIANT_DECODE;
         if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
         const DecodePlan pl = decode_plan(m, n, k, bits, 0);
-        return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+        // (the family's estimate for 4-bit codes dates from before their conversion got cheaper: 1.17 to 1.45 times the
+        // measured time on 40 shapes, median 1.32; it still ranks the family's own plans, but against the tiles it is corrected)
+        const double family = decode_family_estimate_us(m, n, k, bits, pl) * (bits == 4 ? 0.76 : 1.0);
+        return family < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     }
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
     if (is_prefill(variant)) return variant;
@@ -376,7 +384,7 @@ size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant,
 {
     if (m == 0 || n == 0) return 0;
     if (variant == BFAINTB_VARIANT_DECODE) return split_workspace_bytes(decode_plan(m, n, k, bits, forced_split).splits, m, n);
-    if (is_prefill(variant) && tiled_may_split(variant, m, n)) return split_workspace_bytes(tile128_plan(m, n, k, forced_split).splits, m, n);
+    if (is_prefill(variant) && tiled_may_split(variant, m, n)) return split_workspace_bytes(tile128_plan(m, n, k, bits, forced_split).splits, m, n);
     return 0;
 }
 
@@ -500,7 +508,7 @@ uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bit
 {
     const int v = bfaintb_gemm_variant(m, n, k, weight_bits, group_size);
     if (v == BFAINTB_VARIANT_DECODE) return decode_plan(m, n, k, weight_bits, 0).splits;
-    if (v == BFAINTB_VARIANT_PREFILL && tiled_may_split(v, m, n)) return tile128_plan(m, n, k, 0).splits;
+    if (v == BFAINTB_VARIANT_PREFILL && tiled_may_split(v, m, n)) return tile128_plan(m, n, k, weight_bits, 0).splits;
     return 1;
 }
 
@@ -655,7 +663,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
         // row-major weights on small tiles: that form, unless the other one is asked for by name
         small_wreg = tiled_may_split(v, m, n) && bfaintb::prefill128_wreg_serves(p);
         if (small_wreg) {
-            const TilePlan tp = tile128_plan(m, n, k, split_k);
+            const TilePlan tp = tile128_plan(m, n, k, weight_bits, split_k);
             p.k_per_wg = tp.k_per_wg;
             p.splits = tp.splits;
         }
@@ -830,7 +838,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (packed_uses_slab(m, n, k, bits)) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
-    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, true) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits, true) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
