@@ -27,6 +27,7 @@ hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stre
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, hipStream_t stream);
 bool prefill128_wreg_serves(const GemmParams& p);
+hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t decode_prepare_device();
 }  // namespace bfaintb
@@ -128,10 +129,19 @@ static bool prefill_small_tiles(uint32_t m, uint32_t n)
     return (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u) <= 256u;
 }
 
+// Between the two: more than 256 small tiles but at most 256 tiles of 256 rows x 128 columns.  The large tiles would
+// occupy a quarter to a half of the CUs there; the tall ones run one per CU at 0.94 us per K-step against the large tiles'
+// 1.02 on twice the work (8-bit, 64 steps, us tall / large: 1536 x 4096: 61.0 / 66.0; 512 x 11008: 60.3 / 64.7; 2048 x 4096:
+// 71.0 / 75.7; 128 steps, 1024 x 8192: 129 / 141; 4-bit, 768 x 8192: 138 / 140).
+static bool prefill_tall_tiles(uint32_t m, uint32_t n)
+{
+    return !prefill_small_tiles(m, n) && (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u) <= 256u;
+}
+
 static bool is_prefill(int v)
 {
     return v == BFAINTB_VARIANT_PREFILL || v == BFAINTB_VARIANT_PREFILL_256 || v == BFAINTB_VARIANT_PREFILL_128 ||
-           v == BFAINTB_VARIANT_PREFILL_256_LDS || v == BFAINTB_VARIANT_PREFILL_128_LDS;
+           v == BFAINTB_VARIANT_PREFILL_256_LDS || v == BFAINTB_VARIANT_PREFILL_128_LDS || v == BFAINTB_VARIANT_PREFILL_256X128;
 }
 
 // tile size of a tiled-variant launch: forced, or by shape
@@ -695,6 +705,8 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     }
     if (tiled) {
         if (small_wreg) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, st);
+        if ((v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) && !p.reference_arith)
+            return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, st);
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
         return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
@@ -833,6 +845,7 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
 static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
+    if (variant == BFAINTB_VARIANT_PREFILL_256X128) return BFAINTB_ERR_BAD_VARIANT;  // (row-major weights only)
     if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
     if (packed_uses_slab(m, n, k, bits)) return BFAINTB_VARIANT_DECODE;
@@ -1051,6 +1064,7 @@ int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream)
 }
 
 uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n) { return prefill_small_tiles(m, n) ? 128u : 256u; }
+uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n) { return (prefill_small_tiles(m, n) || prefill_tall_tiles(m, n)) ? 128u : 256u; }
 
 const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m)
 {
@@ -1062,6 +1076,7 @@ const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_siz
     if (v == BFAINTB_VARIANT_PREFILL_256_LDS) return "bfaintb_prefill_kernel";
     if (v == BFAINTB_VARIANT_PREFILL_128) return "bfaintb_prefill128_wreg_kernel";
     if (v == BFAINTB_VARIANT_PREFILL_128_LDS) return "bfaintb_prefill128_kernel";
+    if (v == BFAINTB_VARIANT_PREFILL_256X128) return "bfaintb_prefill256x128_wreg_kernel";
     (void)weight_bits;
     (void)group_size;
     return "";

@@ -15,6 +15,7 @@ AUTO, DECODE, PREFILL = 0, 1, 2
 PREFILL_256, PREFILL_128 = 3, 4  # the tiled variant with its tile size forced (tests, tuning)
 PREFILL_256_LDS = 5               # ... and its form with both operands in LDS forced
 PREFILL_128_LDS = 6               # the same for the 128-tile kernel
+PREFILL_256X128 = 7               # tiles of 256 rows x 128 columns, weights in registers
 ACT_NONE, ACT_SILU_GATE = 0, 1
 
 
@@ -127,6 +128,8 @@ def lib():
         L.bfaintb_probe_read.argtypes = [_vp, C.c_size_t, _vp, _vp]
         L.bfaintb_prefill_tile.restype = _u32
         L.bfaintb_prefill_tile.argtypes = [_u32, _u32]
+        L.bfaintb_prefill_tile_cols.restype = _u32
+        L.bfaintb_prefill_tile_cols.argtypes = [_u32, _u32]
         L.bfaintb_kernel_name.restype = C.c_char_p
         L.bfaintb_kernel_name.argtypes = [C.c_int, C.c_int, _u32, _u32]
         L.bfaintb_error_string.restype = C.c_char_p
@@ -176,8 +179,13 @@ def split_k(m, n, k, weight_bits=8, group_size=0):
 
 
 def prefill_tile(m, n):
-    """Tile edge (128 or 256) the PREFILL variant uses for an m x n output."""
+    """Rows of the tiles (128 or 256) the PREFILL variant uses for an m x n output."""
     return lib().bfaintb_prefill_tile(m, n)
+
+
+def prefill_tile_cols(m, n):
+    """Columns of those tiles (128, also for the tiles of 256 rows x 128 columns; or 256)."""
+    return lib().bfaintb_prefill_tile_cols(m, n)
 
 
 def kernel_name(m, weight_bits=8, group_size=0, which=AUTO):

@@ -66,9 +66,12 @@ enum {
     BFAINTB_VARIANT_PREFILL_256_LDS = 5, /* 256x256 tiles with both operands staged in LDS — the form pre-packed weights,
                                           * residuals and the gate epilogue use; row-major weights otherwise run the form
                                           * that keeps the weights in registers (tests, tuning) */
-    BFAINTB_VARIANT_PREFILL_128_LDS = 6  /* 128x128 tiles with both operands staged in LDS — the form pre-packed weights
+    BFAINTB_VARIANT_PREFILL_128_LDS = 6, /* 128x128 tiles with both operands staged in LDS — the form pre-packed weights
                                           * use; row-major weights otherwise run the form that keeps the weights in
                                           * registers (tests, tuning) */
+    BFAINTB_VARIANT_PREFILL_256X128 = 7  /* tiles of 256 rows x 128 columns, weights in registers (row-major weights, this
+                                          * library's arithmetic), whatever the shape (tests, tuning): what PREFILL runs
+                                          * where 128x128 tiles would need a second round and 256x256 tiles leave CUs idle */
 };
 
 /*
@@ -305,9 +308,12 @@ BFAINTB_API int bfaintb_packed_header_check(const bfaintb_packed_header* h);
 /* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */
 BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 
-/* Edge of the square tiles BFAINTB_VARIANT_PREFILL runs an m x n output with: 128 while that makes at most 256 tiles
- * (one per CU), else 256.  Depends only on its arguments. */
+/* Rows (bfaintb_prefill_tile) and columns of the tiles BFAINTB_VARIANT_PREFILL runs an m x n output of row-major
+ * weights with: 128 x 128 while that makes at most 256 tiles (one per CU); else 256 rows x 128 columns while that
+ * makes at most 256; else 256 x 256.  (Pre-packed weights and the reference arithmetic have no 256 x 128 form: 256 x 256
+ * there.)  Depend only on their arguments. */
 BFAINTB_API uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n);
+BFAINTB_API uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n);
 
 /* The split-K factor the decode variant would use for a shape (1 for the prefill variant). */
 BFAINTB_API uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);

@@ -180,14 +180,39 @@ def test_small_tile_forms_agree_bit_for_bit(af, m, n, k, bits, group):
 
 
 def test_tiled_variant_picks_its_tile_size_by_shape(af):
-    """PREFILL runs 128x128 tiles while m x n holds at most 256 of them, 256x256 tiles beyond; either way the result
-    meets the oracle and is the forced form's, bit for bit."""
-    for (m, n, tile) in [(1024, 4096, 128), (2048, 2048, 128), (2064, 2048, 256), (1024, 4224, 256)]:
-        assert af.prefill_tile(m, n) == tile
+    """PREFILL runs 128x128 tiles while m x n holds at most 256 of them, then tiles of 256 rows x 128 columns while those
+    are at most 256, 256x256 tiles beyond; every time the result meets the oracle and is the forced form's, bit for bit."""
+    for (m, n, rows, cols) in [(1024, 4096, 128, 128), (2048, 2048, 128, 128), (2064, 2048, 256, 128), (1024, 4224, 256, 128), (2048, 4096, 256, 128),
+                               (2064, 4096, 256, 256), (520, 16512, 256, 256)]:
+        assert (af.prefill_tile(m, n), af.prefill_tile_cols(m, n)) == (rows, cols)
         p = Problem(m, n, 256, 8, 0, seed=m + n)
         c = run_gemm(p, which=af.PREFILL)
         assert_close_ulp(p, c, f"{m}x{n}")
-        assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128 if tile == 128 else af.PREFILL_256)), f"{m}x{n}"
+        forced = af.PREFILL_128 if rows == 128 else af.PREFILL_256X128 if cols == 128 else af.PREFILL_256
+        assert np.array_equal(c, run_gemm(p, which=forced, force_split_k=1)), f"{m}x{n}"
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [(256, 128, 64, 8, 0), (300, 272, 448, 8, 0), (700, 1008, 1000, 8, 0), (1000, 1008, 384, 4, 0), (520, 528, 512, 8, 64),
+                                              (130, 4112, 256, 4, 128), (257, 272, 8, 4, 0), (2048, 512, 1088, 8, 0), (17, 48, 128, 4, 64)])
+def test_tall_tiles_agree_with_the_large_ones_bit_for_bit(af, m, n, k, bits, group):
+    """Tiles of 256 rows x 128 columns (two waves by two, each converting the weights of its 64 columns) against the 256x256
+    tiles: same products, same order of addition, so the same bits — partial tiles in m and n, K-steps that are not
+    whole, one to seventeen steps, both code widths, grouped scales; and the oracle's tolerance on top."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    c = run_gemm(p, which=af.PREFILL_256X128)
+    assert_close_ulp(p, c, f"256x128 tiles: {m}x{n}x{k} bits={bits} g={group}")
+    assert np.array_equal(c, run_gemm(p, which=af.PREFILL_256))
+
+
+def test_tall_tiles_take_the_epilogues(af):
+    """A shape PREFILL runs on tiles of 256 rows x 128 columns, through the fused entry point: bias and residual, then the
+    SiLU gate (the kernel finishes 128 rows at a time from fp32 sums staged in LDS)."""
+    m, n, k = 2100, 2048, 320
+    assert af.variant(m, n, k) == af.PREFILL and (af.prefill_tile(m, n), af.prefill_tile_cols(m, n)) == (256, 128)
+    p = Problem(m, n, k, 8, 0, seed=71).with_bias().with_residual()
+    assert_close_ulp(p, run_gemm(p), "bias + residual")
+    g = gated_problem(m, n, k, 4, 64, seed=72).with_bias()
+    assert_close_gated(g, run_gemm(g, activation=af.ACT_SILU_GATE), "gated")
 
 
 @pytest.mark.parametrize("m,n,k,bits,group", [(130, 272, 1000, 8, 0), (256, 1040, 2048, 8, 64), (100, 528, 4096, 4, 128), (300, 272, 1088, 4, 0),
