@@ -56,7 +56,8 @@ RECORDED_TRAFFIC = {
     "m2048_n28672_k8192_int4_group128": (896485920, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
     "mid_m256_n4096_k4096_int8_perchannel": (35861798, "profiles/mid_m256_n4096_k4096_int8.txt"),
     "mid_m1024_n4096_k4096_int8_perchannel": (92417830, "profiles/mid_m1024_n4096_k4096_int8.txt"),
-    "mid_m256_n8192_k8192_int8_perchannel": (132209707, "profiles/mid_m256_n8192_k8192_int8.txt"),
+    "mid_m256_n8192_k8192_int8_perchannel": (131112016, "profiles/mid_m256_n8192_k8192_int8.txt"),
+    "mid_m2048_n4096_k4096_int8_perchannel": (168016523, "profiles/mid_m2048_n4096_k4096_int8.txt"),
 }
 
 # Parity counts RECORDED from the GPU test suite (tests/helpers.py: assert_close_ulp logs every check; tests/conftest.py
@@ -377,7 +378,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
-                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m256_n8192_k8192")
+                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM would shard over the columns "
