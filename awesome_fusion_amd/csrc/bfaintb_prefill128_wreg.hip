@@ -187,20 +187,27 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     struct Ops {
         uint32_t w[2][2][4];  // [block of 32 k][column j][dword]: the 8-element operand as 4 packed pairs
     };
-    // the two codes of a load, ready for the conversion: signed bytes (8-bit codes); two's-complement nibbles, the second
-    // shifted down to a low nibble (4-bit codes)
+    // the two codes of a load, ready for the conversion: as stored (8-bit codes: the excess of 128 comes off in the
+    // multiplication, see scaled()); two's-complement nibbles, the second shifted down to a low nibble (4-bit codes)
     auto prepare = [&](uint32_t x, uint32_t& c0, uint32_t& c1) {
         if constexpr (BITS == 8) {
-            c0 = x ^ 0x8080u;
-            c1 = c0;
+            c0 = x;
+            c1 = x;
         } else {
             c0 = x ^ 0x88u;
             c1 = c0 >> 4;
         }
     };
     auto value = [&](uint32_t c, uint32_t j) -> float {
-        if constexpr (BITS == 8) return j == 0 ? sbyte_to_f32<0>(c) : sbyte_to_f32<1>(c);
+        if constexpr (BITS == 8) return j == 0 ? (float)(c & 0xffu) : (float)((c >> 8) & 0xffu);  // v_cvt_f32_ubyte0 / 1
         else return nibble_to_f32_sixteenth<0>(c);
+    };
+    // value x scale.  8-bit codes: u s - 128 s in one fused operation — u s (8 x 8 bits), 128 s and their difference
+    // (u - 128) s are all exact in fp32, so this is the product q s of the signed code, bit for bit (a zero code gives +0
+    // where q s gives -0 for a negative scale: no sum can tell), and the sign flip of the codes is saved.
+    auto scaled = [&](float f, float scale) -> float {
+        if constexpr (BITS == 8) return __builtin_fmaf(f, scale, -128.0f * scale);
+        else return f * scale;
     };
     // one sixteenth of a step's conversion: rows 2 pr, 2 pr + 1 of column j of block blk
     auto convert_pair = [&](Ops& ops, const Raw& raw, uint32_t (&pre)[2][8][2], const float (&sc)[2][2], uint32_t blk, uint32_t j, uint32_t pr) {
@@ -208,7 +215,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             prepare(raw.d[blk][2 * pr], pre[blk][2 * pr][0], pre[blk][2 * pr][1]);
             prepare(raw.d[blk][2 * pr + 1], pre[blk][2 * pr + 1][0], pre[blk][2 * pr + 1][1]);
         }
-        ops.w[blk][j][pr] = pack_bf16_rne(value(pre[blk][2 * pr][j], j) * sc[blk][j], value(pre[blk][2 * pr + 1][j], j) * sc[blk][j]);
+        ops.w[blk][j][pr] = pack_bf16_rne(scaled(value(pre[blk][2 * pr][j], j), sc[blk][j]), scaled(value(pre[blk][2 * pr + 1][j], j), sc[blk][j]));
     };
     auto block_scales = [&](float (&sc)[2][2], const uint32_t (&sr)[2]) {
 #pragma unroll
@@ -320,7 +327,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             } else if (GROUPED && u == 6) {
                 group_scales(s2, kt2);
             }
-            nxt.w[cblk][cj][cpr] = pack_bf16_rne(f0 * sc[cblk][cj], f1 * sc[cblk][cj]);
+            nxt.w[cblk][cj][cpr] = pack_bf16_rne(scaled(f0, sc[cblk][cj]), scaled(f1, sc[cblk][cj]));
             __builtin_amdgcn_sched_barrier(0);
         }
     };

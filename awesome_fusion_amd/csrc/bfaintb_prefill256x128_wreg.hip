@@ -181,16 +181,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     struct Ops {
         uint32_t w[2][4][4];  // [block of 32 k][column j][dword]: the 8-element operand as 4 packed pairs
     };
-    // the four codes of a read, ready for the conversion: signed bytes (8-bit codes); two's-complement nibbles, columns 0
-    // and 2 in the low nibbles of bytes 0 and 1 of `e`, columns 1 and 3 likewise in `o` (4-bit codes)
+    // the four codes of a read, ready for the conversion: as stored (8-bit codes: the excess of 128 comes off in the
+    // multiplication, see scaled()); two's-complement nibbles, columns 0 and 2 in the low nibbles of bytes 0 and 1 of `e`,
+    // columns 1 and 3 likewise in `o` (4-bit codes)
     struct Pre {
         uint32_t e, o;
     };
     auto prepare = [&](uint32_t x) -> Pre {
         Pre q;
         if constexpr (BITS == 8) {
-            q.e = x ^ 0x80808080u;
-            q.o = q.e;
+            q.e = x;
+            q.o = x;
         } else {
             q.e = x ^ 0x8888u;
             q.o = q.e >> 4;
@@ -199,8 +200,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         return q;
     };
     auto value = [&](const Pre& q, uint32_t j) -> float {
-        if constexpr (BITS == 8) return j == 0 ? sbyte_to_f32<0>(q.e) : j == 1 ? sbyte_to_f32<1>(q.e) : j == 2 ? sbyte_to_f32<2>(q.e) : sbyte_to_f32<3>(q.e);
+        if constexpr (BITS == 8) return (float)((q.e >> (8u * j)) & 0xffu);  // v_cvt_f32_ubyte0 .. 3
         else return j == 0 ? nibble_to_f32_sixteenth<0>(q.e) : j == 1 ? nibble_to_f32_sixteenth<0>(q.o) : j == 2 ? nibble_to_f32_sixteenth<1>(q.e) : nibble_to_f32_sixteenth<1>(q.o);
+    };
+    // value x scale.  8-bit codes: u s - 128 s in one fused operation — u s (8 x 8 bits), 128 s and their difference
+    // (u - 128) s are all exact in fp32, so this is the product q s of the signed code, bit for bit (a zero code gives +0
+    // where q s gives -0 for a negative scale: no sum can tell), and the sign flip of the codes is saved.
+    auto scaled = [&](float f, float scale) -> float {
+        if constexpr (BITS == 8) return __builtin_fmaf(f, scale, -128.0f * scale);
+        else return f * scale;
     };
     auto block_scales = [&](float (&sc)[2][4], const ScaleRaw& sr) {
 #pragma unroll
@@ -224,7 +232,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             for (uint32_t pr = 0; pr < 4; ++pr) {
                 const Pre q0 = prepare(read_code(tile, blk, 2u * pr)), q1 = prepare(read_code(tile, blk, 2u * pr + 1u));
 #pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) ops.w[blk][j][pr] = pack_bf16_rne(value(q0, j) * sc[blk][j], value(q1, j) * sc[blk][j]);
+                for (uint32_t j = 0; j < 4; ++j) ops.w[blk][j][pr] = pack_bf16_rne(scaled(value(q0, j), sc[blk][j]), scaled(value(q1, j), sc[blk][j]));
             }
     };
 
@@ -321,7 +329,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 // ---- second slot
                 th_mfma(acc[mt][j1], a_now, wf1);
                 request(2u * u + h);
-                nxt.w[cblk][cj][cpr] = pack_bf16_rne(f0 * sc[cblk][cj], f1 * sc[cblk][cj]);
+                nxt.w[cblk][cj][cpr] = pack_bf16_rne(scaled(f0, sc[cblk][cj]), scaled(f1, sc[cblk][cj]));
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
