@@ -151,8 +151,8 @@ static bool use_small_tiles(int v, uint32_t m, uint32_t n)
 }
 
 // Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
-// k.  Small tiles: a K-step takes 0.62 us on an empty machine and 0.65 us with a workgroup on every CU with row-major
-// weights (the kernel that keeps them in registers; 0.74 and 0.75 us with 4-bit codes), 0.70 and 0.90 us with packed
+// k.  Small tiles: a K-step takes 0.49 us on an empty machine and 0.56 us with a workgroup on every CU with row-major
+// weights (the kernel that keeps them in registers; 0.64 and 0.67 us with 4-bit codes), 0.70 and 0.90 us with packed
 // weights (both operands through LDS).
 // The small-tile kernel over row-major weights may split k: grid y walks the splits, each workgroup runs its share of
 // the K-steps and the workgroup of the last split adds the others' sums (same workspace and protocol as the decode
@@ -181,13 +181,19 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         const uint32_t per = (ksteps + want - 1u) / want;
         t.k_per_wg = per * 64u;
         t.splits = (ksteps + per - 1u) / per;
-        // the hand-over: the producers' device-scope stores have to arrive (some 6 us after the last K-step), then the
+        // the hand-over: the producers' device-scope stores have to arrive (some 3 us after the last K-step), then the
         // reducing workgroup fetches a tile's worth of sums per split through its one CU, slower the more CUs do so at once
-        // (8-bit, n = k = 4096, us with 1 / 2 / 3 / 4 splits: m = 128: 43.4 / 31.1 / 27.5 / 28.3; m = 256: 43.9 / 31.7 /
-        // 28.5 / 29.4; m = 512: 44.3 / 32.9 / 44.1 / 42.3; 8192 x 8192, m = 256: 83.2 / 55.8 / 69.9 / 62.5)
-        const double hand_over = t.splits > 1u ? 2.0 + (t.splits - 1.0) * (3.6 + 0.007 * tiles) : 0.0;
-        // a K-step: 0.62 us (4-bit codes 0.74) on an empty machine, 0.65 (0.75) with a workgroup on every CU
-        t.us = 4.0 + per * ((bits == 4 ? 0.74 : 0.615) + 0.00013 * tiles * t.splits) + hand_over;
+        // (8-bit, n = k = 4096, us with 1 / 2 / 4 splits: m = 128: 35.2 / 27.3 / 26.6; m = 256: 35.6 / 27.8 / 28.6; m = 512:
+        // 35.9 / 30.0; 8192 x 8192, m = 256: 66.0 / 46.0; 4-bit g128, m = 256: 45.8 / 32.8 / 30.3)
+        const double hand_over = t.splits > 1u ? 3.5 + (t.splits - 1.0) * (3.6 + 0.007 * tiles) : 0.0;
+        // a K-step: 0.49 us (4-bit codes 0.64) on an empty machine, rising by 0.01 per 100 workgroups; with a workgroup on
+        // (nearly) every CU 8-bit codes take 0.56 (the clock gives way)
+        const double wgs = tiles * t.splits;
+        const double step_us = bits == 4 ? 0.64 + 0.0001 * wgs : 0.485 + 0.0001 * wgs + (wgs >= 240.0 ? 0.055 : 0.0);
+        t.us = 4.0 + per * step_us + hand_over;
+        // (three splits and more: the hand-over scatters more than this says, and where the row-blocked family is about as
+        // fast it is the safer pick — 192 x 4096 x 4096: 25.5 against 22.9 us, 128 x 4096 x 11008: 39.0 against 34.3)
+        if (t.splits > 2u) t.us *= 1.07;
         return t;
     };
     if (forced_splits) return shape(forced_splits);

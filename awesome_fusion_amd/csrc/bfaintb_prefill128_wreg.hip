@@ -38,6 +38,19 @@ constexpr uint32_t kTwStage = 128 * 128;  // bytes of one A stage
 constexpr uint32_t kTwCodeStage = 64 * 128;  // bytes of one stage of codes (8-bit; half of it used by 4-bit codes)
 
 __device__ __forceinline__ uint32_t tw_swz(uint32_t row, uint32_t chunk) { return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4); }
+
+// acc += a x b with the accumulator pinned to the accumulation registers and updated in place: written as assembly
+// because the compiler gives some of the kernel's matrix instructions a destination other than their source and copies
+// the sums back (21 of 224 instructions, 150 accumulator moves).  Behind the assembly its hazard bookkeeping sees
+// nothing, so: the operands are written long before (LDS reads and conversions, under wait counts the compiler does
+// insert for assembly operands); the accumulators are written by ordinary instructions only at the very start, with the
+// whole prologue between that and the first matrix instruction, and read by them only in the epilogue, behind explicit
+// idle cycles (tw_settle).
+__device__ __forceinline__ void tw_mfma(f32x4_t& acc, const bf16x8_t& a, const bf16x8_t& b)
+{
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void tw_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 }  // namespace
 
 template <int BITS, bool GROUPED>
@@ -305,7 +318,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][0][0], cur.w[blk][0][1], cur.w[blk][0][2], cur.w[blk][0][3]));
             const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][1][0], cur.w[blk][1][1], cur.w[blk][1][2], cur.w[blk][1][3]));
             // ---- slot 0
-            acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_now, wf0, acc[mt][0], 0, 0, 0);
+            tw_mfma(acc[mt][0], a_now, wf0);
             if (u + kAhead < 16) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
             else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - 16u) * 2048u);
             if (cj == 0 && u + 4 < 16) read_codes(u + 4);
@@ -317,7 +330,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             f1 = value(pre[cblk][2 * cpr + 1][cj], cj);
             __builtin_amdgcn_sched_barrier(0);
             // ---- slot 1
-            acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_now, wf1, acc[mt][1], 0, 0, 0);
+            tw_mfma(acc[mt][1], a_now, wf1);
             if (u < 4) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + u * 1024u), 16, (u & 1u) ? vo : ve,
                                                          (kbase + kt3) * kTwK * 2u + u * 16u * p.lda, 0, 0);
@@ -368,6 +381,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // ---- epilogue: fp32 sums -> LDS in [m][n] order (rows 32 q .. 32 q + 31 in the q-th array), then finish row-wise
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing asynchronous may still be writing LDS
+    tw_settle();                                       // the last matrix instructions have written their sums
     __syncthreads();                                   // ... and every wave is done reading the stages
     auto c_rows = [&](uint32_t q) -> float* {
         return reinterpret_cast<float*>(q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_a2 : lds_a3);
