@@ -23,7 +23,7 @@ hipError_t launch_pack_colmajor(uint8_t* dst, const uint8_t* src, uint32_t n, ui
 hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k, uint32_t ldb_bytes, int bits, bool unpack,
                        hipStream_t stream);
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream);
-hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream, bool wreg);
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, hipStream_t stream);
 bool prefill128_wreg_serves(const GemmParams& p);
@@ -931,7 +931,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
         if ((uint64_t)k * 256u * (uint32_t)weight_bits / 8u >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31))
             return BFAINTB_ERR_BAD_SHAPE;
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
-        return (int)bfaintb::launch_prefill_packed(p, weight_bits, st);
+        return (int)bfaintb::launch_prefill_packed(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
     if (!packed_uses_slab(m, n, k, weight_bits)) {
         // beyond a few dozen rows the row-blocked decode family (A reused across 128 or 256 columns) reads the packed

@@ -609,7 +609,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 }
 
 bool prefill_wreg_serves(const GemmParams& p);
-hipError_t launch_prefill_wreg(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 
 template <int BITS, bool GROUPED, bool PACKED, bool REF = false>
 static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream, bool wreg = false)
@@ -626,8 +626,8 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream, boo
         p.tile_count = whole;
         const uint32_t grid = (whole + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
         void (*whole_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 4, PACKED, REF>;
-        // whole tiles of row-major weights: the form that keeps the weights in registers, where it serves the launch
-        hipError_t e = (wreg && !PACKED && !REF && prefill_wreg_serves(p)) ? launch_prefill_wreg(p, BITS, stream)
+        // whole tiles: the form that keeps the weights in registers, where it serves the launch
+        hipError_t e = (wreg && !REF && prefill_wreg_serves(p)) ? launch_prefill_wreg(p, BITS, PACKED, stream)
                                                                            : launch_kernel(whole_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);
         if (e != hipSuccess) return e;
     }
@@ -650,11 +650,11 @@ hipError_t launch_prefill(const GemmParams& p, int bits, hipStream_t stream, boo
 }
 
 // The same kernel over weights in the packed order (p.b is the packed buffer; p.ldb_bytes is unused).
-hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream)
+hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream, bool wreg)
 {
     const bool grouped = p.group_size != 0;
-    if (bits == 8) return grouped ? launch_prefill_t<8, true, true>(p, stream) : launch_prefill_t<8, false, true>(p, stream);
-    return grouped ? launch_prefill_t<4, true, true>(p, stream) : launch_prefill_t<4, false, true>(p, stream);
+    if (bits == 8) return grouped ? launch_prefill_t<8, true, true>(p, stream, wreg) : launch_prefill_t<8, false, true>(p, stream, wreg);
+    return grouped ? launch_prefill_t<4, true, true>(p, stream, wreg) : launch_prefill_t<4, false, true>(p, stream, wreg);
 }
 
 }  // namespace bfaintb

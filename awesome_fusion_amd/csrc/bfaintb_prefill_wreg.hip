@@ -51,7 +51,7 @@ __device__ __forceinline__ void wreg_settle()
 }
 }  // namespace
 
-template <int BITS, bool GROUPED>
+template <int BITS, bool GROUPED, bool PACKED>
 __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmParams p)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kWrStageBytes];
@@ -95,9 +95,14 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
     const __amdgpu_buffer_rsrc_t rsrc_a =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)a_extent, kBufferFlags);
     const uint32_t cols_valid = p.n - n0 < kWrTile ? p.n - n0 : kWrTile;
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
-        kBufferFlags);
+    // packed weights: a block of 16 columns is one run of k x 16 codes (chunks of 1024 bytes: 64 rows of 8-bit, 128 rows of
+    // 4-bit codes); the tile's column blocks follow one another, and one past n reads as zero through the extent
+    const uint32_t slab_bytes = p.k * (BITS == 8 ? 16u : 8u);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b + (size_t)(n0 / 16u) * slab_bytes), 0,
+                                                   (int)(cols_valid / 16u * slab_bytes), kBufferFlags)
+               : __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0,
+                                                   (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)), kBufferFlags);
 
     const uint32_t ksteps = (p.k + kWrK - 1u) / kWrK;
     const uint32_t last_chunks = (p.k - (ksteps - 1u) * kWrK) / 8u;  // valid 16-byte chunks per row of A in the last step
@@ -121,66 +126,138 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
         __builtin_amdgcn_sched_barrier(0);  // the copy's requests stay ahead of the loads that follow: the wait below counts on it
     };
 
-    // W: this lane's 4 columns, rows 8 kq .. 8 kq + 7 of a block of 32 k
-    const uint32_t wcol = 64u * wave + 4u * c16;                 // within the tile
-    const uint32_t b_voff = 8u * kq * p.ldb_bytes + (BITS == 8 ? wcol : wcol / 2u);
-    const bool w_ok = n0 + wcol < p.n;
+    // W: this lane's 4 columns, rows 8 kq .. 8 kq + 7 of a block of 32 k.  Row-major weights: four neighbouring columns
+    // (one dword of a row holds them).  Packed weights: column c16 of each of the wave's four column blocks — the packed
+    // order gives lane 16 kq + c16 of a column block, in 16 bytes, exactly these rows of that column for the chunk's
+    // K-blocks (two for 8-bit codes = this step; four for 4-bit codes, of which a step takes 8 bytes).
+    const uint32_t wcol = PACKED ? 64u * wave + c16 : 64u * wave + 4u * c16;  // the lane's column j is wcol + kColStep * j
+    constexpr uint32_t kColStep = PACKED ? 16u : 1u;
+    const uint32_t b_voff = PACKED ? lane * 16u : 8u * kq * p.ldb_bytes + (BITS == 8 ? wcol : wcol / 2u);
+    const bool w_ok = n0 + wcol < p.n;  // (packed: the lane's four columns are whole column blocks apart, checked each on its own)
+    auto col_ok = [&](uint32_t j) { return n0 + wcol + kColStep * j < p.n; };
+    // packed: where column block j of this wave starts, and where a step's codes are within it
+    auto slab_off = [&](uint32_t j) { return (4u * wave + j) * slab_bytes; };
+    auto step_off = [&](uint32_t kt) { return BITS == 8 ? kt * 1024u : (kt >> 1) * 1024u + (kt & 1u) * 8u; };
     struct Raw {
-        uint32_t d[2][8];   // [block of 32 k][row]
-        uint32_t s[2][2];   // grouped scales of the two blocks: 4 bf16 each
+        // row-major: [block of 32 k][row] (8-bit: a dword of four columns; 4-bit: 16 bits)
+        // packed: [block][2 j + half] = rows 4 half .. + 3 of column j (8-bit); [block][j] = the 8 rows of column j (4-bit)
+        uint32_t d[2][8];
+        uint32_t s[2][PACKED ? 4 : 2];  // grouped scales of the two blocks: row-major 4 bf16 in two dwords, packed one each
+    };
+    // packed: the codes of column block j for step kt, one request
+    auto gload_packed = [&](Raw& raw, uint32_t kt, uint32_t j) {
+        if constexpr (BITS == 8) {
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, b_voff, slab_off(j) + step_off(kt), 0);
+            raw.d[0][2 * j] = v[0], raw.d[0][2 * j + 1] = v[1], raw.d[1][2 * j] = v[2], raw.d[1][2 * j + 1] = v[3];
+        } else {
+            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_b, b_voff, slab_off(j) + step_off(kt), 0);
+            raw.d[0][j] = v[0], raw.d[1][j] = v[1];
+        }
+    };
+    // Scales go through a buffer resource so that the load is issued whatever the lane's column (the wait counts
+    // below count requests): columns past n read other columns' scales, or zero beyond the array; their results are
+    // never stored.
+    const uint32_t scale_rows = GROUPED ? p.k / p.group_size : 1u;
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.scale), 0, (int)(((scale_rows - 1u) * p.lds + p.n) * 2u), kBufferFlags);
+    const uint32_t s_voff = (n0 + wcol) * 2u;
+    // the grouped scales of block blk of step kt (packed: of the lane's column j alone)
+    auto load_group_scales = [&](Raw& raw, uint32_t kt, uint32_t blk, uint32_t j = 0) {
+        uint32_t g = (kt * kWrK + 32u * blk) / p.group_size;
+        if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
+        if constexpr (PACKED) {
+            raw.s[blk][j] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_s, s_voff, g * p.lds * 2u + 32u * j, 0);
+        } else {
+            const u32x2_t sr = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, s_voff, g * p.lds * 2u, 0);
+            raw.s[blk][0] = sr[0];
+            raw.s[blk][1] = sr[1];
+        }
     };
     auto gload = [&](Raw& raw, uint32_t kt) {
+        if constexpr (PACKED) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) gload_packed(raw, kt, j);
+        }
 #pragma unroll
         for (uint32_t blk = 0; blk < 2; ++blk) {
-            const uint32_t row0 = (kt * kWrK + 32u * blk) * p.ldb_bytes;
+            if constexpr (!PACKED) {
+                const uint32_t row0 = (kt * kWrK + 32u * blk) * p.ldb_bytes;
 #pragma unroll
-            for (uint32_t r = 0; r < 8; ++r) {
-                if constexpr (BITS == 8) raw.d[blk][r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
-                else raw.d[blk][r] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
+                for (uint32_t r = 0; r < 8; ++r) {
+                    if constexpr (BITS == 8) raw.d[blk][r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
+                    else raw.d[blk][r] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_b, b_voff, row0 + r * p.ldb_bytes, 0);
+                }
             }
             if constexpr (GROUPED) {
-                uint32_t g = (kt * kWrK + 32u * blk) / p.group_size;
-                const uint32_t groups = p.k / p.group_size;
-                if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do
-                uint2 sr = make_uint2(0, 0);
-                if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + n0 + wcol);
-                raw.s[blk][0] = sr.x;
-                raw.s[blk][1] = sr.y;
+                if constexpr (PACKED) {
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; ++j) load_group_scales(raw, kt, blk, j);
+                } else {
+                    load_group_scales(raw, kt, blk);
+                }
             }
         }
     };
     float cs[4];
     if constexpr (!GROUPED) {
-        uint2 sr = make_uint2(0, 0);
-        if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + n0 + wcol);
-        cs[0] = make_col_scale<BITS>(sr.x & 0xffffu);
-        cs[1] = make_col_scale<BITS>(sr.x >> 16);
-        cs[2] = make_col_scale<BITS>(sr.y & 0xffffu);
-        cs[3] = make_col_scale<BITS>(sr.y >> 16);
+        if constexpr (PACKED) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) cs[j] = make_col_scale<BITS>(__builtin_amdgcn_raw_buffer_load_b16(rsrc_s, s_voff, 32u * j, 0));
+        } else {
+            const u32x2_t sr = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, s_voff, 0, 0);
+            cs[0] = make_col_scale<BITS>(sr[0] & 0xffffu);
+            cs[1] = make_col_scale<BITS>(sr[0] >> 16);
+            cs[2] = make_col_scale<BITS>(sr[1] & 0xffffu);
+            cs[3] = make_col_scale<BITS>(sr[1] >> 16);
+        }
     }
     struct Ops {
         bf16x8_t w[2][4];  // [block of 32 k][column j]
+    };
+    // byte `col` (a compile-time value at every call site) of a dword of signed bytes, as fp32
+    auto sbyte_sel = [&](uint32_t x, uint32_t col) -> float {
+        return col == 0 ? sbyte_to_f32<0>(x) : col == 1 ? sbyte_to_f32<1>(x) : col == 2 ? sbyte_to_f32<2>(x) : sbyte_to_f32<3>(x);
+    };
+    // The signed bytes of a block, s8[8].  Row-major: s8[r] = row r of the lane's 8, byte j = column j.  Packed: s8[2 j + h]
+    // = column j, byte t = row 4 h + t.  weight(s8, r, j): row r of column j as fp32 (r and j compile-time at every call).
+    auto weight = [&](const uint32_t (&s8)[8], uint32_t r, uint32_t j) -> float {
+        return PACKED ? sbyte_sel(s8[2u * j + (r >> 2)], r & 3u) : sbyte_sel(s8[r], j);
+    };
+    // entry e of s8 from the raw codes of block BLK
+    auto signed_bytes = [&](const Raw& raw, auto blk_c, uint32_t e) -> uint32_t {
+        constexpr int BLK = decltype(blk_c)::value;
+        if constexpr (BITS == 8) return codes8_to_s8(raw.d[BLK][e]);
+        else if constexpr (PACKED) return codes4_quad_to_s8x16(raw.d[BLK][e >> 1] >> (16u * (e & 1u)));  // 8 codes of a column: 4 per entry
+        else return codes4_quad_to_s8x16(raw.d[BLK][e]);
+    };
+    auto block_scales = [&](float (&sc)[4], const Raw& raw, auto blk_c) {
+        constexpr int BLK = decltype(blk_c)::value;
+        if constexpr (PACKED) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sc[j] = make_col_scale<BITS>(raw.s[BLK][j]);
+        } else {
+            sc[0] = make_col_scale<BITS>(raw.s[BLK][0] & 0xffffu);
+            sc[1] = make_col_scale<BITS>(raw.s[BLK][0] >> 16);
+            sc[2] = make_col_scale<BITS>(raw.s[BLK][1] & 0xffffu);
+            sc[3] = make_col_scale<BITS>(raw.s[BLK][1] >> 16);
+        }
     };
     // one column of one block: 8 weights -> operand
     auto convert_col = [&](Ops& ops, const uint32_t (&s8)[8], const float (&sc)[4], auto blk_c, auto j_c) {
         constexpr int BLK = decltype(blk_c)::value, J = decltype(j_c)::value;
         uint4 w;
-        w.x = pack_bf16_rne(sbyte_to_f32<J>(s8[0]) * sc[J], sbyte_to_f32<J>(s8[1]) * sc[J]);
-        w.y = pack_bf16_rne(sbyte_to_f32<J>(s8[2]) * sc[J], sbyte_to_f32<J>(s8[3]) * sc[J]);
-        w.z = pack_bf16_rne(sbyte_to_f32<J>(s8[4]) * sc[J], sbyte_to_f32<J>(s8[5]) * sc[J]);
-        w.w = pack_bf16_rne(sbyte_to_f32<J>(s8[6]) * sc[J], sbyte_to_f32<J>(s8[7]) * sc[J]);
+        w.x = pack_bf16_rne(weight(s8, 0, J) * sc[J], weight(s8, 1, J) * sc[J]);
+        w.y = pack_bf16_rne(weight(s8, 2, J) * sc[J], weight(s8, 3, J) * sc[J]);
+        w.z = pack_bf16_rne(weight(s8, 4, J) * sc[J], weight(s8, 5, J) * sc[J]);
+        w.w = pack_bf16_rne(weight(s8, 6, J) * sc[J], weight(s8, 7, J) * sc[J]);
         ops.w[BLK][J] = __builtin_bit_cast(bf16x8_t, w);
     };
-    // the raw rows of one block -> signed bytes, and the block's four column scales
+    // the raw codes of one block -> signed bytes, and the block's four column scales
     auto prepare_block = [&](uint32_t (&s8)[8], float (&sc)[4], const Raw& raw, auto blk_c) {
-        constexpr int BLK = decltype(blk_c)::value;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) s8[r] = BITS == 8 ? codes8_to_s8(raw.d[BLK][r]) : codes4_quad_to_s8x16(raw.d[BLK][r]);
+        for (int e = 0; e < 8; ++e) s8[e] = signed_bytes(raw, blk_c, e);
         if constexpr (GROUPED) {
-            sc[0] = make_col_scale<BITS>(raw.s[BLK][0] & 0xffffu);
-            sc[1] = make_col_scale<BITS>(raw.s[BLK][0] >> 16);
-            sc[2] = make_col_scale<BITS>(raw.s[BLK][1] & 0xffffu);
-            sc[3] = make_col_scale<BITS>(raw.s[BLK][1] >> 16);
+            block_scales(sc, raw, blk_c);
         } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) sc[j] = cs[j];
@@ -194,27 +271,6 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
         convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 1>{});
         convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 2>{});
         convert_col(ops, s8, sc, blk_c, std::integral_constant<int, 3>{});
-    };
-
-    // byte `col` (a compile-time value at every call site) of a dword of signed bytes, as fp32
-    auto sbyte_sel = [&](uint32_t x, uint32_t col) -> float {
-        return col == 0 ? sbyte_to_f32<0>(x) : col == 1 ? sbyte_to_f32<1>(x) : col == 2 ? sbyte_to_f32<2>(x) : sbyte_to_f32<3>(x);
-    };
-    auto load_group_scales = [&](Raw& raw, uint32_t kt, uint32_t blk) {
-        uint32_t g = (kt * kWrK + 32u * blk) / p.group_size;
-        const uint32_t groups = p.k / p.group_size;
-        if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do
-        uint2 sr = make_uint2(0, 0);
-        if (w_ok) sr = *reinterpret_cast<const uint2*>(p.scale + (size_t)g * p.lds + n0 + wcol);
-        raw.s[blk][0] = sr.x;
-        raw.s[blk][1] = sr.y;
-    };
-    auto block_scales = [&](float (&sc)[4], const Raw& raw, auto blk_c) {
-        constexpr int BLK = decltype(blk_c)::value;
-        sc[0] = make_col_scale<BITS>(raw.s[BLK][0] & 0xffffu);
-        sc[1] = make_col_scale<BITS>(raw.s[BLK][0] >> 16);
-        sc[2] = make_col_scale<BITS>(raw.s[BLK][1] & 0xffffu);
-        sc[3] = make_col_scale<BITS>(raw.s[BLK][1] >> 16);
     };
 
     f32x4_t acc[16][4];
@@ -271,14 +327,17 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                     }
                     if (j == 1) {  // (the five instructions of a quarter column are split 3 + 2 over slots j = 1 and j = 3)
                         const uint32_t col = g & 3u;
-                        f_lo = sbyte_sel(s8[2 * i], col) * sc[col];
-                        f_hi = sbyte_sel(s8[2 * i + 1], col);
+                        f_lo = weight(s8, 2 * i, col) * sc[col];
+                        f_hi = weight(s8, 2 * i + 1, col);
                     }
                     if (j == 2) {
                         const uint32_t q = 4u * g + i;  // 0..31
                         if (q < 8) {
                             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16,
                                                                      (q & 1u) ? a_vo : a_ve, kt2 * kWrK * 2u + q * 16u * p.lda, 0, 0);
+                        } else if constexpr (PACKED) {  // 4 requests for the codes, then 8 for the scales
+                            if (q < 12) gload_packed(raw2, kt2, q - 8u);
+                            else if (GROUPED && q < 20) load_group_scales(raw2, kt2, (q - 12u) >> 2, (q - 12u) & 3u);
                         } else if (q < 24) {
                             const uint32_t lb = (q - 8u) >> 3, r = (q - 8u) & 7u;
                             const uint32_t soff = (kt2 * kWrK + 32u * lb + r) * p.ldb_bytes;
@@ -290,10 +349,11 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                     }
                     if (j == 3) wq[blk][g & 3u][i] = pack_bf16_rne(f_lo, f_hi * sc[g & 3u]);
                     if (j == 3 && g == 3) {
-                        // block 1's codes made signed, two rows per slot, into the half of s8 whose conversion is done
-                        // (rows 2 i, 2 i + 1 of block 0 were last used by slot (3, i, 1))
-                        s8[2 * i] = BITS == 8 ? codes8_to_s8(raw1.d[1][2 * i]) : codes4_quad_to_s8x16(raw1.d[1][2 * i]);
-                        s8[2 * i + 1] = BITS == 8 ? codes8_to_s8(raw1.d[1][2 * i + 1]) : codes4_quad_to_s8x16(raw1.d[1][2 * i + 1]);
+                        // block 1's codes made signed, two entries per slot, into the part of s8 whose conversion is done
+                        // (row-major: rows 2 i, 2 i + 1 of block 0 were last used by slot (3, i, 1); packed: column i of
+                        // block 0 was converted in group i, its last rows by slot (i, 3, 1))
+                        s8[2 * i] = signed_bytes(raw1, B1{}, 2 * i);
+                        s8[2 * i + 1] = signed_bytes(raw1, B1{}, 2 * i + 1);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -306,7 +366,9 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                 // it every wave's part has: the next step's first fragments can be fetched at the end of this one, and the
                 // copy this step started (into the stage read two steps ago) overwrites nothing a wave still reads — every
                 // wave that reaches this barrier has passed the previous one, i.e. finished the step before it.
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((GROUPED ? 18 : 16) + 16) : "memory");
+                // (row-major: 16 loads of codes and 2 of scales per step, 8 of the codes before this point; packed: 4 of codes
+                // and 8 of scales, 4 + 4 of them before this point)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PACKED ? (GROUPED ? 12 + 16 : 4 + 12) : (GROUPED ? 18 : 16) + 16) : "memory");
                 barrier_no_fence();  // (a fenced barrier would also wait for the copy this step has just started)
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -327,7 +389,7 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
     convert_block(ops0, rawa, B0{});
     convert_block(ops0, rawa, B1{});
     gload(rawa, ksteps > 1 ? 1 : 0);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GROUPED ? 18 : 16) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PACKED ? (GROUPED ? 12 : 4) : (GROUPED ? 18 : 16)) : "memory");
     __syncthreads();
 #pragma unroll
     for (uint32_t i = 0; i < 4; ++i) af[0][i] = read_frag(C0{}, 0, i);
@@ -355,13 +417,23 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
         // the bare sums, or sums + bias: rounded in registers, staged as bf16 (rows 64 q .. 64 q + 63 in the q-th array)
         float bias[4] = {0.f, 0.f, 0.f, 0.f};
         const bool has_bias = p.bias != nullptr;
-        if (has_bias && w_ok) {
+        if constexpr (PACKED) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (has_bias && col_ok(j)) bias[j] = bf16_bits_to_f32(p.bias[n0 + wcol + kColStep * j]);
+        } else if (has_bias && w_ok) {
             const uint2 raw = *reinterpret_cast<const uint2*>(p.bias + n0 + wcol);
             bias[0] = bf16_bits_to_f32(raw.x & 0xffffu);
             bias[1] = bf16_bits_to_f32(raw.x >> 16);
             bias[2] = bf16_bits_to_f32(raw.y & 0xffffu);
             bias[3] = bf16_bits_to_f32(raw.y >> 16);
         }
+        // Packed weights: a lane's four columns are 16 apart, so it stages four single values per row, and the four
+        // k-groups of a wave (rows 4 apart: the same banks) would collide; the 32-byte groups of a row are therefore
+        // stored at position (group ^ ((row >> 2) & 3)), which the readers below undo.
+        uint32_t pk_base[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) pk_base[j] = 4u * kq * kWrCRowBytes + (((4u * wave + j) ^ kq) << 5) + c16 * 2u;
 #pragma unroll
         for (uint32_t mt = 0; mt < 16; ++mt) {
             uint8_t* base = c_rows(mt >> 2);
@@ -377,7 +449,15 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
                     o.x = pack_bf16_rne(acc[mt][0][r], acc[mt][1][r]);
                     o.y = pack_bf16_rne(acc[mt][2][r], acc[mt][3][r]);
                 }
-                *reinterpret_cast<uint2*>(base + row * kWrCRowBytes + wcol * 2u) = o;
+                if constexpr (PACKED) {
+                    uint8_t* at = base + (16u * (mt & 3u) + r) * kWrCRowBytes;  // + the lane's part, in pk_base
+                    *reinterpret_cast<uint16_t*>(at + pk_base[0]) = (uint16_t)(o.x & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(at + pk_base[1]) = (uint16_t)(o.x >> 16);
+                    *reinterpret_cast<uint16_t*>(at + pk_base[2]) = (uint16_t)(o.y & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(at + pk_base[3]) = (uint16_t)(o.y >> 16);
+                } else {
+                    *reinterpret_cast<uint2*>(base + row * kWrCRowBytes + wcol * 2u) = o;
+                }
             }
         }
         __syncthreads();
@@ -387,7 +467,8 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
             const uint32_t ch = tid & 31u;
             const uint32_t gm = m0 + row, gn = n0 + ch * 8u;
             if (gm < p.m && gn < p.n) {
-                const uint4 v = *reinterpret_cast<const uint4*>(c_rows(row >> 6) + (row & 63u) * kWrCRowBytes + ch * 16u);
+                const uint32_t at = PACKED ? ((((ch >> 1) ^ ((row >> 2) & 3u)) << 5) + (ch & 1u) * 16u) : ch * 16u;
+                const uint4 v = *reinterpret_cast<const uint4*>(c_rows(row >> 6) + (row & 63u) * kWrCRowBytes + at);
                 *reinterpret_cast<uint4*>(p.c + (size_t)gm * p.ldc + gn) = v;
             }
         }
@@ -419,7 +500,12 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
 #pragma unroll
             for (uint32_t r = 0; r < 4; ++r) {
                 const uint32_t row = 16u * (mh & 1u) + 4u * kq + r;  // within the 32 rows of this array
-                *reinterpret_cast<float4*>(base + row * kWrTile + wcol) = make_float4(acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]);
+                if constexpr (PACKED) {
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; ++j) base[row * kWrTile + wcol + kColStep * j] = acc[mt][j][r];
+                } else {
+                    *reinterpret_cast<float4*>(base + row * kWrTile + wcol) = make_float4(acc[mt][0][r], acc[mt][1][r], acc[mt][2][r], acc[mt][3][r]);
+                }
             }
         }
         __syncthreads();
@@ -462,22 +548,29 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
 }
 
 // Runs `tile_count` whole 256x256 tiles from `tile_first` on (the caller splits off a last, thin round for the half-tile kernel).
-template <int BITS, bool GROUPED>
+template <int BITS, bool GROUPED, bool PACKED>
 static hipError_t launch_wreg_t(const GemmParams& p, hipStream_t stream)
 {
     const uint32_t grid = (p.tile_count + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    void (*kernel)(const GemmParams) = bfaintb_prefill_wreg_kernel<BITS, GROUPED>;
+    void (*kernel)(const GemmParams) = bfaintb_prefill_wreg_kernel<BITS, GROUPED, PACKED>;
     return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
 }
 
-// Whether this kernel can serve a launch: row-major weights (the caller's business), this library's own arithmetic.
+// Whether this kernel can serve a launch: this library's own arithmetic (either order of the weights).
 bool prefill_wreg_serves(const GemmParams& p) { return !p.reference_arith; }
 
-hipError_t launch_prefill_wreg(const GemmParams& p, int bits, hipStream_t stream)
+template <bool PACKED>
+static hipError_t launch_wreg_order(const GemmParams& p, int bits, hipStream_t stream)
 {
     const bool grouped = p.group_size != 0;
-    if (bits == 8) return grouped ? launch_wreg_t<8, true>(p, stream) : launch_wreg_t<8, false>(p, stream);
-    return grouped ? launch_wreg_t<4, true>(p, stream) : launch_wreg_t<4, false>(p, stream);
+    if (bits == 8) return grouped ? launch_wreg_t<8, true, PACKED>(p, stream) : launch_wreg_t<8, false, PACKED>(p, stream);
+    return grouped ? launch_wreg_t<4, true, PACKED>(p, stream) : launch_wreg_t<4, false, PACKED>(p, stream);
+}
+
+// packed: p.b is the buffer in the packed order (p.ldb_bytes is unused)
+hipError_t launch_prefill_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream)
+{
+    return packed ? launch_wreg_order<true>(p, bits, stream) : launch_wreg_order<false>(p, bits, stream);
 }
 
 }  // namespace bfaintb

@@ -168,6 +168,36 @@ def test_tile_sizes_and_weight_orders_agree_bit_for_bit(af, m, n, k, bits, group
     assert np.array_equal(run_prepacked(af, p, af.PREFILL_128), run_prepacked(af, p, af.PREFILL_256))
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [(100, 1040, 320, 8, 0), (128, 272, 448, 8, 64), (60, 528, 512, 4, 128), (100, 1040, 384, 4, 0),
+                                              (17, 48, 128, 4, 64), (2064, 4096, 256, 8, 0), (520, 16512, 256, 4, 128), (2100, 4112, 192, 8, 32)])
+def test_large_tiles_keep_packed_weights_in_registers_too(af, m, n, k, bits, group):
+    """Whole 256x256 tiles over packed weights run the kernel that converts the weights into operand registers (a lane
+    takes its operands from the packed order as they are stored; its four columns are 16 apart): against the oracle, and
+    bit for bit against the form with both operands in LDS and against the row-major path.  Shapes whose tiles run whole:
+    up to 128 rows of A, or more than 128 tiles in the last round; partial tiles in m and n, odd numbers of K-steps."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    c = run_prepacked(af, p, af.PREFILL_256)
+    assert_close_ulp(p, c, f"packed, 256x256 tiles, weights in registers: {m}x{n}x{k} bits={bits} g={group}")
+    assert np.array_equal(c, run_prepacked(af, p, af.PREFILL_256_LDS))
+    assert np.array_equal(c, run_gemm(p, which=af.PREFILL_256))
+    p.with_bias()
+    c = run_prepacked(af, p, af.PREFILL_256)
+    assert_close_ulp(p, c, f"... + bias: {m}x{n}x{k} bits={bits} g={group}")
+    assert np.array_equal(c, run_prepacked(af, p, af.PREFILL_256_LDS))
+
+
+@pytest.mark.parametrize("m,n,k,bits,group", [(2064, 4112, 192, 8, 0), (2100, 4128, 128, 4, 128)])
+def test_large_tiles_over_packed_weights_take_the_epilogues(af, m, n, k, bits, group):
+    """Shapes the library runs on whole 256x256 tiles by itself (the fused entry point takes no forced variant): 9 x 17 of
+    them, the last ones partial in m and n."""
+    assert af.prepacked_variant(m, n, k, bits, group) == af.PREFILL and af.prefill_tile(m, n) == 256
+    p = Problem(m, n, k, bits, group, seed=m + k).with_bias().with_residual()
+    assert_close_ulp(p, run_prepacked(af, p), f"packed, 256x256 tiles, bias + residual {m}x{n}x{k}")
+    g = Problem(m, n, k, bits, group, seed=m + k + 1, scale_lo=0.002, scale_hi=0.02 if bits == 8 else 0.2).with_bias()
+    g.residual_bf = oracle.f32_to_bf16_rne(np.random.default_rng(5).uniform(-2, 2, size=(m, n // 2)).astype(np.float32))
+    assert_close_gated(g, run_prepacked(af, g, activation=af.ACT_SILU_GATE), f"packed, 256x256 tiles, gated {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("bits,group", [(8, 0), (4, 128)])
 @pytest.mark.parametrize("which,m", [(1, 16), (1, 32), (1, 64), (3, 64), (4, 64)])
 def test_kernels_dequantise_bit_exact(af, bits, group, which, m):
