@@ -25,7 +25,7 @@ hipError_t launch_pack(uint8_t* dst, const uint8_t* src, uint32_t n, uint32_t k,
 hipError_t launch_decode_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stream, bool wreg);
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
-hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 bool prefill128_wreg_serves(const GemmParams& p);
 hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
@@ -151,10 +151,9 @@ static bool use_small_tiles(int v, uint32_t m, uint32_t n)
 }
 
 // Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
-// k.  Small tiles: a K-step takes 0.49 us on an empty machine and 0.56 us with a workgroup on every CU with row-major
-// weights (the kernel that keeps them in registers; 0.64 and 0.67 us with 4-bit codes), 0.70 and 0.90 us with packed
-// weights (both operands through LDS).
-// The small-tile kernel over row-major weights may split k: grid y walks the splits, each workgroup runs its share of
+// k.  Small tiles: a K-step takes 0.49 us on an empty machine and 0.56 us with a workgroup on every CU (the kernel that
+// keeps the weights in registers; 0.64 and 0.67 us with 4-bit codes), whichever order the weights are stored in.
+// The small-tile kernel may split k: grid y walks the splits, each workgroup runs its share of
 // the K-steps and the workgroup of the last split adds the others' sums (same workspace and protocol as the decode
 // family).  Worth it while tiles x splits still fit one workgroup per CU.
 struct TilePlan {
@@ -210,13 +209,9 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
     return best;
 }
 
-static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits, bool packed = false)
+static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
-    if (prefill_small_tiles(m, n)) {
-        const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
-        if (!packed) return tile128_plan(m, n, k, bits, 0).us;
-        return 4.0 + (k / 64.0) * (0.70 + 0.0008 * tiles);
-    }
+    if (prefill_small_tiles(m, n)) return tile128_plan(m, n, k, bits, 0).us;
     const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
     const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
     return 4.0 + rounds * (k / 64.0) * 1.33;
@@ -710,7 +705,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
         if (e) return e;
     }
     if (tiled) {
-        if (small_wreg) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, st);
+        if (small_wreg) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, false, st);
         if ((v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) && !p.reference_arith)
             return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, st);
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
@@ -857,7 +852,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (packed_uses_slab(m, n, k, bits)) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
-    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits, true) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
@@ -871,10 +866,12 @@ int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weigh
     return packed_variant(m, n, k, weight_bits, BFAINTB_VARIANT_AUTO);
 }
 
-// Scratch of the packed path: only the decode family (where the slab kernel is not used) splits along k.
+// Scratch of the packed path: the decode family (where the slab kernel is not used) and the small tiles split along k.
 static size_t packed_workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int v)
 {
-    if (v != BFAINTB_VARIANT_DECODE || m == 0 || n == 0 || packed_uses_slab(m, n, k, bits)) return 0;
+    if (m == 0 || n == 0) return 0;
+    if (is_prefill(v)) return tiled_may_split(v, m, n) ? split_workspace_bytes(tile128_plan(m, n, k, bits, 0).splits, m, n) : 0;
+    if (v != BFAINTB_VARIANT_DECODE || packed_uses_slab(m, n, k, bits)) return 0;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
     if (pl.splits <= 1) return 0;
     return bfaintb::kWorkspaceHeaderBytes + ((((size_t)(pl.splits - 1u) * m * n * sizeof(float)) + 255u) & ~(size_t)255u);
@@ -930,6 +927,18 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
         // a tile's 16 column blocks and a 256-row panel of A are addressed through 32-bit buffer extents
         if ((uint64_t)k * 256u * (uint32_t)weight_bits / 8u >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31))
             return BFAINTB_ERR_BAD_SHAPE;
+        if (tiled_may_split(v, m, n) && bfaintb::prefill128_wreg_serves(p)) {
+            // small tiles: the kernel that keeps the weights in registers, with the plan (split along k included) and the
+            // workspace protocol of the row-major path
+            const TilePlan tp = tile128_plan(m, n, k, weight_bits, 0);
+            p.k_per_wg = tp.k_per_wg;
+            p.splits = tp.splits;
+            if (p.splits > 1) {
+                e = attach_workspace(p, workspace, workspace_bytes, packed_workspace_need(m, n, k, weight_bits, v));
+                if (e) return e;
+            }
+            return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, true, st);
+        }
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }

@@ -266,8 +266,8 @@ BFAINTB_API int bfaintb_gemm_prepacked_fused(void* c, const void* a, const void*
                                  const bfaintb_epilogue* epilogue, uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc,
                                  int weight_bits, uint32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
 /* Scratch bfaintb_gemm_prepacked needs: 0 where the slab-streaming kernel runs (8-bit codes: m <= 8, m <= 32 when n * k <= 16 Mi and
- * n >= 4096, never when n < 2048 and k >= 12288; 4-bit codes: m <= 48 while n * k <= 24 Mi (m <= 20 when n < 2048 and k >= 12288), m <= 24 below 64 Mi, m <= 8 beyond; 8-bit: m <= 4 beyond 96 Mi) and for the tiled kernels; in between, what the decode family needs when it splits along k:
- * always ask, for the shape at hand.  Same workspace protocol as bfaintb_gemm
+ * n >= 4096, never when n < 2048 and k >= 12288; 4-bit codes: m <= 48 while n * k <= 24 Mi (m <= 20 when n < 2048 and k >= 12288), m <= 24 below 64 Mi, m <= 8 beyond; 8-bit: m <= 4 beyond 96 Mi) and for the large tiles; otherwise what the decode family or the
+ * 128x128 tiles need when they split along k (the plan of the row-major path): always ask, for the shape at hand.  Same workspace protocol as bfaintb_gemm
  * (bfaintb_workspace_init once; one workspace may serve both entry points). */
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
