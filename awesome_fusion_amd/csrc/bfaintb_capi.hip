@@ -841,6 +841,11 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
     return decode_plan_row_blocks(m, n, k, bits, 0, true);
 }
 
+// The family's estimate against the tiles', over packed weights: scaled by what a scan of 11 weight shapes x 9 values of m
+// (96 .. 2048) x both code widths fits best — with these the pick is within 3 % of the best form on 185 of 190 shapes, worst
+// 8 % (8-bit, 128 x 5120 x 13824); with the row-major path's 0.76 for 4-bit codes the family was picked 22 % too slow at
+// 256 x 4096 x 4096 (its kernels over packed 4-bit codes have no 8-wave form).
+constexpr double kPackedFamily8Bit = 0.95, kPackedFamily4Bit = 0.85;
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the
 // row-blocked family without a split along k beyond) or the tiled kernel, by the estimates that choose for row-major weights.
 static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
@@ -849,10 +854,11 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (variant == BFAINTB_VARIANT_PREFILL_256X128) return BFAINTB_ERR_BAD_VARIANT;  // (row-major weights only)
     if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
-    if (packed_uses_slab(m, n, k, bits)) return BFAINTB_VARIANT_DECODE;
+    if (packed_uses_slab(m, n, k, bits) || m <= 64u) return BFAINTB_VARIANT_DECODE;  // (up to 64 rows: as for row-major weights)
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
-    return decode_family_estimate_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    const double family = decode_family_estimate_us(m, n, k, bits, pl) * (bits == 4 ? kPackedFamily4Bit : kPackedFamily8Bit);
+    return family < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)
