@@ -27,7 +27,7 @@ hipError_t launch_prefill_packed(const GemmParams& p, int bits, hipStream_t stre
 hipError_t launch_prefill128(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 hipError_t launch_prefill128_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 bool prefill128_wreg_serves(const GemmParams& p);
-hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, hipStream_t stream);
+hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream);
 hipError_t decode_prepare_device();
 }  // namespace bfaintb
@@ -707,7 +707,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     if (tiled) {
         if (small_wreg) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, false, st);
         if ((v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) && !p.reference_arith)
-            return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, st);
+            return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, false, st);
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
         return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
@@ -851,7 +851,6 @@ constexpr double kPackedFamily8Bit = 0.95, kPackedFamily4Bit = 0.85;
 static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
-    if (variant == BFAINTB_VARIANT_PREFILL_256X128) return BFAINTB_ERR_BAD_VARIANT;  // (row-major weights only)
     if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
     if (packed_uses_slab(m, n, k, bits) || m <= 64u) return BFAINTB_VARIANT_DECODE;  // (up to 64 rows: as for row-major weights)
@@ -944,6 +943,11 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
                 if (e) return e;
             }
             return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, true, st);
+        }
+        if (v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) {
+            p.k_per_wg = k;
+            p.splits = 1;
+            return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, true, st);
         }
         if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);

@@ -1,4 +1,5 @@
-// Tiled variant, 128x128 tiles, weights kept in registers: the form of the small-tile kernel for row-major B.
+// Tiled variant, 128x128 tiles, weights kept in registers: the small-tile kernel, for row-major B (described first) and
+// for B in the packed order (PACKED: what changes is said where the codes are copied and read).
 //
 // Same job and the same reference kernel replaced as bfaintb_prefill128_kernel
 // (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:184-630; the reference's own tile is 32 x 64,

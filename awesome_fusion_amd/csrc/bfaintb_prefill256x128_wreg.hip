@@ -12,7 +12,8 @@
 //   four column groups; around them the fragment of four units ahead, the code reads and the conversion of the next
 //   step's weights (two pairs per unit) and two memory requests.
 // Same reference kernel replaced (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:184-630), same order of addition
-// per output as every other tiled kernel here (ascending k), so the same bits.  No split along k.
+// per output as every other tiled kernel here (ascending k), so the same bits.  No split along k.  Row-major B, or B in
+// the packed order (PACKED: what changes is said where the codes are copied and read).
 #include <utility>
 #include "bfaintb_device.hpp"
 
@@ -39,7 +40,7 @@ __device__ __forceinline__ void th_mfma(f32x4_t& acc, const bf16x8_t& a, const b
 __device__ __forceinline__ void th_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 }  // namespace
 
-template <int BITS, bool GROUPED>
+template <int BITS, bool GROUPED, bool PACKED>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) bfaintb_prefill256x128_wreg_kernel(const GemmParams p)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kThStage];
@@ -93,9 +94,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     const __amdgpu_buffer_rsrc_t rsrc_a =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.a + (size_t)m0 * p.lda), 0, (int)a_extent, kBufferFlags);
     const uint32_t cols_valid = p.n - n0 < kTw ? p.n - n0 : kTw;
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0, (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)),
-        kBufferFlags);
+    // packed weights: a block of 16 columns is one run of k x 16 codes in chunks of 1024 bytes (64 rows of 8-bit, 128 rows
+    // of 4-bit codes); the tile's 8 column blocks follow one another, and one past n reads as zero through the extent
+    const uint32_t slab_bytes = p.k * (BITS == 8 ? 16u : 8u);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        PACKED ? __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b + (size_t)(n0 / 16u) * slab_bytes), 0,
+                                                   (int)(cols_valid / 16u * slab_bytes), kBufferFlags)
+               : __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.b + (BITS == 8 ? n0 : n0 / 2u)), 0,
+                                                   (int)((p.k - 1u) * p.ldb_bytes + (BITS == 8 ? cols_valid : cols_valid / 2u)), kBufferFlags);
 
     const uint32_t ksteps_all = (p.k + kTwK - 1u) / kTwK;
     const uint32_t ksteps = ksteps_all;
@@ -126,28 +132,79 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // position l % kChunks, and fetches the chunk the rotation puts there: position = chunk + kRot * (row / 8 % 4).
     constexpr uint32_t kChunks = kRowBytes / 16u;        // 8 or 4 chunks per row
     constexpr uint32_t kRowsPerCopy = 1024u / kRowBytes; // 8 or 16
-    constexpr uint32_t kCopiesPerWave = 64u / kRowsPerCopy / 4u;  // 2 or 1
+    //
+    // Packed weights: the chunk of a column block that holds the step (1024 bytes: all of it for 8-bit codes; for 4-bit
+    // codes it spans two steps and is copied for each) is one instruction; wave w copies column blocks 2 w and 2 w + 1.
+    // The chunk's 16-byte pieces are the lanes of the packed order: piece 16 kg + nl = rows 8 kg .. + 7 of both K-blocks
+    // (4-bit: of four), column nl.  This kernel's lane (c16, kq) wants columns nl = 4 (c16 % 4) + j, j = 0 .. 3, of column
+    // block 4 wc + c16 / 4: pieces 16 kq + nl.  So that a wave reads each j with one conflict-free instruction, piece
+    // 16 g + 4 c + j of column block b is stored at position 16 j + 4 (g ^ (b % 4)) + c: the 16 lanes of one kq then read
+    // 16 neighbouring pieces' worth of banks.
+    constexpr uint32_t kCopiesPerWave = PACKED ? 2u : 64u / kRowsPerCopy / 4u;  // 2 or 1
     constexpr uint32_t kRot = BITS == 8 ? 4u : 2u;       // a wave's 16 lanes of one kq cover 64 (32) bytes of a row
     uint32_t w_voff[2];  // (fixed extent: see the note on the arrays above)
 #pragma unroll
     for (uint32_t j = 0; j < kCopiesPerWave; ++j) {
-        const uint32_t row = (kCopiesPerWave * wave + j) * kRowsPerCopy + lane / kChunks;  // within the step
-        const uint32_t chunk = ((lane % kChunks) - kRot * ((row >> 3) & 3u)) & (kChunks - 1u);
-        w_voff[j] = row * p.ldb_bytes + chunk * 16u;
+        if constexpr (PACKED) {
+            const uint32_t b = 2u * wave + j;
+            const uint32_t g = ((lane >> 2) & 3u) ^ (b & 3u);
+            w_voff[j] = b * slab_bytes + (16u * g + 4u * (lane & 3u) + (lane >> 4)) * 16u;
+        } else {
+            const uint32_t row = (kCopiesPerWave * wave + j) * kRowsPerCopy + lane / kChunks;  // within the step
+            const uint32_t chunk = ((lane % kChunks) - kRot * ((row >> 3) & 3u)) & (kChunks - 1u);
+            w_voff[j] = row * p.ldb_bytes + chunk * 16u;
+        }
     }
+    // where step kt's codes start, beyond the lane's offset: w_step * (kt >> w_shift)  (spelt out at the two copies: with
+    // a lambda for it among the copy's arguments the host pass drops the kernel's launch stub without a diagnostic)
+    const uint32_t w_step = PACKED ? 1024u : kTwK * p.ldb_bytes;
+    constexpr uint32_t w_shift = (PACKED && BITS == 4) ? 1u : 0u;
     auto dma_w = [&](auto stage_c, uint32_t kt) {
         uint8_t* base = w_tile(stage_c) + kCopiesPerWave * wave * 1024u;
 #pragma unroll
         for (uint32_t j = 0; j < kCopiesPerWave; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16, w_voff[j],
-                                                     (kbase + kt) * kTwK * p.ldb_bytes, 0, 0);
+                                                     ((kbase + kt) >> w_shift) * w_step, 0, 0);
     };
     // Pick: this lane's 4 columns (byte offset wbyte of a row), rows 8 kq .. 8 kq + 7 of block blk of 32 k: row
     // 32 blk + 8 kq + r, whose block of 8 is 4 blk + kq, rotation kRot * kq.  One read per row: ds_read_b32 (u16 for
     // 4-bit codes), column j of the four in byte (nibble) j.
     const uint32_t wcol = 64u * wc + 4u * c16;  // within the tile
     const uint32_t wbyte = wcol * BITS / 8u;
-    const uint32_t w_rd = (8u * kq) * kRowBytes + ((((wbyte >> 4) + kRot * kq) & (kChunks - 1u)) << 4) + (wbyte & 15u);  // + 32 blk rows + r rows
+    // (packed: the piece of the lane's first column; column j's is 256 j bytes on; 4-bit codes: + 8 in odd steps)
+    const uint32_t w_rd = PACKED ? (4u * wc + (c16 >> 2)) * 1024u + ((4u * (kq ^ (c16 >> 2)) + (c16 & 3u)) << 4)
+                                 : (8u * kq) * kRowBytes + ((((wbyte >> 4) + kRot * kq) & (kChunks - 1u)) << 4) + (wbyte & 15u);  // + 32 blk rows + r rows
+    // Packed codes of a step as a lane reads them: [column j][K-block][half]: 8-bit codes: rows 4 half .. + 3 in the bytes
+    // of a dword; 4-bit codes: [j][K-block][0] holds the 8 rows in its nibbles.
+    struct PackedCodes {
+        uint32_t d[4][2][2];
+    };
+    auto read_packed = [&](PackedCodes& pc, const uint8_t* src, uint32_t kt, uint32_t j) {  // src: the stage + w_rd
+        if constexpr (BITS == 8) {
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + 256u * j);
+            pc.d[j][0][0] = v[0], pc.d[j][0][1] = v[1], pc.d[j][1][0] = v[2], pc.d[j][1][1] = v[3];
+        } else {
+            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(src + 256u * j + 8u * ((kbase + kt) & 1u));
+            pc.d[j][0][0] = v[0], pc.d[j][1][0] = v[1];
+        }
+    };
+    // 4-bit: the two's-complement nibbles of a dword of 8 rows: even rows in the low nibbles of `ev`'s bytes, odd rows of `od`'s
+    struct PackedNibbles {
+        uint32_t ev[4][2], od[4][2];  // [column j][K-block]
+    };
+    // rows 2 pr, 2 pr + 1 of column j of K-block blk, as fp32 (8-bit: the stored code; 4-bit: q / 16)
+    auto packed_values = [&](const PackedCodes& pc, PackedNibbles& nb, uint32_t blk, uint32_t j, uint32_t pr, float& f0, float& f1) {
+        if constexpr (BITS == 8) {
+            const uint32_t x = pc.d[j][blk][pr >> 1];
+            f0 = (pr & 1u) ? (float)((x >> 16) & 0xffu) : (float)(x & 0xffu);  // v_cvt_f32_ubyte2 / 0
+            f1 = (pr & 1u) ? (float)(x >> 24) : (float)((x >> 8) & 0xffu);     // v_cvt_f32_ubyte3 / 1
+        } else {
+            if (pr == 0) codes4_to_nibbles(pc.d[j][blk][0], nb.ev[j][blk], nb.od[j][blk]);
+            const uint32_t e = nb.ev[j][blk], o = nb.od[j][blk];
+            f0 = pr == 0 ? nibble_to_f32_sixteenth<0>(e) : pr == 1 ? nibble_to_f32_sixteenth<1>(e) : pr == 2 ? nibble_to_f32_sixteenth<2>(e) : nibble_to_f32_sixteenth<3>(e);
+            f1 = pr == 0 ? nibble_to_f32_sixteenth<0>(o) : pr == 1 ? nibble_to_f32_sixteenth<1>(o) : pr == 2 ? nibble_to_f32_sixteenth<2>(o) : nibble_to_f32_sixteenth<3>(o);
+        }
+    };
     auto read_code = [&](const uint8_t* tile, uint32_t blk, uint32_t r) -> uint32_t {
         if constexpr (BITS == 8) return *reinterpret_cast<const uint32_t*>(tile + (32u * blk + r) * kRowBytes);
         else return *reinterpret_cast<const uint16_t*>(tile + (32u * blk + r) * kRowBytes);
@@ -226,6 +283,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         const uint8_t* tile = w_tile(stage_c) + w_rd;
         float sc[2][4];
         block_scales(sc, sr);
+        if constexpr (PACKED) {
+            PackedCodes pc;
+            PackedNibbles nb;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) read_packed(pc, tile, 0, j);
+#pragma unroll
+            for (uint32_t v = 0; v < 32; ++v) {
+                const uint32_t blk = v >> 4, j = (v >> 2) & 3u, pr = v & 3u;
+                float f0, f1;
+                packed_values(pc, nb, blk, j, pr, f0, f1);
+                ops.w[blk][j][pr] = pack_bf16_rne(scaled(f0, sc[blk][j]), scaled(f1, sc[blk][j]));
+            }
+            return;
+        }
 #pragma unroll
         for (uint32_t blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -279,6 +350,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         const uint8_t* const w_src = w_tile(Next{}) + w_rd;
         uint32_t code[2][8];   // the codes of step kt + 1 as read: [block][row], four codes each
         Pre pre[2];            // the two rows of the pair at hand
+        PackedCodes pc;        // ... or, from packed weights, the lane's 4 x 16 (8) bytes
+        PackedNibbles nb;
         float sc[2][4];
         float f0 = 0.f, f1 = 0.f;
         block_scales(sc, s1);
@@ -287,8 +360,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             code[blk][2u * pr] = read_code(w_src, blk, 2u * pr);
             code[blk][2u * pr + 1u] = read_code(w_src, blk, 2u * pr + 1u);
         };
-        read_rows(0);
-        read_rows(1);
+        if constexpr (PACKED) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) read_packed(pc, w_src, kt + 1u, j);
+        } else {
+            read_rows(0);
+            read_rows(1);
+        }
         __builtin_amdgcn_sched_barrier(0);
         auto request = [&](uint32_t q) {  // the q-th memory request of the step
             if (q < 8) {
@@ -296,7 +374,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                                                          (kbase + kt3) * kTwK * 2u + q * 16u * p.lda, 0, 0);
             } else if (q < 8 + kCopiesPerWave) {
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + (q - 8u) * 1024u), 16, w_voff[q - 8u],
-                                                         (kbase + kt3) * kTwK * p.ldb_bytes, 0, 0);
+                                                         ((kbase + kt3) >> w_shift) * w_step, 0, 0);
             } else if (GROUPED && q == 10) {
                 group_scales(s2, kt2);
             }
@@ -317,14 +395,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 if (h == 0) {
                     if (u + kAhead < kUnits) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
                     else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - kUnits) * 2048u);
-                    if ((u & 1u) == 0u && (u >> 1) + 2u < 8u) read_rows((u >> 1) + 2u);
+                    if constexpr (!PACKED)
+                        if ((u & 1u) == 0u && (u >> 1) + 2u < 8u) read_rows((u >> 1) + 2u);
                 }
-                if (cj == 0) {
-                    pre[0] = prepare(code[cblk][2 * cpr]);
-                    pre[1] = prepare(code[cblk][2 * cpr + 1]);
+                if constexpr (PACKED) {
+                    packed_values(pc, nb, cblk, cj, cpr, f0, f1);
+                } else {
+                    if (cj == 0) {
+                        pre[0] = prepare(code[cblk][2 * cpr]);
+                        pre[1] = prepare(code[cblk][2 * cpr + 1]);
+                    }
+                    f0 = value(pre[0], cj);
+                    f1 = value(pre[1], cj);
                 }
-                f0 = value(pre[0], cj);
-                f1 = value(pre[1], cj);
                 __builtin_amdgcn_sched_barrier(0);
                 // ---- second slot
                 th_mfma(acc[mt][j1], a_now, wf1);
@@ -452,21 +535,28 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
 }
 
-template <int BITS, bool GROUPED>
+template <int BITS, bool GROUPED, bool PACKED>
 static hipError_t launch_prefill256x128_wreg_t(const GemmParams& p, hipStream_t stream)
 {
     const uint32_t tiles = ((p.m + kTh - 1) / kTh) * ((p.n + kTw - 1) / kTw);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    void (*kernel)(const GemmParams) = bfaintb_prefill256x128_wreg_kernel<BITS, GROUPED>;
+    void (*kernel)(const GemmParams) = bfaintb_prefill256x128_wreg_kernel<BITS, GROUPED, PACKED>;
     return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
 }
 
-hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, hipStream_t stream)
+template <bool PACKED>
+static hipError_t launch_prefill256x128_wreg_order(const GemmParams& p, int bits, hipStream_t stream)
+{
+    const bool grouped = p.group_size != 0;
+    if (bits == 8) return grouped ? launch_prefill256x128_wreg_t<8, true, PACKED>(p, stream) : launch_prefill256x128_wreg_t<8, false, PACKED>(p, stream);
+    return grouped ? launch_prefill256x128_wreg_t<4, true, PACKED>(p, stream) : launch_prefill256x128_wreg_t<4, false, PACKED>(p, stream);
+}
+
+// packed: p.b is the buffer in the packed order (p.ldb_bytes is unused)
+hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream)
 {
     if (p.reference_arith || p.splits != 1u) return hipErrorInvalidValue;  // this library's own arithmetic, k unsplit
-    const bool grouped = p.group_size != 0;
-    if (bits == 8) return grouped ? launch_prefill256x128_wreg_t<8, true>(p, stream) : launch_prefill256x128_wreg_t<8, false>(p, stream);
-    return grouped ? launch_prefill256x128_wreg_t<4, true>(p, stream) : launch_prefill256x128_wreg_t<4, false>(p, stream);
+    return packed ? launch_prefill256x128_wreg_order<true>(p, bits, stream) : launch_prefill256x128_wreg_order<false>(p, bits, stream);
 }
 
 }  // namespace bfaintb

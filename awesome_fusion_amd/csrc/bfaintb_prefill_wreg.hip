@@ -1,4 +1,5 @@
-// Tiled variant, 256x256 tiles, weights kept in registers: the form of the prefill kernel for row-major B.
+// Tiled variant, 256x256 tiles, weights kept in registers: the prefill kernel, for row-major B (described first) and for B
+// in the packed order (PACKED: what changes is said where the codes are loaded).
 //
 // Same job and the same reference kernel replaced as bfaintb_prefill_kernel
 // (/root/reference/bfAintBGemm/bf16gemm_kernel_gfx90a.s:184-630).  That kernel stages both operands in LDS and is bound

@@ -59,18 +59,18 @@ enum {
     BFAINTB_VARIANT_DECODE = 1, /* split-K weight-streaming kernel (HBM-bound); m > 32 in row blocks; accepts m <= 32768 */
     BFAINTB_VARIANT_PREFILL = 2, /* LDS-tiled MFMA kernels (MFMA-bound): 256x256 tiles, or 128x128 tiles while m x n
                                   * holds at most 256 of those (the large tiles would leave most CUs idle); while even
-                                  * the small tiles leave CUs idle, the kernel over row-major weights splits k between
-                                  * workgroups (same workspace and hand-over as the decode family's split-K) */
+                                  * the small tiles leave CUs idle, their kernel splits k between workgroups (same
+                                  * workspace and hand-over as the decode family's split-K) */
     BFAINTB_VARIANT_PREFILL_256 = 3, /* the tiled kernel with 256x256 tiles, whatever the shape (tests, tuning) */
     BFAINTB_VARIANT_PREFILL_128 = 4, /* the tiled kernel with 128x128 tiles, whatever the shape (tests, tuning) */
-    BFAINTB_VARIANT_PREFILL_256_LDS = 5, /* 256x256 tiles with both operands staged in LDS — the form pre-packed weights,
-                                          * residuals and the gate epilogue use; row-major weights otherwise run the form
-                                          * that keeps the weights in registers (tests, tuning) */
-    BFAINTB_VARIANT_PREFILL_128_LDS = 6, /* 128x128 tiles with both operands staged in LDS — the form pre-packed weights
-                                          * use; row-major weights otherwise run the form that keeps the weights in
-                                          * registers (tests, tuning) */
-    BFAINTB_VARIANT_PREFILL_256X128 = 7  /* tiles of 256 rows x 128 columns, weights in registers (row-major weights, this
-                                          * library's arithmetic), whatever the shape (tests, tuning): what PREFILL runs
+    BFAINTB_VARIANT_PREFILL_256_LDS = 5, /* 256x256 tiles with both operands staged in LDS — the older form, which the
+                                          * reference's arithmetic and the half tiles of a thin last round still use;
+                                          * otherwise the form that keeps the weights in registers runs (tests, tuning) */
+    BFAINTB_VARIANT_PREFILL_128_LDS = 6, /* 128x128 tiles with both operands staged in LDS — the older form, kept for the
+                                          * reference's arithmetic; otherwise the form that keeps the weights in
+                                          * registers runs (tests, tuning) */
+    BFAINTB_VARIANT_PREFILL_256X128 = 7  /* tiles of 256 rows x 128 columns, weights in registers (this library's
+                                          * arithmetic), whatever the shape (tests, tuning): what PREFILL runs
                                           * where 128x128 tiles would need a second round and 256x256 tiles leave CUs idle */
 };
 
@@ -273,7 +273,7 @@ BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
                                                  int variant);
 /* Same with the kernel family forced (BFAINTB_VARIANT_*: DECODE = the slab-streaming kernel for a few rows of A and the
- * decode family beyond, m <= 32768; PREFILL[_256|_128] = the tiled kernels reading packed weights), and which of
+ * decode family beyond, m <= 32768; PREFILL[_256|_128|_256X128|_256_LDS|_128_LDS] = the tiled kernels reading packed weights), and which of
  * the two bfaintb_gemm_prepacked would run. */
 BFAINTB_API int bfaintb_gemm_prepacked_ex(void* c, const void* a, const void* packed_b, const void* scale, const void* bias, uint32_t m,
                               uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc, int weight_bits, uint32_t group_size,

@@ -188,10 +188,13 @@ def test_prepacked_entry_points_validate_before_launching():
     assert rcp(ldc=64) == -3
     assert rcp(packed_b=None) == -1
     assert rcp(bias=P + 2) == -4
-    assert rcp(which=7) == -7
+    assert rcp(which=9) == -7
     assert rcp(m=0) == 0
     assert af.prepacked_workspace_bytes(1, 4096, 4096) == 0 and af.prepacked_workspace_bytes(4096, 4096, 4096) == 0
     assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) == af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
+    # the small tiles split k over packed weights as over row-major ones: same plan, same scratch
+    assert af.prepacked_variant(384, 2048, 8192, 4, 128) == af.PREFILL
+    assert af.prepacked_workspace_bytes(384, 2048, 8192, 4, 128) == af.workspace_bytes(384, 2048, 8192, 4, 128, af.PREFILL) > 0
     assert rcp(m=64, n=256, k=4096, weight_bits=4, group_size=128) == -6     # the plan splits along k: workspace required
     assert af.prepacked_variant(1, 4096, 4096) == af.DECODE
     assert af.prepacked_variant(64, 4096, 4096) == af.DECODE

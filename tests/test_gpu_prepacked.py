@@ -203,6 +203,31 @@ def test_large_tiles_keep_packed_weights_in_registers_too(af, m, n, k, bits, gro
     assert np.array_equal(c, run_prepacked(af, p, af.PREFILL_256_LDS))
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [(256, 128, 64, 8, 0), (300, 272, 448, 8, 0), (700, 1008, 1024, 8, 0), (1000, 1008, 384, 4, 0), (520, 528, 512, 8, 64),
+                                              (130, 4112, 256, 4, 128), (257, 272, 128, 4, 0), (2048, 512, 1088 + 64, 8, 0), (17, 48, 128, 4, 64)])
+def test_tall_tiles_keep_packed_weights_in_registers_too(af, m, n, k, bits, group):
+    """Tiles of 256 rows x 128 columns over packed weights (a lane's four neighbouring columns are four neighbouring pieces of
+    a packed chunk): against the oracle and bit for bit against the row-major path — partial tiles in m and n, one to
+    eighteen steps, 4-bit chunks of two steps, grouped scales."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    c = run_prepacked(af, p, af.PREFILL_256X128)
+    assert_close_ulp(p, c, f"packed, 256x128 tiles: {m}x{n}x{k} bits={bits} g={group}")
+    assert np.array_equal(c, run_gemm(p, which=af.PREFILL_256X128))
+    p.with_bias()
+    assert_close_ulp(p, run_prepacked(af, p, af.PREFILL_256X128), f"... + bias: {m}x{n}x{k} bits={bits} g={group}")
+
+
+def test_tall_tiles_over_packed_weights_are_what_auto_runs_and_take_the_epilogues(af):
+    m, n, k = 2100, 2048, 320
+    assert af.prepacked_variant(m, n, k) == af.PREFILL and (af.prefill_tile(m, n), af.prefill_tile_cols(m, n)) == (256, 128)
+    p = Problem(m, n, k, 8, 0, seed=81)
+    assert np.array_equal(run_prepacked(af, p), run_prepacked(af, p, af.PREFILL_256X128))
+    p.with_bias().with_residual()
+    assert_close_ulp(p, run_prepacked(af, p), "packed, tall tiles, bias + residual")
+    g = Problem(m, n, 384, 4, 128, seed=82, scale_lo=0.002, scale_hi=0.2).with_bias()
+    assert_close_gated(g, run_prepacked(af, g, activation=af.ACT_SILU_GATE), "packed, tall tiles, gated")
+
+
 @pytest.mark.parametrize("m,n,k,bits,group", [(2064, 4112, 192, 8, 0), (2100, 4128, 128, 4, 128)])
 def test_large_tiles_over_packed_weights_take_the_epilogues(af, m, n, k, bits, group):
     """Shapes the library runs on whole 256x256 tiles by itself (the fused entry point takes no forced variant): 9 x 17 of
