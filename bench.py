@@ -47,17 +47,17 @@ RECORDED_TRAFFIC = {
     # name: (bytes, source)
     "decode_m1_n4096_k4096_int8_perchannel": (17422124, "profiles/decode_m1_n4096_k4096_int8.txt"),
     "decode_m1_n4096_k4096_int8_perchannel_prepacked": (16929572, "profiles/decode_m1_n4096_k4096_int8_prepacked.txt"),
-    "prefill_m4096_n4096_k4096_int8_perchannel": (169307846, "profiles/prefill_m4096_n4096_k4096_int8.txt"),
+    "prefill_m4096_n4096_k4096_int8_perchannel": (171267767, "profiles/prefill_m4096_n4096_k4096_int8.txt"),
     "decode_m1_n11008_k4096_int8_perchannel": (46267304, "profiles/decode_m1_n11008_k4096_int8.txt"),
     "decode_m16_n11008_k4096_int8_perchannel": (49015179, "profiles/decode_m16_n11008_k4096_int8.txt"),
     "decode_m32_n11008_k4096_int8_perchannel": (52631370, "profiles/decode_m32_n11008_k4096_int8.txt"),
     "m1_n28672_k8192_int4_group128": (122577159, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
     "m16_n28672_k8192_int4_group128": (130157043, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
-    "m2048_n28672_k8192_int4_group128": (896485920, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
+    "m2048_n28672_k8192_int4_group128": (910050228, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
     "mid_m256_n4096_k4096_int8_perchannel": (35861798, "profiles/mid_m256_n4096_k4096_int8.txt"),
-    "mid_m1024_n4096_k4096_int8_perchannel": (92417830, "profiles/mid_m1024_n4096_k4096_int8.txt"),
-    "mid_m256_n8192_k8192_int8_perchannel": (131112016, "profiles/mid_m256_n8192_k8192_int8.txt"),
-    "mid_m2048_n4096_k4096_int8_perchannel": (168016523, "profiles/mid_m2048_n4096_k4096_int8.txt"),
+    "mid_m1024_n4096_k4096_int8_perchannel": (92446458, "profiles/mid_m1024_n4096_k4096_int8.txt"),
+    "mid_m256_n8192_k8192_int8_perchannel": (131049442, "profiles/mid_m256_n8192_k8192_int8.txt"),
+    "mid_m2048_n4096_k4096_int8_perchannel": (168006299, "profiles/mid_m2048_n4096_k4096_int8.txt"),
 }
 
 # Parity counts RECORDED from the GPU test suite (tests/helpers.py: assert_close_ulp logs every check; tests/conftest.py
