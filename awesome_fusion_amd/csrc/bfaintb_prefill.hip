@@ -610,14 +610,15 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
 
 bool prefill_wreg_serves(const GemmParams& p);
 hipError_t launch_prefill_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream);
+hipError_t launch_prefill256x128_wreg(const GemmParams& p, int bits, bool packed, hipStream_t stream);
 
 template <int BITS, bool GROUPED, bool PACKED, bool REF = false>
 static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream, bool wreg = false)
 {
     GemmParams p = p0;
     const uint32_t tiles = ((p.m + kBM - 1) / kBM) * ((p.n + kBN - 1) / kBN);
-    // whole rounds of 256 workgroups run 256-row tiles; a last round that would fill less than half of the
-    // CUs runs as twice as many 128-row half tiles instead (also when there is no whole round at all)
+    // whole rounds of 256 workgroups run 256x256 tiles; a last round that would fill less than half of the
+    // CUs runs as twice as many half tiles instead (also when there is no whole round at all)
     const uint32_t rest = tiles % 256u;
     const uint32_t halves = (rest != 0u && rest <= 128u && p.m > 128u) ? rest : 0u;
     const uint32_t whole = tiles - halves;
@@ -634,6 +635,11 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream, boo
     if (halves) {
         p.tile_first = whole;
         p.tile_count = halves;
+        // ... as left and right halves on the kernel of 256x128 tiles that keeps the weights in registers, where that serves
+        if (wreg && !REF && prefill_wreg_serves(p)) {
+            p.splits = 1;
+            return launch_prefill256x128_wreg(p, BITS, PACKED, stream);
+        }
         const uint32_t grid = (2u * halves + 7u) / 8u * 8u;
         void (*half_tiles)(const GemmParams) = bfaintb_prefill_kernel<BITS, GROUPED, 2, PACKED, REF>;
         return launch_kernel(half_tiles, dim3(grid, 1, 1), dim3(512, 1, 1), 0, stream, p);

@@ -76,18 +76,35 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // ---- tile of this workgroup (the order of bfaintb_prefill128_kernel: the ids an XCD receives cover consecutive
     //      logical ids, which walk groups of 8 tile-rows column by column)
+    //      Or, with p.tile_count set: the left and right halves of the 256x256 tiles p.tile_first .. + p.tile_count - 1 in the
+    //      order of bfaintb_prefill_wreg_kernel — the thin last round that kernel leaves to this one.
     const uint32_t tiles_m = (p.m + kTh - 1) / kTh, tiles_n = (p.n + kTw - 1) / kTw;
-    const uint32_t wgs = tiles_m * tiles_n;
-    const uint32_t per_xcd = (wgs + 7u) / 8u;
-    const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= wgs) return;
-    const uint32_t group = logical / (8u * tiles_n);
-    const uint32_t first_m = group * 8u;
-    const uint32_t group_rows = tiles_m - first_m < 8u ? tiles_m - first_m : 8u;
-    const uint32_t in_group = logical - group * 8u * tiles_n;
-    const uint32_t tm = first_m + in_group % group_rows;
-    const uint32_t tn = in_group / group_rows;
-    const uint32_t m0 = tm * kTh, n0 = tn * kTw;
+    uint32_t m0, n0;
+    if (p.tile_count != 0u) {
+        const uint32_t wgs = 2u * p.tile_count;
+        const uint32_t per_xcd = (wgs + 7u) / 8u;
+        const uint32_t local = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (local >= wgs) return;
+        const uint32_t big = p.tile_first + (local >> 1), big_n = (p.n + 255u) / 256u;
+        const uint32_t group = big / (4u * big_n);
+        const uint32_t first_m = group * 4u;
+        const uint32_t group_rows = tiles_m - first_m < 4u ? tiles_m - first_m : 4u;
+        const uint32_t in_group = big - group * 4u * big_n;
+        m0 = (first_m + in_group % group_rows) * kTh;
+        n0 = (in_group / group_rows) * 256u + (local & 1u) * kTw;
+        if (n0 >= p.n) return;  // the right half of a last, narrow tile
+    } else {
+        const uint32_t wgs = tiles_m * tiles_n;
+        const uint32_t per_xcd = (wgs + 7u) / 8u;
+        const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (logical >= wgs) return;
+        const uint32_t group = logical / (8u * tiles_n);
+        const uint32_t first_m = group * 8u;
+        const uint32_t group_rows = tiles_m - first_m < 8u ? tiles_m - first_m : 8u;
+        const uint32_t in_group = logical - group * 8u * tiles_n;
+        m0 = (first_m + in_group % group_rows) * kTh;
+        n0 = (in_group / group_rows) * kTw;
+    }
 
     const uint32_t rows_valid = p.m - m0 < kTh ? p.m - m0 : kTh;
     const uint32_t a_extent = ((rows_valid - 1u) * p.lda + p.k) * 2u;
@@ -538,7 +555,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 template <int BITS, bool GROUPED, bool PACKED>
 static hipError_t launch_prefill256x128_wreg_t(const GemmParams& p, hipStream_t stream)
 {
-    const uint32_t tiles = ((p.m + kTh - 1) / kTh) * ((p.n + kTw - 1) / kTw);
+    const uint32_t tiles = p.tile_count != 0u ? 2u * p.tile_count : ((p.m + kTh - 1) / kTh) * ((p.n + kTw - 1) / kTw);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
     void (*kernel)(const GemmParams) = bfaintb_prefill256x128_wreg_kernel<BITS, GROUPED, PACKED>;
     return launch_kernel(kernel, dim3(grid, 1, 1), dim3(256, 1, 1), 0, stream, p);
