@@ -170,13 +170,15 @@ def test_tile_sizes_and_weight_orders_agree_bit_for_bit(af, m, n, k, bits, group
 
 @pytest.mark.parametrize("m,n,k,bits,group", [(130, 272, 64, 8, 0), (700, 1008, 1024, 8, 0), (300, 528, 512, 8, 64), (1000, 1008, 384, 4, 0),
                                               (130, 4112, 256, 4, 128), (1024, 4096, 1088, 8, 0), (257, 272, 128, 4, 0), (100, 528, 4096, 4, 128),
-                                              (256, 1040, 2048, 8, 64), (64, 4096, 4096, 8, 0), (384, 2048, 8192, 4, 128)])
+                                              (256, 1040, 2048, 8, 64), (64, 4096, 4096, 8, 0), (384, 2048, 8192, 4, 128), (900, 1408, 2432, 4, 128)])
 def test_small_tiles_keep_packed_weights_in_registers_too(af, m, n, k, bits, group):
     """128x128 tiles over packed weights run the kernel that converts the weights into operand registers: the codes of a
     step come into LDS as the packed order stores them and a lane takes its two columns' operands with two reads.  Same
     plan as for row-major weights, the split along k included (the long-k shapes here split), so the two weight orders
     must agree bit for bit; and against the oracle.  Partial tiles in m and n, one to 128 K-steps, 4-bit chunks that
     straddle two steps and two splits."""
+    if (m, k) == (900, 2432):  # two splits of 19 steps: the second starts in the middle of a 4-bit chunk
+        assert af.prepacked_workspace_bytes(m, n, k, bits, group, af.PREFILL_128) == af.workspace_bytes(m, n, k, bits, group, af.PREFILL_128, 2)
     p = Problem(m, n, k, bits, group, seed=m + 2 * n + k)
     c = run_prepacked(af, p, af.PREFILL_128)
     assert_close_ulp(p, c, f"packed, 128x128 tiles, weights in registers: {m}x{n}x{k} bits={bits} g={group}")
