@@ -343,8 +343,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     //   slot 0 of unit u: the A fragment of unit u + kAhead (the last kAhead units fetch the next step's first
     //          fragments: its stage is complete, see the wait below); the two code reads that conversion pair u + 4 needs;
     //          the first half of conversion pair u (two weights: sign flips, two conversions)
-    //   slot 1 of unit u: one memory request (units 0 .. 5: the copies; 6, 7: the group scales); the second half of
-    //          pair u (two multiplications, the rounding pack)
+    //   slot 1 of unit u: one memory request (with group scales: those first, in unit 0; then the copies); the second
+    //          half of pair u (two multiplications, the rounding pack)
     constexpr uint32_t kAhead = 4;
     auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const uint32_t (&s1)[2], uint32_t (&s2)[2]) {
         constexpr uint32_t S = decltype(stage_c)::value;
@@ -413,14 +413,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             __builtin_amdgcn_sched_barrier(0);
             // ---- slot 1
             tw_mfma(acc[mt][1], a_now, wf1);
-            if (u < 4) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + u * 1024u), 16, (u & 1u) ? vo : ve,
-                                                         (kbase + kt3) * kTwK * 2u + u * 16u * p.lda, 0, 0);
-            } else if (u < 4 + kCopiesPerWave) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + (u - 4u) * 1024u), 16, w_voff[u - 4u],
-                                                         ((kbase + kt3) >> w_shift) * w_step, 0, 0);
-            } else if (GROUPED && u == 6) {
+            // (the group scales first: the next step waits for them at its very start, and that wait then leaves the
+            // copies requested behind them in flight — requested last, they made it a wait for everything)
+            constexpr uint32_t kFirstCopy = GROUPED ? 1u : 0u;
+            if (GROUPED && u == 0) {
                 group_scales(s2, kt2);
+            } else if (u >= kFirstCopy && u < kFirstCopy + 4) {
+                const uint32_t q = u - kFirstCopy;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16, (q & 1u) ? vo : ve,
+                                                         (kbase + kt3) * kTwK * 2u + q * 16u * p.lda, 0, 0);
+            } else if (u >= kFirstCopy + 4 && u < kFirstCopy + 4 + kCopiesPerWave) {
+                const uint32_t q = u - kFirstCopy - 4u;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + q * 1024u), 16, w_voff[q],
+                                                         ((kbase + kt3) >> w_shift) * w_step, 0, 0);
             }
             nxt.w[cblk][cj][cpr] = pack_bf16_rne(scaled(f0, sc[cblk][cj]), scaled(f1, sc[cblk][cj]));
             __builtin_amdgcn_sched_barrier(0);

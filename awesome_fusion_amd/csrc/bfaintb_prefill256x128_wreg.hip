@@ -344,8 +344,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // groups).  Around them, per unit: the A fragment of unit u + kAhead (the last kAhead units fetch the next step's
     // first fragments); two of the 32 conversion pairs of the next step's weights (pair v = block v / 16, rows 2 (v / 4 % 4),
     // + 1, column v % 4: slots 0 and 2 flip signs and convert, slots 1 and 3 scale and round); in even units the two code
-    // reads of the row pair two ahead; in slots 1 and 3 one memory request (first the 8 copies of A, then those of the
-    // codes, then the group scales).
+    // reads of the row pair two ahead; in slots 1 and 3 one memory request (the group scales, then the 8 copies of A, then
+    // those of the codes).
     constexpr uint32_t kAhead = 4;
     constexpr uint32_t kUnits = 16;
     auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const ScaleRaw& s1, ScaleRaw& s2) {
@@ -385,15 +385,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             read_rows(1);
         }
         __builtin_amdgcn_sched_barrier(0);
-        auto request = [&](uint32_t q) {  // the q-th memory request of the step
-            if (q < 8) {
+        // (the group scales first: the next step waits for them at its very start, and that wait then leaves the copies
+        // requested behind them in flight — requested last, they made it a wait for everything)
+        auto request = [&](uint32_t slot) {  // the memory request of the step's slot-th request slot
+            constexpr uint32_t kFirstCopy = GROUPED ? 1u : 0u;
+            if (GROUPED && slot == 0) {
+                group_scales(s2, kt2);
+            } else if (slot >= kFirstCopy && slot < kFirstCopy + 8) {
+                const uint32_t q = slot - kFirstCopy;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16, (q & 1u) ? vo : ve,
                                                          (kbase + kt3) * kTwK * 2u + q * 16u * p.lda, 0, 0);
-            } else if (q < 8 + kCopiesPerWave) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + (q - 8u) * 1024u), 16, w_voff[q - 8u],
+            } else if (slot >= kFirstCopy + 8 && slot < kFirstCopy + 8 + kCopiesPerWave) {
+                const uint32_t q = slot - kFirstCopy - 8u;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + q * 1024u), 16, w_voff[q],
                                                          ((kbase + kt3) >> w_shift) * w_step, 0, 0);
-            } else if (GROUPED && q == 10) {
-                group_scales(s2, kt2);
             }
         };
 #pragma unroll
