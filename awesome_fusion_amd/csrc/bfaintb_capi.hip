@@ -658,6 +658,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.ldc = ldc;
     p.lds = n;
     p.group_size = group_size;
+    bfaintb::set_group_division(p);
     p.k_per_wg = k;
     p.splits = 1;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -927,6 +928,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
     p.ldc = ldc;
     p.lds = n;
     p.group_size = group_size;
+    bfaintb::set_group_division(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (is_prefill(v)) {
         // a tile's 16 column blocks and a 256-row panel of A are addressed through 32-bit buffer extents

@@ -491,7 +491,7 @@ bfaintb_decode_kernel(const GemmParams p)
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) st.af[q][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + blk * 32);
                 if constexpr (GROUPED) {
-                    const uint16_t* srow = sptr + (size_t)((kb + 32u * (uint32_t)blk) / p.group_size) * p.lds;
+                    const uint16_t* srow = sptr + (size_t)group_of_row(p, kb + 32u * (uint32_t)blk) * p.lds;
                     if constexpr (PACKED) {
                         // lane j fetches the scales of the workgroup's columns 4j .. 4j+3 (one 8-byte load instead of CPL
                         // 2-byte gathers); compute_stage turns them, through LDS, into this lane's CPL scales

@@ -82,6 +82,8 @@ struct GemmParams {
     uint32_t ldc;        // elements
     uint32_t lds;        // elements per scale row (= n)
     uint32_t group_size; // rows of k per scale group; 0 = one group
+    // the division of a block index (row / 32) by group_size / 32 as a multiplication: see set_group_division()
+    uint32_t group_div_magic, group_div_shift1, group_div_shift2;
     // prefill variant: the logical 256x256 tiles one launch covers
     uint32_t tile_first, tile_count;
     // split-K (decode variant only)
@@ -100,6 +102,32 @@ struct GemmParams {
     unsigned long long* trace;  // timestamp sink (instrumented builds only)
 #endif
 };
+
+// The scale group of a row of B.  The kernels ask for it per block of 32 rows inside their inner loops, where a division
+// by the run-time group size (some 25 dependent scalar instructions) stalls the one wave of a SIMD for longer than a
+// matrix instruction runs: 128x128 tiles, groups of 128 rows, 640 x 4096 x 4096: 41.5 us with the division, 36.8 without.
+// So the host turns the divisor d = group_size / 32 into a multiplier (Granlund and Montgomery's round-up method, exact
+// for every 32-bit dividend): l = ceil(log2 d), magic = floor(2^32 (2^l - d) / d) + 1, and then
+// n / d = (t + ((n - t) >> min(l, 1))) >> max(l - 1, 0) with t = the high half of magic x n.
+inline void set_group_division(GemmParams& p)
+{
+    const uint32_t d = p.group_size / 32u;
+    if (d == 0u) {
+        p.group_div_magic = 1u, p.group_div_shift1 = 0u, p.group_div_shift2 = 0u;  // (no groups: never asked)
+        return;
+    }
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    p.group_div_magic = (uint32_t)((((1ull << l) - d) << 32) / d) + 1u;
+    p.group_div_shift1 = l < 1u ? l : 1u;
+    p.group_div_shift2 = l > 1u ? l - 1u : 0u;
+}
+__device__ __forceinline__ uint32_t group_of_row(const GemmParams& p, uint32_t row)
+{
+    const uint32_t n = row >> 5;
+    const uint32_t t = __umulhi(p.group_div_magic, n);
+    return (t + ((n - t) >> p.group_div_shift1)) >> p.group_div_shift2;
+}
 
 // Launch through hipLaunchKernel so that the error returned belongs to THIS launch:
 // hipGetLastError() would also hand back whatever an earlier, unrelated runtime call left behind.

@@ -233,7 +233,7 @@ __device__ __forceinline__ void decode_packed_body(const GemmParams& p)
                 for (int mb = 0; mb < MB; ++mb) b.a[i][h][mb] = *reinterpret_cast<const uint4*>(aptr[mb] + kChunkRows * c + 32u * h);
             if constexpr (GROUPED) {
 #pragma unroll
-                for (uint32_t h = 0; h < kScalesPerChunk; ++h) b.s[i][h] = sptr[(size_t)((kChunkRows * c + 32u * h) / p.group_size) * p.lds];
+                for (uint32_t h = 0; h < kScalesPerChunk; ++h) b.s[i][h] = sptr[(size_t)group_of_row(p, kChunkRows * c + 32u * h) * p.lds];
             }
         }
     };

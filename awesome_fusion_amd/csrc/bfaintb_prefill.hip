@@ -160,11 +160,10 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     const bool w_ok = ncol < p.n;
     // row-major: cs[j] scales column 4*lane + j.  Packed: cs[2 i + h] scales column nl of block 2 wave + i in K-block h.
     float cs[4];
-    uint32_t cur_group = 0xffffffffu;
-    auto fetch_scales = [&](uint32_t g) {
+    uint32_t cur_group = 0xffffffffu, cur_group1 = 0xffffffffu;
+    auto fetch_scales = [&](uint32_t g, uint32_t g1) {
         if constexpr (PACKED) {
-            // g = group of the step's first K-block; the second K-block is in the next group when groups are 32 rows
-            const uint32_t g1 = (GROUPED && p.group_size == 32u) ? g + 1u : g;
+            // g = group of the step's first K-block, g1 of the second one
 #pragma unroll
             for (uint32_t i = 0; i < 2; ++i) {
                 const uint32_t c = n0 + 16u * (2u * wave + i) + (lane & 15u);
@@ -189,7 +188,7 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
             cs[3] = make_col_scale<BITS>(sr.y >> 16);
         }
     };
-    if constexpr (!GROUPED) fetch_scales(0);
+    if constexpr (!GROUPED) fetch_scales(0, 0);
 
     uint32_t b_reg[8];
 
@@ -266,12 +265,15 @@ __global__ void __launch_bounds__(512) bfaintb_prefill_kernel(const GemmParams p
     };
     auto update_scales = [&](uint32_t kt) {
         if constexpr (GROUPED) {
-            uint32_t g = (kt * (uint32_t)kBK + (PACKED ? 0u : 8u * wave)) / p.group_size;
+            uint32_t g = group_of_row(p, kt * (uint32_t)kBK + (PACKED ? 0u : 8u * wave));
+            uint32_t g1 = PACKED ? group_of_row(p, kt * (uint32_t)kBK + 32u) : g;  // packed: a wave converts both K-blocks of the step
             const uint32_t groups = p.k / p.group_size;
             if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do, their products vanish
-            if (g != cur_group) {
+            if (g1 >= groups) g1 = groups - 1u;
+            if (g != cur_group || g1 != cur_group1) {
                 cur_group = g;
-                fetch_scales(g);
+                cur_group1 = g1;
+                fetch_scales(g, g1);
             }
         }
     };

@@ -120,8 +120,8 @@ bfaintb_prefill128_kernel(const GemmParams p)
     const uint32_t ncol = n0 + (PACKED ? 16u * wave + (lane & 15u) : 2u * lane);
     const bool w_ok = ncol < p.n;
     float cs[2];
-    uint32_t cur_group = 0xffffffffu;
-    auto fetch_scales = [&](uint32_t g) {
+    uint32_t cur_group = 0xffffffffu, cur_group1 = 0xffffffffu;
+    auto fetch_scales = [&](uint32_t g, uint32_t g1) {
         if constexpr (REF) {
             float2 sf = make_float2(0.f, 0.f);
             if (w_ok) sf = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(p.scale) + ncol);
@@ -133,7 +133,7 @@ bfaintb_prefill128_kernel(const GemmParams p)
         if (w_ok) {
             if constexpr (PACKED) {
                 s0 = p.scale[(size_t)g * p.lds + ncol];
-                s1 = p.scale[(size_t)((GROUPED && p.group_size == 32u) ? g + 1u : g) * p.lds + ncol];
+                s1 = p.scale[(size_t)g1 * p.lds + ncol];  // the step's second K-block may lie in the next group
             } else {
                 const uint32_t sr = *reinterpret_cast<const uint32_t*>(p.scale + (size_t)g * p.lds + ncol);
                 s0 = sr & 0xffffu;
@@ -143,15 +143,18 @@ bfaintb_prefill128_kernel(const GemmParams p)
         cs[0] = make_col_scale<BITS>(s0);
         cs[1] = make_col_scale<BITS>(s1);
     };
-    if constexpr (!GROUPED) fetch_scales(0);
+    if constexpr (!GROUPED) fetch_scales(0, 0);
     auto update_scales = [&](uint32_t kt) {
         if constexpr (GROUPED) {
-            uint32_t g = (kt * 64u + (PACKED ? 0u : 8u * wave)) / p.group_size;
+            uint32_t g = group_of_row(p, kt * 64u + (PACKED ? 0u : 8u * wave));
+            uint32_t g1 = PACKED ? group_of_row(p, kt * 64u + 32u) : g;  // packed: a wave converts both K-blocks of the step
             const uint32_t groups = p.k / p.group_size;
             if (g >= groups) g = groups - 1u;  // rows past k in a partial last step: any scale will do, their products vanish
-            if (g != cur_group) {
+            if (g1 >= groups) g1 = groups - 1u;
+            if (g != cur_group || g1 != cur_group1) {
                 cur_group = g;
-                fetch_scales(g);
+                cur_group1 = g1;
+                fetch_scales(g, g1);
             }
         }
     };

@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto group_scales = [&](ScaleRaw& sr, uint32_t kt) {
 #pragma unroll
         for (uint32_t blk = 0; blk < 2; ++blk) {
-            uint32_t g = ((kbase + kt) * kTwK + 32u * blk) / p.group_size;
+            uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk);
             if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
             sr.v[blk] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, s_voff, g * p.lds * 2u, 0);
         }

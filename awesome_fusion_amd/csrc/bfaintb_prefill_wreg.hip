@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
     const uint32_t s_voff = (n0 + wcol) * 2u;
     // the grouped scales of block blk of step kt (packed: of the lane's column j alone)
     auto load_group_scales = [&](Raw& raw, uint32_t kt, uint32_t blk, uint32_t j = 0) {
-        uint32_t g = (kt * kWrK + 32u * blk) / p.group_size;
+        uint32_t g = group_of_row(p, kt * kWrK + 32u * blk);
         if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
         if constexpr (PACKED) {
             raw.s[blk][j] = __builtin_amdgcn_raw_buffer_load_b16(rsrc_s, s_voff, g * p.lds * 2u + 32u * j, 0);

@@ -179,6 +179,17 @@ def test_small_tile_forms_agree_bit_for_bit(af, m, n, k, bits, group):
     assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128_LDS))
 
 
+@pytest.mark.parametrize("m,n,k,bits,group,which", [
+    (1, 256, 960, 8, 96, "AUTO"), (16, 528, 1920, 4, 160, "AUTO"), (40, 512, 1920, 4, 160, "AUTO"), (100, 1040, 2240, 8, 224, "AUTO"),
+    (300, 272, 960, 8, 96, "PREFILL_128"), (300, 272, 960, 8, 96, "PREFILL_256"), (300, 528, 1920, 4, 160, "PREFILL_128_LDS"),
+    (300, 528, 1920, 4, 160, "PREFILL_256_LDS"), (520, 272, 1120, 8, 224, "PREFILL_256X128"), (130, 4112, 672, 4, 96, "PREFILL_256")])
+def test_scale_groups_that_are_no_power_of_two(af, m, n, k, bits, group, which):
+    """The kernels find the scale group of a block of 32 rows by a multiplication the host prepares from the group size;
+    group sizes that are no power of two (any multiple of 32 that divides k is allowed) take the general form of it."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k + group)
+    assert_close_ulp(p, run_gemm(p, which=getattr(af, which)), f"{which}: {m}x{n}x{k} bits={bits} g={group}")
+
+
 def test_tiled_variant_picks_its_tile_size_by_shape(af):
     """PREFILL runs 128x128 tiles while m x n holds at most 256 of them, then tiles of 256 rows x 128 columns while those
     are at most 256, 256x256 tiles beyond; every time the result meets the oracle and is the forced form's, bit for bit."""

@@ -258,6 +258,15 @@ def test_kernels_dequantise_bit_exact(af, bits, group, which, m):
         assert np.array_equal(run_prepacked(af, p, which, pk=pk), p.w_bf[rows]), f"rows {base}.. differ"
 
 
+@pytest.mark.parametrize("m,n,k,bits,group,which", [
+    (1, 256, 960, 8, 96, "AUTO"), (20, 528, 1920, 4, 160, "AUTO"), (80, 1040, 2240, 8, 224, "AUTO"), (64, 256, 1920, 4, 160, "AUTO"),
+    (300, 272, 960, 8, 96, "PREFILL_128"), (300, 528, 1920, 4, 160, "PREFILL_256"), (520, 272, 2240, 8, 224, "PREFILL_256X128"),
+    (300, 528, 1920, 4, 160, "PREFILL_128_LDS")])
+def test_scale_groups_that_are_no_power_of_two(af, m, n, k, bits, group, which):
+    p = Problem(m, n, k, bits, group, seed=m + n + k + group)
+    assert_close_ulp(p, run_prepacked(af, p, getattr(af, which)), f"packed, {which}: {m}x{n}x{k} bits={bits} g={group}")
+
+
 @pytest.mark.parametrize("m", [1, 16])
 def test_headline_shapes(af, m):
     p = Problem(m, 4096, 4096, seed=20 + m)
