@@ -238,13 +238,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.scale), 0, (int)(((scale_rows - 1u) * p.lds + p.n) * 2u), kBufferFlags);
     const uint32_t s_voff = (n0 + wcol) * 2u;
+    auto block_group_scales = [&](uint32_t (&sr)[2], uint32_t kt, uint32_t blk) {
+        uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk);
+        if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
+        sr[blk] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, g * p.lds * 2u, 0);
+    };
     auto group_scales = [&](uint32_t (&sr)[2], uint32_t kt) {
-#pragma unroll
-        for (uint32_t blk = 0; blk < 2; ++blk) {
-            uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk);
-            if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
-            sr[blk] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, g * p.lds * 2u, 0);
-        }
+        block_group_scales(sr, kt, 0);
+        block_group_scales(sr, kt, 1);
     };
     float cs[2] = {0.f, 0.f};  // one scale per column: fixed
     if constexpr (!GROUPED) {
@@ -415,9 +416,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             tw_mfma(acc[mt][1], a_now, wf1);
             // (the group scales first: the next step waits for them at its very start, and that wait then leaves the
             // copies requested behind them in flight — requested last, they made it a wait for everything)
-            constexpr uint32_t kFirstCopy = GROUPED ? 1u : 0u;
-            if (GROUPED && u == 0) {
-                group_scales(s2, kt2);
+            // (one block's scales per slot: finding a group is a chain of five scalar instructions)
+            constexpr uint32_t kFirstCopy = GROUPED ? 2u : 0u;
+            if (GROUPED && u < 2) {
+                block_group_scales(s2, kt2, u);
             } else if (u >= kFirstCopy && u < kFirstCopy + 4) {
                 const uint32_t q = u - kFirstCopy;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16, (q & 1u) ? vo : ve,

@@ -236,13 +236,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     struct ScaleRaw {
         u32x2_t v[2];  // [block of 32 k]: the four columns' bf16 scales
     };
+    auto block_group_scales = [&](ScaleRaw& sr, uint32_t kt, uint32_t blk) {
+        uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk);
+        if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
+        sr.v[blk] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, s_voff, g * p.lds * 2u, 0);
+    };
     auto group_scales = [&](ScaleRaw& sr, uint32_t kt) {
-#pragma unroll
-        for (uint32_t blk = 0; blk < 2; ++blk) {
-            uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk);
-            if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
-            sr.v[blk] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, s_voff, g * p.lds * 2u, 0);
-        }
+        block_group_scales(sr, kt, 0);
+        block_group_scales(sr, kt, 1);
     };
     auto widen_scales = [&](float (&out)[4], const u32x2_t& raw) {
         out[0] = make_col_scale_nibble<BITS>(raw[0] & 0xffffu);
@@ -388,9 +389,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         // (the group scales first: the next step waits for them at its very start, and that wait then leaves the copies
         // requested behind them in flight — requested last, they made it a wait for everything)
         auto request = [&](uint32_t slot) {  // the memory request of the step's slot-th request slot
-            constexpr uint32_t kFirstCopy = GROUPED ? 1u : 0u;
-            if (GROUPED && slot == 0) {
-                group_scales(s2, kt2);
+            // (one block's scales per slot: finding a group is a chain of five scalar instructions)
+            constexpr uint32_t kFirstCopy = GROUPED ? 2u : 0u;
+            if (GROUPED && slot < 2) {
+                block_group_scales(s2, kt2, slot);
             } else if (slot >= kFirstCopy && slot < kFirstCopy + 8) {
                 const uint32_t q = slot - kFirstCopy;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16, (q & 1u) ? vo : ve,
