@@ -51,9 +51,9 @@ RECORDED_TRAFFIC = {
     "decode_m1_n11008_k4096_int8_perchannel": (46267304, "profiles/decode_m1_n11008_k4096_int8.txt"),
     "decode_m16_n11008_k4096_int8_perchannel": (49015179, "profiles/decode_m16_n11008_k4096_int8.txt"),
     "decode_m32_n11008_k4096_int8_perchannel": (52631370, "profiles/decode_m32_n11008_k4096_int8.txt"),
-    "m1_n28672_k8192_int4_group128": (122577159, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
-    "m16_n28672_k8192_int4_group128": (130157043, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
-    "m2048_n28672_k8192_int4_group128": (910479653, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
+    "m1_n28672_k8192_int4_group128": (122555279, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
+    "m16_n28672_k8192_int4_group128": (130160110, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
+    "m2048_n28672_k8192_int4_group128": (907944059, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
     "mid_m256_n4096_k4096_int8_perchannel": (35861798, "profiles/mid_m256_n4096_k4096_int8.txt"),
     "mid_m1024_n4096_k4096_int8_perchannel": (92446458, "profiles/mid_m1024_n4096_k4096_int8.txt"),
     "mid_m256_n8192_k8192_int8_perchannel": (131049442, "profiles/mid_m256_n8192_k8192_int8.txt"),
