@@ -405,6 +405,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             } else {
                 if (cj == 0 && u + 4 < 16) read_codes(u + 4);
                 if (cj == 0) {
+                    if constexpr (BITS == 8) {
+                        // (the two reads stay two registers: left to itself the compiler packs them into one and shifts the
+                        // pair about before converting — six instructions where four byte-selecting conversions do.  Said here,
+                        // where the values are needed, and not at the reads, where it would make the wave wait for them.)
+                        asm("" : "+v"(code[cblk][2 * cpr]));
+                        asm("" : "+v"(code[cblk][2 * cpr + 1]));
+                    }
                     prepare(code[cblk][2 * cpr], pre[cblk][2 * cpr][0], pre[cblk][2 * cpr][1]);
                     prepare(code[cblk][2 * cpr + 1], pre[cblk][2 * cpr + 1][0], pre[cblk][2 * cpr + 1][1]);
                 }
