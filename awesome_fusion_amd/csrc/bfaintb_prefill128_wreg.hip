@@ -55,7 +55,7 @@ __device__ __forceinline__ void tw_settle() { asm volatile("s_nop 15\n\ts_nop 15
 }  // namespace
 
 template <int BITS, bool GROUPED, bool PACKED>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) bfaintb_prefill128_wreg_kernel(const GemmParams p)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) bfaintb_prefill128_wreg_kernel(const GemmParams p)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kTwStage];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kTwStage];
