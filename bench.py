@@ -72,7 +72,7 @@ RECORDED_ACCEPTANCE = {
     "C3_n11008_k4096_m1_4_8_16_32": {"checks": 5, "outputs": 671488, "outside_bound": 12, "worst_ulp": 1.81, "worst_excess_units": 0.08},
     "C4_m4096_n4096_k4096": {"checks": 2, "outputs": 33554432, "outside_bound": 456, "worst_ulp": 2.5, "worst_excess_units": 0.44},
     "C5_int4_g128_n28672_k8192_m1_16_2048sample": {"checks": 5, "outputs": 4644864, "outside_bound": 98, "worst_ulp": 2.25, "worst_excess_units": 0.36},
-    "whole_suite": {"checks": 784, "outputs": 351269280, "outside_bound": 1148, "worst_excess_units": 0.61},
+    "whole_suite": {"checks": 804, "outputs": 355743104, "outside_bound": 1190, "worst_excess_units": 0.61},
 }
 
 C3_ROWS = (1, 16, 32)        # BASELINE config 3 (M in {1,4,8,16,32}): the rows the default line carries; --sweep has all five
