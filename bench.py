@@ -540,10 +540,14 @@ def main():
         for (m, n, k) in ((64, 4096, 4096), (256, 4096, 4096), (256, 8192, 8192), (640, 4096, 4096), (1024, 4096, 4096), (2048, 4096, 4096)):
             w = Workload(f"mid_m{m}_n{n}_k{k}_int8_perchannel", m, n, k, copies=4 if n == 4096 else 2)
             ev_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True)
+            pk_ms, _ = time_graph(af, w, min(K, 100), min(W, 10), rotate=True, packed=True)
             v, split = af.variant(m, n, k), af.split_k(m, n, k)
+            pv = af.prepacked_variant(m, n, k)
             sweep.append({"workload": w.name, **roofline_entry(w, ev_ms, "mfma"),
                           "kernel": "row-blocked decode family" if v == af.DECODE else
-                          f"tiled, {af.prefill_tile(m, n)}x{af.prefill_tile_cols(m, n)} tiles" + (f", k split {split} ways" if split > 1 else "")})
+                          f"tiled, {af.prefill_tile(m, n)}x{af.prefill_tile_cols(m, n)} tiles" + (f", k split {split} ways" if split > 1 else ""),
+                          "prepacked_kernel_us": round(pk_ms * 1e3, 3),
+                          "prepacked_kernel": "row-blocked decode family" if pv == af.DECODE else "tiled, same tiles and plan as row-major weights"})
             del w
             torch.cuda.empty_cache()
         # gated MLP, LLaMA-7B shape: 2 x 11008 interleaved (gate, up) columns over k = 4096
