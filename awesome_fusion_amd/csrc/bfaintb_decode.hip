@@ -366,7 +366,8 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 // REF: the reference kernel's arithmetic (p.reference_arith): p.scale holds one fp32 scale per column, W is narrowed by
 // truncation.
 template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED, bool REF>
-// (packed 4-bit codes always run 4 waves, and their two K-blocks per step want the registers of a 256-thread bound)
+// (packed 4-bit codes always run 4 waves: with 8 — their registers would allow it for one block of 16 rows — the 256-column
+// kernel over packed weights is slower, 28672 x 8192, m = 16: 55 against 42 us)
 __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED && BITS == 4)) ? 512 : 256)
 bfaintb_decode_kernel(const GemmParams p)
 {
