@@ -261,7 +261,12 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
             set_splits(c, k, bits, forced_splits ? forced_splits : s, packed);
             if (!forced_splits && c.splits != s && s != 1u) continue;  // k does not divide that way
             if (!forced_splits && s > 1u && tiles * s > 768u) break;
-            const double t = decode_family_estimate_us(m, n, k, bits, c);
+            double t = decode_family_estimate_us(m, n, k, bits, c);
+            // (packed codes: the kernels of 16-row blocks are the weaker ones there, and the estimate's price of a split sends
+            // 17 to 32 rows against many columns to them — 32000 x 4096, m = 32: 47.8 us in two blocks of 16 rows, 32.0 in one of
+            // 32 with k split in two; 28672 x 4096: 36.9 / 30.5; 13824 x 5120: 29.8 / 25.4.  With two thirds of that price the
+            // pick is within 3 % of the better form on all 45 shapes scanned; for row-major codes the full price picks better.)
+            if (packed) t -= 4.0 * (c.splits - 1.0) * m * n / 1.5e6;
             if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
         }
     }
