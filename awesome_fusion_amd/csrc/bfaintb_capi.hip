@@ -267,6 +267,10 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
             // 32 with k split in two; 28672 x 4096: 36.9 / 30.5; 13824 x 5120: 29.8 / 25.4.  With two thirds of that price the
             // pick is within 3 % of the better form on all 45 shapes scanned; for row-major codes the full price picks better.)
             if (packed) t -= 4.0 * (c.splits - 1.0) * m * n / 1.5e6;
+            // (row-major codes: only the one block of 32 rows with k split in two is priced too high — 17 to 32 rows against
+            // 224 to 250 blocks of columns went to two blocks of 16 rows without a split, a round of workgroups filled exactly:
+            // 32000 x 4096, m = 32: 32.1 us against 28.1; 28672 x 4096: 31.2 / 29.1)
+            else if (c.splits == 2u && mb == 2u) t -= 3.0 * m * n / 1.5e6;
             if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
         }
     }
