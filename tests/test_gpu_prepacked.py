@@ -349,7 +349,8 @@ def test_hip_graph_replays_match_eager(af):
     """Packing and the packed GEMMs hold no memset and no scratch state: captured once, every replay reproduces the
     eager bits, with other work and synchronisations in between."""
     import torch
-    shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (40, 64, 8256, 8, 0), (64, 256, 4096, 4, 128), (600, 512, 512, 8, 0)]
+    # (the last one: 128x128 tiles with k split between workgroups, the hand-over through the workspace inside the graph)
+    shapes = [(1, 4096, 4096, 8, 0), (4, 1040, 2048, 4, 128), (40, 64, 8256, 8, 0), (64, 256, 4096, 4, 128), (600, 512, 512, 8, 0), (384, 2048, 8192, 4, 128)]
     probs = [Problem(m, n, k, bits, g, seed=190 + i) for i, (m, n, k, bits, g) in enumerate(shapes)]
     eager = [run_prepacked(af, p) for p in probs]
     bufs = [dict(a=to_dev(p.a_bf), b=to_dev(p.b_bytes), s=to_dev(p.s_bf), pk=torch.zeros(af.prepack_bytes(p.n, p.k, p.bits), dtype=torch.uint8, device="cuda"),
