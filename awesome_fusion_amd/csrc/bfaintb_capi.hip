@@ -4,6 +4,7 @@
 // (gpu_utils.hpp:5-11, print and exit(0)) every failure is returned to the caller.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <atomic>
@@ -565,6 +566,31 @@ int bfaintb_workspace_status(const void* workspace, void* stream)
     return header[0] == kEmptyWord ? BFAINTB_OK : BFAINTB_ERR_WORKSPACE_POISONED;
 }
 
+// The same two calls for the scratch of bfaintb_gemm_static, whose address the library keeps to itself.
+int bfaintb_static_scratch_status(void* stream)
+{
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DeviceState* dev = nullptr;
+    int rc = device_state(st, &dev);
+    if (rc) return rc;
+    void* ptr = nullptr;
+    rc = static_scratch(*dev, st, &ptr);
+    if (rc) return rc;
+    return bfaintb_workspace_status(ptr, stream);
+}
+
+int bfaintb_static_scratch_reset(void* stream)
+{
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    DeviceState* dev = nullptr;
+    int rc = device_state(st, &dev);
+    if (rc) return rc;
+    void* ptr = nullptr;
+    rc = static_scratch(*dev, st, &ptr);  // (the first call on a device fills it anyway)
+    if (rc) return rc;
+    return init_workspace_on(ptr, BFAINTB_STATIC_SCRATCH_BYTES, st);
+}
+
 int bfaintb_init(void* stream)
 {
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -575,8 +601,21 @@ int bfaintb_init(void* stream)
     return static_scratch(*dev, st, &ptr);
 }
 
+// The two hooks that change what split-K launches do are for the library's own tests: they work only in a process that
+// has BFAINTB_TEST_HOOKS=1 in its environment (read when the first of them is asked for), so that a stray call in a host
+// application cannot turn every split-K result of the process into NaNs.
+static bool test_hooks_armed()
+{
+    static const bool armed = [] {
+        const char* v = getenv("BFAINTB_TEST_HOOKS");
+        return v != nullptr && strcmp(v, "1") == 0;
+    }();
+    return armed;
+}
+
 int bfaintb_debug_control(uint32_t what, uint32_t value)
 {
+    if ((what == BFAINTB_DEBUG_SPLIT_WAIT_LIMIT || what == BFAINTB_DEBUG_WITHHOLD_PARTIALS) && !test_hooks_armed()) return BFAINTB_ERR_UNSUPPORTED;
     switch (what) {
         case BFAINTB_DEBUG_SPLIT_WAIT_LIMIT:
             g_split_wait_limit.store(value ? value : bfaintb::kDefaultSplitWaitLimit);

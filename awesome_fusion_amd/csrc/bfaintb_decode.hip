@@ -642,19 +642,29 @@ bfaintb_decode_kernel(const GemmParams p)
         TRACE_MARK(3);
 
         float4 sum[kMaxR];
+        // The waves' tiles are read with every load of a row in flight at once and added in wave order (wave 0 first:
+        // the order is fixed).  Written for the two workgroup sizes there are, so that the loop over the waves is
+        // unrolled: as a loop with a run-time bound it was a chain of 4 or 8 dependent LDS round trips, and this sum
+        // sits between the end of the weight stream and the hand-over of the partial sums, where nothing hides it.
+        auto add_waves = [&](auto waves_c) {
+            constexpr uint32_t W = decltype(waves_c)::value;
 #pragma unroll
-        for (uint32_t i = 0; i < kMaxR; ++i) {
-            const uint32_t row = rs + i * nrs;
-            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (row < rows_out) {
-                const float* src = red + (size_t)row * kRedStride + 4u * cg;
-                for (uint32_t w = 0; w < nwaves; ++w) {  // fixed order: wave 0 first
-                    const float4 v = *reinterpret_cast<const float4*>(src + (size_t)w * rows_out * kRedStride);
-                    t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+            for (uint32_t i = 0; i < kMaxR; ++i) {
+                const uint32_t row = rs + i * nrs;
+                float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (row < rows_out) {
+                    const float* src = red + (size_t)row * kRedStride + 4u * cg;
+                    float4 v[W];
+#pragma unroll
+                    for (uint32_t w = 0; w < W; ++w) v[w] = *reinterpret_cast<const float4*>(src + (size_t)w * rows_out * kRedStride);
+#pragma unroll
+                    for (uint32_t w = 0; w < W; ++w) { t.x += v[w].x; t.y += v[w].y; t.z += v[w].z; t.w += v[w].w; }
                 }
+                sum[i] = t;
             }
-            sum[i] = t;
-        }
+        };
+        if (nwaves == 8u) add_waves(std::integral_constant<uint32_t, 8>{});
+        else add_waves(std::integral_constant<uint32_t, 4>{});
         const uint32_t first_row = row0 + pass_row0;  // global row of this pass's row 0
         if (p.splits == 1) {
 #pragma unroll

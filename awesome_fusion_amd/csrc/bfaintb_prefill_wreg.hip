@@ -397,6 +397,9 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
 
     using C2 = std::integral_constant<uint32_t, 2>;
     using C3 = std::integral_constant<uint32_t, 3>;
+#ifdef BFAINTB_TRACE
+    const long long tr_c0 = clock64(), tr_w0 = wall_clock64();
+#endif
     uint32_t kt = 0;
     for (; kt + 3 < ksteps; kt += 4) {
         step(C0{}, kt, ops0, ops1, rawa, rawb);
@@ -407,6 +410,18 @@ __global__ void __launch_bounds__(256) bfaintb_prefill_wreg_kernel(const GemmPar
     if (kt < ksteps) step(C0{}, kt, ops0, ops1, rawa, rawb);
     if (kt + 1 < ksteps) step(C1{}, kt + 1, ops1, ops0, rawb, rawa);
     if (kt + 2 < ksteps) step(C2{}, kt + 2, ops0, ops1, rawa, rawb);
+#ifdef BFAINTB_TRACE
+    {   // shader cycles and 100 MHz ticks the K loop took, per wave: words 0, 1 of the wave's 8
+        const long long tr_c1 = clock64(), tr_w1 = wall_clock64();
+        if (lane == 0 && p.trace != nullptr) {
+            unsigned long long* t = p.trace + (size_t)(blockIdx.x * 4u + wave) * 8u;
+            t[0] = (unsigned long long)(tr_c1 - tr_c0);
+            t[1] = (unsigned long long)(tr_w1 - tr_w0);
+            t[2] = (unsigned long long)tr_w0;
+            t[3] = (unsigned long long)tr_w1;
+        }
+    }
+#endif
 
     // ---- epilogue: bf16 tile through LDS (rows 64 q .. 64 q + 63 in the q-th array), then 16-byte row-contiguous stores
     wreg_settle();  // the last matrix instructions have written their accumulators

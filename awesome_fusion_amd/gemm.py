@@ -145,6 +145,10 @@ def lib():
         L.bfaintb_gemm_static_scratch_bytes.argtypes = []
         L.bfaintb_debug_control.restype = C.c_int
         L.bfaintb_debug_control.argtypes = [_u32, _u32]
+        L.bfaintb_static_scratch_status.restype = C.c_int
+        L.bfaintb_static_scratch_status.argtypes = [_vp]
+        L.bfaintb_static_scratch_reset.restype = C.c_int
+        L.bfaintb_static_scratch_reset.argtypes = [_vp]
         _lib = L
     return _lib
 
@@ -230,9 +234,27 @@ ERR_WORKSPACE, ERR_NOT_INITIALISED, ERR_WORKSPACE_POISONED, ERR_STATIC_SCRATCH =
 
 
 def debug_control(what, value):
+    """Test and tuning hooks.  DEBUG_SPLIT_WAIT_LIMIT and DEBUG_WITHHOLD_PARTIALS are refused unless the process has
+    BFAINTB_TEST_HOOKS=1 in its environment."""
     rc = lib().bfaintb_debug_control(what, value)
     if rc:
         raise BfaintbError(rc, "bfaintb_debug_control")
+
+
+def static_scratch_status(stream=None):
+    """bfaintb_workspace_status for the scratch of gemm_static on the current device (synchronises): 0 or
+    ERR_WORKSPACE_POISONED (negative codes are returned, HIP errors raise)."""
+    rc = lib().bfaintb_static_scratch_status(_stream_handle(stream))
+    if rc > 0:
+        raise BfaintbError(rc, "bfaintb_static_scratch_status")
+    return rc
+
+
+def static_scratch_reset(stream=None):
+    """Puts the scratch of gemm_static on the current device back into its at-rest state (asynchronous on the stream)."""
+    rc = lib().bfaintb_static_scratch_reset(_stream_handle(stream))
+    if rc:
+        raise BfaintbError(rc, "bfaintb_static_scratch_reset")
 
 
 def _epilogue(bias, residual, ldr, n, activation=ACT_NONE):

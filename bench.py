@@ -6,7 +6,7 @@
 A step is one GEMM launch through the C ABI on synthetic, seeded inputs already resident in HBM.
 The headline workload is the decode shape the metric is quoted on (bf16 A [1,4096] x int8 B
 [4096,4096], per-channel bf16 scales); the prefill shape (M = 4096), the decode sweep over the MLP
-up-projection shape (N = 11008, M = 1, 16, 32) and the 4-bit group-128 shape (28672 x 8192, M = 1, 16, 2048)
+up-projection shape (N = 11008, M = 1, 4, 8, 16, 32) and the 4-bit group-128 shape (28672 x 8192, M = 1, 16, 2048)
 are measured in the same run and reported under "extra".  The metric definitions follow the reference
 driver's printout (/root/reference/bfAintBGemm/bfAintBGemm.cc:186-195: flops = 2mnk, bytes = 2(mk+mn) + nk)
 with two corrections stated in the output: decimal units, and the scale bytes are counted.
@@ -67,7 +67,7 @@ RECORDED_TRAFFIC = {
 # of 2^-24 * sum|a w|.  Not measured by a run of this file.
 RECORDED_ACCEPTANCE = {
     "source": "tests (-m gpu): tests/conftest.py writes acceptance_counts.json at session end; not measured by this run",
-    "C1_m32_n64_k64": "bit-exact against the golden fixture: no tolerance",
+    "C1_m64_n128_k256": "golden fixture (the reference's own gemm_rrr on the seeded inputs): dequantised W bit-exact; all 8192 outputs of C within 2 bf16 ULP, no near-zero escape",
     "C2_decode_m1_n4096_k4096": {"checks": 11, "outputs": 45056, "outside_bound": 0, "worst_ulp": 1.20, "worst_excess_units": 0.0},
     "C3_n11008_k4096_m1_4_8_16_32": {"checks": 5, "outputs": 671488, "outside_bound": 12, "worst_ulp": 1.81, "worst_excess_units": 0.08},
     "C4_m4096_n4096_k4096": {"checks": 2, "outputs": 33554432, "outside_bound": 456, "worst_ulp": 2.5, "worst_excess_units": 0.44},
@@ -75,7 +75,7 @@ RECORDED_ACCEPTANCE = {
     "whole_suite": {"checks": 804, "outputs": 355743104, "outside_bound": 1190, "worst_excess_units": 0.61},
 }
 
-C3_ROWS = (1, 16, 32)        # BASELINE config 3 (M in {1,4,8,16,32}): the rows the default line carries; --sweep has all five
+C3_ROWS = (1, 4, 8, 16, 32)  # BASELINE config 3: every M of the sweep is in the default line
 C5_ROWS = (1, 16, 2048)      # BASELINE config 5: 4-bit codes, scale groups of 128 rows
 
 
@@ -255,6 +255,87 @@ def time_read_ceiling(af, w, steps, warmup):
     return time_launches(lambda i: af.probe_read(w.b[i % nb]), nb, steps, warmup)[0]
 
 
+class PowerSampler:
+    """Board power (W) and its cap read from the amdgpu hwmon files while a timed region runs: the evidence for which
+    bound a compute-bound launch hits on this part.  Silent when the files are absent or unreadable."""
+
+    def __init__(self, period_s=0.02):
+        import glob
+        self.files = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") or \
+            glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average")
+        self.caps = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")
+        self.period, self.samples, self.stop, self.thread = period_s, [], False, None
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    def __enter__(self):
+        import threading
+        if self.files:
+            def run():
+                while not self.stop:
+                    v = self._read(self.files[0])
+                    if v is not None:
+                        self.samples.append(v)
+                    time.sleep(self.period)
+            self.thread = threading.Thread(target=run, daemon=True)
+            self.thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self.stop = True
+        if self.thread is not None:
+            self.thread.join()
+
+    def summary(self):
+        if not self.samples:
+            return {"note": "no readable hwmon power file on this machine"}
+        # the first samples of a region still show the ramp from the level before it: the upper half is the plateau
+        top = sorted(self.samples)[len(self.samples) // 2:]
+        cap = self._read(self.caps[0]) if self.caps else None
+        return {"board_power_w_plateau": round(sum(top) / len(top), 1), "board_power_w_max": round(max(self.samples), 1),
+                "power_cap_w": cap, "samples": len(self.samples), "source": self.files[0]}
+
+
+def prefill_loop_trace(af, shapes=((256, 4096, 4096), (512, 4096, 4096), (1024, 4096, 4096), (2048, 4096, 4096), (4096, 4096, 4096), (8192, 8192, 4096))):
+    """Needs a library built with -DBFAINTB_TRACE (--lib): the 256x256-tile kernel then writes, per wave, the shader
+    cycles and the 100 MHz ticks its K loop took into the workspace.  Reported by tile count: cycles per K-step of 64
+    (128 matrix instructions per wave: 2048 cycles of matrix pipe) and the shader clock the loop ran at."""
+    import torch
+    rows = []
+    for (m, n, k) in shapes:
+        w = Workload(f"m{m}_n{n}_k{k}", m, n, k, copies=2)
+        tiles = -(-m // 256) * -(-n // 256)
+        ws = torch.zeros(max(tiles, 8) * 4 * 64 + 4096, dtype=torch.uint8, device="cuda")
+
+        def launch(i):
+            af.gemm(w.c, w.a, w.b[i % 2], w.s, m, n, k, which=af.PREFILL_256, workspace=ws, workspace_nbytes=ws.numel())
+        for i in range(100):   # long enough for the clock to settle under this load
+            launch(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(40):
+            launch(i)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 40
+        t = ws[: tiles * 4 * 64].cpu().numpy().view(np.uint64).reshape(-1, 8).astype(np.int64)
+        steps = -(-k // 64)
+        rows.append({"m": m, "n": n, "k": k, "tiles_256x256": tiles, "us_per_launch_eager_loop": round(us, 2),
+                     "k_loop_cycles_per_step": round(float((t[:, 0] / steps).mean()), 1),
+                     "shader_clock_mhz": round(float((t[:, 0] / t[:, 1]).mean() * 100.0), 0),
+                     "matrix_pipe_cycles_per_step": 2048})
+        del w, ws
+        torch.cuda.empty_cache()
+    return rows
+
+
 def time_vendor_bf16_gemm(w, steps, warmup):
     """Context for the prefill figure: the vendor library's plain bf16 x bf16 GEMM (torch.matmul, i.e.
     hipBLASLt) on the same activations and the already dequantised weights, same graph protocol.  It does
@@ -378,7 +459,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
-                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192")
+                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | prefill_trace (needs --lib "
+                    "with a library built with -DBFAINTB_TRACE)")
+    ap.add_argument("--lib", default="", help="load this build of libbfaintb_gemm.so instead of the package's own "
+                    "(an instrumented build, for --only prefill_trace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the GEMM would shard over the columns "
@@ -389,10 +473,17 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     import awesome_fusion_amd as af
+    if args.lib:
+        sys.modules["awesome_fusion_amd.gemm"]._LIB = os.path.abspath(args.lib)
     af.lib()
 
     K, W = args.steps, args.warmup
     out_extra = {}
+
+    if args.only == "prefill_trace":
+        print(json.dumps({"metric": "bfAintBGemm 256x256-tile kernel: K-loop cycles per step and shader clock by tile count (instrumented build)",
+                          "library": af.library_path(), "rows": prefill_loop_trace(af)}))
+        return
 
     # ---- one secondary workload alone (profiling runs)
     if args.only.startswith(("c3_m", "c5_m", "mid_m")):
@@ -474,10 +565,12 @@ def main():
     if args.only in ("", "prefill"):
         w = Workload("prefill_m4096_n4096_k4096_int8_perchannel", 4096, 4096, 4096, copies=2)
         pk = max(20, min(K, 100))
-        ev_ms, wall_ms = time_graph(af, w, pk, max(5, W // 4), rotate=True)
+        with PowerSampler() as power:
+            ev_ms, wall_ms = time_graph(af, w, pk, max(5, W // 4), rotate=True)
         entry = {"value": round(w.flops / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "steps": pk,
                  "ms_per_step": round(wall_ms, 6), "GB/s": round(w.bytes / (wall_ms * 1e-3) / 1e9, 1),
-                 "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma")}
+                 "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma"),
+                 "board_power_during_timed_region": power.summary()}
         try:
             v_ms = time_vendor_bf16_gemm(w, pk, 5)
             entry["vendor_bf16_gemm_same_shape"] = {"TFLOP/s": round(w.flops / (v_ms * 1e-3) / 1e12, 2), "kernel_us": round(v_ms * 1e3, 3),
@@ -503,11 +596,13 @@ def main():
     if args.only == "":
         rows = []
         w32 = config3_workload(32)
-        for m in ((1, 4, 8, 16, 32) if args.sweep else C3_ROWS):
+        read_ms = time_read_ceiling(af, w32, min(K, 200), min(W, 10))   # the same rotation through a kernel that only fetches B
+        for m in C3_ROWS:
             w = w32.rows(m, f"decode_m{m}_n11008_k4096_int8_perchannel")
             steps = min(K, 200)
             ev_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True)
-            rows.append(compact({"workload": w.name, "steps": steps, **roofline_entry(w, ev_ms, "hbm")}))
+            rows.append({**compact({"workload": w.name, "steps": steps, **roofline_entry(w, ev_ms, "hbm")}),
+                         "fetch_only_kernel_us": round(read_ms * 1e3, 3), "frac_of_fetch_only": round(read_ms / ev_ms, 4)})
             if args.sweep and m <= 8:
                 pk_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True, packed=True)
                 rows.append(compact({"workload": w.name + "_prepacked", "steps": steps, **roofline_entry(w, pk_ms, "hbm")}))
@@ -516,6 +611,7 @@ def main():
         torch.cuda.empty_cache()
         rows = []
         w16 = config5_workload(16)
+        read_ms = time_read_ceiling(af, w16, min(K, 100), min(W, 10))
         for m in C5_ROWS:
             if m <= 16:
                 w = w16.rows(m, f"m{m}_n28672_k8192_int4_group128")
@@ -527,6 +623,8 @@ def main():
                 steps = 10
             ev_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True)
             rows.append(compact({"workload": w.name, "steps": steps, **roofline_entry(w, ev_ms, "hbm" if m <= 32 else "mfma")}))
+            if m <= 32:
+                rows[-1].update({"fetch_only_kernel_us": round(read_ms * 1e3, 3), "frac_of_fetch_only": round(read_ms / ev_ms, 4)})
             if args.sweep and m == 1:
                 pk_ms, _ = time_graph(af, w, steps, min(W, 10), rotate=True, packed=True)
                 rows.append(compact({"workload": w.name + "_prepacked", "steps": steps, **roofline_entry(w, pk_ms, "hbm")}))

@@ -220,9 +220,22 @@ BFAINTB_API int bfaintb_init(void* stream);
 BFAINTB_API int bfaintb_gemm_static(void* c, const void* a, const void* b, const void* scale, uint32_t m, uint32_t n, uint32_t k,
                         uint32_t lda, uint32_t ldb, uint32_t ldc, int weight_bits, uint32_t group_size, void* stream);
 BFAINTB_API size_t bfaintb_gemm_static_scratch_bytes(void);
+/*
+ * bfaintb_workspace_status and bfaintb_workspace_init for that scratch, whose address the library keeps to itself.
+ * _status (a synchronising query, like bfaintb_workspace_status) answers BFAINTB_OK, or BFAINTB_ERR_WORKSPACE_POISONED
+ * once a split-K wait has given up on the current device's scratch — two overlapping bfaintb_gemm_static calls on one
+ * GPU are the likely cause — after which later static calls on that GPU may take a stale partial sum for a fresh one.
+ * _reset puts the scratch back into its at-rest state on `stream` (a fill kernel, asynchronous; after bfaintb_init it
+ * may be recorded into a HIP graph); the caller makes sure that no bfaintb_gemm_static call on that GPU is in flight
+ * or follows on another stream before the reset has run.  Both allocate nothing.  No counterpart in the reference.
+ */
+BFAINTB_API int bfaintb_static_scratch_status(void* stream);
+BFAINTB_API int bfaintb_static_scratch_reset(void* stream);
 
 /*
- * Test hooks (no effect on results in normal operation; process-wide, read by each following launch):
+ * Test hooks (no effect on results in normal operation; process-wide, read by each following launch).  The first two
+ * change what split-K launches do and are for the library's own tests: they are refused with BFAINTB_ERR_UNSUPPORTED
+ * unless the process has BFAINTB_TEST_HOOKS=1 in its environment.
  *   BFAINTB_DEBUG_SPLIT_WAIT_LIMIT   value = fetch attempts a reducing workgroup makes before it gives up (0 restores 2^18)
  *   BFAINTB_DEBUG_WITHHOLD_PARTIALS  value != 0: the workgroups of all splits but the last compute and then keep their
  *                                    sums to themselves, so the reducer's wait runs out — the way to exercise the
@@ -240,8 +253,7 @@ BFAINTB_API int bfaintb_debug_control(uint32_t what, uint32_t value);
  * order of the matrix instruction ("mfma16": column blocks of 16, K-chunks of 64 rows, a lane's two 8-row operands
  * adjacent; bfaintb_packed.hip states it byte by byte); bfaintb_gemm_prepacked multiplies by the packed copy.  A
  * block of 16 columns is then one contiguous slab, n / 16 workgroups stream their slabs linearly and own their
- * outputs, and a few rows of A (8 in general; more on small matrices and for 4-bit codes) need no split along k, no workspace
- * and no second pass.  Successor of the
+ * outputs, and a few rows of A need no split along k, no workspace and no second pass.  Successor of the
  * reference's host-side formatter mem_transfer<int8_t, ...> (mem_transfer.hpp:23-32), which writes the
  * bytes the device will read; the reference itself keeps B row-major (bfAintBGemm.cc:101-103).
  *   packed    device buffer of bfaintb_prepack_bytes(n, k, weight_bits) bytes (= n * k * weight_bits / 8), 16-byte aligned;
@@ -265,10 +277,10 @@ BFAINTB_API int bfaintb_gemm_prepacked(void* c, const void* a, const void* packe
 BFAINTB_API int bfaintb_gemm_prepacked_fused(void* c, const void* a, const void* packed_b, const void* scale,
                                  const bfaintb_epilogue* epilogue, uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc,
                                  int weight_bits, uint32_t group_size, void* workspace, size_t workspace_bytes, void* stream);
-/* Scratch bfaintb_gemm_prepacked needs: 0 where the slab-streaming kernel runs (8-bit codes: m <= 8, m <= 32 when n * k <= 16 Mi and
- * n >= 4096, never when n < 2048 and k >= 12288; 4-bit codes: m <= 48 while n * k <= 24 Mi (m <= 20 when n < 2048 and k >= 12288), m <= 24 below 64 Mi, m <= 8 beyond; 8-bit: m <= 4 beyond 96 Mi) and for the large tiles; otherwise what the decode family or the
- * 128x128 tiles need when they split along k (the plan of the row-major path): always ask, for the shape at hand.  Same workspace protocol as bfaintb_gemm
- * (bfaintb_workspace_init once; one workspace may serve both entry points). */
+/* Scratch bfaintb_gemm_prepacked needs: 0 where a kernel that does not split k runs (the slab-streaming kernel for a few
+ * rows of A, the large tiles), otherwise what the decode family or the small tiles need when they split along k — always
+ * ask, for the shape at hand.  Same workspace protocol as bfaintb_gemm (bfaintb_workspace_init once; one workspace may
+ * serve both entry points). */
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 BFAINTB_API size_t bfaintb_gemm_prepacked_workspace_bytes_ex(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size,
                                                  int variant);
@@ -310,8 +322,8 @@ BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int wei
 
 /* Rows (bfaintb_prefill_tile) and columns of the tiles BFAINTB_VARIANT_PREFILL runs an m x n output of row-major
  * weights with: 128 x 128 while that makes at most 256 tiles (one per CU); else 256 rows x 128 columns while that
- * makes at most 256; else 256 x 256.  (Pre-packed weights and the reference arithmetic have no 256 x 128 form: 256 x 256
- * there.)  Depend only on their arguments. */
+ * makes at most 256; else 256 x 256.  Pre-packed weights run the same tiles.  (The reference arithmetic has no
+ * 256 x 128 form: 256 x 256 there.)  Depend only on their arguments. */
 BFAINTB_API uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n);
 BFAINTB_API uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n);
 

@@ -4,6 +4,9 @@ import sys
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# the library's split-K test hooks (bfaintb_debug_control: withheld partial sums, the wait's limit) only work in a
+# process that asks for them before the library reads its environment
+os.environ.setdefault("BFAINTB_TEST_HOOKS", "1")
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 

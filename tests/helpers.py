@@ -134,15 +134,25 @@ NOISE_FACTOR = 2.0   # the escape below: this many times 2^-24 * sum_k |a_k w_k|
 NEAR_ZERO = 0.125    # ... and only for outputs below this fraction of rms(C)
 
 
-def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
+def allowed_outside(outputs, rate=3e-5):
+    """How many outputs of a check may take the near-zero escape: the rate seen at the full-size BASELINE shapes is
+    1.4e-5 to 2.1e-5 of the outputs (228 of 16.7 M at config 4, 98 of 4.6 M at config 5); allowed is 3e-5 of them plus
+    four standard deviations of a count of that mean, and a handful for small problems — so that a kernel whose
+    cancelling outputs are a few times worse than today's fails at the sizes where it can be told from chance
+    (config 4: 593 allowed against 228 seen; the old cap of 2e-4 allowed 3355)."""
+    mean = rate * outputs
+    return max(3, int(mean + 4.0 * np.sqrt(mean)))
+
+
+def assert_close_ulp(p, c_bits, what, rows=None, threads=8):
     """The acceptance bound of this build: every output within 2 bf16 ULP of the fp32
     sequential-K oracle, or within 1e-2 relative where |ref| < 1e-3.
 
     No summation order other than the oracle's own can meet that bound for outputs that cancel to
     (almost) nothing: there a bf16 ULP is smaller than the fp32 rounding noise of the K-term sum on
-    EITHER side.  Such outputs are rare (counted, capped at max_frac of the outputs, and recorded in
-    ACCEPTANCE_LOG); each must be small (|ref| < rms(C) / 8: an output of ordinary size has no such excuse)
-    and must lie within 2 ULP + 8 * 2^-24 * sum_k |a_k w_k| of the fp64-accumulated value.  The second
+    EITHER side.  Such outputs are rare (counted, capped by allowed_outside(), and recorded in
+    ACCEPTANCE_LOG); each must be small (|ref| < rms(C) * NEAR_ZERO: an output of ordinary size has no such excuse)
+    and must lie within 2 ULP + NOISE_FACTOR * 2^-24 * sum_k |a_k w_k| of the fp64-accumulated value.  The second
     term is a few times the rounding error an fp32 sum of those terms makes in any order (measured worst
     over the BASELINE shapes: 1.3 of these units for the device, 4.4 for the sequential oracle); one
     dropped or doubled term of ordinary size is a thousand of them.
@@ -159,7 +169,7 @@ def assert_close_ulp(p, c_bits, what, rows=None, threads=8, max_frac=2e-4):
     nbad_c, _, _ = oracle.check_ulp(c_ref, c_bits)
     assert nbad_c == len(bad), "C and numpy acceptance checks disagree"
     # (a handful is always allowed: over 4000 random problems of a few thousand outputs each, six had 2 or 3 such outputs)
-    assert len(bad) <= max(3, int(max_frac * c_ref.size)), \
+    assert len(bad) <= allowed_outside(c_ref.size), \
         f"{what}: {len(bad)} of {c_ref.size} outputs outside 2 ULP (worst {ulps.max():.2f} ULP)"
     worst_units = 0.0
     if len(bad):

@@ -155,6 +155,21 @@ def test_rejects_bad_arguments_without_launching():
     assert L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 2) == 0 and L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 0) == 0
 
 
+def test_split_k_test_hooks_are_refused_without_the_environment_switch():
+    """The hooks that withhold partial sums or cap the reducer's wait change what every later split-K launch of the
+    process does: a process that has not asked for them (BFAINTB_TEST_HOOKS=1) gets BFAINTB_ERR_UNSUPPORTED."""
+    import subprocess
+    import sys
+    code = ("import os, sys; sys.path.insert(0, %r); os.environ.pop('BFAINTB_TEST_HOOKS', None); os.environ['BFAINTB_TEST_HOOKS'] = sys.argv[1];"
+            "import awesome_fusion_amd as af; L = af.lib();"
+            "print(L.bfaintb_debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 3), L.bfaintb_debug_control(af.DEBUG_WITHHOLD_PARTIALS, 1),"
+            " L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 0))") % ROOT
+    for value, want in (("0", "-5 -5 0"), ("1", "0 0 0")):
+        r = subprocess.run([sys.executable, "-c", code, value], capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        assert r.stdout.split("\n")[-2].strip() == want, (value, r.stdout, r.stderr[-500:])
+
+
 def test_prepacked_entry_points_validate_before_launching():
     L = af.lib()
     assert af.prepack_bytes(4096, 4096, 8) == 4096 * 4096 and af.prepack_bytes(4096, 4096, 4) == 4096 * 4096 // 2

@@ -119,7 +119,7 @@ def test_config2_and_3_decode(af, m):
 def test_config4_prefill_full_size(af):
     p = Problem(4096, 4096, 4096, seed=4)
     c = run_gemm(p)
-    worst, near_zero = assert_close_ulp(p, c, "prefill 4096^3", threads=16, max_frac=1e-4)
+    worst, near_zero = assert_close_ulp(p, c, "prefill 4096^3", threads=16)
     print(f"prefill 4096^3: worst {worst:.3f} ULP, {near_zero} near-zero outputs beyond 2 ULP (within fp32 summation noise)")
 
 

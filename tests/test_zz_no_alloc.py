@@ -67,6 +67,37 @@ def test_static_scratch_refuses_what_does_not_fit(af):
     assert "bfaintb_gemm" in af.error_string(af.ERR_STATIC_SCRATCH)
 
 
+def test_static_scratch_status_and_reset_after_a_give_up(af):
+    """The give-up path on the library's own scratch, forced from the host (producers keep their sums, the wait is capped:
+    every kernel exits normally): the call's outputs are NaN, bfaintb_static_scratch_status reports the poisoned scratch,
+    bfaintb_static_scratch_reset repairs it, and the next call gives bfaintb_gemm's bits again."""
+    import torch
+    af.init()
+    p = Problem(4, 2048, 4096, seed=91)
+    assert af.split_k(p.m, p.n, p.k) > 1
+    c_static, c_plain, _ = _both(af, p)
+    assert np.array_equal(c_static, c_plain)
+    assert af.static_scratch_status() == 0
+    a, b, s = to_dev(p.a_bf), to_dev(p.b_bytes), to_dev(p.s_bf)
+    c = torch.zeros((p.m, p.n), dtype=torch.int16, device="cuda")
+    try:
+        af.debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 3)
+        af.debug_control(af.DEBUG_WITHHOLD_PARTIALS, 1)
+        af.gemm_static(c, a, b, s, p.m, p.n, p.k)
+        torch.cuda.synchronize()
+    finally:
+        af.debug_control(af.DEBUG_WITHHOLD_PARTIALS, 0)
+        af.debug_control(af.DEBUG_SPLIT_WAIT_LIMIT, 0)
+    got = from_dev_u16(c).astype(np.uint32) << 16
+    assert np.isnan(got.view(np.float32)).all(), "every output misses partial sums: all NaN"
+    assert af.static_scratch_status() == af.ERR_WORKSPACE_POISONED
+    af.static_scratch_reset()
+    assert af.static_scratch_status() == 0
+    c_static, c_plain, _ = _both(af, p)
+    assert np.array_equal(c_static, c_plain)
+    assert af.static_scratch_status() == 0
+
+
 def test_static_entry_point_can_be_captured_and_replayed(af):
     """No allocation, no memset, no host-side wait: the call records into a HIP graph; replays, with eager calls on the
     same scratch in between, give the eager result every time."""
