@@ -47,8 +47,26 @@ using bfaintb::kEmptyWord;
 constexpr uint32_t kDecodeAutoMaxM = 32;       // AUTO always runs the decode family up to this m
 constexpr uint32_t kDecodeFamilyAutoMaxM = 4096;  // ... and never beyond this one
 constexpr uint32_t kDecodeMaxM = 32768;        // what the decode family accepts when forced
-constexpr uint32_t kDecodeTargetWgs = 480;        // 4-wave workgroups: a little under two per CU on a 256-CU part
-constexpr uint32_t kDecodeTargetWgsNarrow = 256;  // 8-wave workgroups: one per CU
+// Compute units the plans are made for: those of the device that is current when the first plan is made (256 where there
+// is no device to ask: the part the estimates were fitted on), or what the tuning hook says.  One count per process:
+// workspace sizes and launches must agree, whichever device a later call runs on (a plan for another count is still a
+// correct launch, only not the fastest one).
+std::atomic<uint32_t> g_plan_cus_override{0};
+uint32_t machine_cus()
+{
+    static const uint32_t device_cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            return (uint32_t)n;
+        (void)hipGetLastError();
+        return 256u;
+    }();
+    const uint32_t forced = g_plan_cus_override.load(std::memory_order_relaxed);
+    return forced ? forced : device_cus;
+}
+// workgroups the decode launches aim at: 8-wave workgroups run one per CU; 4-wave ones a little under two per CU
+uint32_t decode_target_wgs_narrow() { return machine_cus(); }
+uint32_t decode_target_wgs() { return machine_cus() * 15u / 8u; }
 constexpr uint32_t kMaxSplits = 64;
 constexpr uint32_t kPackedSlabMaxM = 48;       // packed weights: the slab-streaming kernel never runs more rows of A than this
 
@@ -91,7 +109,7 @@ static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bo
     pl.splits = (k + per - 1) / per;
 }
 
-// Rough time, in microseconds, of the decode family on a 256-CU part for more than 32 rows of A.
+// Rough time, in microseconds, of the decode family for more than 32 rows of A (fitted on a 256-CU part).
 // Every block of 16*mb rows streams and dequantises all weights again: measured 16, 22 and 35 cycles per
 // weight and lane for mb = 1, 2, 4 (the dequantisation plus mb matrix instructions per 8 weights, less well
 // overlapped the fewer waves a SIMD holds); repeats of the stream mostly hit in cache; split-K partial sums
@@ -103,7 +121,8 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
     const double row_blocks = (double)((m + 16u * pl.mb - 1u) / (16u * pl.mb));
     const double col_blocks = (double)((n + pl.cols - 1u) / pl.cols);
     const double waves = row_blocks * col_blocks * pl.splits * pl.waves;
-    const double busy = waves >= 1024.0 ? 1.0 : waves / 1024.0;
+    const double cus = (double)machine_cus();
+    const double busy = waves >= 4.0 * cus ? 1.0 : waves / (4.0 * cus);
     // 8-bit codes, refitted to a scan over row-block size x split factor at m = 40 .. 512 on 4096 x 4096, 11008 x 4096,
     // 4096 x 11008 and 2048 x 8192 (the choice of row block then lands within 0.5 % of the best on all 27 points; the
     // constants before it picked 16-row blocks where 32-row blocks with twice the splits run 6-24 % faster): larger row
@@ -113,30 +132,30 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
     // workgroups beyond one per CU share a CU's arithmetic: the last, partly filled round costs a whole one
     // (measured at n = k = 4096, 64-row blocks: m = 512 -> 256 workgroups, 35 us; m = 640 -> 320 workgroups, 61 us)
     const double wgs = row_blocks * col_blocks * pl.splits;
-    const double ragged = wgs > 256.0 ? (double)(uint64_t)((wgs + 255.0) / 256.0) * 256.0 / wgs : 1.0;
-    const double compute = row_blocks * weights * cycles_per_weight / 65536.0 / 2000.0 / busy * ragged;
-    const double stream_busy = bits == 8 ? (wgs >= 256.0 ? 1.0 : wgs / 256.0) : busy;
+    const double ragged = wgs > cus ? (double)(uint64_t)((wgs + cus - 1.0) / cus) * cus / wgs : 1.0;
+    const double compute = row_blocks * weights * cycles_per_weight / (256.0 * cus) / 2000.0 / busy * ragged;  // 4 SIMDs x 64 lanes per CU at 2 GHz
+    const double stream_busy = bits == 8 ? (wgs >= cus ? 1.0 : wgs / cus) : busy;
     const double stream = weights * bits / 8.0 * (1.0 + (bits == 8 ? 0.5 : 0.3) * (row_blocks - 1.0)) / 3.5e6 / stream_busy;
     const double partial = pl.splits > 1 ? 3.0 + 12.0 * (pl.splits - 1.0) * m * n / 1.5e6 : 0.0;
     return 5.0 + (compute > stream ? compute : stream) + partial;
 }
 
-// The tiled variant runs 128x128 tiles while those fit one per CU (at most 256 of them): four times the workgroups of
+// The tiled variant runs 128x128 tiles while those fit one per CU: four times the workgroups of
 // 256x256 tiles, each with a quarter of the work per K-step.  Measured against the large tiles (8-bit, k = 4096, us):
 // m x n = 256 x 4096: 48 / 59, 1024 x 4096: 58 / 66, 512 x 8192 (4-bit, k = 8192): 112 / 137; with more tiles the
 // large ones win (1536 x 4096: 81 / 72, 512 x 11008: 80 / 68).
 static bool prefill_small_tiles(uint32_t m, uint32_t n)
 {
-    return (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u) <= 256u;
+    return (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u) <= machine_cus();
 }
 
-// Between the two: more than 256 small tiles but at most 256 tiles of 256 rows x 128 columns.  The large tiles would
+// Between the two: more small tiles than CUs, but at most one tile of 256 rows x 128 columns per CU.  The large tiles would
 // occupy a quarter to a half of the CUs there; the tall ones run one per CU at 0.94 us per K-step against the large tiles'
 // 1.02 on twice the work (8-bit, 64 steps, us tall / large: 1536 x 4096: 61.0 / 66.0; 512 x 11008: 60.3 / 64.7; 2048 x 4096:
 // 71.0 / 75.7; 128 steps, 1024 x 8192: 129 / 141; 4-bit, 768 x 8192: 138 / 140).
 static bool prefill_tall_tiles(uint32_t m, uint32_t n)
 {
-    return !prefill_small_tiles(m, n) && (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u) <= 256u;
+    return !prefill_small_tiles(m, n) && (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u) <= machine_cus();
 }
 
 static bool is_prefill(int v)
@@ -151,7 +170,7 @@ static bool use_small_tiles(int v, uint32_t m, uint32_t n)
     return v == BFAINTB_VARIANT_PREFILL_128 || v == BFAINTB_VARIANT_PREFILL_128_LDS || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n));
 }
 
-// Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over 256 CUs, 1.33 us per 64 rows of
+// Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over the CUs, 1.33 us per 64 rows of
 // k.  Small tiles: a K-step takes 0.49 us on an empty machine and 0.56 us with a workgroup on every CU (the kernel that
 // keeps the weights in registers; 0.64 and 0.67 us with 4-bit codes), whichever order the weights are stored in.
 // The small-tile kernel may split k: grid y walks the splits, each workgroup runs its share of
@@ -174,6 +193,7 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
 {
     const uint32_t ksteps = (k + 63u) / 64u;
     const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
+    const double cus = (double)machine_cus();
     auto shape = [&](uint32_t want) {
         TilePlan t;
         if (want > kMaxTileSplits) want = kMaxTileSplits;
@@ -189,7 +209,7 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         // a K-step: 0.49 us (4-bit codes 0.64) on an empty machine, rising by 0.01 per 100 workgroups; with a workgroup on
         // (nearly) every CU 8-bit codes take 0.56 (the clock gives way)
         const double wgs = tiles * t.splits;
-        const double step_us = bits == 4 ? 0.64 + 0.0001 * wgs : 0.485 + 0.0001 * wgs + (wgs >= 240.0 ? 0.055 : 0.0);
+        const double step_us = bits == 4 ? 0.64 + 0.0001 * wgs : 0.485 + 0.0001 * wgs + (wgs >= 0.9375 * cus ? 0.055 : 0.0);
         t.us = 4.0 + per * step_us + hand_over;
         // (three splits and more: the hand-over scatters more than this says, and where the row-blocked family is about as
         // fast it is the safer pick — 192 x 4096 x 4096: 25.5 against 22.9 us, 128 x 4096 x 11008: 39.0 against 34.3)
@@ -200,7 +220,7 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
     TilePlan best = shape(1);
     static const uint32_t kCandidates[] = {2, 3, 4, 6, 8};
     for (uint32_t s : kCandidates) {
-        if (tiles * s > 256.0) break;
+        if (tiles * s > cus) break;
         const TilePlan t = shape(s);
         if (t.splits != s) continue;  // k does not divide that way
         // (at most 256 tiles' worth of sums in all, 14 MiB: within the 32-bit offsets of the kernel and within the scratch of
@@ -214,7 +234,8 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
     if (prefill_small_tiles(m, n)) return tile128_plan(m, n, k, bits, 0).us;
     const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
-    const double rounds = (double)(uint64_t)((tiles + 255.0) / 256.0);
+    const double cus = (double)machine_cus();
+    const double rounds = (double)(uint64_t)((tiles + cus - 1.0) / cus);
     return 4.0 + rounds * (k / 64.0) * 1.33;
 }
 
@@ -243,7 +264,7 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
         if (bits == 8 && forced_splits == 0) {
             // (at most 16 splits, 8 while k is short: 512 x 4096, m = 48: 11.0 us with 16 splits, 7.0 with 8; 1024 x 8192, m = 32:
             // 9.1 with 16, 10.1 with 8)
-            uint32_t s = 256u / tiles;
+            uint32_t s = machine_cus() / (tiles ? tiles : 1u);
             const uint32_t most = k >= 8192u ? 16u : k / 512u > 8u ? k / 512u : 8u;
             if (s > most) s = most;
             for (; s > 1u; --s) {
@@ -261,7 +282,7 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
             if (forced_splits && s != 1u) break;
             set_splits(c, k, bits, forced_splits ? forced_splits : s, packed);
             if (!forced_splits && c.splits != s && s != 1u) continue;  // k does not divide that way
-            if (!forced_splits && s > 1u && tiles * s > 768u) break;
+            if (!forced_splits && s > 1u && tiles * s > 3u * machine_cus()) break;
             double t = decode_family_estimate_us(m, n, k, bits, c);
             // (packed codes: the kernels of 16-row blocks are the weaker ones there, and the estimate's price of a split sends
             // 17 to 32 rows against many columns to them — 32000 x 4096, m = 32: 47.8 us in two blocks of 16 rows, 32.0 in one of
@@ -290,7 +311,7 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
     // those (the 32- and 64-row kernels spend longer in their reductions than such a launch has; 768 x 5120, m = 48: 7.5
     // against 10.8 us; 1536 x 8960: 10.8 / 14.3; 256 x 7168, m = 128: 7.8 / 11.7; with more blocks the larger ones win:
     // 2048 x 8192, m = 128: 20.2 / 16.3)
-    if (bits == 8 && m > 32 && forced_splits == 0 && (uint64_t)((n + 127u) / 128u) * ((m + 15u) / 16u) <= 40u)
+    if (bits == 8 && m > 32 && forced_splits == 0 && (uint64_t)((n + 127u) / 128u) * ((m + 15u) / 16u) <= machine_cus() * 5u / 32u)
         return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u);
     // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
     // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
@@ -321,19 +342,20 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         const uint32_t narrow_blocks = (n + 127u) / 128u;
         uint32_t narrow_splits = 1;
         double best = 0.0;
+        const uint32_t cus = machine_cus();
         for (uint32_t s = 1; s <= cap && s <= 16u; ++s) {
-            const double rounds = (double)((narrow_blocks * s + 255u) / 256u);
+            const double rounds = (double)((narrow_blocks * s + cus - 1u) / cus);
             const double g = rounds / s + 0.04 * s * 4096.0 / k;  // time of the rounds + what a split costs, both relative to one pass over k
             if (best == 0.0 || g < best) { best = g; narrow_splits = s; }
         }
         const uint32_t narrow_wgs = narrow_blocks * narrow_splits;
-        const bool fills_rounds = narrow_wgs * 20u >= ((narrow_wgs + 255u) / 256u) * 256u * 19u;  // >= 95 % of whole rounds
+        const bool fills_rounds = narrow_wgs * 20u >= ((narrow_wgs + cus - 1u) / cus) * cus * 19u;  // >= 95 % of whole rounds
         // m >= 8 on a wide matrix: once 256-column blocks fill their one round with at most 3 splits (more than 64 of
         // them) their partial sums no longer outweigh the better stream (m = 8 / 16 / 32, wide against narrow:
         // 22016 x 4096 20.9 / 22.7 / 28.2 against 21.9 / 23.4 / 31.6 us; 28672 x 8192 46.2 / 48.3 / 54.2 against 49.8 / 53.1 /
         // 61.5; 18944 x 3584 16.9 / 18.3 / 24.0 against 18.0 / 19.9 / 25.1; with fewer blocks narrow stays ahead:
         // 11008 x 4096 13.9 / 14.9 / 17.9 against 13.8 / 16.5 / 22.1; 14336 x 4096 17.2 / 18.5 / 21.4 against 17.6 / 19.0 / 25.1)
-        const bool many_wide_blocks = (n + 255u) / 256u > 64u;
+        const bool many_wide_blocks = (n + 255u) / 256u > cus / 4u;
         // (n not a multiple of 16: only the 8-codes-per-lane shape can read the last columns)
         const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 || (m >= 8 && (!many_wide_blocks || packed)));  // packed weights: the kernels are built for 128 columns
         pl.cols = narrow ? 128u : 256u;
@@ -359,8 +381,8 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 // 8-bit codes with 4 waves: one round on every shape measured (m = 1: 11008 x 4096 12.7 us with 215 workgroups,
                 // 13.2 with 473; 9216 x 4096 11.7 / 13.1; 5120 x 8192 12.8 / 15.7; 18944 x 3584 15.8 / 17.4; 22016 x 4096
                 // 19.6 / 21.8; 28672 x 8192 43.8 / 44.8; a few workgroups past the round are the worst case: 258 -> 15.3 us)
-                const bool one_round = pl.waves == 8u || bits == 8 || (bits == 4 && col_blocks <= 64u);
-                splits = one_round ? kDecodeTargetWgsNarrow / col_blocks : (kDecodeTargetWgs + col_blocks / 2) / col_blocks;
+                const bool one_round = pl.waves == 8u || bits == 8 || (bits == 4 && col_blocks <= cus / 4u);
+                splits = one_round ? decode_target_wgs_narrow() / col_blocks : (decode_target_wgs() + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
                 // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each
                 // and whose partial sums the reducing workgroup must collect: beyond 16 splits (32 once k is long enough
@@ -597,6 +619,7 @@ int bfaintb_init(void* stream)
     DeviceState* dev = nullptr;
     int rc = device_state(st, &dev);
     if (rc) return rc;
+    (void)machine_cus();  // the device's compute units, asked for here rather than by a first plan made under capture
     void* ptr = nullptr;
     return static_scratch(*dev, st, &ptr);
 }
@@ -627,6 +650,10 @@ int bfaintb_debug_control(uint32_t what, uint32_t value)
         case BFAINTB_DEBUG_FORCE_ROW_BLOCK:
             if (value != 0u && value != 1u && value != 2u && value != 4u) return BFAINTB_ERR_UNSUPPORTED;
             g_force_row_block.store(value);
+            return BFAINTB_OK;
+        case BFAINTB_DEBUG_PLAN_COMPUTE_UNITS:
+            if (value > 4096u) return BFAINTB_ERR_UNSUPPORTED;
+            g_plan_cus_override.store(value);
             return BFAINTB_OK;
         default: return BFAINTB_ERR_UNSUPPORTED;
     }
@@ -707,6 +734,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     p.lds = n;
     p.group_size = group_size;
     bfaintb::set_group_division(p);
+    p.cus = machine_cus();
     p.k_per_wg = k;
     p.splits = 1;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -870,7 +898,7 @@ static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
     // 4-bit codes in that corner: up to 20 rows (1024 x 16384, slab / family: m = 17: 22.4 / 24.5 us, 24: 31.4 / 24.8,
     // 32: 35.8 / 25.1; 512 x 12288, m = 24: 22.4 / 21.5; with k = 8192 the slab kernel stays ahead up to its 48 rows)
     if (bits == 4 && n < 2048u && k >= 12288u) return 20u;
-    if (bits == 8) return (weights <= (16ull << 20) && n >= 4096u) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
+    if (bits == 8) return (weights <= (16ull << 20) && n / 16u >= machine_cus()) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
     return weights <= (24ull << 20) ? kPackedSlabMaxM : weights < (64ull << 20) ? 24u : weights == (64ull << 20) ? 16u : 8u;
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
@@ -977,6 +1005,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
     p.lds = n;
     p.group_size = group_size;
     bfaintb::set_group_division(p);
+    p.cus = machine_cus();
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (is_prefill(v)) {
         // a tile's 16 column blocks and a 256-row panel of A are addressed through 32-bit buffer extents
@@ -1136,6 +1165,88 @@ int bfaintb_probe_read(const void* src, size_t bytes, void* sink, void* stream)
     if (misaligned16(src)) return BFAINTB_ERR_ALIGNMENT;
     if (bytes / 16 / 512 / 4 >= (1ull << 31)) return BFAINTB_ERR_BAD_SHAPE;
     return (int)bfaintb::launch_probe_read(src, bytes, sink, static_cast<hipStream_t>(stream));
+}
+
+// What a call would launch, without launching it: the queries above rolled into one description, for callers that want
+// to log or check the library's choice and for the scans that hold the choice against measurements.
+int bfaintb_gemm_plan(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int packed, int variant, uint32_t split_k,
+                      bfaintb_plan* out)
+{
+    if (out == nullptr) return BFAINTB_ERR_NULL_POINTER;
+    memset(out, 0, sizeof(*out));
+    int e = check_format(k, weight_bits, group_size);
+    if (e) return e;
+    e = check_shape(m, n, k, packed ? 8 : weight_bits);
+    if (e) return e;
+    if (packed) {
+        e = check_packed_shape(n, k, weight_bits);
+        if (e) return e;
+    }
+    const int v = packed ? packed_variant(m, n, k, weight_bits, variant) : resolve_variant(m, n, k, weight_bits, variant);
+    if (v < 0) return v;
+    out->compute_units = machine_cus();
+    out->launches = 1;
+    out->splits = 1;
+    out->k_per_workgroup = k;
+    if (m == 0 || n == 0) return BFAINTB_OK;
+    if (v == BFAINTB_VARIANT_DECODE) {
+        out->variant = v;
+        if (packed && packed_uses_slab(m, n, k, weight_bits)) {
+            out->kernel = BFAINTB_KERNEL_DECODE_SLAB;
+            out->tile_rows = m <= 16u ? 16u : 32u;
+            out->tile_cols = 16u;
+            out->waves = 8u;
+            out->workgroups = n / 16u * ((m + out->tile_rows - 1u) / out->tile_rows);
+            return BFAINTB_OK;
+        }
+        const DecodePlan pl = packed ? packed_family_plan(m, n, k, weight_bits) : decode_plan(m, n, k, weight_bits, split_k);
+        out->kernel = BFAINTB_KERNEL_DECODE_FAMILY;
+        out->tile_rows = 16u * pl.mb;
+        out->tile_cols = pl.cols;
+        out->waves = pl.waves;
+        out->splits = pl.splits;
+        out->k_per_workgroup = pl.k_per_wg;
+        out->workgroups = ((n + pl.cols - 1u) / pl.cols) * pl.splits * ((m + 16u * pl.mb - 1u) / (16u * pl.mb));
+        out->workspace_bytes = split_workspace_bytes(pl.splits, m, n);
+        return BFAINTB_OK;
+    }
+    // the tiled kernels
+    if (use_small_tiles(v, m, n)) {
+        out->variant = BFAINTB_VARIANT_PREFILL_128;
+        out->tile_rows = out->tile_cols = 128u;
+        const bool wreg = v != BFAINTB_VARIANT_PREFILL_128_LDS;
+        out->kernel = wreg ? BFAINTB_KERNEL_TILES_128 : BFAINTB_KERNEL_TILES_128_LDS;
+        out->waves = wreg ? 4u : 8u;
+        if (wreg) {
+            const TilePlan tp = tile128_plan(m, n, k, weight_bits, packed ? 0u : split_k);
+            out->splits = tp.splits;
+            out->k_per_workgroup = tp.k_per_wg;
+        }
+        out->workgroups = ((m + 127u) / 128u) * ((n + 127u) / 128u) * out->splits;
+        out->workspace_bytes = split_workspace_bytes(out->splits, m, n);
+        return BFAINTB_OK;
+    }
+    if (v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) {
+        out->variant = BFAINTB_VARIANT_PREFILL_256X128;
+        out->kernel = BFAINTB_KERNEL_TILES_256X128;
+        out->tile_rows = 256u;
+        out->tile_cols = 128u;
+        out->waves = 4u;
+        out->workgroups = ((m + 255u) / 256u) * ((n + 127u) / 128u);
+        return BFAINTB_OK;
+    }
+    out->variant = v == BFAINTB_VARIANT_PREFILL_256_LDS ? v : BFAINTB_VARIANT_PREFILL_256;
+    out->kernel = v == BFAINTB_VARIANT_PREFILL_256_LDS ? BFAINTB_KERNEL_TILES_256_LDS : BFAINTB_KERNEL_TILES_256;
+    out->tile_rows = out->tile_cols = 256u;
+    out->waves = v == BFAINTB_VARIANT_PREFILL_256_LDS ? 8u : 4u;
+    {
+        const uint32_t tiles = ((m + 255u) / 256u) * ((n + 255u) / 256u);
+        const uint32_t halves = bfaintb::thin_round_tiles(tiles, m, machine_cus());
+        out->workgroups = tiles - halves;
+        out->tail_workgroups = 2u * halves;
+        out->launches = (tiles - halves != 0u ? 1u : 0u) + (halves != 0u ? 1u : 0u);
+    }
+    return BFAINTB_OK;
 }
 
 uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n) { return prefill_small_tiles(m, n) ? 128u : 256u; }

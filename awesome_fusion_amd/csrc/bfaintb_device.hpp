@@ -86,6 +86,7 @@ struct GemmParams {
     uint32_t group_div_magic, group_div_shift1, group_div_shift2;
     // prefill variant: the logical 256x256 tiles one launch covers
     uint32_t tile_first, tile_count;
+    uint32_t cus;        // compute units the launch plan is made for (host side only)
     // split-K (decode variant only)
     uint32_t k_per_wg;   // rows of k one workgroup covers (multiple of 32 * decode_blocks_per_step * decode_waves)
     uint32_t decode_waves; // waves per workgroup of the decode variant (4 or 8)
@@ -127,6 +128,15 @@ __device__ __forceinline__ uint32_t group_of_row(const GemmParams& p, uint32_t r
     const uint32_t n = row >> 5;
     const uint32_t t = __umulhi(p.group_div_magic, n);
     return (t + ((n - t) >> p.group_div_shift1)) >> p.group_div_shift2;
+}
+
+// 256x256 tiles: how many of them, at the end, run as a second launch of half tiles.  Tiles beyond whole rounds of one
+// workgroup per CU, when they would fill at most half of the CUs (and every launch with fewer tiles than that), run as
+// twice as many workgroups of half the size.
+inline uint32_t thin_round_tiles(uint32_t tiles, uint32_t m, uint32_t cus)
+{
+    const uint32_t rest = tiles % cus;
+    return (rest != 0u && rest <= cus / 2u && m > 128u) ? rest : 0u;
 }
 
 // Launch through hipLaunchKernel so that the error returned belongs to THIS launch:

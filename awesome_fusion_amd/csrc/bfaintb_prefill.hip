@@ -619,13 +619,12 @@ static hipError_t launch_prefill_t(const GemmParams& p0, hipStream_t stream, boo
 {
     GemmParams p = p0;
     const uint32_t tiles = ((p.m + kBM - 1) / kBM) * ((p.n + kBN - 1) / kBN);
-    // whole rounds of 256 workgroups run 256x256 tiles; a last round that would fill less than half of the
+    // whole rounds of one workgroup per CU run 256x256 tiles; a last round that would fill at most half of the
     // CUs runs as twice as many half tiles instead (also when there is no whole round at all)
-    const uint32_t rest = tiles % 256u;
 #ifdef BFAINTB_TRACE
     const uint32_t halves = 0u;  // instrumented builds time the whole-tile kernel at every tile count
 #else
-    const uint32_t halves = (rest != 0u && rest <= 128u && p.m > 128u) ? rest : 0u;
+    const uint32_t halves = thin_round_tiles(tiles, p.m, p.cus ? p.cus : 256u);
 #endif
     const uint32_t whole = tiles - halves;
     if (whole) {

@@ -145,6 +145,8 @@ def lib():
         L.bfaintb_gemm_static_scratch_bytes.argtypes = []
         L.bfaintb_debug_control.restype = C.c_int
         L.bfaintb_debug_control.argtypes = [_u32, _u32]
+        L.bfaintb_gemm_plan.restype = C.c_int
+        L.bfaintb_gemm_plan.argtypes = [_u32, _u32, _u32, C.c_int, _u32, C.c_int, C.c_int, _u32, C.POINTER(Plan)]
         L.bfaintb_static_scratch_status.restype = C.c_int
         L.bfaintb_static_scratch_status.argtypes = [_vp]
         L.bfaintb_static_scratch_reset.restype = C.c_int
@@ -229,8 +231,30 @@ def gemm_static(c, a, b, scale, m, n, k, lda=None, ldb=None, ldc=None, weight_bi
     return rc
 
 
-DEBUG_SPLIT_WAIT_LIMIT, DEBUG_WITHHOLD_PARTIALS, DEBUG_FORCE_ROW_BLOCK = 1, 2, 3
+DEBUG_SPLIT_WAIT_LIMIT, DEBUG_WITHHOLD_PARTIALS, DEBUG_FORCE_ROW_BLOCK, DEBUG_PLAN_COMPUTE_UNITS = 1, 2, 3, 4
 ERR_WORKSPACE, ERR_NOT_INITIALISED, ERR_WORKSPACE_POISONED, ERR_STATIC_SCRATCH = -6, -8, -9, -10
+
+
+class Plan(C.Structure):
+    """bfaintb_plan: what a call would launch."""
+    _fields_ = [("variant", C.c_int32), ("kernel", _u32), ("tile_rows", _u32), ("tile_cols", _u32), ("waves", _u32), ("splits", _u32),
+                ("k_per_workgroup", _u32), ("workgroups", _u32), ("tail_workgroups", _u32), ("launches", _u32), ("compute_units", _u32),
+                ("reserved", _u32), ("workspace_bytes", C.c_uint64)]
+
+    def as_dict(self):
+        return {f: getattr(self, f) for f, _ in self._fields_ if f != "reserved"}
+
+
+KERNEL_DECODE_FAMILY, KERNEL_DECODE_SLAB, KERNEL_TILES_128, KERNEL_TILES_128_LDS, KERNEL_TILES_256X128, KERNEL_TILES_256, KERNEL_TILES_256_LDS = range(1, 8)
+
+
+def plan(m, n, k, weight_bits=8, group_size=0, packed=False, which=AUTO, force_split_k=0):
+    """What gemm (or gemm_prepacked, packed=True) would launch for this shape: a Plan.  Host only."""
+    out = Plan()
+    rc = lib().bfaintb_gemm_plan(m, n, k, weight_bits, group_size, int(bool(packed)), which, force_split_k, C.byref(out))
+    if rc:
+        raise BfaintbError(rc, "bfaintb_gemm_plan")
+    return out
 
 
 def debug_control(what, value):

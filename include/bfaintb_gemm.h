@@ -242,10 +242,15 @@ BFAINTB_API int bfaintb_static_scratch_reset(void* stream);
  *                                    give-up path with every kernel exiting normally
  *   BFAINTB_DEBUG_FORCE_ROW_BLOCK    value = 1, 2 or 4: beyond 32 rows of A the decode family runs blocks of 16 x value rows
  *                                    whatever its estimates say (tuning; results do not depend on it); 0 restores the choice
+ *   BFAINTB_DEBUG_PLAN_COMPUTE_UNITS value = the number of compute units the launch plans are made for instead of the
+ *                                    device's own (tuning, partitioned devices; every plan is a correct launch on any
+ *                                    device; workspace sizes follow the plan, so set it before asking for them);
+ *                                    0 restores the device's count
  */
 #define BFAINTB_DEBUG_SPLIT_WAIT_LIMIT 1u
 #define BFAINTB_DEBUG_WITHHOLD_PARTIALS 2u
 #define BFAINTB_DEBUG_FORCE_ROW_BLOCK 3u
+#define BFAINTB_DEBUG_PLAN_COMPUTE_UNITS 4u
 BFAINTB_API int bfaintb_debug_control(uint32_t what, uint32_t value);
 
 /*
@@ -317,13 +322,48 @@ BFAINTB_API int bfaintb_packed_header_init(bfaintb_packed_header* h, uint32_t n,
                                int has_bias);
 BFAINTB_API int bfaintb_packed_header_check(const bfaintb_packed_header* h);
 
+/*
+ * What a call would launch, without launching anything: the kernel, the shape of a workgroup's share, the split along
+ * k and the scratch it needs.  packed != 0 describes bfaintb_gemm_prepacked, else bfaintb_gemm; variant and split_k as
+ * for bfaintb_gemm_ex (BFAINTB_VARIANT_AUTO, 0 = the library's own choice).  Host only; returns 0 or a negative error.
+ * The plan is made for the compute units of the device that was current when the library first made one (256 when
+ * there is none), reported in compute_units.  No counterpart in the reference, whose grid is fixed by the shape
+ * (bfAintBGemm.cc:105-109).
+ */
+enum {
+    BFAINTB_KERNEL_DECODE_FAMILY = 1, /* weight streaming with split-K, in row blocks beyond 32 rows of A */
+    BFAINTB_KERNEL_DECODE_SLAB = 2,   /* packed weights: one column block of 16 per workgroup, no split */
+    BFAINTB_KERNEL_TILES_128 = 3,     /* 128 x 128 tiles, weights in registers, may split k */
+    BFAINTB_KERNEL_TILES_128_LDS = 4, /* 128 x 128 tiles, both operands through LDS */
+    BFAINTB_KERNEL_TILES_256X128 = 5, /* tiles of 256 rows x 128 columns, weights in registers */
+    BFAINTB_KERNEL_TILES_256 = 6,     /* 256 x 256 tiles, weights in registers */
+    BFAINTB_KERNEL_TILES_256_LDS = 7  /* 256 x 256 tiles, both operands through LDS */
+};
+typedef struct bfaintb_plan {
+    int32_t variant;           /* BFAINTB_VARIANT_DECODE, or the tiled variant with its tile size resolved */
+    uint32_t kernel;           /* BFAINTB_KERNEL_* */
+    uint32_t tile_rows;        /* rows of A per workgroup */
+    uint32_t tile_cols;        /* columns of B per workgroup */
+    uint32_t waves;            /* waves per workgroup */
+    uint32_t splits;           /* workgroups along k per tile */
+    uint32_t k_per_workgroup;  /* rows of k one workgroup covers */
+    uint32_t workgroups;       /* of the launch (the first one, if there are two) */
+    uint32_t tail_workgroups;  /* of a second launch over a last, thin round of tiles, or 0 */
+    uint32_t launches;         /* 1 or 2 */
+    uint32_t compute_units;    /* what the plan was made for */
+    uint32_t reserved;
+    uint64_t workspace_bytes;  /* what bfaintb_gemm[_prepacked]_workspace_bytes_ex reports for the same arguments */
+} bfaintb_plan;
+BFAINTB_API int bfaintb_gemm_plan(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size, int packed, int variant,
+                                  uint32_t split_k, bfaintb_plan* out);
+
 /* Which variant bfaintb_gemm would run (BFAINTB_VARIANT_*), or a negative error. */
 BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size);
 
 /* Rows (bfaintb_prefill_tile) and columns of the tiles BFAINTB_VARIANT_PREFILL runs an m x n output of row-major
  * weights with: 128 x 128 while that makes at most 256 tiles (one per CU); else 256 rows x 128 columns while that
- * makes at most 256; else 256 x 256.  Pre-packed weights run the same tiles.  (The reference arithmetic has no
- * 256 x 128 form: 256 x 256 there.)  Depend only on their arguments. */
+ * makes at most 256; else 256 x 256 (256 = the device's compute units: one tile per unit).  Pre-packed weights run
+ * the same tiles.  (The reference arithmetic has no 256 x 128 form: 256 x 256 there.) */
 BFAINTB_API uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n);
 BFAINTB_API uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n);
 

@@ -155,6 +155,45 @@ def test_rejects_bad_arguments_without_launching():
     assert L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 2) == 0 and L.bfaintb_debug_control(af.DEBUG_FORCE_ROW_BLOCK, 0) == 0
 
 
+def test_plan_query_agrees_with_the_other_queries_and_follows_the_compute_units():
+    """bfaintb_gemm_plan describes a launch without making it: it must say what variant / split_k / workspace_bytes say,
+    and plans made for another number of compute units (the tuning hook; on a device, its own count) stay within it."""
+    for (m, n, k, bits, g) in [(1, 4096, 4096, 8, 0), (16, 11008, 4096, 8, 0), (32, 28672, 8192, 4, 128), (256, 4096, 4096, 8, 0),
+                               (384, 2048, 8192, 8, 0), (1024, 4096, 4096, 8, 0), (2048, 4096, 4096, 8, 0), (4096, 4096, 4096, 8, 0),
+                               (2048, 28672, 8192, 4, 128)]:
+        pl = af.plan(m, n, k, bits, g)
+        v = af.variant(m, n, k, bits, g)
+        assert (pl.variant == af.DECODE) == (v == af.DECODE), (m, n, k)
+        assert pl.splits == af.split_k(m, n, k, bits, g) and pl.workspace_bytes == af.workspace_bytes(m, n, k, bits, g)
+        assert pl.compute_units == 256 or pl.compute_units > 0
+        if pl.variant != af.DECODE:
+            assert pl.tile_rows == af.prefill_tile(m, n) and pl.tile_cols == af.prefill_tile_cols(m, n)
+        pk = af.plan(m, n, k, bits, g, packed=True)
+        assert pk.workspace_bytes == af.prepacked_workspace_bytes(m, n, k, bits, g)
+    # the headline shapes on a 256-unit part (what this container, without a device, plans for)
+    if af.plan(1, 4096, 4096).compute_units == 256:
+        d = af.plan(1, 4096, 4096)
+        assert (d.kernel, d.tile_cols, d.waves, d.splits, d.workgroups) == (af.KERNEL_DECODE_FAMILY, 128, 8, 8, 256)
+        t = af.plan(4096, 4096, 4096)
+        assert (t.kernel, t.tile_rows, t.tile_cols, t.workgroups, t.launches) == (af.KERNEL_TILES_256, 256, 256, 256, 1)
+        c5 = af.plan(2048, 28672, 8192, 4, 128)
+        assert (c5.kernel, c5.workgroups, c5.tail_workgroups, c5.launches) == (af.KERNEL_TILES_256, 768, 256, 2)
+        assert af.plan(1, 4096, 4096, packed=True).kernel == af.KERNEL_DECODE_SLAB
+    try:
+        for cus in (64, 304):
+            af.debug_control(af.DEBUG_PLAN_COMPUTE_UNITS, cus)
+            d = af.plan(1, 4096, 4096)
+            assert d.compute_units == cus and d.workgroups <= cus, (cus, d.as_dict())       # 8-wave workgroups: one round
+            assert d.workspace_bytes == af.workspace_bytes(1, 4096, 4096)
+            for (m, n) in ((512, 2048), (1024, 4096), (2048, 4096)):
+                t = af.plan(m, n, 4096, which=af.PREFILL)
+                tiles = -(-m // t.tile_rows) * -(-n // t.tile_cols)
+                assert t.tile_rows == 256 and t.tile_cols == 256 or tiles * t.splits <= cus, (cus, m, n, t.as_dict())
+    finally:
+        af.debug_control(af.DEBUG_PLAN_COMPUTE_UNITS, 0)
+    assert af.plan(1, 4096, 4096).compute_units != 64
+
+
 def test_split_k_test_hooks_are_refused_without_the_environment_switch():
     """The hooks that withhold partial sums or cap the reducer's wait change what every later split-K launch of the
     process does: a process that has not asked for them (BFAINTB_TEST_HOOKS=1) gets BFAINTB_ERR_UNSUPPORTED."""

@@ -178,3 +178,21 @@ def test_random_ragged_case(af, case):
              "prefill_256_lds": af.PREFILL_256_LDS}[case["variant"]]
     c = run_ragged(af, p, which, af.ACT_SILU_GATE if gated else af.ACT_NONE, case["pad"])
     (assert_close_gated if gated else assert_close_ulp)(p, c, str(case))
+
+
+@pytest.mark.parametrize("cus", [64, 304])
+def test_plans_for_another_compute_unit_count_are_still_correct_launches(af, cus):
+    """The launch plans follow the device's compute units; a plan made for another count (the tuning hook) changes the
+    split factors, the tile sizes and the second launch over a thin last round, and never the result's contract."""
+    shapes = [(1, 4096, 4096, 8, 0), (16, 1024, 4096, 8, 0), (24, 2064, 2048, 4, 128), (72, 1536, 2048, 8, 0), (300, 512, 1024, 8, 0),
+              (700, 1280, 512, 4, 64), (520, 4096, 256, 8, 0), (2100, 2304, 256, 8, 0)]
+    try:
+        af.debug_control(af.DEBUG_PLAN_COMPUTE_UNITS, cus)
+        for i, (m, n, k, bits, g) in enumerate(shapes):
+            assert af.plan(m, n, k, bits, g).compute_units == cus
+            p = Problem(m, n, k, bits, g, seed=300 + i)
+            assert_close_ulp(p, run_gemm(p), f"planned for {cus} compute units: {m}x{n}x{k} int{bits} g{g}")
+            if k % 128 == 0:  # (whole K-chunks of either code width)
+                assert_close_ulp(p, run_prepacked(af, p), f"planned for {cus} compute units, packed: {m}x{n}x{k} int{bits} g{g}")
+    finally:
+        af.debug_control(af.DEBUG_PLAN_COMPUTE_UNITS, 0)
