@@ -336,6 +336,60 @@ def prefill_loop_trace(af, shapes=((256, 4096, 4096), (512, 4096, 4096), (1024, 
     return rows
 
 
+PLAN_CHECK_SHAPES = [
+    # (m, n, k, weight_bits, group_size): the library's own choice held against every alternative it could be forced to
+    (1, 4096, 4096, 8, 0), (16, 4096, 4096, 8, 0), (32, 4096, 4096, 8, 0), (1, 11008, 4096, 8, 0), (8, 11008, 4096, 8, 0),
+    (32, 11008, 4096, 8, 0), (1, 28672, 8192, 4, 128), (16, 28672, 8192, 4, 128), (4, 1024, 8192, 8, 0), (32, 2048, 8192, 4, 128),
+    (48, 4096, 4096, 8, 0), (64, 4096, 4096, 8, 0), (96, 11008, 4096, 8, 0), (128, 4096, 4096, 8, 0), (128, 28672, 8192, 4, 128),
+    (192, 4096, 11008, 8, 0), (256, 4096, 4096, 8, 0), (256, 8192, 8192, 8, 0), (256, 8192, 8192, 4, 128), (384, 2048, 8192, 8, 0),
+    (512, 4096, 4096, 8, 0), (512, 11008, 4096, 8, 0), (640, 4096, 4096, 8, 0), (768, 8192, 8192, 8, 0), (1024, 4096, 4096, 8, 0),
+    (1024, 4096, 4096, 4, 128), (1536, 4096, 4096, 8, 0), (2048, 4096, 4096, 8, 0), (2048, 4096, 11008, 8, 0), (4096, 4096, 4096, 8, 0),
+]
+
+
+def plan_check(af, steps=40):
+    """For every shape of PLAN_CHECK_SHAPES: the kernel time of the library's own plan (BFAINTB_VARIANT_AUTO) and of every
+    alternative it can be forced to — the decode family with other split factors, the three tile sizes — same buffers,
+    same graph protocol.  Run after a kernel or plan change; rows where the own choice is more than 5 % off the best
+    alternative are the ones to look at."""
+    import torch
+    rows = []
+    for (m, n, k, bits, group) in PLAN_CHECK_SHAPES:
+        b_bytes = n * k * bits // 8
+        copies = max(2, min(40, (640 << 20) // b_bytes)) if m <= 32 else 2
+        w = Workload(f"m{m}_n{n}_k{k}_int{bits}_g{group}", m, n, k, bits, group, copies=copies)
+        own = af.plan(m, n, k, bits, group)
+        alts = [("own choice", af.AUTO, 0)]
+        if m <= 1024:  # (beyond, the row-blocked family takes milliseconds)
+            for sk in sorted({1, 2, 4, 8, 16, max(1, own.splits // 2), own.splits * 2} - ({own.splits} if own.variant == af.DECODE else set())):
+                alts.append((f"decode family, k split {sk} ways", af.DECODE, sk))
+        if m > 32:
+            alts += [("128x128 tiles", af.PREFILL_128, 0), ("256x128 tiles", af.PREFILL_256X128, 0), ("256x256 tiles", af.PREFILL_256, 0)]
+        timed = []
+        for name, which, sk in alts:
+            need = af.workspace_bytes(m, n, k, bits, group, which, sk)
+            ws = None
+            if need:
+                ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+                af.workspace_init(ws)
+            try:
+                ev = time_launches(lambda i: af.gemm(w.c, w.a, w.b[i % copies], w.s, m, n, k, weight_bits=bits, group_size=group,
+                                                     workspace=ws, which=which, force_split_k=sk), copies, steps if m <= 256 else 10, 5)[0]
+            except Exception as exc:  # a forced form that cannot run this shape
+                timed.append((name, None, str(exc)[:80]))
+                continue
+            timed.append((name, round(ev * 1e3, 2), None))
+        best = min((t for t in timed if t[1] is not None), key=lambda t: t[1])
+        own_us = timed[0][1]
+        rows.append({"m": m, "n": n, "k": k, "weight_bits": bits, "group_size": group,
+                     "own": {"kernel": own.kernel, "tile": [own.tile_rows, own.tile_cols], "splits": own.splits, "workgroups": own.workgroups, "us": own_us},
+                     "best": {"what": best[0], "us": best[1]}, "own_over_best": round(own_us / best[1], 3),
+                     "all": {t[0]: (t[1] if t[1] is not None else t[2]) for t in timed}})
+        del w
+        torch.cuda.empty_cache()
+    return rows
+
+
 def time_vendor_bf16_gemm(w, steps, warmup):
     """Context for the prefill figure: the vendor library's plain bf16 x bf16 GEMM (torch.matmul, i.e.
     hipBLASLt) on the same activations and the already dequantised weights, same graph protocol.  It does
@@ -459,8 +513,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
-                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | prefill_trace (needs --lib "
-                    "with a library built with -DBFAINTB_TRACE)")
+                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | plan_check (the library's plans "
+                    "against forced alternatives) | prefill_trace (needs --lib with a library built with -DBFAINTB_TRACE)")
     ap.add_argument("--lib", default="", help="load this build of libbfaintb_gemm.so instead of the package's own "
                     "(an instrumented build, for --only prefill_trace)")
     args = ap.parse_args()
@@ -480,6 +534,12 @@ def main():
     K, W = args.steps, args.warmup
     out_extra = {}
 
+    if args.only == "plan_check":
+        rows = plan_check(af)
+        off = [r for r in rows if r["own_over_best"] > 1.05]
+        print(json.dumps({"metric": "bfAintBGemm launch plans against forced alternatives", "shapes": len(rows), "more_than_5_percent_off": len(off),
+                          "compute_units": af.plan(1, 4096, 4096).compute_units, "rows": rows}))
+        return
     if args.only == "prefill_trace":
         print(json.dumps({"metric": "bfAintBGemm 256x256-tile kernel: K-loop cycles per step and shader clock by tile count (instrumented build)",
                           "library": af.library_path(), "rows": prefill_loop_trace(af)}))
