@@ -45,19 +45,21 @@ MIN_LAUNCHES = 400            # launches inside one event pair (several replays 
 # file: the output names the source beside the figure.
 RECORDED_TRAFFIC = {
     # name: (bytes, source)
-    "decode_m1_n4096_k4096_int8_perchannel": (17422124, "profiles/decode_m1_n4096_k4096_int8.txt"),
+    "decode_m1_n4096_k4096_int8_perchannel": (17424987, "profiles/decode_m1_n4096_k4096_int8.txt"),
     "decode_m1_n4096_k4096_int8_perchannel_prepacked": (16929572, "profiles/decode_m1_n4096_k4096_int8_prepacked.txt"),
-    "prefill_m4096_n4096_k4096_int8_perchannel": (171267767, "profiles/prefill_m4096_n4096_k4096_int8.txt"),
-    "decode_m1_n11008_k4096_int8_perchannel": (46267304, "profiles/decode_m1_n11008_k4096_int8.txt"),
-    "decode_m16_n11008_k4096_int8_perchannel": (49015179, "profiles/decode_m16_n11008_k4096_int8.txt"),
-    "decode_m32_n11008_k4096_int8_perchannel": (52631370, "profiles/decode_m32_n11008_k4096_int8.txt"),
-    "m1_n28672_k8192_int4_group128": (122555279, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
-    "m16_n28672_k8192_int4_group128": (130160110, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
-    "m2048_n28672_k8192_int4_group128": (907944059, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
-    "mid_m256_n4096_k4096_int8_perchannel": (35861798, "profiles/mid_m256_n4096_k4096_int8.txt"),
-    "mid_m1024_n4096_k4096_int8_perchannel": (92446458, "profiles/mid_m1024_n4096_k4096_int8.txt"),
-    "mid_m256_n8192_k8192_int8_perchannel": (131049442, "profiles/mid_m256_n8192_k8192_int8.txt"),
-    "mid_m2048_n4096_k4096_int8_perchannel": (168006299, "profiles/mid_m2048_n4096_k4096_int8.txt"),
+    "prefill_m4096_n4096_k4096_int8_perchannel": (171267562, "profiles/prefill_m4096_n4096_k4096_int8.txt"),
+    "decode_m1_n11008_k4096_int8_perchannel": (46258715, "profiles/decode_m1_n11008_k4096_int8.txt"),
+    "decode_m4_n11008_k4096_int8_perchannel": (48334036, "profiles/decode_m4_n11008_k4096_int8.txt"),
+    "decode_m8_n11008_k4096_int8_perchannel": (47187147, "profiles/decode_m8_n11008_k4096_int8.txt"),
+    "decode_m16_n11008_k4096_int8_perchannel": (48972850, "profiles/decode_m16_n11008_k4096_int8.txt"),
+    "decode_m32_n11008_k4096_int8_perchannel": (52579634, "profiles/decode_m32_n11008_k4096_int8.txt"),
+    "m1_n28672_k8192_int4_group128": (122557732, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
+    "m16_n28672_k8192_int4_group128": (130166040, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
+    "m2048_n28672_k8192_int4_group128": (908258153, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
+    "mid_m256_n4096_k4096_int8_perchannel": (35834805, "profiles/mid_m256_n4096_k4096_int8.txt"),
+    "mid_m1024_n4096_k4096_int8_perchannel": (92435211, "profiles/mid_m1024_n4096_k4096_int8.txt"),
+    "mid_m256_n8192_k8192_int8_perchannel": (131059871, "profiles/mid_m256_n8192_k8192_int8.txt"),
+    "mid_m2048_n4096_k4096_int8_perchannel": (168014478, "profiles/mid_m2048_n4096_k4096_int8.txt"),
 }
 
 # Parity counts RECORDED from the GPU test suite (tests/helpers.py: assert_close_ulp logs every check; tests/conftest.py
@@ -302,6 +304,76 @@ class PowerSampler:
                 "power_cap_w": cap, "samples": len(self.samples), "source": self.files[0]}
 
 
+def sustained_power(launch, nb, seconds=1.5):
+    """Replays a graph of 20 launches back to back for `seconds` with the board power sampled alongside: the kernel time
+    and the power once the part has settled under the load (the short timed region above is over before the power has
+    reached its plateau)."""
+    import torch
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(20):
+            launch(i % nb)
+    g.replay()
+    torch.cuda.synchronize()
+    with PowerSampler() as power:
+        t_end = time.perf_counter() + seconds
+        while time.perf_counter() < t_end:      # settle
+            for _ in range(10):
+                g.replay()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+    return {"kernel_us_after_settling": round(e0.elapsed_time(e1) * 1e3 / 400, 3), "seconds_under_load": seconds, **power.summary()}
+
+
+def decode_timeline(af, shapes=((1, 4096, 4096), (1, 11008, 4096), (32, 11008, 4096))):
+    """Needs a library built with -DBFAINTB_TRACE (--lib): the decode kernel's waves then write 100 MHz time stamps behind
+    the split-K area of the workspace — entry, last step multiplied, workgroup's sums ready, producer's stores issued,
+    reducer holds every partial sum, reducer done — and the number of fetch attempts a reducer made.  One cold launch
+    after twenty warm ones, eight times; the last one is reported, in microseconds after the first workgroup's entry."""
+    import torch
+    names = ["entry", "reducer holds every partial sum", "wave has multiplied its last step", "workgroup's sums ready (LDS, barrier)",
+             "producer's stores issued", "reducer done", "a first fetch attempt came back incomplete"]
+    out = []
+    for (m, n, k) in shapes:
+        w = Workload(f"m{m}_n{n}_k{k}", m, n, k, copies=40 if n * k <= 4096 * 4096 else 14)
+        need = af.workspace_bytes(m, n, k)
+        off = (need + 255) & ~255
+        ws = torch.zeros(off + (8 << 20), dtype=torch.uint8, device="cuda")
+        af.workspace_init(ws)
+        pl = af.plan(m, n, k)
+        waves = pl.waves
+        nwg = pl.workgroups
+        nb = len(w.b)
+        for rep in range(8):
+            for i in range(20):
+                af.gemm(w.c, w.a, w.b[(i + rep) % nb], w.s, m, n, k, workspace=ws, workspace_nbytes=need)
+            torch.cuda.synchronize()
+            ws[off:].zero_()
+            torch.cuda.synchronize()
+            af.gemm(w.c, w.a, w.b[(21 + rep) % nb], w.s, m, n, k, workspace=ws, workspace_nbytes=need)
+            torch.cuda.synchronize()
+        t = ws[off:off + nwg * waves * 64].cpu().numpy().view(np.uint64).reshape(nwg * waves, 8).astype(np.int64)
+        t0 = t[:, 0][t[:, 0] > 0].min()
+        r = (t - t0) / 100.0
+        row = {"m": m, "n": n, "k": k, "splits": pl.splits, "workgroups": nwg, "waves_per_workgroup": waves, "events_us": {}}
+        for i, name in enumerate(names):
+            col = r[:, i][t[:, i] > 0]
+            if len(col):
+                row["events_us"][name] = {"min": round(float(col.min()), 2), "median": round(float(np.median(col)), 2),
+                                          "p90": round(float(np.percentile(col, 90)), 2), "max": round(float(col.max()), 2), "waves": int(len(col))}
+        tries = t[:, 7][t[:, 7] > 0]
+        row["fetch_attempts_per_reducing_wave"] = {int(a): int(c) for a, c in zip(*np.unique(tries, return_counts=True))}
+        out.append(row)
+        del w, ws
+        torch.cuda.empty_cache()
+    return out
+
+
 def prefill_loop_trace(af, shapes=((256, 4096, 4096), (512, 4096, 4096), (1024, 4096, 4096), (2048, 4096, 4096), (4096, 4096, 4096), (8192, 8192, 4096))):
     """Needs a library built with -DBFAINTB_TRACE (--lib): the 256x256-tile kernel then writes, per wave, the shader
     cycles and the 100 MHz ticks its K loop took into the workspace.  Reported by tile count: cycles per K-step of 64
@@ -500,7 +572,7 @@ def config5_workload(m_max):
 
 
 def compact(entry):
-    return {k: entry[k] for k in ("workload", "bound", "kernel_us", "achieved", "unit", "frac", "algorithmic_bytes", "flops", "steps") if k in entry}
+    return {k: entry[k] for k in ("workload", "bound", "kernel_us", "achieved", "unit", "frac", "traffic", "algorithmic_bytes", "flops", "steps") if k in entry}
 
 
 def main():
@@ -514,7 +586,7 @@ def main():
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
                     "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | plan_check (the library's plans "
-                    "against forced alternatives) | prefill_trace (needs --lib with a library built with -DBFAINTB_TRACE)")
+                    "against forced alternatives) | prefill_trace, decode_timeline (both need --lib with a library built with -DBFAINTB_TRACE)")
     ap.add_argument("--lib", default="", help="load this build of libbfaintb_gemm.so instead of the package's own "
                     "(an instrumented build, for --only prefill_trace)")
     args = ap.parse_args()
@@ -539,6 +611,10 @@ def main():
         off = [r for r in rows if r["own_over_best"] > 1.05]
         print(json.dumps({"metric": "bfAintBGemm launch plans against forced alternatives", "shapes": len(rows), "more_than_5_percent_off": len(off),
                           "compute_units": af.plan(1, 4096, 4096).compute_units, "rows": rows}))
+        return
+    if args.only == "decode_timeline":
+        print(json.dumps({"metric": "bfAintBGemm decode kernel: time stamps of one cold launch (instrumented build)", "library": af.library_path(),
+                          "rows": decode_timeline(af)}))
         return
     if args.only == "prefill_trace":
         print(json.dumps({"metric": "bfAintBGemm 256x256-tile kernel: K-loop cycles per step and shader clock by tile count (instrumented build)",
@@ -625,12 +701,11 @@ def main():
     if args.only in ("", "prefill"):
         w = Workload("prefill_m4096_n4096_k4096_int8_perchannel", 4096, 4096, 4096, copies=2)
         pk = max(20, min(K, 100))
-        with PowerSampler() as power:
-            ev_ms, wall_ms = time_graph(af, w, pk, max(5, W // 4), rotate=True)
+        ev_ms, wall_ms = time_graph(af, w, pk, max(5, W // 4), rotate=True)
         entry = {"value": round(w.flops / (wall_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s", "steps": pk,
                  "ms_per_step": round(wall_ms, 6), "GB/s": round(w.bytes / (wall_ms * 1e-3) / 1e9, 1),
-                 "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma"),
-                 "board_power_during_timed_region": power.summary()}
+                 "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma")}
+        entry["sustained"] = sustained_power(lambda i: af.gemm(w.c, w.a, w.b[i], w.s, w.m, w.n, w.k), len(w.b))
         try:
             v_ms = time_vendor_bf16_gemm(w, pk, 5)
             entry["vendor_bf16_gemm_same_shape"] = {"TFLOP/s": round(w.flops / (v_ms * 1e-3) / 1e12, 2), "kernel_us": round(v_ms * 1e3, 3),
