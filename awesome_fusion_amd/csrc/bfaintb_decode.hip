@@ -361,6 +361,81 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
     }
 }
 
+// The reducing workgroup's part where a thread has one row and the launch at most 8 splits (the 128-column kernels up to
+// 16 rows of A): the same hand-over as reduce_splits — same words, same order of addition, same bits — with TWO fetch
+// attempts in flight, the second issued kPollGap x 64 cycles after the first and each issued again as soon as it has come
+// back incomplete.  A fetch is a round trip of about a microsecond past the L2, and whether the first one samples the
+// workspace before or after the last producer's store has landed varies from launch to launch; with one attempt at a
+// time a miss costs a whole further round trip, with two the workspace is sampled about twice per round trip.  Measured
+// on one box (us, one attempt / two): 4096 x 4096, m = 1 / 4 / 16: 7.46 / 7.21, 7.75 / 7.49-7.67, 8.70 / 8.21;
+// 11008 x 4096, m = 8 / 16: 12.77 / 12.39, 13.75 / 13.25; 1024 x 8192, m = 4: 7.89 / 7.41.  The 256-column kernels keep the
+// single attempt: with two they were 1.5 to 6 % slower (11008 x 4096, m = 1: 11.88 / 12.59; 4-bit 28672 x 8192: 29.7 / 30.2).
+// The selection of the winning attempt is written as copies under uniform branches: indexing the two register sets by a
+// run-time flag sent both through scratch memory (0.8 us at m = 1, 5 us at m = 16).
+constexpr int kPollGap = 8;
+template <uint32_t NL, uint32_t NSUM>
+__device__ __forceinline__ void reduce_splits_two_in_flight(const GemmParams& p, const float4 (&sum)[NSUM], uint32_t first_row, uint32_t rows,
+                                                            uint32_t rs, uint32_t col, bool col_ok)
+{
+    if (!col_ok || rs >= rows) return;
+    const uint32_t others = p.splits - 1u;  // 1 .. NL
+    const uint32_t split_bytes = p.m * p.n * 4u;
+    const __amdgpu_buffer_rsrc_t ws = __builtin_amdgcn_make_buffer_rsrc(p.partials, 0, (int)p.partial_bytes, kBufferFlags);
+    const uint32_t off = ((first_row + rs) * p.n + col) * 4u;
+    // (always NL loads, so that the wait counts are compile-time numbers: splits that do not exist re-read split 0)
+    auto fetch = [&](u32x4_t (&v)[NL]) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (uint32_t j = 0; j < NL; ++j)
+            v[j] = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)off, (int)((j < others ? j : 0u) * split_bytes), kAuxDeviceScope);
+    };
+    auto whole = [&](const u32x4_t (&v)[NL]) -> bool {
+        bool ok = true;
+#pragma unroll
+        for (uint32_t j = 0; j < NL; ++j)
+#pragma unroll
+            for (int h = 0; h < 4; ++h)
+                if (j < others && v[j][h] == kEmptyWord) ok = false;
+        return ok;
+    };
+    u32x4_t a[NL], b[NL];
+    fetch(a);
+    __builtin_amdgcn_s_sleep(kPollGap);
+    fetch(b);
+    uint32_t tries = 2;
+    bool complete = false;
+    u32x4_t win[NL];
+    auto take = [&](const u32x4_t (&v)[NL]) {
+#pragma unroll
+        for (uint32_t j = 0; j < NL; ++j) win[j] = v[j];
+    };
+    for (;;) {
+        if (whole(a)) { take(a); complete = true; break; }
+        if (tries >= p.split_wait_limit) { take(a); break; }
+        fetch(a);
+        ++tries;
+        if (whole(b)) { take(b); complete = true; break; }
+        if (tries >= p.split_wait_limit) { take(b); break; }
+        fetch(b);
+        ++tries;
+    }
+    if (!complete) __hip_atomic_store(p.ws_header, kWorkspaceGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const u32x4_t empty4 = {kEmptyWord, kEmptyWord, kEmptyWord, kEmptyWord};
+    float4 total = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (uint32_t j = 0; j < NL; ++j) {
+        if (j < others) {
+            __builtin_amdgcn_raw_buffer_store_b128(empty4, ws, (int)off, (int)(j * split_bytes), kAuxDeviceScope);
+            const u32x4_t v = win[j];
+            total.x += __uint_as_float(v[0]);
+            total.y += __uint_as_float(v[1]);
+            total.z += __uint_as_float(v[2]);
+            total.w += __uint_as_float(v[3]);
+        }
+    }
+    finish_row4(p, make_float4(total.x + sum[0].x, total.y + sum[0].y, total.z + sum[0].z, total.w + sum[0].w), first_row + rs, col);
+}
+
 // PACKED: p.b holds the weights in the packed order; the workgroup's kCols columns are CPL column blocks of 16, and
 // accumulator c of a lane belongs to column block c (local column 16 c + 4 kg + r instead of (4 kg + r) CPL + c).
 // REF: the reference kernel's arithmetic (p.reference_arith): p.scale holds one fp32 scale per column, W is narrowed by
@@ -699,7 +774,12 @@ bfaintb_decode_kernel(const GemmParams p)
             // never arrives leaves a NaN in the output instead of hanging the kernel.
             // Rows a thread has in this pass: a power of two up to kMaxR; the fewer, the more splits are fetched at once.
             const uint32_t rows_per_thread = (rows_out + nrs - 1u) / nrs;
-            if (rows_per_thread <= 1u) reduce_splits<1>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
+            constexpr bool kTwoAttempts = CPL == 8;  // (see reduce_splits_two_in_flight)
+            if (kTwoAttempts && rows_per_thread <= 1u && p.splits <= 2u) reduce_splits_two_in_flight<1>(p, sum, first_row, rows_out, rs, col, col_ok);
+            else if (kTwoAttempts && rows_per_thread <= 1u && p.splits <= 3u) reduce_splits_two_in_flight<2>(p, sum, first_row, rows_out, rs, col, col_ok);
+            else if (kTwoAttempts && rows_per_thread <= 1u && p.splits <= 5u) reduce_splits_two_in_flight<4>(p, sum, first_row, rows_out, rs, col, col_ok);
+            else if (kTwoAttempts && rows_per_thread <= 1u && p.splits <= 8u) reduce_splits_two_in_flight<7>(p, sum, first_row, rows_out, rs, col, col_ok);
+            else if (rows_per_thread <= 1u) reduce_splits<1>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
             else if (rows_per_thread <= 2u) reduce_splits<(kMaxR < 2u ? kMaxR : 2u)>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
             else if (rows_per_thread <= 4u) reduce_splits<(kMaxR < 4u ? kMaxR : 4u)>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
             else reduce_splits<kMaxR>(p, sum, first_row, rows_out, rs, nrs, col, col_ok);
