@@ -367,9 +367,10 @@ __device__ __forceinline__ void reduce_splits(const GemmParams& p, const float4 
 // back incomplete.  A fetch is a round trip of about a microsecond past the L2, and whether the first one samples the
 // workspace before or after the last producer's store has landed varies from launch to launch; with one attempt at a
 // time a miss costs a whole further round trip, with two the workspace is sampled about twice per round trip.  Measured
-// on one box (us, one attempt / two): 4096 x 4096, m = 1 / 4 / 16: 7.46 / 7.21, 7.75 / 7.49-7.67, 8.70 / 8.21;
-// 11008 x 4096, m = 8 / 16: 12.77 / 12.39, 13.75 / 13.25; 1024 x 8192, m = 4: 7.89 / 7.41.  The 256-column kernels keep the
-// single attempt: with two they were 1.5 to 6 % slower (11008 x 4096, m = 1: 11.88 / 12.59; 4-bit 28672 x 8192: 29.7 / 30.2).
+// on one box (us, one attempt / two): 4096 x 4096, m = 1 / 4 / 16: 7.43 / 7.32, 7.71 / 7.86, 8.69 / 8.44;
+// 11008 x 4096, m = 8 / 16: 12.79 / 12.42, 13.74 / 13.33; 1024 x 8192, m = 4: 7.83 / 7.50; 2048 x 4096, m = 12: 7.84 / 7.51.
+// The 256-column kernels keep the single attempt: with two they were 1.5 to 6 % slower (11008 x 4096, m = 1: 11.88 / 12.59;
+// 4-bit 28672 x 8192: 29.7 / 30.2).
 // The selection of the winning attempt is written as copies under uniform branches: indexing the two register sets by a
 // run-time flag sent both through scratch memory (0.8 us at m = 1, 5 us at m = 16).
 constexpr int kPollGap = 8;
@@ -434,6 +435,13 @@ __device__ __forceinline__ void reduce_splits_two_in_flight(const GemmParams& p,
         }
     }
     finish_row4(p, make_float4(total.x + sum[0].x, total.y + sum[0].y, total.z + sum[0].z, total.w + sum[0].w), first_row + rs, col);
+    // The attempt that did not win may still be in flight.  Its destination registers stay this function's until it has
+    // come back: with nothing holding them, the compiler handed them to the constants of the emptying stores above while
+    // the loads were still due to write them (a workspace word of the second split left holding a partial sum: found
+    // by the at-rest check of the test suite).  The wait is behind every store this thread issues, where it costs nothing.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (uint32_t j = 0; j < NL; ++j) asm volatile("" ::"v"(a[j]), "v"(b[j]));
 }
 
 // PACKED: p.b holds the weights in the packed order; the workgroup's kCols columns are CPL column blocks of 16, and

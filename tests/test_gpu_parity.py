@@ -249,6 +249,33 @@ def test_tiled_split_k_matches_oracle_and_is_deterministic(af, m, n, k, bits, gr
         assert af.workspace_status(helpers._ws.t) == 0
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 1024, 4096), (16, 640, 2048), (9, 2064, 4096)])
+def test_decode_hand_over_leaves_the_workspace_at_rest_for_every_split_factor(af, m, n, k):
+    """The reducer of the 128-column decode kernels keeps two fetch attempts in flight and has one instantiation per
+    number of splits it fetches (1, 2, up to 4, up to 7 others); beyond 8 splits the single-attempt form runs.  Every
+    split factor: the oracle's bound, the same bits on every run, and every workspace word empty again afterwards
+    (an attempt still in flight when the words are emptied must not disturb the emptying stores)."""
+    import torch
+    p = Problem(m, n, k, seed=m + n)
+    a, b, s = to_dev(p.a_bf), to_dev(p.b_bytes), to_dev(p.s_bf)
+    for split in (2, 3, 4, 5, 7, 8, 16):
+        need = af.workspace_bytes(m, n, k, which=af.DECODE, force_split_k=split)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        af.workspace_init(ws)
+        c = torch.zeros((m, n), dtype=torch.int16, device="cuda")
+        first = None
+        for rep in range(20):
+            af.gemm(c, a, b, s, m, n, k, workspace=ws, which=af.DECODE, force_split_k=split)
+            torch.cuda.synchronize()
+            got = from_dev_u16(c).copy()
+            if first is None:
+                first = got
+                assert_close_ulp(p, got, f"decode, k split {split} ways: {m}x{n}x{k}")
+            assert np.array_equal(got, first), f"split {split}, run {rep}: not reproducible"
+            assert bool((ws[256:] == 0xFF).all()), f"split {split}, run {rep}: workspace not at rest"
+        assert af.workspace_status(ws) == 0
+
+
 def test_tiled_split_k_is_what_auto_runs_and_takes_the_epilogues(af):
     """A shape whose plan is the small tiles with k split (long k, few tiles): AUTO gives the forced form's bits, and the
     bias / residual / gate epilogues run on the reduced sums."""
