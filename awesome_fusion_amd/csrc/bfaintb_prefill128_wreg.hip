@@ -54,9 +54,12 @@ __device__ __forceinline__ void tw_mfma(f32x4_t& acc, const bf16x8_t& a, const b
 __device__ __forceinline__ void tw_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 }  // namespace
 
-template <int BITS, bool GROUPED, bool PACKED>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) bfaintb_prefill128_wreg_kernel(const GemmParams p)
+template <int BITS, bool GROUPED, bool PACKED, int KH>
+__global__ void __launch_bounds__(256 * KH) __attribute__((amdgpu_waves_per_eu(KH, KH))) bfaintb_prefill128_wreg_kernel(const GemmParams p)
 {
+    static_assert(KH == 1 || KH == 2, "one wave per SIMD, or two that share a K-step by its blocks of 32 k");
+    constexpr uint32_t kWaves = 4u * KH;
+    constexpr uint32_t NB = 2u / KH;  // blocks of 32 k of a K-step that a wave multiplies
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kTwStage];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[kTwStage];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a2[kTwStage];
@@ -84,7 +87,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // 0..3: the wave's 32 columns
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wc = wave & 3u;                  // the wave's 32 columns
+    const uint32_t kh = KH == 2 ? wave >> 2 : 0u;   // two waves per column group: the block of 32 k this one multiplies
+    // local block lb of this wave is block blk_of(lb) of the step
+    auto blk_of = [&](uint32_t lb) { return KH == 2 ? kh : lb; };
     const uint32_t c16 = lane & 15u, kq = lane >> 4;
 
     // ---- tile of this workgroup (the order of bfaintb_prefill128_kernel: the ids an XCD receives cover consecutive
@@ -125,20 +132,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     const uint32_t last_chunks = (p.k - (ksteps_all - 1u) * kTwK) / 8u;  // valid 16-byte chunks per row of A in the last step
     auto clamp = [&](uint32_t t) { return t < ksteps ? t : ksteps - 1u; };
 
-    // A copy: instruction j of wave w fills rows 32 w + 8 j .. + 7; lane l lands at row + l / 8, chunk position l % 8, so
+    // A copy: instruction j of wave w fills rows 8 (kACopies w + j) .. + 7; lane l lands at row + l / 8, chunk position l % 8, so
     // it fetches chunk (l % 8) ^ ((row >> 1) & 7) = (l % 8) ^ (l / 16) for even j and that ^ 4 for odd j; the row advance
     // of j and the K advance sit in the scalar offset.  A chunk past the end of k (partial last step) is fetched from
     // beyond the extent and reads as zero; rows of B past k read as zero codes, finite weights, and multiply those zeros.
-    const uint32_t a_row = 32u * wave + (lane >> 3);
+    constexpr uint32_t kACopies = 4u / KH;  // per wave and step: 8 rows each
+    const uint32_t a_row = 8u * kACopies * wave + (lane >> 3);
     const uint32_t chunk_e = (lane & 7u) ^ ((lane >> 4) & 7u), chunk_o = chunk_e ^ 4u;
     const uint32_t a_voff_e = (a_row * p.lda + chunk_e * 8u) * 2u, a_voff_o = (a_row * p.lda + chunk_o * 8u) * 2u;
     const uint32_t a_last_e = chunk_e < last_chunks ? a_voff_e : a_extent, a_last_o = chunk_o < last_chunks ? a_voff_o : a_extent;
     auto dma_a = [&](auto stage_c, uint32_t kt) {
-        uint8_t* base = a_tile(stage_c) + wave * 4096u;
+        uint8_t* base = a_tile(stage_c) + wave * (1024u * kACopies);
         const bool last = kbase + kt + 1u == ksteps_all;
         const uint32_t ve = last ? a_last_e : a_voff_e, vo = last ? a_last_o : a_voff_o;
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
+        for (uint32_t j = 0; j < kACopies; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16,
                                                      (j & 1u) ? vo : ve, (kbase + kt) * kTwK * 2u + j * 16u * p.lda, 0, 0);
     };
@@ -156,16 +164,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // block odd)): the 16 lanes of one kq then read 16 neighbouring pieces' worth of banks.
     constexpr uint32_t kChunks = kRowBytes / 16u;        // 8 or 4 chunks per row
     constexpr uint32_t kRowsPerCopy = 1024u / kRowBytes; // 8 or 16
-    constexpr uint32_t kCopiesPerWave = PACKED ? 2u : 64u / kRowsPerCopy / 4u;  // 2 or 1
+    // (eight waves, 4-bit codes in rows: four instructions for eight waves — waves 4 .. 7 repeat the copies of waves
+    // 0 .. 3, same bytes to the same place, so that every wave has the same number of requests in flight for the one
+    // wait count at the top of a step)
+    constexpr uint32_t kCopies = PACKED ? 8u : 64u / kRowsPerCopy;  // per step: 8, or 4 for 4-bit codes in rows
+    constexpr uint32_t kCopiesPerWave = kCopies >= kWaves ? kCopies / kWaves : 1u;
+    const uint32_t wcopier = kCopies >= kWaves ? wave : wave & (kCopies - 1u);
     constexpr uint32_t kRot = BITS == 8 ? 2u : 1u;       // a wave's 16 lanes of one kq cover 32 (16) bytes of a row
     uint32_t w_voff[2];  // (fixed extent: see the note on the arrays above)
 #pragma unroll
     for (uint32_t j = 0; j < kCopiesPerWave; ++j) {
         if constexpr (PACKED) {
-            const uint32_t at = (lane & 31u) ^ (8u * j);  // 8 g + c of the piece this lane's position holds
-            w_voff[j] = (2u * wave + j) * slab_bytes + (16u * (at >> 3) + 2u * (at & 7u) + (lane >> 5)) * 16u;
+            const uint32_t cblock = kCopiesPerWave * wcopier + j;  // the column block this instruction copies
+            const uint32_t at = (lane & 31u) ^ (8u * (cblock & 1u));  // 8 g + c of the piece this lane's position holds
+            w_voff[j] = cblock * slab_bytes + (16u * (at >> 3) + 2u * (at & 7u) + (lane >> 5)) * 16u;
         } else {
-            const uint32_t row = (kCopiesPerWave * wave + j) * kRowsPerCopy + lane / kChunks;  // within the step
+            const uint32_t row = (kCopiesPerWave * wcopier + j) * kRowsPerCopy + lane / kChunks;  // within the step
             const uint32_t chunk = ((lane % kChunks) - kRot * ((row >> 3) & 3u)) & (kChunks - 1u);
             w_voff[j] = row * p.ldb_bytes + chunk * 16u;
         }
@@ -175,35 +189,41 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     const uint32_t w_step = PACKED ? 1024u : kTwK * p.ldb_bytes;
     constexpr uint32_t w_shift = (PACKED && BITS == 4) ? 1u : 0u;
     auto dma_w = [&](auto stage_c, uint32_t kt) {
-        uint8_t* base = w_tile(stage_c) + kCopiesPerWave * wave * 1024u;
+        uint8_t* base = w_tile(stage_c) + kCopiesPerWave * wcopier * 1024u;
 #pragma unroll
         for (uint32_t j = 0; j < kCopiesPerWave; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16, w_voff[j], ((kbase + kt) >> w_shift) * w_step, 0, 0);
     };
     // Pick: this lane's 2 columns (byte offset wbyte of a row), rows 8 kq .. 8 kq + 7 of block blk of 32 k: row
     // 32 blk + 8 kq + r, whose block of 8 is 4 blk + kq, rotation kRot * kq
-    const uint32_t wcol = 32u * wave + 2u * c16;  // within the tile
+    const uint32_t wcol = 32u * wc + 2u * c16;  // within the tile
     const uint32_t wbyte = wcol * BITS / 8u;
     // (packed: the piece of the lane's first column; the second one's is 512 bytes on; 4-bit codes: + 8 in odd steps)
-    const uint32_t w_rd = PACKED ? (2u * wave + (c16 >> 3)) * 1024u + (((8u * kq + (c16 & 7u)) ^ (8u * (c16 >> 3))) << 4)
+    const uint32_t w_rd = PACKED ? (2u * wc + (c16 >> 3)) * 1024u + (((8u * kq + (c16 & 7u)) ^ (8u * (c16 >> 3))) << 4)
                                  : (8u * kq) * kRowBytes + ((((wbyte >> 4) + kRot * kq) & (kChunks - 1u)) << 4) + (wbyte & 15u);  // + 32 blk rows + r rows
     // Packed codes of a step as a lane reads them: [column j][K-block][half]: 8-bit codes: rows 4 half .. + 3 in the bytes
     // of a dword; 4-bit codes: [j][K-block][0] holds the 8 rows in its nibbles.
+    // (K-block: the wave's own; with two waves per column group each reads its half of the piece)
     struct PackedCodes {
-        uint32_t d[2][2][2];
+        uint32_t d[2][NB][2];
     };
     auto read_packed = [&](PackedCodes& pc, const uint8_t* src, uint32_t kt, uint32_t j) {  // src: the stage + w_rd
-        if constexpr (BITS == 8) {
+        if constexpr (BITS == 8 && KH == 1) {
             const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + 512u * j);
             pc.d[j][0][0] = v[0], pc.d[j][0][1] = v[1], pc.d[j][1][0] = v[2], pc.d[j][1][1] = v[3];
-        } else {
+        } else if constexpr (BITS == 8) {
+            const u32x2_t v = *reinterpret_cast<const u32x2_t*>(src + 512u * j + 8u * kh);
+            pc.d[j][0][0] = v[0], pc.d[j][0][1] = v[1];
+        } else if constexpr (KH == 1) {
             const u32x2_t v = *reinterpret_cast<const u32x2_t*>(src + 512u * j + 8u * ((kbase + kt) & 1u));
             pc.d[j][0][0] = v[0], pc.d[j][1][0] = v[1];
+        } else {
+            pc.d[j][0][0] = *reinterpret_cast<const uint32_t*>(src + 512u * j + 8u * ((kbase + kt) & 1u) + 4u * kh);
         }
     };
     // 4-bit: the two's-complement nibbles of a dword of 8 rows: even rows in the low nibbles of `ev`'s bytes, odd rows of `od`'s
     struct PackedNibbles {
-        uint32_t ev[2][2], od[2][2];  // [column j][K-block]
+        uint32_t ev[2][NB], od[2][NB];  // [column j][K-block]
     };
     // rows 2 pr, 2 pr + 1 of column j of K-block blk, as fp32 (8-bit: the stored code; 4-bit: q / 16)
     auto packed_values = [&](const PackedCodes& pc, PackedNibbles& nb, uint32_t blk, uint32_t j, uint32_t pr, float& f0, float& f1) {
@@ -219,16 +239,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
     };
     struct Raw {
-        uint32_t d[2][8];  // [block of 32 k][row]: two codes
+        uint32_t d[NB][8];  // [the wave's block of 32 k][row]: two codes
     };
     auto pick = [&](Raw& raw, auto stage_c) {
         const uint8_t* tile = w_tile(stage_c) + w_rd;
 #pragma unroll
-        for (uint32_t blk = 0; blk < 2; ++blk)
+        for (uint32_t lb = 0; lb < NB; ++lb)
 #pragma unroll
             for (uint32_t r = 0; r < 8; ++r) {
-                if constexpr (BITS == 8) raw.d[blk][r] = *reinterpret_cast<const uint16_t*>(tile + (32u * blk + r) * kRowBytes);
-                else raw.d[blk][r] = *(tile + (32u * blk + r) * kRowBytes);
+                if constexpr (BITS == 8) raw.d[lb][r] = *reinterpret_cast<const uint16_t*>(tile + (32u * blk_of(lb) + r) * kRowBytes);
+                else raw.d[lb][r] = *(tile + (32u * blk_of(lb) + r) * kRowBytes);
             }
     };
     // Scales go through a buffer resource so that the load is issued whatever the lane's column (the wait counts
@@ -238,14 +258,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.scale), 0, (int)(((scale_rows - 1u) * p.lds + p.n) * 2u), kBufferFlags);
     const uint32_t s_voff = (n0 + wcol) * 2u;
-    auto block_group_scales = [&](uint32_t (&sr)[2], uint32_t kt, uint32_t blk) {
-        uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk);
+    auto block_group_scales = [&](uint32_t (&sr)[NB], uint32_t kt, uint32_t lb) {
+        uint32_t g = group_of_row(p, (kbase + kt) * kTwK + 32u * blk_of(lb));
         if (g >= scale_rows) g = scale_rows - 1u;  // rows past k in a partial last step: any scale will do
-        sr[blk] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, g * p.lds * 2u, 0);
+        sr[lb] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_s, s_voff, g * p.lds * 2u, 0);
     };
-    auto group_scales = [&](uint32_t (&sr)[2], uint32_t kt) {
-        block_group_scales(sr, kt, 0);
-        block_group_scales(sr, kt, 1);
+    auto group_scales = [&](uint32_t (&sr)[NB], uint32_t kt) {
+#pragma unroll
+        for (uint32_t lb = 0; lb < NB; ++lb) block_group_scales(sr, kt, lb);
     };
     float cs[2] = {0.f, 0.f};  // one scale per column: fixed
     if constexpr (!GROUPED) {
@@ -254,7 +274,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         cs[1] = make_col_scale_nibble<BITS>(sr >> 16);
     }
     struct Ops {
-        uint32_t w[2][2][4];  // [block of 32 k][column j][dword]: the 8-element operand as 4 packed pairs
+        uint32_t w[NB][2][4];  // [the wave's block of 32 k][column j][dword]: the 8-element operand as 4 packed pairs
     };
     // the two codes of a load, ready for the conversion: as stored (8-bit codes: the excess of 128 comes off in the
     // multiplication, see scaled()); two's-complement nibbles, the second shifted down to a low nibble (4-bit codes)
@@ -278,17 +298,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         if constexpr (BITS == 8) return __builtin_fmaf(f, scale, -128.0f * scale);
         else return f * scale;
     };
-    // one sixteenth of a step's conversion: rows 2 pr, 2 pr + 1 of column j of block blk
-    auto convert_pair = [&](Ops& ops, const Raw& raw, uint32_t (&pre)[2][8][2], const float (&sc)[2][2], uint32_t blk, uint32_t j, uint32_t pr) {
+    // one sixteenth of a step's conversion: rows 2 pr, 2 pr + 1 of column j of the wave's block blk
+    auto convert_pair = [&](Ops& ops, const Raw& raw, uint32_t (&pre)[NB][8][2], const float (&sc)[NB][2], uint32_t blk, uint32_t j, uint32_t pr) {
         if (j == 0) {
             prepare(raw.d[blk][2 * pr], pre[blk][2 * pr][0], pre[blk][2 * pr][1]);
             prepare(raw.d[blk][2 * pr + 1], pre[blk][2 * pr + 1][0], pre[blk][2 * pr + 1][1]);
         }
         ops.w[blk][j][pr] = pack_bf16_rne(scaled(value(pre[blk][2 * pr][j], j), sc[blk][j]), scaled(value(pre[blk][2 * pr + 1][j], j), sc[blk][j]));
     };
-    auto block_scales = [&](float (&sc)[2][2], const uint32_t (&sr)[2]) {
+    auto block_scales = [&](float (&sc)[NB][2], const uint32_t (&sr)[NB]) {
 #pragma unroll
-        for (uint32_t blk = 0; blk < 2; ++blk) {
+        for (uint32_t blk = 0; blk < NB; ++blk) {
             if constexpr (GROUPED) {
                 sc[blk][0] = make_col_scale_nibble<BITS>(sr[blk] & 0xffffu);
                 sc[blk][1] = make_col_scale_nibble<BITS>(sr[blk] >> 16);
@@ -298,23 +318,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             }
         }
     };
-    auto convert_all = [&](Ops& ops, const Raw& raw, const uint32_t (&sr)[2]) {
-        uint32_t pre[2][8][2];
-        float sc[2][2];
+    auto convert_all = [&](Ops& ops, const Raw& raw, const uint32_t (&sr)[NB]) {
+        uint32_t pre[NB][8][2];
+        float sc[NB][2];
         block_scales(sc, sr);
 #pragma unroll
-        for (uint32_t u = 0; u < 16; ++u) convert_pair(ops, raw, pre, sc, u >> 3, (u >> 2) & 1u, u & 3u);
+        for (uint32_t u = 0; u < 8u * NB; ++u) convert_pair(ops, raw, pre, sc, u >> 3, (u >> 2) & 1u, u & 3u);
     };
     // the same from packed codes: step kt, whose codes are in the stage behind src
-    auto convert_all_packed = [&](Ops& ops, const uint8_t* src, uint32_t kt, const uint32_t (&sr)[2]) {
+    auto convert_all_packed = [&](Ops& ops, const uint8_t* src, uint32_t kt, const uint32_t (&sr)[NB]) {
         PackedCodes pc;
         PackedNibbles nb;
-        float sc[2][2];
+        float sc[NB][2];
         block_scales(sc, sr);
         read_packed(pc, src, kt, 0);
         read_packed(pc, src, kt, 1);
 #pragma unroll
-        for (uint32_t u = 0; u < 16; ++u) {
+        for (uint32_t u = 0; u < 8u * NB; ++u) {
             const uint32_t blk = u >> 3, j = (u >> 2) & 1u, pr = u & 3u;
             float f0, f1;
             packed_values(pc, nb, blk, j, pr, f0, f1);
@@ -330,9 +350,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // fragment (mt, blk): row 16 mt + c16 of the tile, chunk 4 blk + kq (the swizzle repeats every 16 rows)
     bf16x8_t af[4];  // the fragments of the next few units, carried from step to step
-    uint32_t a_rd[2];
+    uint32_t a_rd[NB];
 #pragma unroll
-    for (uint32_t blk = 0; blk < 2; ++blk) a_rd[blk] = tw_swz(c16, 4u * blk + kq);
+    for (uint32_t lb = 0; lb < NB; ++lb) a_rd[lb] = tw_swz(c16, 4u * blk_of(lb) + kq);
 
     // One K-step.  `cur`: the operands of this step; `nxt` receives those of step kt + 1, converted from the codes in stage
     // S + 1; stage S holds this step's A; the copies of step kt + 3 go into stage S + 3 = S - 1, which every wave finished
@@ -347,28 +367,29 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     //   slot 1 of unit u: one memory request (with group scales: those first, in unit 0; then the copies); the second
     //          half of pair u (two multiplications, the rounding pack)
     constexpr uint32_t kAhead = 4;
-    auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const uint32_t (&s1)[2], uint32_t (&s2)[2]) {
+    constexpr uint32_t kUnits = 8u * NB;
+    auto step = [&](auto stage_c, uint32_t kt, const Ops& cur, Ops& nxt, const uint32_t (&s1)[NB], uint32_t (&s2)[NB]) {
         constexpr uint32_t S = decltype(stage_c)::value;
         using Next = std::integral_constant<uint32_t, (S + 1u) & 3u>;
         using Target = std::integral_constant<uint32_t, (S + 3u) & 3u>;
         // At most the requests of the step before this one may still be in flight: then this wave's part of this step's
         // AND the next step's A (requested three and two steps ago) and of the next step's codes (two steps ago) has
         // landed.  Behind the barrier every wave's has.
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + kCopiesPerWave + (GROUPED ? 2 : 0)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kACopies + kCopiesPerWave + (GROUPED ? NB : 0)) : "memory");
         barrier_no_fence();  // (a fenced barrier would also wait for the copies of the steps ahead)
         const uint32_t kt3 = clamp(kt + 3), kt2 = clamp(kt + 2);
         const bool last3 = kbase + kt3 + 1u == ksteps_all;
         const uint32_t ve = last3 ? a_last_e : a_voff_e, vo = last3 ? a_last_o : a_voff_o;
-        uint8_t* const a_dst = a_tile(Target{}) + wave * 4096u;
-        uint8_t* const w_dst = w_tile(Target{}) + kCopiesPerWave * wave * 1024u;
+        uint8_t* const a_dst = a_tile(Target{}) + wave * (1024u * kACopies);
+        uint8_t* const w_dst = w_tile(Target{}) + kCopiesPerWave * wcopier * 1024u;
         const uint8_t* const a_src = a_tile(stage_c);
         const uint8_t* const a_nxt = a_tile(Next{});
         const uint8_t* const w_src = w_tile(Next{}) + w_rd;
-        uint32_t code[2][8];   // the codes of step kt + 1 as read: [block][row], two codes each
-        uint32_t pre[2][8][2];
+        uint32_t code[NB][8];   // the codes of step kt + 1 as read: [block][row], two codes each
+        uint32_t pre[NB][8][2];
         PackedCodes pc;        // ... or, from packed weights, the lane's 2 x 16 (8) bytes
         PackedNibbles nb;
-        float sc[2][2];
+        float sc[NB][2];
         float f0 = 0.f, f1 = 0.f;
         block_scales(sc, s1);
         // pair v = (block v / 8, rows 2 (v / 2 % 4), + 1, column v % 2): its two rows are read by the pair with column 0
@@ -377,8 +398,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (uint32_t h = 0; h < 2; ++h) {
                 const uint32_t r = 2u * pr + h;
-                if constexpr (BITS == 8) code[blk][r] = *reinterpret_cast<const uint16_t*>(w_src + (32u * blk + r) * kRowBytes);
-                else code[blk][r] = *(w_src + (32u * blk + r) * kRowBytes);
+                if constexpr (BITS == 8) code[blk][r] = *reinterpret_cast<const uint16_t*>(w_src + (32u * blk_of(blk) + r) * kRowBytes);
+                else code[blk][r] = *(w_src + (32u * blk_of(blk) + r) * kRowBytes);
             }
         };
         if constexpr (PACKED) {
@@ -390,7 +411,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (uint32_t u = 0; u < 16; ++u) {
+        for (uint32_t u = 0; u < kUnits; ++u) {
             const uint32_t blk = u >> 3, mt = u & 7u;
             const uint32_t cblk = u >> 3, cpr = (u >> 1) & 3u, cj = u & 1u;  // conversion pair u
             const bf16x8_t a_now = af[u % kAhead];
@@ -398,12 +419,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][1][0], cur.w[blk][1][1], cur.w[blk][1][2], cur.w[blk][1][3]));
             // ---- slot 0
             tw_mfma(acc[mt][0], a_now, wf0);
-            if (u + kAhead < 16) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
-            else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - 16u) * 2048u);
+            if (u + kAhead < kUnits) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
+            else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - kUnits) * 2048u);
             if constexpr (PACKED) {
                 packed_values(pc, nb, cblk, cj, cpr, f0, f1);
             } else {
-                if (cj == 0 && u + 4 < 16) read_codes(u + 4);
+                if (cj == 0 && u + 4 < kUnits) read_codes(u + 4);
                 if (cj == 0) {
                     if constexpr (BITS == 8) {
                         // (the two reads stay two registers: left to itself the compiler packs them into one and shifts the
@@ -424,15 +445,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             // (the group scales first: the next step waits for them at its very start, and that wait then leaves the
             // copies requested behind them in flight — requested last, they made it a wait for everything)
             // (one block's scales per slot: finding a group is a chain of five scalar instructions)
-            constexpr uint32_t kFirstCopy = GROUPED ? 2u : 0u;
-            if (GROUPED && u < 2) {
+            constexpr uint32_t kFirstCopy = GROUPED ? NB : 0u;
+            if (GROUPED && u < NB) {
                 block_group_scales(s2, kt2, u);
-            } else if (u >= kFirstCopy && u < kFirstCopy + 4) {
+            } else if (u >= kFirstCopy && u < kFirstCopy + kACopies) {
                 const uint32_t q = u - kFirstCopy;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16, (q & 1u) ? vo : ve,
                                                          (kbase + kt3) * kTwK * 2u + q * 16u * p.lda, 0, 0);
-            } else if (u >= kFirstCopy + 4 && u < kFirstCopy + 4 + kCopiesPerWave) {
-                const uint32_t q = u - kFirstCopy - 4u;
+            } else if (u >= kFirstCopy + kACopies && u < kFirstCopy + kACopies + kCopiesPerWave) {
+                const uint32_t q = u - kFirstCopy - kACopies;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_dst + q * 1024u), 16, w_voff[q],
                                                          ((kbase + kt3) >> w_shift) * w_step, 0, 0);
             }
@@ -443,7 +464,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // ---- prologue: A tiles and codes of steps 0, 1, 2 -> stages 0, 1, 2; operands of step 0
     Ops ops0, ops1;
-    uint32_t sa[2] = {0u, 0u}, sb[2] = {0u, 0u};  // group scales, alternating: sb = step 0 (then 2, ...), sa = step 1 (then 3, ...)
+    uint32_t sa[NB] = {}, sb[NB] = {};  // group scales, alternating: sb = step 0 (then 2, ...), sa = step 1 (then 3, ...)
     dma_w(C0{}, 0);
     dma_a(C0{}, 0);
     dma_w(C1{}, clamp(1));
@@ -484,14 +505,31 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto c_rows = [&](uint32_t q) -> float* {
         return reinterpret_cast<float*>(q == 0 ? lds_a0 : q == 1 ? lds_a1 : q == 2 ? lds_a2 : lds_a3);
     };
+    // (two waves per column group: the wave of the second blocks stages its sums, the wave of the first blocks adds its
+    // own to them — first blocks + second blocks, whatever the timing)
+    auto stage_sums = [&](bool add) {
 #pragma unroll
-    for (uint32_t mt = 0; mt < 8; ++mt) {
-        float* base = c_rows(mt >> 1);
+        for (uint32_t mt = 0; mt < 8; ++mt) {
+            float* base = c_rows(mt >> 1);
 #pragma unroll
-        for (uint32_t r = 0; r < 4; ++r) {
-            const uint32_t row = 16u * (mt & 1u) + 4u * kq + r;  // within the 32 rows of this array
-            *reinterpret_cast<float2*>(base + row * kTw + wcol) = make_float2(acc[mt][0][r], acc[mt][1][r]);
+            for (uint32_t r = 0; r < 4; ++r) {
+                const uint32_t row = 16u * (mt & 1u) + 4u * kq + r;  // within the 32 rows of this array
+                float2* at = reinterpret_cast<float2*>(base + row * kTw + wcol);
+                float2 v = make_float2(acc[mt][0][r], acc[mt][1][r]);
+                if (add) {
+                    const float2 o = *at;
+                    v = make_float2(v.x + o.x, v.y + o.y);
+                }
+                *at = v;
+            }
         }
+    };
+    if constexpr (KH == 2) {
+        if (kh == 1u) stage_sums(false);
+        __syncthreads();
+        if (kh == 0u) stage_sums(true);
+    } else {
+        stage_sums(false);
     }
     __syncthreads();
     const bool gated = p.activation == kActSiluGate;
@@ -550,8 +588,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     };
     auto finish_tile = [&]() {
 #pragma unroll
-        for (uint32_t pass = 0; pass < 8; ++pass) {
-            const uint32_t row = 16u * pass + (tid >> 4);
+        for (uint32_t pass = 0; pass < 8u / KH; ++pass) {
+            const uint32_t row = 16u * KH * pass + (tid >> 4);
             if (m0 + row >= p.m || gn >= p.n) continue;
             float v[8];
             staged(row, v);
@@ -567,25 +605,26 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // last split (dispatched after them: blockIdx.y is the slow index) fetches them, again while any word is still empty,
     // adds them in split order with its own sums last, finishes the outputs and leaves the words empty.  Only it waits, and
     // only on workgroups that wait for nothing; the wait is bounded all the same.
-    // Who moves what: thread t has the four columns 4 (t % 32) .. + 3 of tile rows t / 32 + 8 i, i = 0 .. 15, so that one
+    // Who moves what: thread t has the four columns 4 (t % 32) .. + 3 of tile rows t / 32 + kHStride i, i = 0 .. kHeld - 1, so that one
     // instruction of a wave covers two whole rows of the tile (512 contiguous bytes each): whole cache lines go out and come
     // in.  What the hand-over costs all the same is the reducing workgroup's fetch: 64 KiB per split through one CU, which
     // draws some 15-20 GB/s from beyond its L2 (3-5 us per split; measured with the fetch, the producers' stores and the
     // emptying switched off in turn), plus about 6 us for the producers' stores to arrive.
     const __amdgpu_buffer_rsrc_t ws = __builtin_amdgcn_make_buffer_rsrc(p.partials, 0, (int)p.partial_bytes, kBufferFlags);
     const uint32_t split_bytes = p.m * p.n * 4u;
+    constexpr uint32_t kHStride = 8u * KH, kHeld = 16u / KH;
     const uint32_t hrow = tid >> 5, hcol = 4u * (tid & 31u);
     const uint32_t rows_here = p.m - m0 < kTw ? p.m - m0 : kTw;  // rows of this tile that exist
-    const uint32_t mine = (n0 + hcol < p.n && hrow < rows_here) ? (rows_here - hrow + 7u) / 8u : 0u;  // of the thread's 16 rows
-    auto word_off = [&](uint32_t i) { return ((m0 + hrow + 8u * i) * p.n + n0 + hcol) * 4u; };
+    const uint32_t mine = (n0 + hcol < p.n && hrow < rows_here) ? (rows_here - hrow + kHStride - 1u) / kHStride : 0u;  // of the thread's kHeld rows
+    auto word_off = [&](uint32_t i) { return ((m0 + hrow + kHStride * i) * p.n + n0 + hcol) * 4u; };
     auto held = [&](uint32_t i) -> float4* {
-        const uint32_t row = hrow + 8u * i;
+        const uint32_t row = hrow + kHStride * i;
         return reinterpret_cast<float4*>(c_rows(row >> 5) + (row & 31u) * kTw + hcol);
     };
     if (ks != p.splits - 1u) {
         if (p.debug_flags & kDebugWithholdPartials) return;  // test hook: lets the reducer's wait run out
 #pragma unroll
-        for (uint32_t i = 0; i < 16; ++i) {
+        for (uint32_t i = 0; i < kHeld; ++i) {
             if (i >= mine) continue;
             const float4 v = *held(i);
             const u32x4_t w4 = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
@@ -593,9 +632,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         return;
     }
-    float4 total[16];
+    float4 total[kHeld];
 #pragma unroll
-    for (uint32_t i = 0; i < 16; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t i = 0; i < kHeld; ++i) total[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     // First wait, at the price of one word per thread and split, until the producers' last stores show: a fetch of whole
     // tiles that comes too early moves 64 KiB per split of nothing through this CU.  (What a thread stored last is not
     // bound to arrive last: the fetch below checks every word on its own.)
@@ -617,11 +656,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         // two splits' words of all the thread's rows are fetched together (more bytes in flight per CU, fewer round trips),
         // and fetched again together while any is empty
         const bool pair = sp + 2u < p.splits;  // the same for every thread
-        u32x4_t w[2][16];
+        u32x4_t w[2][kHeld];
         // bit 16 j + i: words (j, i) are wanted and have not been seen complete yet; only those are fetched again
         uint32_t missing = 0u;
 #pragma unroll
-        for (uint32_t i = 0; i < 16; ++i)
+        for (uint32_t i = 0; i < kHeld; ++i)
             if (i < mine) missing |= (1u << i) | (pair ? 1u << (16u + i) : 0u);
         for (uint32_t tries = 0; missing != 0u && tries < fetch_limit; ++tries) {
             if (tries) __builtin_amdgcn_s_sleep(2);
@@ -629,13 +668,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (uint32_t j = 0; j < 2; ++j)
 #pragma unroll
-                for (uint32_t i = 0; i < 16; ++i)
+                for (uint32_t i = 0; i < kHeld; ++i)
                     if (missing & (1u << (16u * j + i)))
                         w[j][i] = __builtin_amdgcn_raw_buffer_load_b128(ws, (int)word_off(i), (int)((sp + j) * split_bytes), kAuxDeviceScope);
 #pragma unroll
             for (uint32_t j = 0; j < 2; ++j)
 #pragma unroll
-                for (uint32_t i = 0; i < 16; ++i)
+                for (uint32_t i = 0; i < kHeld; ++i)
                     if ((missing & (1u << (16u * j + i))) && w[j][i][0] != kEmptyWord && w[j][i][1] != kEmptyWord && w[j][i][2] != kEmptyWord &&
                         w[j][i][3] != kEmptyWord)
                         missing &= ~(1u << (16u * j + i));
@@ -647,7 +686,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
         for (uint32_t j = 0; j < 2; ++j)  // in split order
 #pragma unroll
-            for (uint32_t i = 0; i < 16; ++i) {
+            for (uint32_t i = 0; i < kHeld; ++i) {
                 if (i >= mine || (j == 1u && !pair)) continue;
                 total[i].x += __uint_as_float(w[j][i][0]);
                 total[i].y += __uint_as_float(w[j][i][1]);
@@ -657,7 +696,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
     // the other splits' sums plus this workgroup's own, back where the finishing pass takes them from
 #pragma unroll
-    for (uint32_t i = 0; i < 16; ++i) {
+    for (uint32_t i = 0; i < kHeld; ++i) {
         if (i >= mine) continue;
         float4* own = held(i);
         const float4 o = *own;
@@ -669,7 +708,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     const u32x4_t empty4 = {kEmptyWord, kEmptyWord, kEmptyWord, kEmptyWord};
     for (uint32_t sp = 0; sp + 1u < p.splits; ++sp) {
 #pragma unroll
-        for (uint32_t i = 0; i < 16; ++i)
+        for (uint32_t i = 0; i < kHeld; ++i)
             if (i < mine) __builtin_amdgcn_raw_buffer_store_b128(empty4, ws, (int)word_off(i), (int)(sp * split_bytes), kAuxDeviceScope);
     }
 }
@@ -679,8 +718,8 @@ static hipError_t launch_prefill128_wreg_t(const GemmParams& p, hipStream_t stre
 {
     const uint32_t tiles = ((p.m + kTw - 1) / kTw) * ((p.n + kTw - 1) / kTw);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED>;
-    return launch_kernel(kernel, dim3(grid, p.splits, 1), dim3(256, 1, 1), 0, stream, p);
+    void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED, 2>;
+    return launch_kernel(kernel, dim3(grid, p.splits, 1), dim3(512, 1, 1), 0, stream, p);
 }
 
 // Whether this kernel can serve a launch: this library's own arithmetic (either order of the weights).
