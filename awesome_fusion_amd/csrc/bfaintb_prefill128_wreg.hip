@@ -6,13 +6,18 @@
 // /root/reference/bfAintBGemm/bfAintBGemm.cc:105-109).  That kernel converts W into LDS and every wave reads both
 // operands back: a K-step takes 0.75 us whatever the load on the machine, three times its matrix-instruction time.
 // Here, as in bfaintb_prefill_wreg_kernel, only A goes through LDS:
-//   256 threads = 4 waves side by side along n; a wave owns ALL 128 rows x 32 columns of the tile = 8 x 2 accumulators
-//   of v_mfma_f32_16x16x32_bf16, converts exactly the weights it multiplies by, straight into the instruction's
-//   operand registers, and each weight of the tile is converted once.
+//   4 column groups side by side along n, KH waves each (the launch uses KH = 2: 512 threads, two waves per SIMD);
+//   a wave owns ALL 128 rows x 32 columns of the tile = 8 x 2 accumulators of v_mfma_f32_16x16x32_bf16, converts exactly
+//   the weights it multiplies by, straight into the instruction's operand registers, and each weight of the tile is
+//   converted once.  With KH = 2 the two waves of a column group share a K-step by its blocks of 32 k (wave kh takes
+//   block kh of every step) and the epilogue adds their sums, first blocks + second blocks: an output is the sum of
+//   two chains of matrix instructions, not of one as in the other tiled kernels, so it agrees with them to rounding,
+//   not bit for bit (it is reproducible run to run: nothing depends on timing).  The second wave per SIMD gives
+//   the in-order issue something to run while the other waits for LDS: 2-11 % on every shape measured.
 //   The vector-memory path takes about 20 cycles per instruction of a wave whatever it moves (measured: with the codes
 //   fetched by 16 two-byte loads per wave and step, 80 instructions per CU and step took 1600 cycles and the kernel was
 //   no faster than its predecessor; without them a step took 0.48 us instead of 0.80).  So the codes, too, come in by the
-//   asynchronous copy — 16 bytes per lane, 8 KiB (4 for 4-bit codes) per step in 2 (1) instructions per wave — into
+//   asynchronous copy — 16 bytes per lane, 8 KiB (4 for 4-bit codes) per step in 8 (4) instructions of the workgroup — into
 //   four LDS stages of their own, kept as stored (rows of the tile's 128 codes), and each lane picks its codes out of
 //   LDS: lane (c16 = lane % 16, kq = lane / 16) reads, per block of 32 k and for each of the 8 rows k0 + 8 kq + r, the
 //   codes of columns 2 c16, 2 c16 + 1 of the wave's 32 (one ds_read_u16; u8 for 4-bit codes): code j of those 8 reads
@@ -22,9 +27,9 @@
 //   kernels; the copies of step kt + 3 (A and codes) start at step kt, behind the step's one barrier (which also says
 //   every wave is done reading the stages they overwrite).  96 KiB of LDS in all.
 //   Per K-step a CU reads 64 KiB of A fragments and 8 KiB of codes from LDS and the copy engine writes 24.
-// Each of the step's 16 (block of 32 k, row block) pairs runs two matrix instructions and carries one sixteenth of
-// the conversion of the next step's weights (two weights: five instructions), so conversion and matrix work
-// alternate finely without hand-placed fences.
+// Each of a wave's 8 (KH = 1: 16) units (block of 32 k, row block) of a step runs two matrix instructions and carries
+// one conversion pair of the next step's weights (two weights: five instructions), so conversion and matrix work
+// alternate finely.
 // Accumulator (mt, j), register r of lane (c16, q = lane / 16): row 16 mt + 4 q + r, column 32 w + 2 c16 + j of the tile.
 // Epilogue: as bfaintb_prefill128_kernel — fp32 sums staged in LDS in [m][n] order, each thread finishes 8 neighbouring
 // columns of a row (bias, SiLU gate, residual, the one rounding) and stores them with one 16-byte write.
@@ -54,8 +59,9 @@ __device__ __forceinline__ void tw_mfma(f32x4_t& acc, const bf16x8_t& a, const b
 __device__ __forceinline__ void tw_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 }  // namespace
 
-template <int BITS, bool GROUPED, bool PACKED, int KH>
-__global__ void __launch_bounds__(256 * KH) __attribute__((amdgpu_waves_per_eu(KH, KH))) bfaintb_prefill128_wreg_kernel(const GemmParams p)
+template <int BITS, bool GROUPED, bool PACKED, int KH, bool COPIER>
+__global__ void __launch_bounds__(256 * KH + (COPIER ? 64 : 0)) __attribute__((amdgpu_waves_per_eu(KH + (COPIER ? 1 : 0), KH + (COPIER ? 1 : 0))))
+bfaintb_prefill128_wreg_kernel(const GemmParams p)
 {
     static_assert(KH == 1 || KH == 2, "one wave per SIMD, or two that share a K-step by its blocks of 32 k");
     constexpr uint32_t kWaves = 4u * KH;
@@ -194,6 +200,55 @@ __global__ void __launch_bounds__(256 * KH) __attribute__((amdgpu_waves_per_eu(K
         for (uint32_t j = 0; j < kCopiesPerWave; ++j)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(base + j * 1024u), 16, w_voff[j], ((kbase + kt) >> w_shift) * w_step, 0, 0);
     };
+    // The copying wave (COPIER: one wave more than those that compute): every copy of the K loop is its request, so that
+    // the computing waves' only memory requests are their group scales and the wait for those — which the compiler
+    // places, and which counts every request of the wave ahead of them — no longer holds a wave until copies of later
+    // steps have landed (grouped scales: 9-11 % on the whole kernel; with one scale per column, where the computing
+    // waves load nothing in the loop, the copying wave changes -1 .. +4 % and is not used).
+    // Instruction j of a step's A fills rows 8 j .. 8 j + 7 (the lane's offsets are those of rows 0 .. 7, the row advance
+    // sits in the scalar offset); the codes go as the computing waves would copy them.  The first three steps' copies
+    // are shared out over the computing waves (the prologue below): one wave would issue them one after the other.
+    if (COPIER && wave == kWaves) {
+        const uint32_t pa_e = ((lane >> 3) * p.lda + chunk_e * 8u) * 2u, pa_o = ((lane >> 3) * p.lda + chunk_o * 8u) * 2u;
+        const uint32_t pl_e = chunk_e < last_chunks ? pa_e : a_extent, pl_o = chunk_o < last_chunks ? pa_o : a_extent;
+        uint32_t pw[8];
+#pragma unroll
+        for (uint32_t j = 0; j < kCopies; ++j) {
+            if constexpr (PACKED) {
+                const uint32_t at = (lane & 31u) ^ (8u * (j & 1u));
+                pw[j] = j * slab_bytes + (16u * (at >> 3) + 2u * (at & 7u) + (lane >> 5)) * 16u;
+            } else {
+                const uint32_t row = j * kRowsPerCopy + lane / kChunks;
+                const uint32_t chunk = ((lane % kChunks) - kRot * ((row >> 3) & 3u)) & (kChunks - 1u);
+                pw[j] = row * p.ldb_bytes + chunk * 16u;
+            }
+        }
+        auto copy_step = [&](uint32_t stage, uint32_t kt) {
+            uint8_t* const a_base = stage == 0u ? lds_a0 : stage == 1u ? lds_a1 : stage == 2u ? lds_a2 : lds_a3;
+            uint8_t* const w_base = stage == 0u ? lds_w0 : stage == 1u ? lds_w1 : stage == 2u ? lds_w2 : lds_w3;
+            const bool last = kbase + kt + 1u == ksteps_all;
+            const uint32_t ve = last ? pl_e : pa_e, vo = last ? pl_o : pa_o;
+#pragma unroll
+            for (uint32_t j = 0; j < 16u; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_base + j * 1024u), 16, (j & 1u) ? vo : ve,
+                                                         (kbase + kt) * kTwK * 2u + j * 16u * p.lda, 0, 0);
+#pragma unroll
+            for (uint32_t j = 0; j < kCopies; ++j)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)(w_base + j * 1024u), 16, pw[j],
+                                                         ((kbase + kt) >> w_shift) * w_step, 0, 0);
+        };
+        barrier_no_fence();  // (the first three steps' copies are shared out over the computing waves: see the prologue)
+        for (uint32_t kt = 0; kt < ksteps; ++kt) {
+            // the computing waves start step kt behind this barrier: the copies of steps up to kt + 1 have landed when at
+            // most those of step kt + 2 (requested behind the last barrier) are in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(16 + kCopies) : "memory");
+            barrier_no_fence();
+            copy_step((kt + 3u) & 3u, clamp(kt + 3u));  // into the stage of step kt - 1, which every wave has left
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // the epilogue's first barrier: nothing is writing LDS any more
+        return;               // (a wave that has ended no longer counts at the barriers that follow)
+    }
     // Pick: this lane's 2 columns (byte offset wbyte of a row), rows 8 kq .. 8 kq + 7 of block blk of 32 k: row
     // 32 blk + 8 kq + r, whose block of 8 is 4 blk + kq, rotation kRot * kq
     const uint32_t wcol = 32u * wc + 2u * c16;  // within the tile
@@ -375,7 +430,7 @@ __global__ void __launch_bounds__(256 * KH) __attribute__((amdgpu_waves_per_eu(K
         // At most the requests of the step before this one may still be in flight: then this wave's part of this step's
         // AND the next step's A (requested three and two steps ago) and of the next step's codes (two steps ago) has
         // landed.  Behind the barrier every wave's has.
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kACopies + kCopiesPerWave + (GROUPED ? NB : 0)) : "memory");
+        if constexpr (!COPIER) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kACopies + kCopiesPerWave + (GROUPED ? NB : 0)) : "memory");
         barrier_no_fence();  // (a fenced barrier would also wait for the copies of the steps ahead)
         const uint32_t kt3 = clamp(kt + 3), kt2 = clamp(kt + 2);
         const bool last3 = kbase + kt3 + 1u == ksteps_all;
@@ -448,6 +503,7 @@ __global__ void __launch_bounds__(256 * KH) __attribute__((amdgpu_waves_per_eu(K
             constexpr uint32_t kFirstCopy = GROUPED ? NB : 0u;
             if (GROUPED && u < NB) {
                 block_group_scales(s2, kt2, u);
+            } else if (COPIER) {
             } else if (u >= kFirstCopy && u < kFirstCopy + kACopies) {
                 const uint32_t q = u - kFirstCopy;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)(a_dst + q * 1024u), 16, (q & 1u) ? vo : ve,
@@ -718,8 +774,9 @@ static hipError_t launch_prefill128_wreg_t(const GemmParams& p, hipStream_t stre
 {
     const uint32_t tiles = ((p.m + kTw - 1) / kTw) * ((p.n + kTw - 1) / kTw);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
-    void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED, 2>;
-    return launch_kernel(kernel, dim3(grid, p.splits, 1), dim3(512, 1, 1), 0, stream, p);
+    // two waves per column group; with grouped scales, the copying wave on top
+    void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED, 2, GROUPED>;
+    return launch_kernel(kernel, dim3(grid, p.splits, 1), dim3(512 + (GROUPED ? 64 : 0), 1, 1), 0, stream, p);
 }
 
 // Whether this kernel can serve a launch: this library's own arithmetic (either order of the weights).
