@@ -115,7 +115,10 @@ static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bo
 // overlapped the fewer waves a SIMD holds); repeats of the stream mostly hit in cache; split-K partial sums
 // are written, read and cleared, and cost two more trips to memory; with fewer than one wave per SIMD both the
 // arithmetic and the stream slow down in proportion.  Fitted to measurements at N = 4096, 11008 and 28672.
-static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
+struct FamilyEstimate {
+    double core, partial;  // the stream or the arithmetic, whichever is longer; the split's hand-over
+};
+static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl, FamilyEstimate* parts = nullptr)
 {
     const double weights = (double)n * k;
     const double row_blocks = (double)((m + 16u * pl.mb - 1u) / (16u * pl.mb));
@@ -137,7 +140,24 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
     const double stream_busy = bits == 8 ? (wgs >= cus ? 1.0 : wgs / cus) : busy;
     const double stream = weights * bits / 8.0 * (1.0 + (bits == 8 ? 0.5 : 0.3) * (row_blocks - 1.0)) / 3.5e6 / stream_busy;
     const double partial = pl.splits > 1 ? 3.0 + 12.0 * (pl.splits - 1.0) * m * n / 1.5e6 : 0.0;
+    if (parts != nullptr) *parts = FamilyEstimate{compute > stream ? compute : stream, partial};
     return 5.0 + (compute > stream ? compute : stream) + partial;
+}
+
+// The same estimate, corrected to what the family's own plan takes in absolute terms: the estimate above ranks the
+// family's plans among themselves (row-block size x split factor) and is left as fitted for that; against the tiles
+// its absolute value decides, and there it is 1.3 - 1.75 times the measured time wherever k is split (the hand-over
+// term is several times too large for row blocks of up to 32 rows, about 1.5 times for 64-row blocks) and within 8 %
+// without a split.  Corrections fitted on 62 shapes (m = 48 .. 1024 over 4096 x 4096, 11008 x 4096, 4096 x 11008,
+// 8192 x 8192, 2048 x 8192, 28672 x 8192, both code widths: the pick is then the faster form on 58 of them, within 10 %
+// on the other four); 4-bit codes: 0.76 of the whole estimate, which dates from before their conversion got cheaper.
+static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
+{
+    FamilyEstimate e;
+    const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
+    if (bits == 4) return 0.76 * ranked;
+    if (pl.splits > 1u) return 0.87 * (5.0 + e.core + (pl.mb == 4u ? 0.65 : 0.2) * e.partial);
+    return (pl.mb == 4u ? 1.05 : 0.93) * (5.0 + e.core);
 }
 
 // The tiled variant runs 128x128 tiles while those fit one per CU: four times the workgroups of
@@ -170,9 +190,8 @@ static bool use_small_tiles(int v, uint32_t m, uint32_t n)
     return v == BFAINTB_VARIANT_PREFILL_128 || v == BFAINTB_VARIANT_PREFILL_128_LDS || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n));
 }
 
-// Rough time of the tiled variant.  Large tiles: whole rounds of 256x256 tiles over the CUs, 1.33 us per 64 rows of
-// k.  Small tiles: a K-step takes 0.49 us on an empty machine and 0.56 us with a workgroup on every CU (the kernel that
-// keeps the weights in registers; 0.64 and 0.67 us with 4-bit codes), whichever order the weights are stored in.
+// Rough time of the tiled variant (prefill_estimate_us, below the plan of the small tiles).  Small tiles: a K-step takes 0.40 us on an empty machine and 0.55 us with a workgroup on every CU (the kernel that
+// keeps the weights in registers), whichever order the weights are stored in.
 // The small-tile kernel may split k: grid y walks the splits, each workgroup runs its share of
 // the K-steps and the workgroup of the last split adds the others' sums (same workspace and protocol as the decode
 // family).  Worth it while tiles x splits still fit one workgroup per CU.
@@ -194,6 +213,7 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
     const uint32_t ksteps = (k + 63u) / 64u;
     const double tiles = (double)((m + 127u) / 128u) * (double)((n + 127u) / 128u);
     const double cus = (double)machine_cus();
+    const double fill = (double)m / (double)((m + 127u) / 128u * 128u);  // the share of the tiles' rows that exist
     auto shape = [&](uint32_t want) {
         TilePlan t;
         if (want > kMaxTileSplits) want = kMaxTileSplits;
@@ -201,15 +221,19 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         const uint32_t per = (ksteps + want - 1u) / want;
         t.k_per_wg = per * 64u;
         t.splits = (ksteps + per - 1u) / per;
-        // the hand-over: the producers' device-scope stores have to arrive (some 3 us after the last K-step), then the
-        // reducing workgroup fetches a tile's worth of sums per split through its one CU, slower the more CUs do so at once
-        // (8-bit, n = k = 4096, us with 1 / 2 / 4 splits: m = 128: 35.2 / 27.3 / 26.6; m = 256: 35.6 / 27.8 / 28.6; m = 512:
-        // 35.9 / 30.0; 8192 x 8192, m = 256: 66.0 / 46.0; 4-bit g128, m = 256: 45.8 / 32.8 / 30.3)
-        const double hand_over = t.splits > 1u ? 3.5 + (t.splits - 1.0) * (3.6 + 0.007 * tiles) : 0.0;
-        // a K-step: 0.49 us (4-bit codes 0.64) on an empty machine, rising by 0.01 per 100 workgroups; with a workgroup on
-        // (nearly) every CU 8-bit codes take 0.56 (the clock gives way)
+        // the hand-over: the producers' device-scope stores have to arrive, then the reducing workgroup fetches the rows
+        // of a tile that exist, per split, through its one CU, slower the more CUs do so at once.  What the measured times
+        // leave after the K-steps (8-bit, us): 48 / 64 / 96 / 128 x 4096 x 4096, 4 splits of 32 tiles: 7.0 / 8.0 / 9.7 / 11.4;
+        // 384 x 2048 x 8192, 4 x 48: 9.6; 384 x 4096 x 4096, 2 x 96: 4.5; 256 x 8192 x 8192, 2 x 128: 5.9; 512 x 4096 x
+        // 4096, 2 x 128: 7.6.
+        const double hand_over = t.splits > 1u ? 3.0 + (t.splits - 1.0) * (0.6 + 1.6 * fill + 0.008 * tiles) : 0.0;
+        // a K-step (two waves per column group): 0.40 us (4-bit codes 0.41) on a nearly empty machine, rising with the
+        // cube of the share of the CUs that hold a workgroup as the clock gives way (8-bit, n = k = 4096, us per step at
+        // 160 / 192 / 224 / 256 workgroups: 0.425 / 0.44 / 0.50 / 0.55; 4-bit g128: 0.49 at 224, 0.55 - 0.56 at 256);
+        // rows of a tile that do not exist are not copied (28672 x 8192 4-bit, m = 64 / 96 / 128: 0.435 / 0.45 / 0.48)
         const double wgs = tiles * t.splits;
-        const double step_us = bits == 4 ? 0.64 + 0.0001 * wgs : 0.485 + 0.0001 * wgs + (wgs >= 0.9375 * cus ? 0.055 : 0.0);
+        const double load = wgs >= cus ? 1.0 : wgs / cus;
+        const double step_us = ((bits == 4 ? 0.41 : 0.40) + 0.15 * load * load * load) * (0.8 + 0.2 * fill);
         t.us = 4.0 + per * step_us + hand_over;
         // (three splits and more: the hand-over scatters more than this says, and where the row-blocked family is about as
         // fast it is the safer pick — 192 x 4096 x 4096: 25.5 against 22.9 us, 128 x 4096 x 11008: 39.0 against 34.3)
@@ -233,10 +257,18 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
 static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
     if (prefill_small_tiles(m, n)) return tile128_plan(m, n, k, bits, 0).us;
-    const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
     const double cus = (double)machine_cus();
+    if (prefill_tall_tiles(m, n)) {
+        // one tile of 256 rows x 128 columns per CU at most (8-bit, us per K-step: 512 x 11008 x 4096, 172 tiles: 0.87;
+        // 768 x 8192 x 8192 and 1536 x 4096 x 4096, 192: 0.84 and 0.88; 2048 x 4096 x 4096 and x 11008, 256: 1.02 and 0.98)
+        const double tiles = (double)((m + 255u) / 256u) * (double)((n + 127u) / 128u);
+        const double load = tiles / cus;
+        return 4.0 + (k / 64.0) * (0.83 + 0.17 * load * load * load);
+    }
+    // whole rounds of 256x256 tiles at what the board's power allows (4096^3: 1.55 us per K-step and round)
+    const double tiles = (double)((m + 255u) / 256u) * (double)((n + 255u) / 256u);
     const double rounds = (double)(uint64_t)((tiles + cus - 1.0) / cus);
-    return 4.0 + rounds * (k / 64.0) * 1.33;
+    return 4.0 + rounds * (k / 64.0) * 1.5;
 }
 
 // The decode family in row blocks: grid z walks blocks of 16*mb rows.  128 columns x 64 rows (mb = 4, 4 waves: one
@@ -404,16 +436,10 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
 int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 {
     if (variant == BFAINTB_VARIANT_AUTO) {
-        // (up to 64 rows one block of rows streams B once at full matrix-instruction height, while tiles of 128 rows run half
-        // empty: the family wins on every shape measured — 11008 x 4096, m = 64: 24.6 against 29.6 us, 8192 x 8192: 29.8
-        // against 35.0, 4-bit 31.2 against 39.0 — whatever the estimates, which are not that fine, say)
-        if (m <= kDecodeAutoMaxM || m <= 64u) return BFAINTB_VARIANT_DECODE;
+        if (m <= kDecodeAutoMaxM) return BFAINTB_VARIANT_DECODE;
         if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
         const DecodePlan pl = decode_plan(m, n, k, bits, 0);
-        // (the family's estimate for 4-bit codes dates from before their conversion got cheaper: 1.17 to 1.45 times the
-        // measured time on 40 shapes, median 1.32; it still ranks the family's own plans, but against the tiles it is corrected)
-        const double family = decode_family_estimate_us(m, n, k, bits, pl) * (bits == 4 ? 0.76 : 1.0);
-        return family < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+        return decode_family_time_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
     }
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
     if (is_prefill(variant)) return variant;
@@ -918,11 +944,19 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
     return decode_plan_row_blocks(m, n, k, bits, 0, true);
 }
 
-// The family's estimate against the tiles', over packed weights: scaled by what a scan of 11 weight shapes x 9 values of m
-// (96 .. 2048) x both code widths fits best — with these the pick is within 3 % of the best form on 185 of 190 shapes, worst
-// 8 % (8-bit, 128 x 5120 x 13824); with the row-major path's 0.76 for 4-bit codes the family was picked 22 % too slow at
-// 256 x 4096 x 4096 (its kernels over packed 4-bit codes have no 8-wave form).
-constexpr double kPackedFamily8Bit = 0.95, kPackedFamily4Bit = 0.85;
+// The family's estimate against the tiles', over packed weights, corrected as decode_family_time_us corrects it for
+// row-major weights, with what a scan of 11 weight shapes x 9 values of m (96 .. 2048) x both code widths fits: the
+// family's kernels over packed weights run at 0.72 (row blocks up to 32 rows) to 0.78 (64 rows) of the estimate's stream and
+// arithmetic, and the hand-over costs 0.35 and 0.7 of its term; the factors in use (0.76, 0.84) sit a little above that,
+// where the pick on the scan's shapes is best: where the two forms are close the tiles are the steadier choice.  4-bit
+// codes: 0.70 of the whole (their packed kernels have no 8-wave form).
+static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
+{
+    FamilyEstimate e;
+    const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
+    if (bits == 4) return 0.70 * ranked;
+    return (pl.mb == 4u ? 0.84 : 0.76) * (5.0 + e.core + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
+}
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the
 // row-blocked family without a split along k beyond) or the tiled kernel, by the estimates that choose for row-major weights.
 static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
@@ -933,8 +967,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (packed_uses_slab(m, n, k, bits) || m <= 64u) return BFAINTB_VARIANT_DECODE;  // (up to 64 rows: as for row-major weights)
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
-    const double family = decode_family_estimate_us(m, n, k, bits, pl) * (bits == 4 ? kPackedFamily4Bit : kPackedFamily8Bit);
-    return family < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
+    return packed_family_time_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
 }
 
 int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint32_t group_size)

@@ -416,6 +416,10 @@ PLAN_CHECK_SHAPES = [
     (192, 4096, 11008, 8, 0), (256, 4096, 4096, 8, 0), (256, 8192, 8192, 8, 0), (256, 8192, 8192, 4, 128), (384, 2048, 8192, 8, 0),
     (512, 4096, 4096, 8, 0), (512, 11008, 4096, 8, 0), (640, 4096, 4096, 8, 0), (768, 8192, 8192, 8, 0), (1024, 4096, 4096, 8, 0),
     (1024, 4096, 4096, 4, 128), (1536, 4096, 4096, 8, 0), (2048, 4096, 4096, 8, 0), (2048, 4096, 11008, 8, 0), (4096, 4096, 4096, 8, 0),
+    # where the row-blocked decode family and the small tiles cross (48 .. 256 rows), both code widths
+    (64, 11008, 4096, 8, 0), (64, 8192, 8192, 8, 0), (96, 4096, 4096, 8, 0), (192, 4096, 4096, 8, 0), (128, 4096, 11008, 8, 0),
+    (896, 4096, 4096, 8, 0), (64, 8192, 8192, 4, 128), (64, 28672, 8192, 4, 128), (96, 4096, 4096, 4, 128), (128, 4096, 4096, 4, 128),
+    (192, 4096, 4096, 4, 128), (256, 4096, 4096, 4, 128),
 ]
 
 

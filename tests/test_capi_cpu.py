@@ -46,7 +46,7 @@ def test_variant_choice_and_split():
     assert af.variant(1, 4096, 4096) == af.DECODE
     assert af.variant(32, 4096, 4096) == af.DECODE
     assert af.variant(33, 4096, 4096) == af.DECODE      # row blocks of the decode family: 256x256 tiles would idle most CUs
-    assert af.variant(256, 4096, 4096) == af.DECODE
+    assert af.variant(128, 4096, 4096) == af.DECODE     # 15.7 us against 22 for 32 small tiles with k split four ways
     assert af.variant(2048, 4096, 4096) == af.PREFILL
     assert af.variant(512, 28672, 8192, 4, 128) == af.PREFILL
     assert af.variant(4096, 4096, 4096) == af.PREFILL
