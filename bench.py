@@ -45,20 +45,20 @@ MIN_LAUNCHES = 400            # launches inside one event pair (several replays 
 # file: the output names the source beside the figure.
 RECORDED_TRAFFIC = {
     # name: (bytes, source)
-    "decode_m1_n4096_k4096_int8_perchannel": (17424987, "profiles/decode_m1_n4096_k4096_int8.txt"),
+    "decode_m1_n4096_k4096_int8_perchannel": (17453820, "profiles/decode_m1_n4096_k4096_int8.txt"),
     "decode_m1_n4096_k4096_int8_perchannel_prepacked": (16929572, "profiles/decode_m1_n4096_k4096_int8_prepacked.txt"),
     "prefill_m4096_n4096_k4096_int8_perchannel": (171267562, "profiles/prefill_m4096_n4096_k4096_int8.txt"),
-    "decode_m1_n11008_k4096_int8_perchannel": (46258715, "profiles/decode_m1_n11008_k4096_int8.txt"),
-    "decode_m4_n11008_k4096_int8_perchannel": (48334036, "profiles/decode_m4_n11008_k4096_int8.txt"),
-    "decode_m8_n11008_k4096_int8_perchannel": (47187147, "profiles/decode_m8_n11008_k4096_int8.txt"),
-    "decode_m16_n11008_k4096_int8_perchannel": (48972850, "profiles/decode_m16_n11008_k4096_int8.txt"),
-    "decode_m32_n11008_k4096_int8_perchannel": (52579634, "profiles/decode_m32_n11008_k4096_int8.txt"),
-    "m1_n28672_k8192_int4_group128": (122557732, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
-    "m16_n28672_k8192_int4_group128": (130166040, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
-    "m2048_n28672_k8192_int4_group128": (908258153, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
-    "mid_m256_n4096_k4096_int8_perchannel": (35834805, "profiles/mid_m256_n4096_k4096_int8.txt"),
-    "mid_m1024_n4096_k4096_int8_perchannel": (92435211, "profiles/mid_m1024_n4096_k4096_int8.txt"),
-    "mid_m256_n8192_k8192_int8_perchannel": (131059871, "profiles/mid_m256_n8192_k8192_int8.txt"),
+    "decode_m1_n11008_k4096_int8_perchannel": (46256875, "profiles/decode_m1_n11008_k4096_int8.txt"),
+    "decode_m4_n11008_k4096_int8_perchannel": (48373503, "profiles/decode_m4_n11008_k4096_int8.txt"),
+    "decode_m8_n11008_k4096_int8_perchannel": (47149725, "profiles/decode_m8_n11008_k4096_int8.txt"),
+    "decode_m16_n11008_k4096_int8_perchannel": (48989005, "profiles/decode_m16_n11008_k4096_int8.txt"),
+    "decode_m32_n11008_k4096_int8_perchannel": (52592926, "profiles/decode_m32_n11008_k4096_int8.txt"),
+    "m1_n28672_k8192_int4_group128": (122554256, "profiles/decode_m1_n28672_k8192_int4_group128.txt"),
+    "m16_n28672_k8192_int4_group128": (130124529, "profiles/decode_m16_n28672_k8192_int4_group128.txt"),
+    "m2048_n28672_k8192_int4_group128": (907765746, "profiles/prefill_m2048_n28672_k8192_int4_group128.txt"),
+    "mid_m256_n4096_k4096_int8_perchannel": (49120900, "profiles/mid_m256_n4096_k4096_int8.txt"),
+    "mid_m1024_n4096_k4096_int8_perchannel": (92341147, "profiles/mid_m1024_n4096_k4096_int8.txt"),
+    "mid_m256_n8192_k8192_int8_perchannel": (131513630, "profiles/mid_m256_n8192_k8192_int8.txt"),
     "mid_m2048_n4096_k4096_int8_perchannel": (168014478, "profiles/mid_m2048_n4096_k4096_int8.txt"),
 }
 
