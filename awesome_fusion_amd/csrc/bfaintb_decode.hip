@@ -412,6 +412,9 @@ __device__ __forceinline__ void reduce_splits_two_in_flight(const GemmParams& p,
     };
     for (;;) {
         if (whole(a)) { take(a); complete = true; break; }
+#ifdef BFAINTB_TRACE
+        if (tries == 2) TRACE_MARK(6);  // the first attempt has come back incomplete
+#endif
         if (tries >= p.split_wait_limit) { take(a); break; }
         fetch(a);
         ++tries;
@@ -420,6 +423,11 @@ __device__ __forceinline__ void reduce_splits_two_in_flight(const GemmParams& p,
         fetch(b);
         ++tries;
     }
+#ifdef BFAINTB_TRACE
+    // (attempts issued, the two up front included: 2 = the first one was whole)
+    if ((threadIdx.x & 63) == 0) p.trace[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + 7] = tries;
+    TRACE_MARK(1);
+#endif
     if (!complete) __hip_atomic_store(p.ws_header, kWorkspaceGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const u32x4_t empty4 = {kEmptyWord, kEmptyWord, kEmptyWord, kEmptyWord};
     float4 total = make_float4(0.f, 0.f, 0.f, 0.f);
