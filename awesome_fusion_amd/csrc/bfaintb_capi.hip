@@ -945,16 +945,19 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
 }
 
 // The family's estimate against the tiles', over packed weights, corrected as decode_family_time_us corrects it for
-// row-major weights, with what a scan of 11 weight shapes x 9 values of m (96 .. 2048) x both code widths fits: the
-// family's kernels over packed weights run at 0.72 (row blocks up to 32 rows) to 0.78 (64 rows) of the estimate's stream and
-// arithmetic, and the hand-over costs 0.35 and 0.7 of its term; the factors in use (0.76, 0.84) sit a little above that,
-// where the pick on the scan's shapes is best: where the two forms are close the tiles are the steadier choice.  4-bit
-// codes: 0.70 of the whole (their packed kernels have no 8-wave form).
+// row-major weights, with what a scan of 11 weight shapes x 12 values of m (40 .. 2048) x both code widths fits.  8-bit
+// codes: the family's kernels over packed weights run at 0.72 (row blocks up to 32 rows) to 0.78 (64 rows) of the
+// estimate's stream and arithmetic, and the hand-over costs 0.35 and 0.7 of its term; the factors in use (0.76, 0.84)
+// sit a little above that, where the pick on the scan's shapes is best.  4-bit codes: the family measures 0.69 - 0.84 of
+// the whole estimate (their packed kernels have no 8-wave form) and the tiles over packed 4-bit codes 0.82 - 0.98 of
+// theirs; 0.84 against the tiles' estimate as it stands picks best (2 of 116 shapes more than 3 % off, worst 9 %;
+// 8-bit: 3 of 128, worst 15 % at 40 x 11008 x 4096).  Up to 64 rows the family used to be the rule, as it once was
+// for row-major weights: 4-bit codes against 11008 and 28672 columns then ran 22 - 39 % over the tiles' time.
 static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
 {
     FamilyEstimate e;
     const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
-    if (bits == 4) return 0.70 * ranked;
+    if (bits == 4) return 0.84 * ranked;
     return (pl.mb == 4u ? 0.84 : 0.76) * (5.0 + e.core + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
 }
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the
@@ -964,7 +967,7 @@ static int packed_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int vari
     if (variant == BFAINTB_VARIANT_DECODE) return m <= kDecodeMaxM ? variant : BFAINTB_ERR_BAD_VARIANT;
     if (is_prefill(variant)) return variant;
     if (variant != BFAINTB_VARIANT_AUTO) return BFAINTB_ERR_BAD_VARIANT;
-    if (packed_uses_slab(m, n, k, bits) || m <= 64u) return BFAINTB_VARIANT_DECODE;  // (up to 64 rows: as for row-major weights)
+    if (packed_uses_slab(m, n, k, bits) || m <= kDecodeAutoMaxM) return BFAINTB_VARIANT_DECODE;
     if (m > kDecodeFamilyAutoMaxM) return BFAINTB_VARIANT_PREFILL;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
     return packed_family_time_us(m, n, k, bits, pl) < prefill_estimate_us(m, n, k, bits) ? BFAINTB_VARIANT_DECODE : BFAINTB_VARIANT_PREFILL;
