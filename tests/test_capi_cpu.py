@@ -252,6 +252,10 @@ def test_prepacked_entry_points_validate_before_launching():
     assert rcp(m=64, n=256, k=4096, weight_bits=4, group_size=128) == -6     # the plan splits along k: workspace required
     assert af.prepacked_variant(1, 4096, 4096) == af.DECODE
     assert af.prepacked_variant(64, 4096, 4096) == af.DECODE
+    # 48 .. 64 rows of 4-bit codes against many columns: the small tiles (54.5 against 74.5 us measured at 64 x 28672 x 8192),
+    # in either weight order; the row-blocked family where it is the faster one
+    assert af.prepacked_variant(64, 28672, 8192, 4, 128) == af.PREFILL == af.variant(64, 28672, 8192, 4, 128)
+    assert af.variant(64, 4096, 4096) == af.DECODE and af.variant(192, 4096, 4096, 4, 128) == af.PREFILL
     assert af.prepacked_variant(4096, 4096, 4096) == af.PREFILL
     assert af.prepacked_variant(1, 4096, 4160, 4, 0) == -2
     assert L.bfaintb_gemm_prepacked_variant(1, 100, 4096, 8, 0) == -2
