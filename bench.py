@@ -710,6 +710,15 @@ def main():
                  "ms_per_step": round(wall_ms, 6), "GB/s": round(w.bytes / (wall_ms * 1e-3) / 1e9, 1),
                  "config": {"workload": w.name}, "roofline": roofline_entry(w, ev_ms, "mfma")}
         entry["sustained"] = sustained_power(lambda i: af.gemm(w.c, w.a, w.b[i], w.s, w.m, w.n, w.k), len(w.b))
+        # the same launch on all-zero activations: same instructions, same memory traffic, nothing switching in the matrix
+        # pipe's operands — what the part does with this kernel when power is not what limits it
+        a_keep = w.a
+        w.a = torch.zeros_like(a_keep)
+        z_ms, _ = time_graph(af, w, pk, max(5, W // 4), rotate=True)
+        w.a = a_keep
+        entry["same_kernel_on_zero_activations"] = {"kernel_us": round(z_ms * 1e3, 3), "TFLOP/s": round(w.flops / (z_ms * 1e-3) / 1e12, 2),
+                                                    "frac": round(w.flops / (z_ms * 1e-3) / 1e12 / 2500.0, 4),
+                                                    "note": "identical instruction stream and bytes; the difference to the figure above is operand switching under the board's power cap"}
         try:
             v_ms = time_vendor_bf16_gemm(w, pk, 5)
             entry["vendor_bf16_gemm_same_shape"] = {"TFLOP/s": round(w.flops / (v_ms * 1e-3) / 1e12, 2), "kernel_us": round(v_ms * 1e3, 3),
