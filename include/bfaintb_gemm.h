@@ -62,7 +62,10 @@ enum {
                                   * the small tiles leave CUs idle, their kernel splits k between workgroups (same
                                   * workspace and hand-over as the decode family's split-K) */
     BFAINTB_VARIANT_PREFILL_256 = 3, /* the tiled kernel with 256x256 tiles, whatever the shape (tests, tuning) */
-    BFAINTB_VARIANT_PREFILL_128 = 4, /* the tiled kernel with 128x128 tiles, whatever the shape (tests, tuning) */
+    BFAINTB_VARIANT_PREFILL_128 = 4, /* the tiled kernel with 128x128 tiles, whatever the shape (tests, tuning).  Its fp32
+                                      * sums are those of two chains of matrix instructions added at the end (even and odd
+                                      * blocks of 32 k), so it agrees with the other tiled forms to rounding, not in
+                                      * every bit; like every form it gives the same bits on every run */
     BFAINTB_VARIANT_PREFILL_256_LDS = 5, /* 256x256 tiles with both operands staged in LDS — the older form, which the
                                           * reference's arithmetic and the half tiles of a thin last round still use;
                                           * otherwise the form that keeps the weights in registers runs (tests, tuning) */
