@@ -330,6 +330,57 @@ def sustained_power(launch, nb, seconds=1.5):
     return {"kernel_us_after_settling": round(e0.elapsed_time(e1) * 1e3 / 400, 3), "seconds_under_load": seconds, **power.summary()}
 
 
+POWER_SCAN_SHAPES = [
+    # (m, n, k, weight_bits, group_size): tiled kernels with a workgroup on every CU, with fewer, and the decode family
+    (4096, 4096, 4096, 8, 0), (2048, 4096, 4096, 8, 0), (1024, 4096, 4096, 8, 0), (1024, 4096, 4096, 4, 128), (256, 8192, 8192, 8, 0),
+    (128, 28672, 8192, 4, 128), (640, 4096, 4096, 8, 0), (256, 4096, 4096, 8, 0), (1, 4096, 4096, 8, 0), (32, 11008, 4096, 8, 0),
+    (1, 28672, 8192, 4, 128),
+]
+
+
+def power_scan(af):
+    """Board power under sustained launches of the library's own choice for POWER_SCAN_SHAPES (which kernels run at the
+    power cap), and config 4 again on operands of other value distributions (same instructions, same bytes: what the
+    cap costs)."""
+    import torch
+    rows = []
+    for (m, n, k, bits, group) in POWER_SCAN_SHAPES:
+        w = Workload(f"m{m}_n{n}_k{k}_int{bits}_g{group}", m, n, k, bits, group, copies=4 if n * k <= 8192 * 8192 else 2)
+        ws = w.workspace(af)
+        af.gemm(w.c, w.a, w.b[0], w.s, m, n, k, weight_bits=bits, group_size=group, workspace=ws)  # (first call outside capture)
+        torch.cuda.synchronize()
+        r = sustained_power(lambda i: af.gemm(w.c, w.a, w.b[i], w.s, m, n, k, weight_bits=bits, group_size=group, workspace=ws), len(w.b))
+        pl = af.plan(m, n, k, bits, group)
+        rows.append({"m": m, "n": n, "k": k, "weight_bits": bits, "group_size": group, "kernel": pl.kernel, "workgroups": pl.workgroups,
+                     "splits": pl.splits, "TFLOP/s": round(w.flops / r["kernel_us_after_settling"] / 1e6, 1), **r})
+        del w, ws
+        torch.cuda.empty_cache()
+    operands = []
+    m = n = k = 4096
+    for name in ("uniform codes, N(0,1) activations", "codes of N(0, 127/4) weights (absmax quantisation)", "codes of N(0, 127/8) weights",
+                 "all codes zero", "all activations zero"):
+        torch.manual_seed(1)
+        a = torch.randn((m, k), device="cuda").to(torch.bfloat16)
+        if name.startswith("codes of N(0, 127/4)"):
+            q = torch.clamp(torch.round(torch.randn((k, n), device="cuda") * (127 / 4)), -128, 127)
+        elif name.startswith("codes of N(0, 127/8)"):
+            q = torch.clamp(torch.round(torch.randn((k, n), device="cuda") * (127 / 8)), -128, 127)
+        elif name == "all codes zero":
+            q = torch.zeros((k, n), device="cuda")
+        else:
+            q = torch.randint(-128, 128, (k, n), device="cuda")
+        if name == "all activations zero":
+            a.zero_()
+        bs = [(q + 128).to(torch.uint8).contiguous() for _ in range(2)]
+        sc = (torch.rand((1, n), device="cuda") * 0.009 + 0.001).to(torch.bfloat16)
+        c = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        ev, _, _ = time_launches(lambda i: af.gemm(c, a, bs[i % 2], sc, m, n, k), 2, 50, 10)
+        operands.append({"operands": name, "kernel_us": round(ev * 1e3, 2), "frac_of_2.5_PFLOP/s": round(2.0 * m * n * k / (ev * 1e-3) / 2.5e15, 4)})
+        del a, bs, c
+        torch.cuda.empty_cache()
+    return {"sustained": rows, "config4_by_operands": operands}
+
+
 def decode_timeline(af, shapes=((1, 4096, 4096), (1, 11008, 4096), (32, 11008, 4096))):
     """Needs a library built with -DBFAINTB_TRACE (--lib): the decode kernel's waves then write 100 MHz time stamps behind
     the split-K area of the workspace — entry, last step multiplied, workgroup's sums ready, producer's stores issued,
@@ -590,7 +641,8 @@ def main():
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
                     "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | plan_check (the library's plans "
-                    "against forced alternatives) | prefill_trace, decode_timeline (both need --lib with a library built with -DBFAINTB_TRACE)")
+                    "against forced alternatives) | power_scan (board power by shape; config 4 by operand values) | prefill_trace, decode_timeline "
+                    "(both need --lib with a library built with -DBFAINTB_TRACE)")
     ap.add_argument("--lib", default="", help="load this build of libbfaintb_gemm.so instead of the package's own "
                     "(an instrumented build, for --only prefill_trace)")
     args = ap.parse_args()
@@ -619,6 +671,9 @@ def main():
     if args.only == "decode_timeline":
         print(json.dumps({"metric": "bfAintBGemm decode kernel: time stamps of one cold launch (instrumented build)", "library": af.library_path(),
                           "rows": decode_timeline(af)}))
+        return
+    if args.only == "power_scan":
+        print(json.dumps({"metric": "bfAintBGemm: board power under sustained launches, and config 4 by operand values", **power_scan(af)}))
         return
     if args.only == "prefill_trace":
         print(json.dumps({"metric": "bfAintBGemm 256x256-tile kernel: K-loop cycles per step and shader clock by tile count (instrumented build)",
