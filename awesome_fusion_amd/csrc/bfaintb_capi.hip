@@ -333,6 +333,19 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
 
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
 {
+    // 4-bit codes in rows also have a 128-column form (a lane loads 4 bytes of a row, 16 lanes half a cache line): twice the
+    // column blocks, so half the splits for the same number of workgroups, and 8 waves from one row on.  It takes the launch
+    // shape 8-bit codes of the same n x k would get — measured against the 256-column plan over 15 weight shapes x 10
+    // values of m.  It wins wherever the weights are few: up to 8 MiB of codes every m gains (1024 x 8192: 9.4 -> 8.0 us at
+    // m = 1, 13.7 -> 9.4 at 16, 18.4 -> 10.0 at 48; 256 x 7168: 16.3 -> 9.5 at 64; 4096 x 4096: 8.0 -> 7.8, 10.7 -> 8.8,
+    // 15.3 -> 12.3 at m = 1, 16, 64); and from 17 rows on up to 40 MiB (11008 x 4096, m = 24 / 32: 18.8 / 19.5 -> 15.4 / 16.5;
+    // 4096 x 11008, m = 24 .. 128: 9 - 17 %; 5120 x 13824, m = 24 / 32: 24.2 / 24.4 -> 20.6 / 21.9; 8192 x 8192: 1 - 7 %).  Few
+    // rows against many weights stream better in whole lines (8192 x 8192, m = 1 .. 16: 15 - 30 % slower; 32000 x 4096: 25 - 32 %;
+    // 28672 x 8192: 2 - 17 %), and so do packed weights, whose kernels are built for 256 columns.
+    if (bits == 4 && !packed) {
+        const uint64_t code_bytes = (uint64_t)n * k / 2u;
+        if (code_bytes <= (8ull << 20) || (m > 16u && code_bytes <= (40ull << 20))) return decode_plan(m, n, k, 8, forced_splits, false);
+    }
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built
     // for 4 waves): the two 16-row blocks run 8 waves each (m = 32, 1024 x 4096: 10.5 against 13.7 us, 17 rows: 10.6 / 17.2; 2048 x 8192:

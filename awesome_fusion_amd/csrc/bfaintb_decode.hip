@@ -12,7 +12,8 @@
 //   Within a wave, lane = (kg, nl) with nl = lane%16, kg = lane/16.  Per step the lane loads, from
 //   each of the 8 rows k0 + 8*kg + r, the CPL consecutive weights of columns n0 + CPL*nl .. +CPL-1
 //   (128-bit or 64-bit loads): a wave request covers 4 rows x 16 lanes of contiguous bytes, whole
-//   128-byte lines or more.  Nothing of B goes through LDS.
+//   128-byte lines or more — except 4-bit codes in the 128-column shape (32-bit loads, half a line per row), which the
+//   host picks where the weights are few and workgroups count for more than whole lines.  Nothing of B goes through LDS.
 //   The products run on v_mfma_f32_16x16x32_bf16 with the operands swapped (C^T = W^T A^T): for
 //   c = 0..CPL-1 the dequantised weights of column CPL*nl + c, rows 8*kg..8*kg+7, are exactly the
 //   8-element operand of lane (nl, kg); the activations A[mi][k0 + 8*kg .. +7] of row mi = lane%16
@@ -30,7 +31,7 @@ namespace bfaintb {
 
 template <int BITS, int CPL>
 struct RawStep {
-    static constexpr int kDwords = CPL * BITS / 32;  // 4 or 2
+    static constexpr int kDwords = CPL * BITS / 32;  // 4, 2 or 1
     uint32_t d[8][kDwords];  // 8 rows x CPL codes
 };
 
@@ -61,9 +62,11 @@ __device__ __forceinline__ void load_raw(RawStep<BITS, CPL>& raw, const uint8_t*
         if constexpr (RawStep<BITS, CPL>::kDwords == 4) {
             const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(src));
             raw.d[r][0] = v[0]; raw.d[r][1] = v[1]; raw.d[r][2] = v[2]; raw.d[r][3] = v[3];
-        } else {
+        } else if constexpr (RawStep<BITS, CPL>::kDwords == 2) {
             const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(src));
             raw.d[r][0] = v[0]; raw.d[r][1] = v[1];
+        } else {
+            raw.d[r][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(src));
         }
     }
 }
@@ -76,9 +79,8 @@ __device__ __forceinline__ void prepare_row(uint32_t (&out)[CPL / 4], const uint
 #pragma unroll
         for (int i = 0; i < CPL / 4; ++i) out[i] = codes8_to_s8(in[i]);
     } else {
-        static_assert(BITS == 8 || CPL == 16, "4-bit codes: 16 columns per lane");
         codes4_to_nibbles(in[0], out[0], out[1]);
-        codes4_to_nibbles(in[1], out[2], out[3]);
+        if constexpr (CPL == 16) codes4_to_nibbles(in[1], out[2], out[3]);
     }
 }
 
@@ -524,7 +526,7 @@ bfaintb_decode_kernel(const GemmParams p)
         }
     }
     const uint32_t kblock0 = kb / 32u;  // first K-block of this wave
-    static_assert(kLaneBytes == 16 || kLaneBytes == 8, "lane loads 16 or 8 bytes of a row");
+    static_assert(kLaneBytes == 16 || kLaneBytes == 8 || (kLaneBytes == 4 && !PACKED), "lane loads 16, 8 or (4-bit codes, 128 columns) 4 bytes of a row");
 
     // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg.
     // Lanes whose row is past the last one re-read the last one; their accumulator columns are never stored.
@@ -862,7 +864,7 @@ hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)
         return p.decode_cols == 128u ? launch_decode_ref<8>(p, stream) : launch_decode_ref<16>(p, stream);
     }
     if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8, false>(p, stream) : launch_decode_b<8, 16, false>(p, stream);
-    return launch_decode_b<4, 16, false>(p, stream);
+    return p.decode_cols == 128u ? launch_decode_b<4, 8, false>(p, stream) : launch_decode_b<4, 16, false>(p, stream);
 }
 
 // The same family over weights in the packed order (p.b = the packed buffer): the shapes the plan uses beyond 32 rows of A,

@@ -245,7 +245,10 @@ def test_prepacked_entry_points_validate_before_launching():
     assert rcp(which=9) == -7
     assert rcp(m=0) == 0
     assert af.prepacked_workspace_bytes(1, 4096, 4096) == 0 and af.prepacked_workspace_bytes(4096, 4096, 4096) == 0
-    assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) == af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
+    # (4-bit codes: packed weights keep the 256-column plan, row-major ones of so small a matrix run 128 columns per workgroup)
+    assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) > 0 and af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
+    assert af.plan(64, 256, 4096, 4, 128, which=af.DECODE).tile_cols == 128 and af.plan(64, 256, 4096, 4, 128, packed=True, which=af.DECODE).tile_cols == 256
+    assert af.plan(1, 28672, 8192, 4, 128).tile_cols == 256 and af.plan(24, 11008, 4096, 4, 128).tile_cols == 128
     # the small tiles split k over packed weights as over row-major ones: same plan, same scratch
     assert af.prepacked_variant(384, 2048, 8192, 4, 128) == af.PREFILL
     assert af.prepacked_workspace_bytes(384, 2048, 8192, 4, 128) == af.workspace_bytes(384, 2048, 8192, 4, 128, af.PREFILL) > 0
@@ -255,7 +258,7 @@ def test_prepacked_entry_points_validate_before_launching():
     # 48 .. 64 rows of 4-bit codes against many columns: the small tiles (54.5 against 74.5 us measured at 64 x 28672 x 8192),
     # in either weight order; the row-blocked family where it is the faster one
     assert af.prepacked_variant(64, 28672, 8192, 4, 128) == af.PREFILL == af.variant(64, 28672, 8192, 4, 128)
-    assert af.variant(64, 4096, 4096) == af.DECODE and af.variant(192, 4096, 4096, 4, 128) == af.PREFILL
+    assert af.variant(64, 4096, 4096) == af.DECODE and af.variant(192, 4096, 4096, 4, 128) == af.DECODE and af.variant(512, 4096, 4096, 4, 128) == af.PREFILL
     assert af.prepacked_variant(4096, 4096, 4096) == af.PREFILL
     assert af.prepacked_variant(1, 4096, 4160, 4, 0) == -2
     assert L.bfaintb_gemm_prepacked_variant(1, 100, 4096, 8, 0) == -2
