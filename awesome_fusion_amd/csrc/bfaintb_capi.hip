@@ -68,7 +68,6 @@ uint32_t machine_cus()
 uint32_t decode_target_wgs_narrow() { return machine_cus(); }
 uint32_t decode_target_wgs() { return machine_cus() * 15u / 8u; }
 constexpr uint32_t kMaxSplits = 64;
-constexpr uint32_t kPackedSlabMaxM = 48;       // packed weights: the slab-streaming kernel never runs more rows of A than this
 
 int check_format(uint32_t k, int bits, uint32_t group_size)
 {
@@ -925,20 +924,27 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
 // (48: 15.6 / 13.6), but 5120 x 5120 14.0 / 10.5, 15.9 / 10.7, 22.8 / 15.8; 32000 x 4096 35.3 / 25.7, 38.3 / 25.1,
 // 63.2 / 35.1; 8192 x 8192 22.5 / 21.4, 22.6 / 21.3, 33.6 / 29.4: beyond 8 rows only the matrix whose 256 slabs make
 // exactly one round of workgroups keeps the slab kernel.
-// 4-bit codes: 48 rows up to 24 Mi weights (4096 x 4096, m = 16: 6.5 us, the family 9 and more), 24 below 64 Mi (4096 x
-// 11008: m = 20: 20.8 / 23.6, 24: 22.3 / 23.5), 16 at 64 Mi (8192 x 8192: m = 20: 26.5 / 25.9), 8 beyond (32000 x 4096:
-// m = 12: 28.0 / 26.4; 28672 x 8192: m = 12: 44.5 / 39.9).
+// 4-bit codes: see the rule itself.
 static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
 {
     const uint64_t weights = (uint64_t)n * k;
     // 8-bit codes, a narrow matrix with long columns: n/16 workgroups that each walk all of k alone take 0.75 us per 1024
     // rows whatever n is; the family splits k instead (1024 x 16384, m = 1: 12.7 us the slab kernel, 10.2 the split)
     if (bits == 8 && n < 2048u && k >= 12288u) return 0u;
-    // 4-bit codes in that corner: up to 20 rows (1024 x 16384, slab / family: m = 17: 22.4 / 24.5 us, 24: 31.4 / 24.8,
-    // 32: 35.8 / 25.1; 512 x 12288, m = 24: 22.4 / 21.5; with k = 8192 the slab kernel stays ahead up to its 48 rows)
-    if (bits == 4 && n < 2048u && k >= 12288u) return 20u;
     if (bits == 8) return (weights <= (16ull << 20) && n / 16u >= machine_cus()) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
-    return weights <= (24ull << 20) ? kPackedSlabMaxM : weights < (64ull << 20) ? 24u : weights == (64ull << 20) ? 16u : 8u;
+    // 4-bit codes, against the family in its 128-column form (slab / family, us).  Few slabs (n below 2048): the family
+    // from 12 rows on, from 8 with long columns (1024 x 8192, m = 8 / 12 / 16 / 24 / 48: 7.3 / 7.2, 8.8 / 7.7, 10.2 / 7.8,
+    // 16.1 / 8.1, 18.0 / 9.4; 256 x 7168, m = 16 / 32: 8.9 / 7.2, 15.4 / 7.4; 1536 x 8960, m = 8 / 16: 8.9 / 9.4, 11.4 / 9.9;
+    // 1024 x 16384, m = 8 / 16: 13.8 / 9.8, 18.4 / 10.5).  Up to 8 MiB of codes: 20 rows where the slabs make a whole round
+    // of workgroups (4096 x 4096, m = 16 / 20 / 24 / 32 / 48: 5.9 / 7.3, 8.6 / 8.8, 9.1 / 8.7, 10.4 / 9.0, 14.9 / 11.1), 16
+    // otherwise (2048 x 4096, m = 16 / 20 / 32: 5.4 / 6.7, 7.9 / 6.8, 10.1 / 7.1).  Up to 40 MiB, where the family has that
+    // form from 17 rows on: 16 (4096 x 11008, m = 16 / 20 / 24: 13.5 / 21.7, 20.0 / 14.7, 21.4 / 14.9; 11008 x 4096: 13.5 /
+    // 16.4, 19.3 / 14.5, 21.3 / 14.7; 5120 x 5120, m = 20: 16.3 / 11.1; 8192 x 8192, m = 16 / 20: 18.3 / 19.9, 26.1 / 16.3).
+    // Beyond: 8 (32000 x 4096, m = 12: 28.0 / 26.4; 28672 x 8192, m = 12: 44.5 / 39.9).
+    const uint64_t code_bytes = weights / 2u;
+    if (n < 2048u) return k >= 12288u ? 4u : 8u;
+    if (code_bytes <= (8ull << 20)) return n / 16u >= machine_cus() ? 20u : 16u;
+    return code_bytes <= (40ull << 20) ? 16u : 8u;
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
@@ -953,6 +959,17 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
     if (bits == 8) {
         const DecodePlan pl = decode_plan(m, n, k, bits, 0, true);
         if (pl.cols == 128u) return pl;
+    }
+    // 4-bit codes: where row-major weights run the 128-column form (see decode_plan), so do packed ones — 8 column blocks
+    // of 16 per workgroup, 8 waves — with the launch shape 8-bit codes would get (1024 x 8192, m = 64 / 128: 18.3 / 17.5 ->
+    // 8.9 / 11.4 us; 4096 x 4096: 15.7 / 20.7 -> 10.6 / 14.9; 256 x 7168, m = 64: 17.3 -> 7.4; 8192 x 8192, m = 24 / 32: 24.3 /
+    // 24.1 -> 16.8 / 18.0; 11008 x 4096, m = 32: 20.8 -> 15.9)
+    if (bits == 4) {
+        const uint64_t code_bytes = (uint64_t)n * k / 2u;
+        if (code_bytes <= (8ull << 20) || (m > 16u && code_bytes <= (40ull << 20))) {
+            const DecodePlan pl = decode_plan(m, n, k, 8, 0, true);
+            if (pl.cols == 128u) return pl;
+        }
     }
     return decode_plan_row_blocks(m, n, k, bits, 0, true);
 }
@@ -970,7 +987,7 @@ static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 {
     FamilyEstimate e;
     const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
-    if (bits == 4) return 0.84 * ranked;
+    if (bits == 4) return (pl.cols == 128u ? 0.74 : 0.84) * ranked;  // (the 128-column form measures 0.52 - 0.79 of its estimate)
     return (pl.mb == 4u ? 0.84 : 0.76) * (5.0 + e.core + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
 }
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the

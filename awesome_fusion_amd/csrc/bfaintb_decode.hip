@@ -461,7 +461,7 @@ __device__ __forceinline__ void reduce_splits_two_in_flight(const GemmParams& p,
 template <int BITS, int CPL, int MB, bool GROUPED, bool PACKED, bool REF>
 // (packed 4-bit codes always run 4 waves: with 8 — their registers would allow it for one block of 16 rows — the 256-column
 // kernel over packed weights is slower, 28672 x 8192, m = 16: 55 against 42 us)
-__global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED && BITS == 4)) ? 512 : 256)
+__global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED && BITS == 4 && CPL == 16)) ? 512 : 256)
 bfaintb_decode_kernel(const GemmParams p)
 {
     static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
@@ -526,7 +526,7 @@ bfaintb_decode_kernel(const GemmParams p)
         }
     }
     const uint32_t kblock0 = kb / 32u;  // first K-block of this wave
-    static_assert(kLaneBytes == 16 || kLaneBytes == 8 || (kLaneBytes == 4 && !PACKED), "lane loads 16, 8 or (4-bit codes, 128 columns) 4 bytes of a row");
+    static_assert(kLaneBytes == 16 || kLaneBytes == 8 || kLaneBytes == 4, "row-major weights: a lane loads 16, 8 or (4-bit codes, 128 columns) 4 bytes of a row");
 
     // activation operand: row mi = 16*mb + lane%16, 8 consecutive k starting at k0 + 8*kg.
     // Lanes whose row is past the last one re-read the last one; their accumulator columns are never stored.
@@ -812,7 +812,7 @@ static hipError_t launch_decode_t(const GemmParams& p, hipStream_t stream)
     constexpr uint32_t kCols = 16u * CPL;
     constexpr uint32_t kRows = 16u * MB;
     const uint32_t waves = p.decode_waves;
-    if ((MB > 2 || (PACKED && BITS == 4)) && waves != 4u) return hipErrorInvalidValue;  // kernels compiled for 256 threads
+    if ((MB > 2 || (PACKED && BITS == 4 && CPL == 16)) && waves != 4u) return hipErrorInvalidValue;  // kernels compiled for 256 threads
     const dim3 grid((p.n + kCols - 1u) / kCols, p.splits, (p.m + kRows - 1u) / kRows);
     if (grid.z > 65535u) return hipErrorInvalidValue;
     const uint32_t pass_rows = 16u * (uint32_t)decode_rows16_per_pass(CPL, MB);
@@ -872,7 +872,7 @@ hipError_t launch_decode(const GemmParams& p, int bits, hipStream_t stream)
 hipError_t launch_decode_family_packed(const GemmParams& p, int bits, hipStream_t stream)
 {
     if (bits == 8) return p.decode_cols == 128u ? launch_decode_b<8, 8, true>(p, stream) : hipErrorInvalidValue;
-    return launch_decode_b<4, 16, true>(p, stream);
+    return p.decode_cols == 128u ? launch_decode_b<4, 8, true>(p, stream) : launch_decode_b<4, 16, true>(p, stream);
 }
 
 // Allows every kernel of the family its largest dynamic LDS size on the current device.  Runs once per device, from the

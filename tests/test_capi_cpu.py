@@ -245,9 +245,10 @@ def test_prepacked_entry_points_validate_before_launching():
     assert rcp(which=9) == -7
     assert rcp(m=0) == 0
     assert af.prepacked_workspace_bytes(1, 4096, 4096) == 0 and af.prepacked_workspace_bytes(4096, 4096, 4096) == 0
-    # (4-bit codes: packed weights keep the 256-column plan, row-major ones of so small a matrix run 128 columns per workgroup)
-    assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) > 0 and af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
-    assert af.plan(64, 256, 4096, 4, 128, which=af.DECODE).tile_cols == 128 and af.plan(64, 256, 4096, 4, 128, packed=True, which=af.DECODE).tile_cols == 256
+    # (4-bit codes of so small a matrix run 128 columns per workgroup in either weight order: the same plan again)
+    assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) == af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
+    assert af.plan(64, 256, 4096, 4, 128, which=af.DECODE).tile_cols == 128 == af.plan(64, 256, 4096, 4, 128, packed=True, which=af.DECODE).tile_cols
+    assert af.plan(12, 28672, 8192, 4, 128, packed=True, which=af.DECODE).tile_cols == 256   # many weights: whole lines
     assert af.plan(1, 28672, 8192, 4, 128).tile_cols == 256 and af.plan(24, 11008, 4096, 4, 128).tile_cols == 128
     # the small tiles split k over packed weights as over row-major ones: same plan, same scratch
     assert af.prepacked_variant(384, 2048, 8192, 4, 128) == af.PREFILL
