@@ -330,7 +330,8 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
     return best;
 }
 
-DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false)
+// nibbles: the plan is for 4-bit codes in the 128-column form, which takes the launch shapes of 8-bit codes (bits == 8 here)
+DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false, bool nibbles = false)
 {
     // 4-bit codes in rows also have a 128-column form (a lane loads 4 bytes of a row, 16 lanes half a cache line): twice the
     // column blocks, so half the splits for the same number of workgroups, and 8 waves from one row on.  It takes the launch
@@ -343,7 +344,7 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
     // 28672 x 8192: 2 - 17 %), and so do packed weights, whose kernels are built for 256 columns.
     if (bits == 4 && !packed) {
         const uint64_t code_bytes = (uint64_t)n * k / 2u;
-        if (code_bytes <= (8ull << 20) || (m > 16u && code_bytes <= (40ull << 20))) return decode_plan(m, n, k, 8, forced_splits, false);
+        if (code_bytes <= (8ull << 20) || (m > 16u && code_bytes <= (40ull << 20))) return decode_plan(m, n, k, 8, forced_splits, false, true);
     }
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built
@@ -388,6 +389,20 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         double best = 0.0;
         const uint32_t cus = machine_cus();
         for (uint32_t s = 1; s <= cap && s <= 16u; ++s) {
+            // (only the factors k divides into: another one would be rounded to its neighbour, whose workgroups may fill
+            // the rounds far worse — 4-bit codes, 11008 x 8192: 5 splits, 430 workgroups, would have become 4 and 344:
+            // 24.3 us at m = 16 against 22.0 with 2 splits)
+            DecodePlan probe{};
+            probe.cols = 128u;
+            probe.waves = 8u;
+            set_splits(probe, k, bits, s, packed);
+            if (probe.splits != s) continue;
+            // 4-bit codes in this form: one round of workgroups at most.  Measured over packed weights at m = 4 / 16 / 32,
+            // best factor within a round against the best beyond: 12288 x 12288 2 splits 26.3 / 28.3 / 33.8 us, 5 splits
+            // 28.8 / 30.6 / 36.2; 22016 x 4096 1 split 20.2 / 21.6 / 24.4, 4 splits 21.1 / 22.5 / 28.0; 14336 x 8192 2 splits
+            // 21.1 / 23.7 / 27.1, 4 splits 23.6 / 25.9 / 30.9; only 16384 x 8192 likes two rounds (4 splits 26.1 / 27.4 / 32.3
+            // against 2 splits 29.2 / 29.9 / 32.4)
+            if (nibbles && s > 1u && narrow_blocks * s > cus) break;
             const double rounds = (double)((narrow_blocks * s + cus - 1u) / cus);
             const double g = rounds / s + 0.04 * s * 4096.0 / k;  // time of the rounds + what a split costs, both relative to one pass over k
             if (best == 0.0 || g < best) { best = g; narrow_splits = s; }
@@ -401,7 +416,9 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         // 11008 x 4096 13.9 / 14.9 / 17.9 against 13.8 / 16.5 / 22.1; 14336 x 4096 17.2 / 18.5 / 21.4 against 17.6 / 19.0 / 25.1)
         const bool many_wide_blocks = (n + 255u) / 256u > cus / 4u;
         // (n not a multiple of 16: only the 8-codes-per-lane shape can read the last columns)
-        const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 || (m >= 8 && (!many_wide_blocks || packed)));  // packed weights: the kernels are built for 128 columns
+        // (packed weights: the kernels are built for 128 columns; packed 4-bit codes: the 256-column form, 4 waves, is at
+        // best 6 % ahead — 16384 x 8192 and 32000 x 4096 up to 16 rows — and up to 30 % behind)
+        const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 || (m >= 8 && (!many_wide_blocks || packed)) || (nibbles && packed));
         pl.cols = narrow ? 128u : 256u;
         // 4-bit codes, 8 to 16 rows: the same 256 columns with 8 waves (twice the waves to hide the activation loads and
         // the matrix instructions behind; n = k = 4096, m = 16: 11.6 against 14.7 us, 1024 x 8192: 14.1 / 17.4,
@@ -932,23 +949,46 @@ static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
     // rows whatever n is; the family splits k instead (1024 x 16384, m = 1: 12.7 us the slab kernel, 10.2 the split)
     if (bits == 8 && n < 2048u && k >= 12288u) return 0u;
     if (bits == 8) return (weights <= (16ull << 20) && n / 16u >= machine_cus()) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
-    // 4-bit codes, against the family in its 128-column form (slab / family, us).  Few slabs (n below 2048): the family
-    // from 12 rows on, from 8 with long columns (1024 x 8192, m = 8 / 12 / 16 / 24 / 48: 7.3 / 7.2, 8.8 / 7.7, 10.2 / 7.8,
-    // 16.1 / 8.1, 18.0 / 9.4; 256 x 7168, m = 16 / 32: 8.9 / 7.2, 15.4 / 7.4; 1536 x 8960, m = 8 / 16: 8.9 / 9.4, 11.4 / 9.9;
-    // 1024 x 16384, m = 8 / 16: 13.8 / 9.8, 18.4 / 10.5).  Up to 8 MiB of codes: 20 rows where the slabs make a whole round
-    // of workgroups (4096 x 4096, m = 16 / 20 / 24 / 32 / 48: 5.9 / 7.3, 8.6 / 8.8, 9.1 / 8.7, 10.4 / 9.0, 14.9 / 11.1), 16
-    // otherwise (2048 x 4096, m = 16 / 20 / 32: 5.4 / 6.7, 7.9 / 6.8, 10.1 / 7.1).  Up to 40 MiB, where the family has that
-    // form from 17 rows on: 16 (4096 x 11008, m = 16 / 20 / 24: 13.5 / 21.7, 20.0 / 14.7, 21.4 / 14.9; 11008 x 4096: 13.5 /
-    // 16.4, 19.3 / 14.5, 21.3 / 14.7; 5120 x 5120, m = 20: 16.3 / 11.1; 8192 x 8192, m = 16 / 20: 18.3 / 19.9, 26.1 / 16.3).
-    // Beyond: 8 (32000 x 4096, m = 12: 28.0 / 26.4; 28672 x 8192, m = 12: 44.5 / 39.9).
-    const uint64_t code_bytes = weights / 2u;
-    if (n < 2048u) return k >= 12288u ? 4u : 8u;
-    if (code_bytes <= (8ull << 20)) return n / 16u >= machine_cus() ? 20u : 16u;
-    return code_bytes <= (40ull << 20) ? 16u : 8u;
+    return 0u;  // 4-bit codes: packed_uses_slab compares the two kernels' times
+}
+
+static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bits);
+
+// 4-bit codes: the slab kernel against the family's 128-column form, by what each was measured to take (28 weight shapes
+// from 256 x 7168 to 28672 x 8192, m = 1 .. 32, us).
+// The slab kernel is bound by its CUs' vector arithmetic: a workgroup walks its 16 columns at 2040 rows per us, two
+// workgroups that share a CU at half that each, so a launch takes as many such walks as the fullest CU has slabs —
+// n / 16 over 256 CUs, rounded up (5120 x 5120, 320 slabs: 7.3 us, the same as 8192 x 5120 would take; 4096 x 4096: 3.5) —
+// and each further row of A costs 3.6 % of the walk up to 6 rows, 8 % from there (two blocks of 16 rows from m = 17: 2.6
+// to 3.8 walks) — a least-squares fit, 7 % rms.
+// The family's 128-column form streams at about 3.5 TB/s with every CU busy, pays the split's hand-over, and hardly
+// grows with m up to 16 rows (15 % more from 17).
+// Where the two are close either choice is within a few per cent; where they are not the gap is up to 80 % (5120 x 13824,
+// m = 16: slab 31.0, family 17.2; 13824 x 5120: 26.0 / 15.5; 4096 x 2048, m = 32: 5.5 / 6.9; 1024 x 16384, m = 1: 10.5 / 9.0).
+static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
+{
+    const double cus = (double)machine_cus();
+    const double slabs = n / 16.0;
+    const double walks = slabs <= 4.0 * cus ? (double)(uint64_t)((slabs + cus - 1.0) / cus) : slabs / cus;
+    const double rows = m <= 6u ? 1.0 + 0.036 * (m - 1.0) : m <= 16u ? 1.18 + 0.082 * (m - 6.0) : 1.34 + 0.077 * m;
+    return 2.1 + walks * k / 2040.0 * rows;
+}
+static double packed4_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
+{
+    const double cus = (double)machine_cus();
+    const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits * ((m + 16u * pl.mb - 1u) / (16u * pl.mb));
+    const double rounds = (double)(uint64_t)((wgs + cus - 1.0) / cus);
+    const double fill = wgs / (rounds * cus);
+    const double mbytes = (double)n * k / 2.0e6;
+    return 3.5 + 0.073 * m + 0.11 * (pl.splits - 1.0) + mbytes / (3.38 * pow(fill, 0.62)) * (1.0 + 0.0013 * m + (m > 16u ? 0.148 : 0.0));
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
-    return m <= packed_slab_max_m(n, k, bits);
+    if (bits == 8) return m <= packed_slab_max_m(n, k, bits);
+    if (m > kDecodeAutoMaxM) return false;
+    const DecodePlan pl = packed_family_plan(m, n, k, bits);
+    if (pl.cols != 128u) return m <= 8u;
+    return packed4_slab_time_us(m, n, k) <= packed4_family_time_us(m, n, k, pl);
 }
 
 // The family's plan over packed weights.  8-bit codes: the one row-major weights get, as long as it uses the 128 columns
@@ -960,16 +1000,15 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
         const DecodePlan pl = decode_plan(m, n, k, bits, 0, true);
         if (pl.cols == 128u) return pl;
     }
-    // 4-bit codes: where row-major weights run the 128-column form (see decode_plan), so do packed ones — 8 column blocks
-    // of 16 per workgroup, 8 waves — with the launch shape 8-bit codes would get (1024 x 8192, m = 64 / 128: 18.3 / 17.5 ->
-    // 8.9 / 11.4 us; 4096 x 4096: 15.7 / 20.7 -> 10.6 / 14.9; 256 x 7168, m = 64: 17.3 -> 7.4; 8192 x 8192, m = 24 / 32: 24.3 /
-    // 24.1 -> 16.8 / 18.0; 11008 x 4096, m = 32: 20.8 -> 15.9)
+    // 4-bit codes: the 128-column form (8 column blocks of 16 per workgroup, 8 waves) with the launch shape 8-bit codes
+    // would get, wherever that shape has 128 columns.  Against the 256-column form, whose kernels over packed 4-bit codes
+    // run 4 waves (us, 128 / 256 columns): 1024 x 8192, m = 64 / 128: 8.9 / 18.3, 11.4 / 17.5; 4096 x 4096: 10.6 / 15.7,
+    // 14.9 / 20.7; 8192 x 8192, m = 16 / 32: 15.5 / 19.9, 18.3 / 24.1; 28672 x 8192, m = 12 / 32 / 48: 37.0 / 49.4, 42.3 / 47.1,
+    // 52.0 / 70.6; 8192 x 28672: 37.0 / 41.4, 43.9 / 50.3, 52.8 / 68.5; 8192 x 11008, m = 16 / 64: 19.0 / 23.9, 30.5 / 36.2; the
+    // other way round at most 6 % (16384 x 8192, m = 12: 29.5 / 27.8; 32000 x 4096: 27.6 / 26.3).
     if (bits == 4) {
-        const uint64_t code_bytes = (uint64_t)n * k / 2u;
-        if (code_bytes <= (8ull << 20) || (m > 16u && code_bytes <= (40ull << 20))) {
-            const DecodePlan pl = decode_plan(m, n, k, 8, 0, true);
-            if (pl.cols == 128u) return pl;
-        }
+        const DecodePlan pl = decode_plan(m, n, k, 8, 0, true, true);
+        if (pl.cols == 128u) return pl;
     }
     return decode_plan_row_blocks(m, n, k, bits, 0, true);
 }
@@ -987,7 +1026,7 @@ static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 {
     FamilyEstimate e;
     const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
-    if (bits == 4) return (pl.cols == 128u ? 0.74 : 0.84) * ranked;  // (the 128-column form measures 0.52 - 0.79 of its estimate)
+    if (bits == 4) return (pl.cols == 128u ? 0.70 : 0.84) * ranked;  // (the 128-column form measures 0.52 - 0.79 of its estimate)
     return (pl.mb == 4u ? 0.84 : 0.76) * (5.0 + e.core + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
 }
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the

@@ -248,7 +248,11 @@ def test_prepacked_entry_points_validate_before_launching():
     # (4-bit codes of so small a matrix run 128 columns per workgroup in either weight order: the same plan again)
     assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) == af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
     assert af.plan(64, 256, 4096, 4, 128, which=af.DECODE).tile_cols == 128 == af.plan(64, 256, 4096, 4, 128, packed=True, which=af.DECODE).tile_cols
-    assert af.plan(12, 28672, 8192, 4, 128, packed=True, which=af.DECODE).tile_cols == 256   # many weights: whole lines
+    # packed 4-bit codes up to 32 rows: the slab kernel (16 columns) while the rows are few, then the 128-column form
+    assert af.plan(4, 28672, 8192, 4, 128, packed=True).tile_cols == 16 and af.plan(12, 28672, 8192, 4, 128, packed=True).tile_cols == 128
+    assert af.plan(16, 5120, 13824, 4, 128, packed=True).tile_cols == 128 and af.plan(32, 4096, 2048, 4, 128, packed=True).tile_cols == 16
+    # (one round of workgroups, and only the split factors k divides into)
+    assert af.plan(16, 11008, 8192, 4, 128, packed=True).splits == 2 and af.plan(16, 12288, 12288, 4, 128, packed=True).workgroups == 192
     assert af.plan(1, 28672, 8192, 4, 128).tile_cols == 256 and af.plan(24, 11008, 4096, 4, 128).tile_cols == 128
     # the small tiles split k over packed weights as over row-major ones: same plan, same scratch
     assert af.prepacked_variant(384, 2048, 8192, 4, 128) == af.PREFILL
@@ -256,9 +260,11 @@ def test_prepacked_entry_points_validate_before_launching():
     assert rcp(m=64, n=256, k=4096, weight_bits=4, group_size=128) == -6     # the plan splits along k: workspace required
     assert af.prepacked_variant(1, 4096, 4096) == af.DECODE
     assert af.prepacked_variant(64, 4096, 4096) == af.DECODE
-    # 48 .. 64 rows of 4-bit codes against many columns: the small tiles (54.5 against 74.5 us measured at 64 x 28672 x 8192),
-    # in either weight order; the row-blocked family where it is the faster one
-    assert af.prepacked_variant(64, 28672, 8192, 4, 128) == af.PREFILL == af.variant(64, 28672, 8192, 4, 128)
+    # 48 .. 64 rows of 4-bit codes against many columns: row-major weights run the small tiles (54.5 against 74.5 us measured
+    # at 64 x 28672 x 8192); packed ones have the family's 128-column form at every size, which is level with the tiles
+    # there (54.1 / 53.1 us) and ahead on fewer columns (48 x 11008 x 8192: 30.7 / 33.3); from 96 rows the tiles
+    assert af.variant(64, 28672, 8192, 4, 128) == af.PREFILL and af.prepacked_variant(96, 28672, 8192, 4, 128) == af.PREFILL
+    assert af.prepacked_variant(48, 11008, 8192, 4, 128) == af.DECODE and af.plan(48, 11008, 8192, 4, 128, packed=True).tile_cols == 128
     assert af.variant(64, 4096, 4096) == af.DECODE and af.variant(192, 4096, 4096, 4, 128) == af.DECODE and af.variant(512, 4096, 4096, 4, 128) == af.PREFILL
     assert af.prepacked_variant(4096, 4096, 4096) == af.PREFILL
     assert af.prepacked_variant(1, 4096, 4160, 4, 0) == -2
