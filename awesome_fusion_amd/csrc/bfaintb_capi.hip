@@ -397,12 +397,15 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
             probe.waves = 8u;
             set_splits(probe, k, bits, s, packed);
             if (probe.splits != s) continue;
-            // 4-bit codes in this form: one round of workgroups at most.  Measured over packed weights at m = 4 / 16 / 32,
-            // best factor within a round against the best beyond: 12288 x 12288 2 splits 26.3 / 28.3 / 33.8 us, 5 splits
-            // 28.8 / 30.6 / 36.2; 22016 x 4096 1 split 20.2 / 21.6 / 24.4, 4 splits 21.1 / 22.5 / 28.0; 14336 x 8192 2 splits
-            // 21.1 / 23.7 / 27.1, 4 splits 23.6 / 25.9 / 30.9; only 16384 x 8192 likes two rounds (4 splits 26.1 / 27.4 / 32.3
-            // against 2 splits 29.2 / 29.9 / 32.4)
-            if (nibbles && s > 1u && narrow_blocks * s > cus) break;
+            // Packed weights, and 4-bit codes in this form: one round of workgroups at most.  Measured over packed weights,
+            // best factor within a round against the best beyond, us.  4-bit codes at m = 4 / 16 / 32: 12288 x 12288 2 splits
+            // 26.3 / 28.3 / 33.8, 5 splits 28.8 / 30.6 / 36.2; 22016 x 4096 1 split 20.2 / 21.6 / 24.4, 4 splits 21.1 / 22.5 / 28.0;
+            // 14336 x 8192 2 splits 21.1 / 23.7 / 27.1, 4 splits 23.6 / 25.9 / 30.9; only 16384 x 8192 likes two rounds (4 splits
+            // 26.1 / 27.4 / 32.3 against 2 splits 29.2 / 29.9 / 32.4).  8-bit codes at m = 8 / 16 / 32: 11008 x 8192 2 splits
+            // 20.0 / 21.0 / 24.3, 8 splits 24.5 / 25.3 / 29.9; 22016 x 4096 1 split 18.7 / 19.5 / 22.0, 4 splits 23.3 / 23.9 / 27.9;
+            // 12288 x 12288 2 splits 30.5 / 32.7 / 36.3, 5 splits 30.6 / 31.6 / 36.1.  (8-bit codes in rows are within 7 % of
+            // their best factor as the formula below picks it: 11008 x 8192, m = 8: 5 splits 22.5, 2 splits 21.0.)
+            if ((nibbles || packed) && s > 1u && narrow_blocks * s > cus) break;
             const double rounds = (double)((narrow_blocks * s + cus - 1u) / cus);
             const double g = rounds / s + 0.04 * s * 4096.0 / k;  // time of the rounds + what a split costs, both relative to one pass over k
             if (best == 0.0 || g < best) { best = g; narrow_splits = s; }
@@ -936,57 +939,64 @@ int bfaintb_prepack_colmajor(void* packed, const void* b, uint32_t n, uint32_t k
 
 // Packed weights, "DECODE": the slab-streaming kernel (one workgroup per 16 columns over all of k, no split, every block
 // of 16 rows of A converts the slab again) or the decode family reading packed slabs (128 or 256 columns per workgroup,
-// split along k).  The slab kernel wins while the rows are few.  Measured, slab / family in us —
-// 8-bit codes: m = 8 is the slab kernel's everywhere; at m = 12, 16, 32: 4096 x 4096 6.2 / 9.0, 6.9 / 9.5, 10.7 / 12.1
-// (48: 15.6 / 13.6), but 5120 x 5120 14.0 / 10.5, 15.9 / 10.7, 22.8 / 15.8; 32000 x 4096 35.3 / 25.7, 38.3 / 25.1,
-// 63.2 / 35.1; 8192 x 8192 22.5 / 21.4, 22.6 / 21.3, 33.6 / 29.4: beyond 8 rows only the matrix whose 256 slabs make
-// exactly one round of workgroups keeps the slab kernel.
-// 4-bit codes: see the rule itself.
-static uint32_t packed_slab_max_m(uint32_t n, uint32_t k, int bits)
-{
-    const uint64_t weights = (uint64_t)n * k;
-    // 8-bit codes, a narrow matrix with long columns: n/16 workgroups that each walk all of k alone take 0.75 us per 1024
-    // rows whatever n is; the family splits k instead (1024 x 16384, m = 1: 12.7 us the slab kernel, 10.2 the split)
-    if (bits == 8 && n < 2048u && k >= 12288u) return 0u;
-    if (bits == 8) return (weights <= (16ull << 20) && n / 16u >= machine_cus()) ? 32u : weights <= (96ull << 20) ? 8u : 4u;
-    return 0u;  // 4-bit codes: packed_uses_slab compares the two kernels' times
-}
-
+// split along k).  The slab kernel wins while the rows are few; how few depends on the shape, so packed_uses_slab
+// compares what each was measured to take.
 static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bits);
 
-// 4-bit codes: the slab kernel against the family's 128-column form, by what each was measured to take (28 weight shapes
-// from 256 x 7168 to 28672 x 8192, m = 1 .. 32, us).
-// The slab kernel is bound by its CUs' vector arithmetic: a workgroup walks its 16 columns at 2040 rows per us, two
-// workgroups that share a CU at half that each, so a launch takes as many such walks as the fullest CU has slabs —
-// n / 16 over 256 CUs, rounded up (5120 x 5120, 320 slabs: 7.3 us, the same as 8192 x 5120 would take; 4096 x 4096: 3.5) —
-// and each further row of A costs 3.6 % of the walk up to 6 rows, 8 % from there (two blocks of 16 rows from m = 17: 2.6
-// to 3.8 walks) — a least-squares fit, 7 % rms.
-// The family's 128-column form streams at about 3.5 TB/s with every CU busy, pays the split's hand-over, and hardly
-// grows with m up to 16 rows (15 % more from 17).
-// Where the two are close either choice is within a few per cent; where they are not the gap is up to 80 % (5120 x 13824,
-// m = 16: slab 31.0, family 17.2; 13824 x 5120: 26.0 / 15.5; 4096 x 2048, m = 32: 5.5 / 6.9; 1024 x 16384, m = 1: 10.5 / 9.0).
-static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
+// The slab kernel against the family, by what each was measured to take: 28 weight shapes from 256 x 7168 to 28672 x 8192,
+// m = 1 .. 32, both code widths; least-squares fits, 7 - 9 % rms (us).
+// The slab kernel: a workgroup walks its 16 columns alone, two workgroups that share a CU at half the pace each, so a
+// launch takes as many walks as the fullest CU has slabs — n / 16 over 256 CUs, rounded up (4-bit codes, 5120 x 5120,
+// 320 slabs: 7.3 us, what 8192 x 5120 would take; 4096 x 4096: 3.5).  4-bit codes are bound by the CUs' vector
+// arithmetic (2040 rows per us and walk); 8-bit codes by that (1544 rows per us) or by memory (6.2 TB/s).  Each
+// further row of A costs 1.4 - 3.6 % of the walk up to 6 rows and 6 - 8 % from there (two blocks of 16 rows from m = 17).
+// The family's 128-column form streams at about 3.4 TB/s (4-bit) or 5.6 TB/s (8-bit) with every CU busy, pays the
+// split's hand-over, and hardly grows with m up to 16 rows (11 - 15 % more from 17).
+// Where the two are close either choice is within a few per cent; where they are not the gap is up to 80 % (4-bit codes,
+// 5120 x 13824, m = 16: slab 31.0, family 17.2; 13824 x 5120: 26.0 / 15.5; 4096 x 2048, m = 32: 5.5 / 6.9; 1024 x 16384,
+// m = 1: 10.5 / 9.0.  8-bit codes, m = 8: 5120 x 13824 23.2 / 16.3; 13824 x 5120 20.2 / 15.0; 5120 x 5120 11.3 / 9.2;
+// 2048 x 4096, m = 12: 5.5 / 6.9).  Picks on the scan: 4-bit 13 of 248 more than 5 % off, 8-bit 13 of 196 (fixed row
+// limits, as before: 22 of 196, up to 42 %).
+static double packed_slab_walks(uint32_t n)
 {
     const double cus = (double)machine_cus();
     const double slabs = n / 16.0;
-    const double walks = slabs <= 4.0 * cus ? (double)(uint64_t)((slabs + cus - 1.0) / cus) : slabs / cus;
-    const double rows = m <= 6u ? 1.0 + 0.036 * (m - 1.0) : m <= 16u ? 1.18 + 0.082 * (m - 6.0) : 1.34 + 0.077 * m;
-    return 2.1 + walks * k / 2040.0 * rows;
+    return slabs <= 4.0 * cus ? (double)(uint64_t)((slabs + cus - 1.0) / cus) : slabs / cus;
 }
-static double packed4_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
+static double packed_family_fill(uint32_t m, uint32_t n, const DecodePlan& pl)
 {
     const double cus = (double)machine_cus();
     const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits * ((m + 16u * pl.mb - 1u) / (16u * pl.mb));
     const double rounds = (double)(uint64_t)((wgs + cus - 1.0) / cus);
-    const double fill = wgs / (rounds * cus);
-    const double mbytes = (double)n * k / 2.0e6;
-    return 3.5 + 0.073 * m + 0.11 * (pl.splits - 1.0) + mbytes / (3.38 * pow(fill, 0.62)) * (1.0 + 0.0013 * m + (m > 16u ? 0.148 : 0.0));
+    return wgs / (rounds * cus);
+}
+static double packed8_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
+{
+    const double walks = packed_slab_walks(n);
+    const double rows = m <= 6u ? 1.0 + 0.0136 * (m - 1.0) : m <= 16u ? 1.068 + 0.0578 * (m - 6.0) : 0.856 + 0.0608 * m;
+    const double walk_us = walks * k / 1544.0, stream_us = (double)n * k / 6.16e6;
+    return 2.07 + 0.017 * m * walks + (walk_us > stream_us ? walk_us : stream_us) * rows;
+}
+static double packed8_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
+{
+    const double stream_us = (double)n * k / 1.0e6 / (5.63 * pow(packed_family_fill(m, n, pl), 0.638));
+    return 3.0 + 0.0885 * m + 0.118 * (pl.splits - 1.0) + stream_us * (1.0 - 0.0037 * m + (m > 16u ? 0.1076 : 0.0)) * (pl.cols == 256u ? 1.1 : 1.0);
+}
+static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
+{
+    const double rows = m <= 6u ? 1.0 + 0.036 * (m - 1.0) : m <= 16u ? 1.18 + 0.082 * (m - 6.0) : 1.34 + 0.077 * m;
+    return 2.1 + packed_slab_walks(n) * k / 2040.0 * rows;
+}
+static double packed4_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
+{
+    const double stream_us = (double)n * k / 2.0e6 / (3.38 * pow(packed_family_fill(m, n, pl), 0.62));
+    return 3.5 + 0.073 * m + 0.11 * (pl.splits - 1.0) + stream_us * (1.0 + 0.0013 * m + (m > 16u ? 0.148 : 0.0));
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
-    if (bits == 8) return m <= packed_slab_max_m(n, k, bits);
     if (m > kDecodeAutoMaxM) return false;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
+    if (bits == 8) return packed8_slab_time_us(m, n, k) <= packed8_family_time_us(m, n, k, pl);
     if (pl.cols != 128u) return m <= 8u;
     return packed4_slab_time_us(m, n, k) <= packed4_family_time_us(m, n, k, pl);
 }
