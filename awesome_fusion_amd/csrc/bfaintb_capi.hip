@@ -93,13 +93,14 @@ std::atomic<uint32_t> g_force_row_block{0};
 // rows of k per workgroup, workgroups along k.
 struct DecodePlan {
     uint32_t cols, waves, mb, k_per_wg, splits;
+    uint32_t unit_bits = 0;  // width of the codes where it is not the `bits` the plan is made with (4-bit codes planned as 8-bit ones)
 };
 
 // Rows of k per workgroup and the number of splits that results, for `splits` wanted.
 static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bool packed = false)
 {
     // rows one workgroup covers per pipeline step of its waves
-    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(bits, (int)pl.cols / 16, packed) * pl.waves;
+    const uint32_t unit = 32u * (uint32_t)bfaintb::decode_blocks_per_step(pl.unit_bits ? (int)pl.unit_bits : bits, (int)pl.cols / 16, packed, (int)pl.mb) * pl.waves;
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
     uint32_t per = (k + splits - 1) / splits;
@@ -276,7 +277,7 @@ static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits)
 // are fixed by the code width here: what the kernels over packed weights need.)  max_mb: the largest row block to
 // consider, in units of 16 rows; wide8: blocks of 16 rows of 4-bit codes run 8 waves instead of 4.
 DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false,
-                                  uint32_t max_mb = 4u, bool wide8 = false)
+                                  uint32_t max_mb = 4u, bool wide8 = false, bool nibbles = false)
 {
     DecodePlan best{};
     double best_t = 0.0;
@@ -284,6 +285,7 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
     for (uint32_t mb = bits == 8 ? max_mb : (max_mb < 2u ? max_mb : 2u); mb >= 1u; mb >>= 1) {
         if (only_mb != 0u && mb != only_mb && only_mb <= (bits == 8 ? max_mb : 2u)) continue;
         DecodePlan c;
+        c.unit_bits = nibbles ? 4u : 0u;
         c.cols = bits == 8 ? 128u : 256u;
         c.waves = ((bits == 8 && mb <= 2u) || (wide8 && mb == 1u)) ? 8u : 4u;  // wide8: 4-bit codes, 256 columns x 8 waves
         c.mb = mb;
@@ -351,24 +353,25 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
     // for 4 waves): the two 16-row blocks run 8 waves each (m = 32, 1024 x 4096: 10.5 against 13.7 us, 17 rows: 10.6 / 17.2; 2048 x 8192:
     // 15.3 / 18.4; 4096 x 4096: 14.3 / 16.6; larger matrices lose: 4096 x 11008: 26.5 / 21.8)
     if (bits == 4 && m > 16 && m <= 32 && forced_splits == 0 && !packed && (weight_bytes <= (8ull << 20) || n <= 2048u))
-        return decode_plan_row_blocks(m, n, k, bits, 0, false, 1u, true);
+        return decode_plan_row_blocks(m, n, k, bits, 0, false, 1u, true, nibbles);
     // 8-bit codes, more than 32 rows, but so few columns that even 16-row blocks make at most 40 workgroups per split: only
     // those (the 32- and 64-row kernels spend longer in their reductions than such a launch has; 768 x 5120, m = 48: 7.5
     // against 10.8 us; 1536 x 8960: 10.8 / 14.3; 256 x 7168, m = 128: 7.8 / 11.7; with more blocks the larger ones win:
     // 2048 x 8192, m = 128: 20.2 / 16.3)
     if (bits == 8 && m > 32 && forced_splits == 0 && (uint64_t)((n + 127u) / 128u) * ((m + 15u) / 16u) <= machine_cus() * 5u / 32u)
-        return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u);
+        return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u, false, nibbles);
     // More than 32 rows of A; 4-bit codes from 17 rows on: three blocks of 16 rows with their own workgroups beat one
     // 32-row block (n = k = 4096, m = 32: 15.8 against 21.4 us; 28672 x 8192, group 128: 46.5 against 53.0 us).
-    if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed);
+    if (m > 32 || (bits == 4 && m > 16)) return decode_plan_row_blocks(m, n, k, bits, forced_splits, packed, 4u, false, nibbles);
     DecodePlan pl;
+    pl.unit_bits = nibbles ? 4u : 0u;
     // 8-bit codes, 17 to 32 rows, a small or narrow matrix: one 32-row block per workgroup cannot fill the machine without
     // splitting k further than it likes; two blocks of 16 rows with their own workgroups (the second stream hits in cache)
     // and the split that fills one round do (m = 32, n x k = 1024 x 4096: 7.0 against 8.9 us; 2048 x 8192: 10.9 against
     // 14.0; 1024 x 16384: 11.7 against 16.3; 4096 x 2048: 7.9 against 9.3; 4096 x 4096: 10.7 against 10.8; beyond 16 MiB
     // at more than 2048 columns the one block wins: 3072 x 8192: 15.4 against 14.4)
     if (bits == 8 && m > 16 && forced_splits == 0 && (weight_bytes <= (16ull << 20) || n <= 2048u))
-        return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u);
+        return decode_plan_row_blocks(m, n, k, bits, 0, packed, 1u, false, nibbles);
     {
         // 8-bit codes, 128 columns x 8 waves ("narrow": a lane loads 8 bytes of a row, 16 lanes one 128-byte line)
         // needs half the splits of 256 columns x 4 waves ("wide") for the same number of waves, so half the
@@ -393,8 +396,10 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
             // the rounds far worse — 4-bit codes, 11008 x 8192: 5 splits, 430 workgroups, would have become 4 and 344:
             // 24.3 us at m = 16 against 22.0 with 2 splits)
             DecodePlan probe{};
+            probe.unit_bits = nibbles ? 4u : 0u;
             probe.cols = 128u;
             probe.waves = 8u;
+            probe.mb = m <= 16 ? 1u : 2u;
             set_splits(probe, k, bits, s, packed);
             if (probe.splits != s) continue;
             // Packed weights, and 4-bit codes in this form: one round of workgroups at most.  Measured over packed weights,

@@ -154,6 +154,20 @@ __device__ __forceinline__ void load_packed_pair(PackedStep<BITS, CPL>& first, P
     }
 }
 
+// 4-bit codes: a lane's whole share of a K-chunk of 128 rows (its four K-blocks) with one 16-byte load per column block
+template <int CPL>
+__device__ __forceinline__ void load_packed_chunk4(PackedStep<4, CPL> (&blocks)[4], const uint8_t* const (&slab)[CPL], uint32_t lane_off)
+{
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(slab[c] + lane_off));
+        blocks[0].d[c][0] = v[0];
+        blocks[1].d[c][0] = v[1];
+        blocks[2].d[c][0] = v[2];
+        blocks[3].d[c][0] = v[3];
+    }
+}
+
 template <int BITS, int CPL, int MB>
 __device__ __forceinline__ void mac_step_packed(const PackedStep<BITS, CPL>& raw, const float (&cs)[CPL], const uint4 (&afrag)[MB],
                                                 f32x4_t (&acc)[MB][CPL])
@@ -465,7 +479,7 @@ __global__ void __launch_bounds__((MB <= 2 && (CPL == 8 || MB == 1) && !(PACKED 
 bfaintb_decode_kernel(const GemmParams p)
 {
     static_assert(!REF || (BITS == 8 && !GROUPED && !PACKED), "the reference's arithmetic: 8-bit codes, row-major, one scale per column");
-    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED);  // blocks of 32 rows per pipeline step
+    constexpr int KB = decode_blocks_per_step(BITS, CPL, PACKED, MB);  // blocks of 32 rows per pipeline step
     constexpr uint32_t kCols = 16u * CPL;             // columns per workgroup
     constexpr uint32_t kRedStride = kCols + 4u;       // floats per row of a wave's tile in LDS (+4: spreads rows over banks)
     constexpr uint32_t kLaneBytes = CPL * BITS / 8;   // bytes of one row a lane loads
@@ -568,7 +582,15 @@ bfaintb_decode_kernel(const GemmParams p)
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
                 const size_t blk = (size_t)step * KB + q;
-                if constexpr (PACKED && KB == 2) {
+                if constexpr (PACKED && KB == 4) {
+                    // the step is one K-chunk of 4-bit codes: the lane's 16 bytes of it
+                    if constexpr (BITS == 4) {
+                        if (q == 0) {
+                            const uint32_t kblock = kblock0 + (uint32_t)blk;
+                            load_packed_chunk4<CPL>(st.raw, slab, (kUniformSlabs ? (uint32_t)lane * 16u : 0u) + (kblock / kBlocksPerChunk) * 1024u);
+                        }
+                    }
+                } else if constexpr (PACKED && KB == 2) {
                     // the step's two K-blocks (an even one and its successor) lie side by side in a lane's share of the chunk
                     if (q == 0) {
                         const uint32_t kblock = kblock0 + (uint32_t)blk;
@@ -599,36 +621,38 @@ bfaintb_decode_kernel(const GemmParams p)
             }
             __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic that follows
         };
-        // row-major weights with grouped scales: blocks of 32 rows until the next group begins (0: the block at hand opens
-        // one — so does the wave's first, wherever in a group it lies), and how many the group after that spans
+        // grouped scales: blocks of 32 rows until the next group begins (0: the block at hand opens one — so does the wave's
+        // first, wherever in a group it lies), and how many the group after that spans
         uint32_t blocks_to_group = 0u;
         uint32_t next_group_blocks = 0u;
-        if constexpr (GROUPED && !PACKED) {
+        if constexpr (GROUPED) {
             const uint32_t kb_uniform = __builtin_amdgcn_readfirstlane(kb);
             next_group_blocks = (p.group_size - kb_uniform % p.group_size) / 32u;
         }
         auto compute_stage = [&](Stage& st) {
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
-                if constexpr (GROUPED && PACKED) {
-                    // scale of column 4j + e goes to T[(4j + e) % 16][(4j + e) / 16]; lane (nl, kg) then reads row nl: its CPL
-                    // scales, in column-block order.  The table is this wave's own; LDS serves a wave's requests in order.
-                    if ((uint32_t)lane < kCols / 4u) {
-                        const uint32_t d[2] = {st.sraw[q][0].x, st.sraw[q][0].y};
-#pragma unroll
-                        for (uint32_t e = 0; e < 4; ++e) {
-                            const uint32_t cix = 4u * (uint32_t)lane + e;
-                            sc_table[(cix & 15u) * CPL + (cix >> 4)] = (uint16_t)(e & 1u ? d[e >> 1] >> 16 : d[e >> 1] & 0xffffu);
-                        }
-                    }
-                    uint4 mine[CPL / 8];
-#pragma unroll
-                    for (int i = 0; i < CPL / 8; ++i) mine[i] = *reinterpret_cast<const uint4*>(sc_table + (uint32_t)nl * CPL + 8u * i);
-                    apply_scales<BITS, CPL>(cs, mine);
-                } else if constexpr (GROUPED) {
+                if constexpr (GROUPED) {
                     // the scales change only where a group of rows begins: widen them there, not for every block
                     if (blocks_to_group == 0u) {
-                        apply_scales<BITS, CPL>(cs, st.sraw[q]);
+                        if constexpr (PACKED) {
+                            // scale of column 4j + e goes to T[(4j + e) % 16][(4j + e) / 16]; lane (nl, kg) then reads row nl: its
+                            // CPL scales, in column-block order.  The table is this wave's own; LDS serves a wave's requests in order.
+                            if ((uint32_t)lane < kCols / 4u) {
+                                const uint32_t d[2] = {st.sraw[q][0].x, st.sraw[q][0].y};
+#pragma unroll
+                                for (uint32_t e = 0; e < 4; ++e) {
+                                    const uint32_t cix = 4u * (uint32_t)lane + e;
+                                    sc_table[(cix & 15u) * CPL + (cix >> 4)] = (uint16_t)(e & 1u ? d[e >> 1] >> 16 : d[e >> 1] & 0xffffu);
+                                }
+                            }
+                            uint4 mine[CPL / 8];
+#pragma unroll
+                            for (int i = 0; i < CPL / 8; ++i) mine[i] = *reinterpret_cast<const uint4*>(sc_table + (uint32_t)nl * CPL + 8u * i);
+                            apply_scales<BITS, CPL>(cs, mine);
+                        } else {
+                            apply_scales<BITS, CPL>(cs, st.sraw[q]);
+                        }
                         blocks_to_group = next_group_blocks;
                         next_group_blocks = p.group_size / 32u;
                     }

@@ -60,10 +60,17 @@ inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 
 // Decode variant: blocks of 32 rows of k a wave loads per pipeline step (cpl = weights per lane and
 // row).  Row-major weights: one; two blocks for the 8-byte-per-row layouts measured no faster (more bytes in
-// flight per wave, fewer waves per CU).  Packed weights: two, so that a lane fetches its two neighbouring K-blocks of a
-// column block with one load (16 bytes for 8-bit codes: its whole share of a 64-row chunk; 8 bytes for 4-bit codes:
-// half of its share of a 128-row chunk) instead of two loads of half a sector each.
-__host__ __device__ constexpr int decode_blocks_per_step(int /*bits*/, int /*cpl*/, bool packed) { return packed ? 2 : 1; }
+// flight per wave, fewer waves per CU).  Packed weights: a lane's whole 16-byte share of a K-chunk with one load where the
+// registers allow it — two blocks (a 64-row chunk) for 8-bit codes, four (a 128-row chunk) for 4-bit codes in the
+// 128-column form with one block of 16 rows of A (mb = 1).  Half a share per load (8 bytes at a stride of 16) touches
+// every line of the chunk twice, a step apart, and the second touch misses in cache: 40 % more bytes fetched than the
+// matrix holds (32000 x 4096, m = 16, counted) and 30 - 60 % longer launches where it was tried for 8-bit codes.  Packed
+// 4-bit codes with more row blocks, or in the 256-column form, have no registers for four blocks per stage (two row
+// blocks: 22 spilled) and stay at two.
+__host__ __device__ constexpr int decode_blocks_per_step(int bits, int cpl, bool packed, int mb)
+{
+    return packed ? (bits == 4 && cpl == 8 && mb == 1 ? 4 : 2) : 1;
+}
 
 struct GemmParams {
     uint16_t* c;
