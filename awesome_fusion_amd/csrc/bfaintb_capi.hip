@@ -953,10 +953,10 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
 // The slab kernel: a workgroup walks its 16 columns alone, two workgroups that share a CU at half the pace each, so a
 // launch takes as many walks as the fullest CU has slabs — n / 16 over 256 CUs, rounded up (4-bit codes, 5120 x 5120,
 // 320 slabs: 7.3 us, what 8192 x 5120 would take; 4096 x 4096: 3.5).  4-bit codes are bound by the CUs' vector
-// arithmetic (2040 rows per us and walk); 8-bit codes by that (1544 rows per us) or by memory (6.2 TB/s).  Each
+// arithmetic (1975 rows per us and walk); 8-bit codes by that (1544 rows per us) or by memory (6.2 TB/s).  Each
 // further row of A costs 1.4 - 3.6 % of the walk up to 6 rows and 6 - 8 % from there (two blocks of 16 rows from m = 17).
-// The family's 128-column form streams at about 3.4 TB/s (4-bit) or 5.6 TB/s (8-bit) with every CU busy, pays the
-// split's hand-over, and hardly grows with m up to 16 rows (11 - 15 % more from 17).
+// The family's 128-column form streams at about 4.4 TB/s (4-bit) or 5.6 TB/s (8-bit) with every CU busy, pays the
+// split's hand-over, and hardly grows with m up to 16 rows (11 - 26 % more from 17).
 // Where the two are close either choice is within a few per cent; where they are not the gap is up to 80 % (4-bit codes,
 // 5120 x 13824, m = 16: slab 31.0, family 17.2; 13824 x 5120: 26.0 / 15.5; 4096 x 2048, m = 32: 5.5 / 6.9; 1024 x 16384,
 // m = 1: 10.5 / 9.0.  8-bit codes, m = 8: 5120 x 13824 23.2 / 16.3; 13824 x 5120 20.2 / 15.0; 5120 x 5120 11.3 / 9.2;
@@ -989,13 +989,13 @@ static double packed8_family_time_us(uint32_t m, uint32_t n, uint32_t k, const D
 }
 static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
 {
-    const double rows = m <= 6u ? 1.0 + 0.036 * (m - 1.0) : m <= 16u ? 1.18 + 0.082 * (m - 6.0) : 1.34 + 0.077 * m;
-    return 2.1 + packed_slab_walks(n) * k / 2040.0 * rows;
+    const double rows = m <= 6u ? 1.0 + 0.031 * (m - 1.0) : m <= 16u ? 1.155 + 0.078 * (m - 6.0) : 1.267 + 0.0776 * m;
+    return 2.58 + packed_slab_walks(n) * k / 1975.0 * rows;
 }
 static double packed4_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
 {
-    const double stream_us = (double)n * k / 2.0e6 / (3.38 * pow(packed_family_fill(m, n, pl), 0.62));
-    return 3.5 + 0.073 * m + 0.11 * (pl.splits - 1.0) + stream_us * (1.0 + 0.0013 * m + (m > 16u ? 0.148 : 0.0));
+    const double stream_us = (double)n * k / 2.0e6 / (4.37 * pow(packed_family_fill(m, n, pl), 0.58));
+    return 4.71 + 0.067 * m + 0.144 * (pl.splits - 1.0) + stream_us * (1.0 + 0.0003 * m + (m > 16u ? 0.258 : 0.0));
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
 {

@@ -522,7 +522,7 @@ bfaintb_decode_kernel(const GemmParams p)
     constexpr uint32_t kBlocksPerChunk = BITS == 8 ? 2u : 4u;
     constexpr uint32_t kBlockBytes = 16u / kBlocksPerChunk;
     // column block c of the workgroup (blocks past the last one re-read it; what they compute is never stored)
-    constexpr bool kUniformSlabs = BITS == 8;
+    constexpr bool kUniformSlabs = BITS == 8 || (CPL == 8 && MB == 2);
     const uint8_t* slab[CPL];
     uint32_t pk_col[CPL];
     if constexpr (PACKED) {
@@ -532,9 +532,10 @@ bfaintb_decode_kernel(const GemmParams p)
         for (int c = 0; c < CPL; ++c) {
             uint32_t gb = cb * CPL + (uint32_t)c;
             if (gb >= nblocks) gb = nblocks - 1u;
-            // 8-bit codes: the same for every lane (scalar registers; the lane's share is in the load's offset): the 8-wave
-            // kernels have no vector registers to spare.  4-bit codes: 16 bases do not fit the scalar file, and the 256-thread
-            // kernels have room for per-lane pointers (measured 4-19 % faster that way).
+            // 8-bit codes, and 4-bit codes with two row blocks in the 128-column form: the same for every lane (scalar registers;
+            // the lane's share is in the load's offset): those 8-wave kernels have no vector registers to spare.  Other 4-bit
+            // kernels: 16 bases do not fit the scalar file, and there is room for per-lane pointers (measured 4-19 % faster
+            // that way).
             slab[c] = p.b + (size_t)gb * slab_bytes + (kUniformSlabs ? 0u : (size_t)lane * 16u);
             pk_col[c] = 16u * gb + (uint32_t)nl;
         }

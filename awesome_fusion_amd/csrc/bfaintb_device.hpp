@@ -62,14 +62,15 @@ inline void fill_argv(void** argv, Tuple& t, std::index_sequence<I...>)
 // row).  Row-major weights: one; two blocks for the 8-byte-per-row layouts measured no faster (more bytes in
 // flight per wave, fewer waves per CU).  Packed weights: a lane's whole 16-byte share of a K-chunk with one load where the
 // registers allow it — two blocks (a 64-row chunk) for 8-bit codes, four (a 128-row chunk) for 4-bit codes in the
-// 128-column form with one block of 16 rows of A (mb = 1).  Half a share per load (8 bytes at a stride of 16) touches
+// 128-column form with one or two blocks of 16 rows of A.  Half a share per load (8 bytes at a stride of 16) touches
 // every line of the chunk twice, a step apart, and the second touch misses in cache: 40 % more bytes fetched than the
 // matrix holds (32000 x 4096, m = 16, counted) and 30 - 60 % longer launches where it was tried for 8-bit codes.  Packed
-// 4-bit codes with more row blocks, or in the 256-column form, have no registers for four blocks per stage (two row
-// blocks: 22 spilled) and stay at two.
+// 4-bit codes with four row blocks, or in the 256-column form, have no registers for four blocks per stage and stay at
+// two (two row blocks fit with the slab bases in scalar registers: 7 registers spilled with grouped scales, and still
+// 9 - 14 % faster on matrices from 32 MiB).
 __host__ __device__ constexpr int decode_blocks_per_step(int bits, int cpl, bool packed, int mb)
 {
-    return packed ? (bits == 4 && cpl == 8 && mb == 1 ? 4 : 2) : 1;
+    return packed ? (bits == 4 && cpl == 8 && mb <= 2 ? 4 : 2) : 1;
 }
 
 struct GemmParams {

@@ -245,11 +245,13 @@ def test_prepacked_entry_points_validate_before_launching():
     assert rcp(which=9) == -7
     assert rcp(m=0) == 0
     assert af.prepacked_workspace_bytes(1, 4096, 4096) == 0 and af.prepacked_workspace_bytes(4096, 4096, 4096) == 0
-    # (4-bit codes of so small a matrix run 128 columns per workgroup in either weight order: the same plan again)
-    assert af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) == af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE) > 0
+    # (4-bit codes of so small a matrix run 128 columns per workgroup in either weight order; packed ones walk k in whole
+    # K-chunks of 128 rows per wave, so their split factors are coarser)
+    assert 0 < af.prepacked_workspace_bytes(64, 256, 4096, 4, 128) <= af.workspace_bytes(64, 256, 4096, 4, 128, af.DECODE)
+    assert af.plan(16, 8192, 8192, 4, 128, packed=True).k_per_workgroup % 1024 == 0 and af.plan(64, 256, 4096, 4, 128, packed=True).k_per_workgroup % 512 == 0
     assert af.plan(64, 256, 4096, 4, 128, which=af.DECODE).tile_cols == 128 == af.plan(64, 256, 4096, 4, 128, packed=True, which=af.DECODE).tile_cols
     # packed 4-bit codes up to 32 rows: the slab kernel (16 columns) while the rows are few, then the 128-column form
-    assert af.plan(4, 28672, 8192, 4, 128, packed=True).tile_cols == 16 and af.plan(12, 28672, 8192, 4, 128, packed=True).tile_cols == 128
+    assert af.plan(8, 4096, 4096, 4, 128, packed=True).tile_cols == 16 and af.plan(12, 28672, 8192, 4, 128, packed=True).tile_cols == 128
     assert af.plan(16, 5120, 13824, 4, 128, packed=True).tile_cols == 128 and af.plan(32, 4096, 2048, 4, 128, packed=True).tile_cols == 16
     # (one round of workgroups, and only the split factors k divides into)
     assert af.plan(16, 11008, 8192, 4, 128, packed=True).splits == 2 and af.plan(16, 12288, 12288, 4, 128, packed=True).workgroups == 192
