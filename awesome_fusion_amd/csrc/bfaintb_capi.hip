@@ -335,18 +335,20 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
 // nibbles: the plan is for 4-bit codes in the 128-column form, which takes the launch shapes of 8-bit codes (bits == 8 here)
 DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t forced_splits, bool packed = false, bool nibbles = false)
 {
-    // 4-bit codes in rows also have a 128-column form (a lane loads 4 bytes of a row, 16 lanes half a cache line): twice the
-    // column blocks, so half the splits for the same number of workgroups, and 8 waves from one row on.  It takes the launch
-    // shape 8-bit codes of the same n x k would get — measured against the 256-column plan over 15 weight shapes x 10
-    // values of m.  It wins wherever the weights are few: up to 8 MiB of codes every m gains (1024 x 8192: 9.4 -> 8.0 us at
-    // m = 1, 13.7 -> 9.4 at 16, 18.4 -> 10.0 at 48; 256 x 7168: 16.3 -> 9.5 at 64; 4096 x 4096: 8.0 -> 7.8, 10.7 -> 8.8,
-    // 15.3 -> 12.3 at m = 1, 16, 64); and from 17 rows on up to 40 MiB (11008 x 4096, m = 24 / 32: 18.8 / 19.5 -> 15.4 / 16.5;
-    // 4096 x 11008, m = 24 .. 128: 9 - 17 %; 5120 x 13824, m = 24 / 32: 24.2 / 24.4 -> 20.6 / 21.9; 8192 x 8192: 1 - 7 %).  Few
-    // rows against many weights stream better in whole lines (8192 x 8192, m = 1 .. 16: 15 - 30 % slower; 32000 x 4096: 25 - 32 %;
-    // 28672 x 8192: 2 - 17 %), and so do packed weights, whose kernels are built for 256 columns.
+    // 4-bit codes in rows also have a 128-column form (a lane loads 4 bytes of a row, 16 lanes half a cache line — the
+    // kernel gives the two halves of a line to workgroups that share an L2): twice the column blocks, so half the splits
+    // for the same number of workgroups, and 8 waves from one row on.  It takes the launch shape 8-bit codes of the same
+    // n x k would get.  Measured against the 256-column plan over 15 weight shapes x m = 1 .. 64 (us, 128 / 256 columns): up
+    // to 24 MiB of codes every m gains (2048 x 8192: 7.8 / 9.6 at m = 1, 9.8 / 14.1 at 16, 12.4 / 17.7 at 64; 4096 x 4096:
+    // 6.8 / 7.9, 8.0 / 10.7, 11.4 / 15.4; 6144 x 4096: 8.4 / 9.1, 10.0 / 11.3, 16.1 / 21.2; 4096 x 11008: 11.0 / 11.3, 13.4 /
+    // 16.3, 21.4 / 26.3; 11008 x 4096: 11.3 / 11.2, 12.3 / 13.2, 14.6 / 18.9 at 24); up to 40 MiB from 16 rows on (8192 x
+    // 8192, m = 16 / 24 / 32: 15.4 / 15.8, 17.4 / 21.3, 18.7 / 21.4; 5120 x 13824: 17.4 / 19.4, 19.6 / 24.3, 20.9 / 24.5; with
+    // fewer rows the two are level).  More weights stream better in whole lines per workgroup (14336 x 8192, m = 8 /
+    // 16: 22.8 / 19.9, 25.1 / 21.2; 16384 x 8192, m = 1 .. 16: 12 - 15 % slower; 12288 x 12288, m = 8 .. 32: 10 - 44 %; 8192 x
+    // 28672, m = 1 .. 32: 9 - 31 %; 28672 x 8192: 2 - 5 %).
     if (bits == 4 && !packed) {
         const uint64_t code_bytes = (uint64_t)n * k / 2u;
-        if (code_bytes <= (8ull << 20) || (m > 16u && code_bytes <= (40ull << 20))) return decode_plan(m, n, k, 8, forced_splits, false, true);
+        if (code_bytes <= (24ull << 20) || (m >= 16u && code_bytes <= (40ull << 20))) return decode_plan(m, n, k, 8, forced_splits, false, true);
     }
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built

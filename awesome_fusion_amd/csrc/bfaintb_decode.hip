@@ -490,7 +490,15 @@ bfaintb_decode_kernel(const GemmParams p)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same for the wave's lanes: what follows from it stays scalar
     const int nl = lane & 15;
     const int kg = lane >> 4;
-    const uint32_t cb = blockIdx.x;
+    // 4-bit codes in rows, 128 columns per workgroup: a workgroup reads half of every 128-byte line and its neighbour the
+    // other half.  Workgroups go to the XCDs (each with its own L2) in turn, so neighbours i and i + 1 would fetch every
+    // line once each; within a run of 16 column blocks the two halves of a line are given to workgroups 8 apart instead,
+    // which share an L2.
+    uint32_t cb = blockIdx.x;
+    if constexpr (BITS == 4 && CPL == 8 && !PACKED) {
+        const uint32_t run = cb & ~15u;
+        if (run + 16u <= gridDim.x) cb = run + 2u * (cb & 7u) + ((cb >> 3) & 1u);
+    }
     const uint32_t ks = blockIdx.y;
     // rows of A and C this workgroup covers: block blockIdx.z of 16*MB rows
     const uint32_t row0 = blockIdx.z * (16u * MB);
