@@ -587,7 +587,21 @@ bfaintb_decode_kernel(const GemmParams p)
         uint16_t* sc_table = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(red) + p.decode_scale_lds) + (uint32_t)wave * 16u * CPL;
         uint32_t sc_col = cb * kCols + 4u * (uint32_t)lane;
         if (sc_col + 4u > p.n) sc_col = p.n - 4u;
+        // Packed 8-bit codes, one scale per column: a workgroup starts its walk along k at a step of its own (and wraps
+        // round).  Slabs lie k x 16 bytes apart; when that is a large power of two, every workgroup's loads of a step
+        // differ only in address bits that do not choose the memory channel, and the launch crowds onto a few of them
+        // (8192 x 8192, m = 16: 20.7 us, 16.6 with k = 8064 — same plan, fewer bytes by 1.6 %).  The order in which a
+        // wave adds its steps differs from workgroup to workgroup, so it is fixed by the launch shape, as before.
+        constexpr bool kRotateSteps = PACKED && BITS == 8 && !GROUPED;
+        int first_step = 0;
+        if constexpr (kRotateSteps) {
+            if (nsteps > 1) first_step = (int)((cb + ks) % (uint32_t)nsteps);
+        }
         auto load_stage = [&](Stage& st, int step) {
+            if constexpr (kRotateSteps) {
+                step += first_step;
+                if (step >= nsteps) step -= nsteps;
+            }
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
                 const size_t blk = (size_t)step * KB + q;
