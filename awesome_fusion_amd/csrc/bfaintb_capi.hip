@@ -962,8 +962,8 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
 // Where the two are close either choice is within a few per cent; where they are not the gap is up to 80 % (4-bit codes,
 // 5120 x 13824, m = 16: slab 31.0, family 17.2; 13824 x 5120: 26.0 / 15.5; 4096 x 2048, m = 32: 5.5 / 6.9; 1024 x 16384,
 // m = 1: 10.5 / 9.0.  8-bit codes, m = 8: 5120 x 13824 23.2 / 16.3; 13824 x 5120 20.2 / 15.0; 5120 x 5120 11.3 / 9.2;
-// 2048 x 4096, m = 12: 5.5 / 6.9).  Picks on the scan: 4-bit 13 of 248 more than 5 % off, 8-bit 13 of 196 (fixed row
-// limits, as before: 22 of 196, up to 42 %).
+// 2048 x 4096, m = 12: 5.5 / 6.9).  Picks on the scan, weights cold: 4-bit 9 of 252 more than 5 % off the faster kernel
+// (worst 12 %), 8-bit 17 of 252 (worst 14 %); fixed row limits, as before: 22 of 196, up to 42 %.
 static double packed_slab_walks(uint32_t n)
 {
     const double cus = (double)machine_cus();
