@@ -640,7 +640,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="time only this workload, cold B, nothing else (for a kernel trace or a counter "
                     "run of one kernel): decode | prefill | decode_cold | decode_packed_cold | c3_m1 | c3_m16 | c3_m32 | "
-                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | plan_check (the library's plans "
+                    "c5_m1 | c5_m16 | c5_m2048 | mid_m256 | mid_m1024 | mid_m2048 | mid_m256_n8192_k8192 | shape_m<m>_n<n>_k<k>_int<8|4>[_g<group>][_packed] (any one shape) | plan_check (the library's plans "
                     "against forced alternatives) | power_scan (board power by shape; config 4 by operand values) | prefill_trace, decode_timeline "
                     "(both need --lib with a library built with -DBFAINTB_TRACE)")
     ap.add_argument("--lib", default="", help="load this build of libbfaintb_gemm.so instead of the package's own "
@@ -678,6 +678,28 @@ def main():
     if args.only == "prefill_trace":
         print(json.dumps({"metric": "bfAintBGemm 256x256-tile kernel: K-loop cycles per step and shader clock by tile count (instrumented build)",
                           "library": af.library_path(), "rows": prefill_loop_trace(af)}))
+        return
+
+    # ---- any one shape alone, either weight order (profiling runs): shape_m<m>_n<n>_k<k>_int<8|4>[_g<group>][_packed]
+    if args.only.startswith("shape_m"):
+        import re
+        parsed = re.fullmatch(r"shape_m(\d+)_n(\d+)_k(\d+)_int(4|8)(?:_g(\d+))?(_packed)?", args.only)
+        assert parsed, f"--only {args.only}: not a shape name"
+        m, n, k, bits = (int(parsed.group(i)) for i in (1, 2, 3, 4))
+        group = int(parsed.group(5) or 0)
+        packed = parsed.group(6) is not None
+        b_bytes = n * k * bits // 8
+        w = Workload(args.only, m, n, k, bits=bits, group=group, copies=max(2, min(40, 2 * LLC_BYTES // b_bytes + 2)) if m <= 32 else 2)
+        steps = min(K, 100) if m <= 64 else 10
+        ev_ms, wall_ms = time_graph(af, w, steps, min(W, 10), rotate=True, packed=packed)
+        bound = "hbm" if m <= 64 else "mfma"
+        pl = af.plan(m, n, k, bits, group, packed=packed)
+        print(json.dumps({"metric": f"bfAintBGemm {w.name}", "value": roofline_entry(w, wall_ms, bound)["achieved"],
+                          "unit": "GB/s" if bound == "hbm" else "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": min(W, 10),
+                          "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                          "dtype": "bf16", "data": "synthetic", "config": {"workload": w.name, "packed": packed},
+                          "plan": {"tile": [pl.tile_rows, pl.tile_cols], "waves": pl.waves, "splits": pl.splits, "workgroups": pl.workgroups},
+                          "roofline": roofline_entry(w, ev_ms, bound)}))
         return
 
     # ---- one secondary workload alone (profiling runs)
