@@ -1044,7 +1044,16 @@ static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
     FamilyEstimate e;
     const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
     if (bits == 4) return (pl.cols == 128u ? 0.70 : 0.84) * ranked;  // (the 128-column form measures 0.52 - 0.79 of its estimate)
-    return (pl.mb == 4u ? 0.84 : 0.76) * (5.0 + e.core + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
+    // (a row block that is not full costs less: 64-row blocks at m = 40 / 48 / 64 measure 0.87 / 0.91 / 1.0 of the tiles' time
+    // over 11 weight shapes where the estimate had them level — the rows past m are neither converted for nor multiplied)
+    const double block_rows = 16.0 * pl.mb;
+    const double fill = m < block_rows ? m / block_rows : 1.0;  // (with more blocks than one the estimate is right as it stands: 96 x 8192 x 8192)
+    // (and a round of workgroups that leaves CUs idle slows the stream less than in proportion: 172 and 192 workgroups of 64
+    // rows x 128 columns run at 0.80 and 0.85 of the pace of 256, not 0.67 and 0.75 — 11008 x 8192, 22016 x 4096, 12288 x 12288)
+    const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits * (double)(uint64_t)((m + block_rows - 1.0) / block_rows);
+    const double cus = (double)machine_cus();
+    const double idle = wgs < cus ? pow(wgs / cus, 0.45) : 1.0;
+    return (pl.mb == 4u ? 0.84 : 0.76) * (0.65 + 0.35 * fill) * (5.0 + e.core * idle + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
 }
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the
 // row-blocked family without a split along k beyond) or the tiled kernel, by the estimates that choose for row-major weights.
