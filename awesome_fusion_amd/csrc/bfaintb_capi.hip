@@ -428,7 +428,11 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         // (n not a multiple of 16: only the 8-codes-per-lane shape can read the last columns)
         // (packed weights: the kernels are built for 128 columns; packed 4-bit codes: the 256-column form, 4 waves, is at
         // best 6 % ahead — 16384 x 8192 and 32000 x 4096 up to 16 rows — and up to 30 % behind)
-        const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 || (m >= 8 && (!many_wide_blocks || packed)) || (nibbles && packed));
+        // (... and up to 96 MiB of weights: beyond, 256-column blocks win again unless the narrow ones fill their rounds — m = 8 /
+        // 16, wide against narrow: 12288 x 12288 29.3 / 31.9 against 34.3 / 37.4 us; 14336 x 8192 24.8 / 26.9 against 26.2 / 28.3;
+        // 32000 x 4096, 250 narrow blocks, stays narrow: 25.0 / 25.2 against 23.7 / 24.5)
+        const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 ||
+                                          (m >= 8 && (packed || (!many_wide_blocks && weight_bytes <= (96ull << 20)))) || (nibbles && packed));
         pl.cols = narrow ? 128u : 256u;
         // 4-bit codes, 8 to 16 rows: the same 256 columns with 8 waves (twice the waves to hide the activation loads and
         // the matrix instructions behind; n = k = 4096, m = 16: 11.6 against 14.7 us, 1024 x 8192: 14.1 / 17.4,
