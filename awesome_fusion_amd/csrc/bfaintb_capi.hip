@@ -155,7 +155,19 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 {
     FamilyEstimate e;
     const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
-    if (bits == 4) return 0.76 * ranked;
+    if (bits == 4) {
+        // (one row block that is not full costs less, a full one a little more than the 0.76 says: 64-row blocks of the
+        // 128-column form at m = 40 / 48 / 64 against the tiles, us: 11008 x 8192 32.4 / 36.3, 33.6 / 36.5, 36.5 / 36.8;
+        // 32000 x 4096 31.1 / 32.6, 32.1 / 32.6, 34.9 / 33.1; 16384 x 8192 34.4 / 36.8, 37.0 / 37.0, 40.6 / 38.8)
+        const double block_rows = 16.0 * pl.mb;
+        if (m <= block_rows && pl.cols == 128u) {
+            // (and CUs left idle slow the stream less than in proportion, as over packed weights: 86 column blocks x 2 splits)
+            const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits, cus = (double)machine_cus();
+            const double idle = wgs < cus ? pow(wgs / cus, 0.45) : 1.0;
+            return 0.80 * (0.65 + 0.35 * m / block_rows) * (5.0 + e.core * idle + e.partial);
+        }
+        return 0.76 * ranked;
+    }
     if (pl.splits > 1u) return 0.87 * (5.0 + e.core + (pl.mb == 4u ? 0.65 : 0.2) * e.partial);
     return (pl.mb == 4u ? 1.05 : 0.93) * (5.0 + e.core);
 }
@@ -343,12 +355,16 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
     // 6.8 / 7.9, 8.0 / 10.7, 11.4 / 15.4; 6144 x 4096: 8.4 / 9.1, 10.0 / 11.3, 16.1 / 21.2; 4096 x 11008: 11.0 / 11.3, 13.4 /
     // 16.3, 21.4 / 26.3; 11008 x 4096: 11.3 / 11.2, 12.3 / 13.2, 14.6 / 18.9 at 24); up to 40 MiB from 16 rows on (8192 x
     // 8192, m = 16 / 24 / 32: 15.4 / 15.8, 17.4 / 21.3, 18.7 / 21.4; 5120 x 13824: 17.4 / 19.4, 19.6 / 24.3, 20.9 / 24.5; with
-    // fewer rows the two are level).  More weights stream better in whole lines per workgroup (14336 x 8192, m = 8 /
+    // fewer rows the two are level); up to 64 MiB from 17 rows on, where the 256-column form needs row blocks of its own
+    // (8192 x 11008, m = 20 / 24 / 32: 21.3 / 24.7, 22.1 / 25.9, 23.5 / 26.3; 11008 x 8192: 23.3 / 27.1, 24.2 / 27.6, 26.2 / 28.7;
+    // 32000 x 4096: 22.8 / 26.0, 23.6 / 25.8, 25.3 / 26.7; 14336 x 8192 and 16384 x 8192: level; 12288 x 12288, 72 MiB: 38.0 /
+    // 34.9, 42.8 / 37.3).  More weights stream better in whole lines per workgroup (14336 x 8192, m = 8 /
     // 16: 22.8 / 19.9, 25.1 / 21.2; 16384 x 8192, m = 1 .. 16: 12 - 15 % slower; 12288 x 12288, m = 8 .. 32: 10 - 44 %; 8192 x
     // 28672, m = 1 .. 32: 9 - 31 %; 28672 x 8192: 2 - 5 %).
     if (bits == 4 && !packed) {
         const uint64_t code_bytes = (uint64_t)n * k / 2u;
-        if (code_bytes <= (24ull << 20) || (m >= 16u && code_bytes <= (40ull << 20))) return decode_plan(m, n, k, 8, forced_splits, false, true);
+        if (code_bytes <= (24ull << 20) || (m >= 16u && code_bytes <= (40ull << 20)) || (m > 16u && code_bytes <= (64ull << 20)))
+            return decode_plan(m, n, k, 8, forced_splits, false, true);
     }
     const uint64_t weight_bytes = (uint64_t)n * k * (uint32_t)bits / 8u;
     // 4-bit codes, 17 to 32 rows, a small or narrow matrix (row-major only: the kernels over packed 4-bit codes are built
