@@ -168,7 +168,10 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
         }
         return 0.76 * ranked;
     }
-    if (pl.splits > 1u) return 0.87 * (5.0 + e.core + (pl.mb == 4u ? 0.65 : 0.2) * e.partial);
+    // (64-row blocks: the hand-over at 0.9 of its term — at 0.65 the family ran up to 13 % over the tiles' time at 48 - 64 rows
+    // against 8192 x 11008 and 8192 x 8192; 5 of 105 shapes scanned are then more than 2.5 % off, the worst 96 x 4096 x 11008
+    // at 13 %.  Scaling a single block by its fill, which suits 4-bit codes, sends those same shapes back to the family.)
+    if (pl.splits > 1u) return 0.87 * (5.0 + e.core + (pl.mb == 4u ? 0.9 : 0.2) * e.partial);
     return (pl.mb == 4u ? 1.05 : 0.93) * (5.0 + e.core);
 }
 
