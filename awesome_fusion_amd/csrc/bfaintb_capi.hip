@@ -179,9 +179,17 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 // 256x256 tiles, each with a quarter of the work per K-step.  Measured against the large tiles (8-bit, k = 4096, us):
 // m x n = 256 x 4096: 48 / 59, 1024 x 4096: 58 / 66, 512 x 8192 (4-bit, k = 8192): 112 / 137; with more tiles the
 // large ones win (1536 x 4096: 81 / 72, 512 x 11008: 80 / 68).
+// (One gap: a few tall tiles more than CUs — 640 x 11008 makes 258 — would go to 129 large tiles on half the machine, 82 us;
+// the small tiles take it in two rounds, 430 of them, in 66 us.  So: also up to two rounds of small tiles where the tall
+// ones do not fit one round and the large ones fill at most 55 % of the CUs.)
 static bool prefill_small_tiles(uint32_t m, uint32_t n)
 {
-    return (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u) <= machine_cus();
+    const uint64_t cus = machine_cus();
+    const uint64_t small = (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u);
+    if (small <= cus) return true;
+    const uint64_t tall = (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u);
+    const uint64_t large = (uint64_t)((m + 255u) / 256u) * ((n + 255u) / 256u);
+    return small <= 2u * cus && tall > cus && large * 20u <= cus * 11u;
 }
 
 // Between the two: more small tiles than CUs, but at most one tile of 256 rows x 128 columns per CU.  The large tiles would
@@ -249,7 +257,7 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         const double wgs = tiles * t.splits;
         const double load = wgs >= cus ? 1.0 : wgs / cus;
         const double step_us = ((bits == 4 ? 0.41 : 0.40) + 0.15 * load * load * load) * (0.8 + 0.2 * fill);
-        t.us = 4.0 + per * step_us + hand_over;
+        t.us = 4.0 + (wgs > cus ? 2.0 : 1.0) * per * step_us + hand_over;  // (more small tiles than CUs: two rounds of them)
         // (three splits and more: the hand-over scatters more than this says, and where the row-blocked family is about as
         // fast it is the safer pick — 192 x 4096 x 4096: 25.5 against 22.9 us, 128 x 4096 x 11008: 39.0 against 34.3)
         if (t.splits > 2u) t.us *= 1.07;

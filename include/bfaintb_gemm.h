@@ -365,8 +365,10 @@ BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int wei
 
 /* Rows (bfaintb_prefill_tile) and columns of the tiles BFAINTB_VARIANT_PREFILL runs an m x n output of row-major
  * weights with: 128 x 128 while that makes at most 256 tiles (one per CU); else 256 rows x 128 columns while that
- * makes at most 256; else 256 x 256 (256 = the device's compute units: one tile per unit).  Pre-packed weights run
- * the same tiles.  (The reference arithmetic has no 256 x 128 form: 256 x 256 there.) */
+ * makes at most 256; else 256 x 256 (256 = the device's compute units: one tile per unit) — except that up to 512
+ * tiles of 128 x 128 run in two rounds where the 256 x 128 ones just miss one round and the 256 x 256 ones would fill
+ * at most 55 % of the units (640 x 11008).  Pre-packed weights run the same tiles.  (The reference arithmetic has no
+ * 256 x 128 form: 256 x 256 there.) */
 BFAINTB_API uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n);
 BFAINTB_API uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n);
 

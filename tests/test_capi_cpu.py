@@ -59,6 +59,9 @@ def test_variant_choice_and_split():
     assert af.split_k(512, 4096, 4096) == 2 and af.split_k(640, 4096, 4096) == 1
     # 128x128 tiles up to one per CU, 256x256 beyond; forced forms are accepted as variants
     assert af.prefill_tile(1024, 4096) == 128 and af.prefill_tile(1025, 4096) == 256
+    # (the gap: 258 tall tiles just miss one round and the large ones would use half the machine: two rounds of small tiles)
+    assert af.prefill_tile(640, 11008) == 128 and af.plan(640, 11008, 4096).workgroups == 430 and af.plan(640, 11008, 4096).splits == 1
+    assert af.prefill_tile(704, 11008) == 256 and af.prefill_tile(512, 11008) == 256 and af.prefill_tile_cols(512, 11008) == 128
     assert af.prefill_tile(128, 28672) == 128 and af.prefill_tile(4096, 4096) == 256 and af.prefill_tile(1, 16) == 128
     # the small tiles over row-major weights split k while tiles x splits fit one workgroup per CU: same workspace layout as
     # the decode family's; the large tiles, the both-operands-in-LDS form and an unsplit launch need none
