@@ -182,11 +182,16 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 // (One gap: a few tall tiles more than CUs — 640 x 11008 makes 258 — would go to 129 large tiles on half the machine, 82 us;
 // the small tiles take it in two rounds, 430 of them, in 66 us.  So: also up to two rounds of small tiles where the tall
 // ones do not fit one round and the large ones fill at most 55 % of the CUs.)
-static bool prefill_small_tiles(uint32_t m, uint32_t n)
+static bool prefill_small_tiles(uint32_t m, uint32_t n, int bits)
 {
     const uint64_t cus = machine_cus();
     const uint64_t small = (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u);
     if (small <= cus) return true;
+    // 4-bit codes: two rounds of small tiles beat one of tall ones while the second round is about a third full (the tall
+    // kernel converts every weight in two waves; us, small / tall, on two boxes: 1152 x 4096 x 4096, 288 tiles: 65.8 / 70.7
+    // and 68.9 / 70.9; 512 x 11008 x 4096, 344: 65.9 / 71.1; with 384 to 448 tiles the second box had them level or the tall
+    // ones ahead by 2 %, and packed weights by up to 4 %; 8-bit codes the other way throughout: 63.1 / 59.2 at 288 tiles)
+    if (bits == 4 && small * 20u <= cus * 27u) return true;
     const uint64_t tall = (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u);
     const uint64_t large = (uint64_t)((m + 255u) / 256u) * ((n + 255u) / 256u);
     return small <= 2u * cus && tall > cus && large * 20u <= cus * 11u;
@@ -196,9 +201,9 @@ static bool prefill_small_tiles(uint32_t m, uint32_t n)
 // occupy a quarter to a half of the CUs there; the tall ones run one per CU at 0.94 us per K-step against the large tiles'
 // 1.02 on twice the work (8-bit, 64 steps, us tall / large: 1536 x 4096: 61.0 / 66.0; 512 x 11008: 60.3 / 64.7; 2048 x 4096:
 // 71.0 / 75.7; 128 steps, 1024 x 8192: 129 / 141; 4-bit, 768 x 8192: 138 / 140).
-static bool prefill_tall_tiles(uint32_t m, uint32_t n)
+static bool prefill_tall_tiles(uint32_t m, uint32_t n, int bits)
 {
-    return !prefill_small_tiles(m, n) && (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u) <= machine_cus();
+    return !prefill_small_tiles(m, n, bits) && (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u) <= machine_cus();
 }
 
 static bool is_prefill(int v)
@@ -208,9 +213,9 @@ static bool is_prefill(int v)
 }
 
 // tile size of a tiled-variant launch: forced, or by shape
-static bool use_small_tiles(int v, uint32_t m, uint32_t n)
+static bool use_small_tiles(int v, uint32_t m, uint32_t n, int bits)
 {
-    return v == BFAINTB_VARIANT_PREFILL_128 || v == BFAINTB_VARIANT_PREFILL_128_LDS || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n));
+    return v == BFAINTB_VARIANT_PREFILL_128 || v == BFAINTB_VARIANT_PREFILL_128_LDS || (v == BFAINTB_VARIANT_PREFILL && prefill_small_tiles(m, n, bits));
 }
 
 // Rough time of the tiled variant (prefill_estimate_us, below the plan of the small tiles).  Small tiles: a K-step takes 0.40 us on an empty machine and 0.55 us with a workgroup on every CU (the kernel that
@@ -279,9 +284,9 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
 
 static double prefill_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits)
 {
-    if (prefill_small_tiles(m, n)) return tile128_plan(m, n, k, bits, 0).us;
+    if (prefill_small_tiles(m, n, bits)) return tile128_plan(m, n, k, bits, 0).us;
     const double cus = (double)machine_cus();
-    if (prefill_tall_tiles(m, n)) {
+    if (prefill_tall_tiles(m, n, bits)) {
         // one tile of 256 rows x 128 columns per CU at most (8-bit, us per K-step: 512 x 11008 x 4096, 172 tiles: 0.87;
         // 768 x 8192 x 8192 and 1536 x 4096 x 4096, 192: 0.84 and 0.88; 2048 x 4096 x 4096 and x 11008, 256: 1.02 and 0.98)
         const double tiles = (double)((m + 255u) / 256u) * (double)((n + 127u) / 128u);
@@ -517,13 +522,13 @@ int resolve_variant(uint32_t m, uint32_t n, uint32_t k, int bits, int variant)
 }
 
 // whether a tiled-variant launch over row-major weights goes to the small-tile kernel that can split k
-static bool tiled_may_split(int v, uint32_t m, uint32_t n) { return use_small_tiles(v, m, n) && v != BFAINTB_VARIANT_PREFILL_128_LDS; }
+static bool tiled_may_split(int v, uint32_t m, uint32_t n, int bits) { return use_small_tiles(v, m, n, bits) && v != BFAINTB_VARIANT_PREFILL_128_LDS; }
 
 size_t workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int variant, uint32_t forced_split)
 {
     if (m == 0 || n == 0) return 0;
     if (variant == BFAINTB_VARIANT_DECODE) return split_workspace_bytes(decode_plan(m, n, k, bits, forced_split).splits, m, n);
-    if (is_prefill(variant) && tiled_may_split(variant, m, n)) return split_workspace_bytes(tile128_plan(m, n, k, bits, forced_split).splits, m, n);
+    if (is_prefill(variant) && tiled_may_split(variant, m, n, bits)) return split_workspace_bytes(tile128_plan(m, n, k, bits, forced_split).splits, m, n);
     return 0;
 }
 
@@ -647,7 +652,7 @@ uint32_t bfaintb_gemm_split_k(uint32_t m, uint32_t n, uint32_t k, int weight_bit
 {
     const int v = bfaintb_gemm_variant(m, n, k, weight_bits, group_size);
     if (v == BFAINTB_VARIANT_DECODE) return decode_plan(m, n, k, weight_bits, 0).splits;
-    if (v == BFAINTB_VARIANT_PREFILL && tiled_may_split(v, m, n)) return tile128_plan(m, n, k, weight_bits, 0).splits;
+    if (v == BFAINTB_VARIANT_PREFILL && tiled_may_split(v, m, n, weight_bits)) return tile128_plan(m, n, k, weight_bits, 0).splits;
     return 1;
 }
 
@@ -845,7 +850,7 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
         return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
 #endif
         // row-major weights on small tiles: that form, unless the other one is asked for by name
-        small_wreg = tiled_may_split(v, m, n) && bfaintb::prefill128_wreg_serves(p);
+        small_wreg = tiled_may_split(v, m, n, weight_bits) && bfaintb::prefill128_wreg_serves(p);
         if (small_wreg) {
             const TilePlan tp = tile128_plan(m, n, k, weight_bits, split_k);
             p.k_per_wg = tp.k_per_wg;
@@ -879,9 +884,9 @@ static int gemm_impl(void* c, const void* a, const void* b, const void* scale, c
     }
     if (tiled) {
         if (small_wreg) return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, false, st);
-        if ((v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) && !p.reference_arith)
+        if ((v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n, weight_bits))) && !p.reference_arith)
             return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, false, st);
-        if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
+        if (use_small_tiles(v, m, n, weight_bits)) return (int)bfaintb::launch_prefill128(p, weight_bits, false, st);
         return (int)bfaintb::launch_prefill(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
 #ifdef BFAINTB_TRACE
@@ -1114,7 +1119,7 @@ int bfaintb_gemm_prepacked_variant(uint32_t m, uint32_t n, uint32_t k, int weigh
 static size_t packed_workspace_need(uint32_t m, uint32_t n, uint32_t k, int bits, int v)
 {
     if (m == 0 || n == 0) return 0;
-    if (is_prefill(v)) return tiled_may_split(v, m, n) ? split_workspace_bytes(tile128_plan(m, n, k, bits, 0).splits, m, n) : 0;
+    if (is_prefill(v)) return tiled_may_split(v, m, n, bits) ? split_workspace_bytes(tile128_plan(m, n, k, bits, 0).splits, m, n) : 0;
     if (v != BFAINTB_VARIANT_DECODE || packed_uses_slab(m, n, k, bits)) return 0;
     const DecodePlan pl = packed_family_plan(m, n, k, bits);
     if (pl.splits <= 1) return 0;
@@ -1173,7 +1178,7 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
         // a tile's 16 column blocks and a 256-row panel of A are addressed through 32-bit buffer extents
         if ((uint64_t)k * 256u * (uint32_t)weight_bits / 8u >= (1ull << 31) || (uint64_t)256 * lda * 2u >= (1ull << 31))
             return BFAINTB_ERR_BAD_SHAPE;
-        if (tiled_may_split(v, m, n) && bfaintb::prefill128_wreg_serves(p)) {
+        if (tiled_may_split(v, m, n, weight_bits) && bfaintb::prefill128_wreg_serves(p)) {
             // small tiles: the kernel that keeps the weights in registers, with the plan (split along k included) and the
             // workspace protocol of the row-major path
             const TilePlan tp = tile128_plan(m, n, k, weight_bits, 0);
@@ -1185,12 +1190,12 @@ static int gemm_prepacked_impl(void* c, const void* a, const void* packed_b, con
             }
             return (int)bfaintb::launch_prefill128_wreg(p, weight_bits, true, st);
         }
-        if (v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) {
+        if (v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n, weight_bits))) {
             p.k_per_wg = k;
             p.splits = 1;
             return (int)bfaintb::launch_prefill256x128_wreg(p, weight_bits, true, st);
         }
-        if (use_small_tiles(v, m, n)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
+        if (use_small_tiles(v, m, n, weight_bits)) return (int)bfaintb::launch_prefill128(p, weight_bits, true, st);
         return (int)bfaintb::launch_prefill_packed(p, weight_bits, st, v != BFAINTB_VARIANT_PREFILL_256_LDS);
     }
     if (!packed_uses_slab(m, n, k, weight_bits)) {
@@ -1373,7 +1378,7 @@ int bfaintb_gemm_plan(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint3
         return BFAINTB_OK;
     }
     // the tiled kernels
-    if (use_small_tiles(v, m, n)) {
+    if (use_small_tiles(v, m, n, weight_bits)) {
         out->variant = BFAINTB_VARIANT_PREFILL_128;
         out->tile_rows = out->tile_cols = 128u;
         const bool wreg = v != BFAINTB_VARIANT_PREFILL_128_LDS;
@@ -1388,7 +1393,7 @@ int bfaintb_gemm_plan(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint3
         out->workspace_bytes = split_workspace_bytes(out->splits, m, n);
         return BFAINTB_OK;
     }
-    if (v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n))) {
+    if (v == BFAINTB_VARIANT_PREFILL_256X128 || (v == BFAINTB_VARIANT_PREFILL && prefill_tall_tiles(m, n, weight_bits))) {
         out->variant = BFAINTB_VARIANT_PREFILL_256X128;
         out->kernel = BFAINTB_KERNEL_TILES_256X128;
         out->tile_rows = 256u;
@@ -1411,8 +1416,8 @@ int bfaintb_gemm_plan(uint32_t m, uint32_t n, uint32_t k, int weight_bits, uint3
     return BFAINTB_OK;
 }
 
-uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n) { return prefill_small_tiles(m, n) ? 128u : 256u; }
-uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n) { return (prefill_small_tiles(m, n) || prefill_tall_tiles(m, n)) ? 128u : 256u; }
+uint32_t bfaintb_prefill_tile(uint32_t m, uint32_t n) { return prefill_small_tiles(m, n, 8) ? 128u : 256u; }
+uint32_t bfaintb_prefill_tile_cols(uint32_t m, uint32_t n) { return (prefill_small_tiles(m, n, 8) || prefill_tall_tiles(m, n, 8)) ? 128u : 256u; }
 
 const char* bfaintb_kernel_name(int variant, int weight_bits, uint32_t group_size, uint32_t m)
 {
