@@ -587,12 +587,11 @@ bfaintb_decode_kernel(const GemmParams p)
         uint16_t* sc_table = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(red) + p.decode_scale_lds) + (uint32_t)wave * 16u * CPL;
         uint32_t sc_col = cb * kCols + 4u * (uint32_t)lane;
         if (sc_col + 4u > p.n) sc_col = p.n - 4u;
-        // Packed 8-bit codes, one scale per column: a workgroup starts its walk along k at a step of its own (and wraps
-        // round).  Slabs lie k x 16 bytes apart; when that is a large power of two, every workgroup's loads of a step
+        // Packed 8-bit codes: a workgroup starts its walk along k at a step of its own (and wraps round).  Slabs lie k x 16 bytes apart; when that is a large power of two, every workgroup's loads of a step
         // differ only in address bits that do not choose the memory channel, and the launch crowds onto a few of them
         // (8192 x 8192, m = 16: 20.7 us, 16.6 with k = 8064 — same plan, fewer bytes by 1.6 %).  The order in which a
         // wave adds its steps differs from workgroup to workgroup, so it is fixed by the launch shape, as before.
-        constexpr bool kRotateSteps = PACKED && BITS == 8 && !GROUPED;
+        constexpr bool kRotateSteps = PACKED && BITS == 8;
         int first_step = 0;
         if constexpr (kRotateSteps) {
             if (nsteps > 1) first_step = (int)((cb + ks) % (uint32_t)nsteps);
@@ -648,11 +647,22 @@ bfaintb_decode_kernel(const GemmParams p)
         // first, wherever in a group it lies), and how many the group after that spans
         uint32_t blocks_to_group = 0u;
         uint32_t next_group_blocks = 0u;
+        // (a walk that starts at step first_step wraps round to the wave's first row after nsteps - first_step steps, and
+        // the count starts again there)
+        uint32_t steps_to_wrap = 0u;
         if constexpr (GROUPED) {
-            const uint32_t kb_uniform = __builtin_amdgcn_readfirstlane(kb);
+            const uint32_t kb_uniform = __builtin_amdgcn_readfirstlane(kb) + 32u * (uint32_t)KB * (uint32_t)first_step;
             next_group_blocks = (p.group_size - kb_uniform % p.group_size) / 32u;
+            steps_to_wrap = (uint32_t)(nsteps - first_step);
         }
         auto compute_stage = [&](Stage& st) {
+            if constexpr (GROUPED && kRotateSteps) {
+                if (steps_to_wrap == 0u) {
+                    blocks_to_group = 0u;
+                    next_group_blocks = (p.group_size - __builtin_amdgcn_readfirstlane(kb) % p.group_size) / 32u;
+                }
+                --steps_to_wrap;
+            }
 #pragma unroll
             for (int q = 0; q < KB; ++q) {
                 if constexpr (GROUPED) {
