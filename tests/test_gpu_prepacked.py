@@ -131,7 +131,13 @@ def test_plan_corners_both_weight_orders(af, m, n, k, bits, group):
     (49, 128, 512, 8, 0), (64, 4096, 1024, 8, 0), (100, 272, 448, 8, 64), (130, 48, 1024, 8, 32), (200, 1040, 256, 8, 0), (300, 144, 2048, 8, 128),
     (64, 256, 512, 4, 0), (97, 528, 1024, 4, 128), (150, 80, 640, 4, 32), (260, 1296, 384, 4, 128),
     # shapes whose plan splits along k (few column groups, long k): partial sums meet in the workspace
-    (64, 256, 4096, 4, 128), (80, 128, 8192, 8, 0), (100, 512, 4096, 4, 0)])
+    (64, 256, 4096, 4, 128), (80, 128, 8192, 8, 0), (100, 512, 4096, 4, 0),
+    # 8-bit codes whose waves walk several steps from a start of their own (one scale per column, and scale groups that
+    # begin before, at and after that start: 32, 128, 192 and 2048 rows), 4-bit codes walking whole chunks with one and two row blocks
+    (20, 1024, 8192, 8, 0), (33, 1024, 8192, 8, 128), (16, 2048, 6144, 8, 192), (70, 512, 8192, 8, 32), (24, 1024, 8192, 8, 2048),
+    (16, 2048, 8192, 4, 128), (32, 1024, 8192, 4, 256), (40, 2048, 4096, 4, 64),
+    # ... and three and four steps per wave (the walk wraps round inside a scale group of 384 rows, and between groups of 32)
+    (20, 4096, 12288, 8, 384), (20, 11008, 4096, 8, 32), (16, 4096, 11008, 8, 0)])
 def test_row_blocked_family_over_packed_weights(af, m, n, k, bits, group):
     """Beyond 48 rows of A the forced DECODE variant is the row-blocked decode family reading packed slabs (8 column
     blocks per workgroup for 8-bit codes, 16 for 4-bit; partial last groups re-read the last block)."""
