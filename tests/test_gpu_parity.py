@@ -256,6 +256,16 @@ def test_tiled_split_k_matches_oracle_and_is_deterministic(af, m, n, k, bits, gr
         assert af.workspace_status(helpers._ws.t) == 0
 
 
+@pytest.mark.parametrize("m,n,k,group", [(1, 2048, 1024, 128), (5, 2432, 512, 0), (20, 4224, 1024, 64), (33, 4112, 512, 128), (16, 6144, 2048, 128)])
+def test_4bit_128_column_form_gives_the_halves_of_a_line_to_paired_workgroups(af, m, n, k, group):
+    """4-bit codes in rows, 128 columns per workgroup: within every whole run of 16 column blocks the kernel hands blocks
+    2j and 2j + 1 (the two halves of a 128-byte line) to workgroups 8 apart; blocks past the last whole run keep their
+    order.  One run, a run and a remainder, two runs and a partial last block, three runs: the oracle's bound."""
+    p = Problem(m, n, k, 4, group, seed=m + n + k)
+    assert af.plan(m, n, k, 4, group, which=af.DECODE).tile_cols == 128
+    assert_close_ulp(p, run_gemm(p, which=af.DECODE), f"4-bit 128-column form {m}x{n}x{k} g{group}")
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 1024, 4096), (16, 640, 2048), (9, 2064, 4096)])
 def test_decode_hand_over_leaves_the_workspace_at_rest_for_every_split_factor(af, m, n, k):
     """The reducer of the 128-column decode kernels keeps two fetch attempts in flight and has one instantiation per
