@@ -208,6 +208,16 @@ def test_tiled_variant_picks_its_tile_size_by_shape(af):
         assert_close_ulp(p, c, f"{m}x{n}")
         forced = af.PREFILL_128 if rows == 128 else af.PREFILL_256X128 if cols == 128 else af.PREFILL_256
         assert np.array_equal(c, run_gemm(p, which=forced, force_split_k=1)), f"{m}x{n}"
+    # two rounds of 128x128 tiles: where 256x128 tiles just miss one round and 256x256 ones would use half the machine
+    # (8-bit codes, 640 x 11008: 430 tiles), and for 4-bit codes up to 345 tiles (1152 x 4096: 288)
+    for (m, n, bits, group, tiles) in [(640, 11008, 8, 0, 430), (1152, 4096, 4, 128, 288), (1152, 4096, 8, 0, 0)]:
+        pl = af.plan(m, n, 256, bits, group, which=af.PREFILL)
+        assert (pl.tile_rows, pl.tile_cols, pl.workgroups) == ((128, 128, tiles) if tiles else (256, 128, 160))
+        p = Problem(m, n, 256, bits, group, seed=m + n + bits)
+        c = run_gemm(p, which=af.PREFILL)
+        assert_close_ulp(p, c, f"{m}x{n} b{bits}")
+        if tiles:
+            assert np.array_equal(c, run_gemm(p, which=af.PREFILL_128, force_split_k=1)), f"{m}x{n} b{bits}"
 
 
 @pytest.mark.parametrize("m,n,k,bits,group", [(256, 128, 64, 8, 0), (300, 272, 448, 8, 0), (700, 1008, 1000, 8, 0), (1000, 1008, 384, 4, 0), (520, 528, 512, 8, 64),
