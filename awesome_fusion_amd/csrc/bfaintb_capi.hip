@@ -463,7 +463,9 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
         // (... and up to 96 MiB of weights: beyond, 256-column blocks win again unless the narrow ones fill their rounds — m = 8 /
         // 16, wide against narrow: 12288 x 12288 29.3 / 31.9 against 34.3 / 37.4 us; 14336 x 8192 24.8 / 26.9 against 26.2 / 28.3;
         // 32000 x 4096, 250 narrow blocks, stays narrow: 25.0 / 25.2 against 23.7 / 24.5)
-        const bool narrow = bits == 8 && (few || fills_rounds || n % 16u != 0 ||
+        // (whole rounds decide up to 160 MiB: 8192 x 28672, 224 MiB, 4 splits x 64 blocks: narrow 41.5 - 47.9 us at m = 1 .. 16, wide
+        // 39.7 - 45.5)
+        const bool narrow = bits == 8 && (few || (fills_rounds && weight_bytes <= (160ull << 20)) || n % 16u != 0 ||
                                           (m >= 8 && (packed || (!many_wide_blocks && weight_bytes <= (96ull << 20)))) || (nibbles && packed));
         pl.cols = narrow ? 128u : 256u;
         // 4-bit codes, 8 to 16 rows: the same 256 columns with 8 waves (twice the waves to hide the activation loads and
