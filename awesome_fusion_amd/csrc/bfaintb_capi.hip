@@ -493,6 +493,25 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 const bool one_round = pl.waves == 8u || bits == 8 || (bits == 4 && col_blocks <= cus / 4u);
                 splits = one_round ? decode_target_wgs_narrow() / col_blocks : (decode_target_wgs() + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
+                // More column blocks of 4-bit codes, 4 waves: rounds of one workgroup per CU count here as well, and a few
+                // workgroups past a round cost 10 - 20 %.  The same cost as for the narrow form (rounds over the splits + what
+                // a split costs) ranks the factors as measured (m = 1, k = 4096, us by splits: 22016 columns 5: 16.4, 6: 17.1,
+                // 7: 17.7, 8: 15.6; 26624 4: 18.0, 5: 21.5, 6: 20.2, 7: 18.9; 33280 3: 21.7, 4: 24.0, 5: 22.7, 6: 23.4;
+                // 45056 2: 29.0, 3: 30.7, 4: 25.4, 5: 28.6; 34816 x 8192 3: 37.9, 4: 41.5, 5: 37.1, 6: 40.3; m = 4 alike).
+                if (!one_round) {
+                    double least = 0.0;
+                    for (uint32_t s = 1; s <= cap && s <= 16u; ++s) {
+                        DecodePlan probe = pl;
+                        set_splits(probe, k, bits, s, packed);
+                        if (probe.splits != s) continue;
+                        // (between one and a half and three rounds: two workgroups of 4 waves per CU are what keeps the
+                        // memory system busy - 22016 x 4096 with 2 splits, 172 workgroups, one round: 18.3 us)
+                        if (col_blocks * s * 2u < cus * 3u || col_blocks * s > cus * 3u) continue;
+                        const double rounds = (double)((col_blocks * s + cus - 1u) / cus);
+                        const double g = rounds / s + 0.04 * s * 4096.0 / k;
+                        if (least == 0.0 || g < least) { least = g; splits = s; }
+                    }
+                }
                 // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each
                 // and whose partial sums the reducing workgroup must collect: beyond 16 splits (32 once k is long enough
                 // for four steps per wave) the launch gets slower again.  Measured at m = 1, 16 splits against what the

@@ -184,6 +184,11 @@ def test_plan_query_agrees_with_the_other_queries_and_follows_the_compute_units(
         c5 = af.plan(2048, 28672, 8192, 4, 128)
         assert (c5.kernel, c5.workgroups, c5.tail_workgroups, c5.launches) == (af.KERNEL_TILES_256, 768, 256, 2)
         assert af.plan(1, 4096, 4096, packed=True).kernel == af.KERNEL_DECODE_SLAB
+        # many 256-column blocks of 4-bit codes, 4 waves: never a few workgroups past a round of one per unit
+        for (n, k, wgs) in ((22016, 4096, 430), (26624, 4096, 416), (33280, 4096, 390), (45056, 4096, 704), (28672, 8192, 448)):
+            w = af.plan(1, n, k, 4, 128)
+            assert (w.tile_cols, w.waves, w.workgroups) == (256, 4, wgs), (n, k, w.as_dict())
+            assert w.workgroups % 256 >= 128
     try:
         for cus in (64, 304):
             af.debug_control(af.DEBUG_PLAN_COMPUTE_UNITS, cus)
