@@ -166,6 +166,10 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
             const double idle = wgs < cus ? pow(wgs / cus, 0.45) : 1.0;
             return 0.80 * (0.65 + 0.35 * m / block_rows) * (5.0 + e.core * idle + e.partial);
         }
+        // (32-row blocks in more than a round and a half of workgroups take 0.82 - 0.86 of it: 48 / 64 x 128256 x 4096 161 / 163 us,
+        // 48 / 64 x 50304 x 4096 79 / 81, where the tiles take 138 / 146 and 66 / 67)
+        const double wgs = (double)((m + 16u * pl.mb - 1u) / (16u * pl.mb)) * (double)((n + pl.cols - 1u) / pl.cols) * pl.splits;
+        if (pl.mb == 2u && wgs * 2.0 > 3.0 * (double)machine_cus()) return 0.84 * ranked;
         return 0.76 * ranked;
     }
     // (64-row blocks: the hand-over at 0.9 of its term — at 0.65 the family ran up to 13 % over the tiles' time at 48 - 64 rows
@@ -187,6 +191,11 @@ static bool prefill_small_tiles(uint32_t m, uint32_t n, int bits)
     const uint64_t cus = machine_cus();
     const uint64_t small = (uint64_t)((m + 127u) / 128u) * ((n + 127u) / 128u);
     if (small <= cus) return true;
+    // One row of tiles: 256-row tiles would spend half their matrix instructions or more on rows that do not exist, however
+    // many rounds the small ones take (us, small / large, 8-bit and 4-bit codes: 64 x 128256 x 4096, 1002 small tiles, 152 / 187
+    // and 148 / 203; 128 x 128256 x 4096 171 / 202 and 163 / 210; 96 x 50304 x 4096, 393 tiles, 71 / 86 and 69 / 101;
+    // 128 x 36864 x 8192, 288 tiles, 134 / 157 and 135 / 135; from 129 rows on the large tiles win: 192 x 50304 x 4096 132 / 97)
+    if (m <= 128u) return true;
     // 4-bit codes: two rounds of small tiles beat one of tall ones while the second round is about a third full (the tall
     // kernel converts every weight in two waves; us, small / tall, on two boxes: 1152 x 4096 x 4096, 288 tiles: 65.8 / 70.7
     // and 68.9 / 70.9; 512 x 11008 x 4096, 344: 65.9 / 71.1; with 384 to 448 tiles the second box had them level or the tall
@@ -260,9 +269,14 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         // 160 / 192 / 224 / 256 workgroups: 0.425 / 0.44 / 0.50 / 0.55; 4-bit g128: 0.49 at 224, 0.55 - 0.56 at 256);
         // rows of a tile that do not exist are not copied (28672 x 8192 4-bit, m = 64 / 96 / 128: 0.435 / 0.45 / 0.48)
         const double wgs = tiles * t.splits;
-        const double load = wgs >= cus ? 1.0 : wgs / cus;
-        const double step_us = ((bits == 4 ? 0.41 : 0.40) + 0.15 * load * load * load) * (0.8 + 0.2 * fill);
-        t.us = 4.0 + (wgs > cus ? 2.0 : 1.0) * per * step_us + hand_over;  // (more small tiles than CUs: two rounds of them)
+        auto step_us = [&](double load) { return ((bits == 4 ? 0.41 : 0.40) + 0.15 * load * load * load) * (0.8 + 0.2 * fill); };
+        // (more small tiles than CUs: whole rounds of them and a last one at the pace of its own load — 96 x 36864 x 8192, 288
+        // tiles: 128 us, 122 over packed weights; 640 x 11008 x 4096, 430: 66; 96 x 50304 x 4096, 393: 72; beyond two rounds the
+        // steps take 10 - 18 % longer than this: 64 / 96 / 128 x 128256 x 4096, four rounds: 152 / 162 / 171 us with 8-bit
+        // codes, 148 / 154 / 163 with 4-bit ones)
+        const double whole = (double)(uint64_t)(wgs / cus), rest = wgs - whole * cus;
+        const double steps_us = whole * step_us(1.0) + (rest > 0.0 ? step_us(rest / cus) : 0.0);
+        t.us = 4.0 + (wgs > 2.0 * cus ? 1.12 : 1.0) * per * steps_us + hand_over;
         // (three splits and more: the hand-over scatters more than this says, and where the row-blocked family is about as
         // fast it is the safer pick — 192 x 4096 x 4096: 25.5 against 22.9 us, 128 x 4096 x 11008: 39.0 against 34.3)
         if (t.splits > 2u) t.us *= 1.07;
@@ -450,7 +464,10 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
             if (best == 0.0 || g < best) { best = g; narrow_splits = s; }
         }
         const uint32_t narrow_wgs = narrow_blocks * narrow_splits;
-        const bool fills_rounds = narrow_wgs * 20u >= ((narrow_wgs + cus - 1u) / cus) * cus * 19u;  // >= 95 % of whole rounds
+        // (one round, at least 95 % full.  Several rounds of narrow workgroups lose to the wide form however well they fill them,
+        // m = 1 / 8 / 16: 36864 x 4096, 6 splits x 288 blocks = 6.75 rounds, 39.8 / 43.3 / 47.9 us, its best factor, 2, 37.1 /
+        // 39.4 / 42.7, wide 31.5 / 33.2 / 35.4; 24576 x 4096, 4 x 192 = 3 rounds, 23.6 / 25.7 / 28.2 against 20.5 / 21.8 / 23.5)
+        const bool fills_rounds = narrow_wgs <= cus && narrow_wgs * 20u >= cus * 19u;
         // m >= 8 on a wide matrix: once 256-column blocks fill their one round with at most 3 splits (more than 64 of
         // them) their partial sums no longer outweigh the better stream (m = 8 / 16 / 32, wide against narrow:
         // 22016 x 4096 20.9 / 22.7 / 28.2 against 21.9 / 23.4 / 31.6 us; 28672 x 8192 46.2 / 48.3 / 54.2 against 49.8 / 53.1 /
@@ -493,6 +510,15 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 const bool one_round = pl.waves == 8u || bits == 8 || (bits == 4 && col_blocks <= cus / 4u);
                 splits = one_round ? decode_target_wgs_narrow() / col_blocks : (decode_target_wgs() + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
+                // One workgroup per column block that leaves 40 % or more of the CUs idle: three splits, one and a half rounds,
+                // once k is long enough to pay for them (m = 8 / 16, 1 split against 3: 4-bit 38400 x 8192 50.4 / 50.8 against
+                // 42.1 / 43.4 us, 34816 x 8192 51.2 / 53.9 against 43.4 / 46.3; 8-bit, m = 1 / 8 / 16, 36864 x 8192 59.2 / 62.5 / 66.4
+                // against 52.8 / 56.6 / 59.9; no difference at k = 4096: 4-bit 38400 x 4096 27.7 / 28.1 against 27.3 / 28.8)
+                if (one_round && splits == 1u && col_blocks * 5u <= cus * 3u && col_blocks * 2u > cus && k > 4096u && cap >= 3u) {
+                    DecodePlan probe = pl;
+                    set_splits(probe, k, bits, 3u, packed);
+                    if (probe.splits == 3u) splits = 3u;
+                }
                 // More column blocks of 4-bit codes, 4 waves: rounds of one workgroup per CU count here as well, and a few
                 // workgroups past a round cost 10 - 20 %.  The same cost as for the narrow form (rounds over the splits + what
                 // a split costs) ranks the factors as measured (m = 1, k = 4096, us by splits: 22016 columns 5: 16.4, 6: 17.1,

@@ -189,6 +189,18 @@ def test_plan_query_agrees_with_the_other_queries_and_follows_the_compute_units(
             w = af.plan(1, n, k, 4, 128)
             assert (w.tile_cols, w.waves, w.workgroups) == (256, 4, wgs), (n, k, w.as_dict())
             assert w.workgroups % 256 >= 128
+        # 8-bit codes: 128-column blocks only where they fit one round (36864 columns would take 6.75 rounds of them) ...
+        w = af.plan(1, 36864, 4096)
+        assert (w.tile_cols, w.waves, w.splits, w.workgroups) == (256, 4, 1, 144)
+        # ... and a half-filled round of 256-column blocks takes three splits once k is beyond 4096
+        assert [af.plan(mm, 36864, 8192, bb, gg).workgroups for (mm, bb, gg) in ((1, 8, 0), (16, 8, 0), (8, 4, 128), (16, 4, 128))] == [432] * 4
+        # one row of tiles is always 128 x 128 tiles, whatever their number; more rows go back to large tiles
+        assert (af.prefill_tile(96, 36864), af.prefill_tile(128, 128256), af.prefill_tile(129, 36864)) == (128, 128, 256)
+        for packed in (False, True):
+            t = af.plan(96, 36864, 8192, packed=packed)
+            assert (t.tile_rows, t.tile_cols, t.workgroups) == (128, 128, 288), (packed, t.as_dict())
+            t = af.plan(64, 128256, 4096, 4, 128, packed=packed)
+            assert t.workgroups == 1002 and (t.tile_rows == 128) == (not packed), (packed, t.as_dict())
     try:
         for cus in (64, 304):
             af.debug_control(af.DEBUG_PLAN_COMPUTE_UNITS, cus)

@@ -210,7 +210,9 @@ def test_tiled_variant_picks_its_tile_size_by_shape(af):
         assert np.array_equal(c, run_gemm(p, which=forced, force_split_k=1)), f"{m}x{n}"
     # two rounds of 128x128 tiles: where 256x128 tiles just miss one round and 256x256 ones would use half the machine
     # (8-bit codes, 640 x 11008: 430 tiles), and for 4-bit codes up to 345 tiles (1152 x 4096: 288)
-    for (m, n, bits, group, tiles) in [(640, 11008, 8, 0, 430), (1152, 4096, 4, 128, 288), (1152, 4096, 8, 0, 0)]:
+    # and one row of them however many: 256-row tiles would be half empty or worse (96 x 36992: 289 tiles; 40 x 50304, 4-bit: 393)
+    for (m, n, bits, group, tiles) in [(640, 11008, 8, 0, 430), (1152, 4096, 4, 128, 288), (1152, 4096, 8, 0, 0), (96, 36992, 8, 0, 289),
+                                       (40, 50304, 4, 128, 393)]:
         pl = af.plan(m, n, 256, bits, group, which=af.PREFILL)
         assert (pl.tile_rows, pl.tile_cols, pl.workgroups) == ((128, 128, tiles) if tiles else (256, 128, 160))
         p = Problem(m, n, 256, bits, group, seed=m + n + bits)

@@ -119,6 +119,10 @@ def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
     (2, 9216, 4096, 8, 0),       # 8-bit, 256 columns x 4 waves on a large matrix: the split that fills one round (7 x 36 workgroups)
     (16, 16640, 2048, 8, 0),     # 8 rows and more, over 64 blocks of 256 columns: those blocks (row-major) instead of 128-column ones
     (24, 16640, 2048, 8, 64),    # the same with two 16-row accumulators per wave
+    (1, 22016, 4096, 4, 128),    # 4-bit, 4 waves, 86 blocks of 256 columns: 5 splits, not the 6 that land 4 workgroups past two rounds
+    (4, 45056, 2048, 4, 128),    # ... 176 blocks: 4 splits, 2.75 rounds
+    (8, 33024, 4224, 8, 0),      # 129 blocks of 256 columns, half a round: three splits once k is beyond 4096
+    (16, 33024, 4224, 4, 128),   # the same for 4-bit codes with 8 waves
 ])
 def test_plan_corners_both_weight_orders(af, m, n, k, bits, group):
     """Shapes on either side of the launch-plan rules for small, narrow and long matrices, kernel left to the library."""

@@ -58,12 +58,12 @@ def test_static_scratch_matches_caller_workspace_on_calls_in_a_row(af):
 
 def test_static_scratch_refuses_what_does_not_fit(af):
     L = af.lib()
-    # 32 rows x 28672 columns, k long enough for 8 splits: 24.5 MiB of partial sums
-    m, n, k = 32, 28672, 28672
-    need = L.bfaintb_gemm_workspace_bytes(m, n, k, 8, 0)
+    # 32 rows x 22016 columns of 4-bit codes, k long enough for 8 splits: 18.8 MiB of partial sums
+    m, n, k = 32, 22016, 28672
+    need = L.bfaintb_gemm_workspace_bytes(m, n, k, 4, 128)
     assert need > L.bfaintb_gemm_static_scratch_bytes() == 16 << 20
     P = 1 << 20  # never dereferenced: the call is refused before any launch
-    assert L.bfaintb_gemm_static(P, P, P, P, m, n, k, k, n, n, 8, 0, None) == af.ERR_STATIC_SCRATCH
+    assert L.bfaintb_gemm_static(P, P, P, P, m, n, k, k, n, n, 4, 128, None) == af.ERR_STATIC_SCRATCH
     assert "bfaintb_gemm" in af.error_string(af.ERR_STATIC_SCRATCH)
 
 
