@@ -1075,11 +1075,17 @@ static double packed8_family_time_us(uint32_t m, uint32_t n, uint32_t k, const D
 static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
 {
     const double rows = m <= 6u ? 1.0 + 0.031 * (m - 1.0) : m <= 16u ? 1.155 + 0.078 * (m - 6.0) : 1.267 + 0.0776 * m;
-    return 2.58 + packed_slab_walks(n) * k / 1975.0 * rows;
+    // (more than seven slabs per CU: 5 % less than that — 32000 / 50304 / 128256 / 151936 x 4096, m = 1: 17.6 / 26.2 / 63.4 / 74.8 us;
+    // 28672 x 8192, seven, is as the formula says: 31.1)
+    const double many = n / 16.0 > 7.0 * (double)machine_cus() ? 0.95 : 1.0;
+    return 2.58 + many * packed_slab_walks(n) * k / 1975.0 * rows;
 }
 static double packed4_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
 {
-    const double stream_us = (double)n * k / 2.0e6 / (4.37 * pow(packed_family_fill(m, n, pl), 0.58));
+    // (more than one round of workgroups: 8 % more than the fill says — 50304 / 128256 / 151936 x 4096, m = 1: 35.6 / 71.6 / 86.8 us,
+    // m = 16: 37.4 / 75.4 / 91.5)
+    const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits * ((m + 16u * pl.mb - 1u) / (16u * pl.mb));
+    const double stream_us = (double)n * k / 2.0e6 / (4.37 * pow(packed_family_fill(m, n, pl), 0.58)) * (wgs > (double)machine_cus() ? 1.08 : 1.0);
     return 4.71 + 0.067 * m + 0.144 * (pl.splits - 1.0) + stream_us * (1.0 + 0.0003 * m + (m > 16u ? 0.258 : 0.0));
 }
 static bool packed_uses_slab(uint32_t m, uint32_t n, uint32_t k, int bits)
