@@ -538,6 +538,21 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                         if (least == 0.0 || g < least) { least = g; splits = s; }
                     }
                 }
+                // More column blocks than two rounds, fewer than 8 rows: the same cost picks among 1 to 4 splits (m = 1, 151936 x
+                // 4096, 594 blocks, us with 1 / 2 / 3 / 4 splits: 8-bit 102.7 / 96.1 / 95.7 / 98.2, 4-bit 85.6 / 80.0 / 80.7 / 83.0;
+                // 128256 x 4096, 501 blocks, 1.96 rounds, stays whole: 78.4 / 80.5 and 56.9 / 58.7; from 8 rows on the partial
+                // sums take the gain back: m = 8, 594 blocks: 103.2 / 101.4 / 104.4)
+                if (col_blocks > 2u * cus && m < 8u) {
+                    double least = 0.0;
+                    for (uint32_t s = 1; s <= cap && s <= 4u; ++s) {
+                        DecodePlan probe = pl;
+                        set_splits(probe, k, bits, s, packed);
+                        if (probe.splits != s) continue;
+                        const double rounds = (double)((col_blocks * s + cus - 1u) / cus);
+                        const double g = rounds / s + 0.04 * s * 4096.0 / k;
+                        if (least == 0.0 || g < least) { least = g; splits = s; }
+                    }
+                }
                 // a narrow matrix reaches that target only with very many splits, whose waves then run a single step each
                 // and whose partial sums the reducing workgroup must collect: beyond 16 splits (32 once k is long enough
                 // for four steps per wave) the launch gets slower again.  Measured at m = 1, 16 splits against what the
