@@ -59,11 +59,14 @@ __device__ __forceinline__ void tw_mfma(f32x4_t& acc, const bf16x8_t& a, const b
 __device__ __forceinline__ void tw_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 }  // namespace
 
-template <int BITS, bool GROUPED, bool PACKED, int KH, bool COPIER>
+// MT: the blocks of 16 rows of the tile that are multiplied (8, or 4 for an m of at most 64: the rows beyond take no
+// matrix instructions, no fragment reads and no accumulators; everything about the weights stays as it is).
+template <int BITS, bool GROUPED, bool PACKED, int KH, bool COPIER, int MT>
 __global__ void __launch_bounds__(256 * KH + (COPIER ? 64 : 0)) __attribute__((amdgpu_waves_per_eu(KH + (COPIER ? 1 : 0), KH + (COPIER ? 1 : 0))))
 bfaintb_prefill128_wreg_kernel(const GemmParams p)
 {
     static_assert(KH == 1 || KH == 2, "one wave per SIMD, or two that share a K-step by its blocks of 32 k");
+    static_assert(MT == 8 || MT == 4, "whole tiles, or their first 64 rows");
     constexpr uint32_t kWaves = 4u * KH;
     constexpr uint32_t NB = 2u / KH;  // blocks of 32 k of a K-step that a wave multiplies
     __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[kTwStage];
@@ -473,9 +476,11 @@ bfaintb_prefill128_wreg_kernel(const GemmParams p)
             const bf16x8_t wf0 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][0][0], cur.w[blk][0][1], cur.w[blk][0][2], cur.w[blk][0][3]));
             const bf16x8_t wf1 = __builtin_bit_cast(bf16x8_t, make_uint4(cur.w[blk][1][0], cur.w[blk][1][1], cur.w[blk][1][2], cur.w[blk][1][3]));
             // ---- slot 0
-            tw_mfma(acc[mt][0], a_now, wf0);
-            if (u + kAhead < kUnits) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
-            else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - kUnits) * 2048u);
+            if (mt < (uint32_t)MT) tw_mfma(acc[mt][0], a_now, wf0);
+            if (((u + kAhead) & 7u) < (uint32_t)MT) {  // (the fragment of a row block that is multiplied)
+                if (u + kAhead < kUnits) af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_src + a_rd[(u + kAhead) >> 3] + ((u + kAhead) & 7u) * 2048u);
+                else af[u % kAhead] = *reinterpret_cast<const bf16x8_t*>(a_nxt + a_rd[0] + (u + kAhead - kUnits) * 2048u);
+            }
             if constexpr (PACKED) {
                 packed_values(pc, nb, cblk, cj, cpr, f0, f1);
             } else {
@@ -496,7 +501,7 @@ bfaintb_prefill128_wreg_kernel(const GemmParams p)
             }
             __builtin_amdgcn_sched_barrier(0);
             // ---- slot 1
-            tw_mfma(acc[mt][1], a_now, wf1);
+            if (mt < (uint32_t)MT) tw_mfma(acc[mt][1], a_now, wf1);
             // (the group scales first: the next step waits for them at its very start, and that wait then leaves the
             // copies requested behind them in flight — requested last, they made it a wait for everything)
             // (one block's scales per slot: finding a group is a chain of five scalar instructions)
@@ -565,7 +570,7 @@ bfaintb_prefill128_wreg_kernel(const GemmParams p)
     // own to them — first blocks + second blocks, whatever the timing)
     auto stage_sums = [&](bool add) {
 #pragma unroll
-        for (uint32_t mt = 0; mt < 8; ++mt) {
+        for (uint32_t mt = 0; mt < (uint32_t)MT; ++mt) {
             float* base = c_rows(mt >> 1);
 #pragma unroll
             for (uint32_t r = 0; r < 4; ++r) {
@@ -775,7 +780,9 @@ static hipError_t launch_prefill128_wreg_t(const GemmParams& p, hipStream_t stre
     const uint32_t tiles = ((p.m + kTw - 1) / kTw) * ((p.n + kTw - 1) / kTw);
     const uint32_t grid = (tiles + 7u) / 8u * 8u;  // a whole number of workgroups per XCD; ids past the last tile exit at once
     // two waves per column group; with grouped scales, the copying wave on top
-    void (*kernel)(const GemmParams) = bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED, 2, GROUPED>;
+    // (at most 64 rows in all: the form that multiplies only the first four blocks of 16 rows)
+    void (*kernel)(const GemmParams) = p.m <= 64u ? bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED, 2, GROUPED, 4>
+                                                  : bfaintb_prefill128_wreg_kernel<BITS, GROUPED, PACKED, 2, GROUPED, 8>;
     return launch_kernel(kernel, dim3(grid, p.splits, 1), dim3(512 + (GROUPED ? 64 : 0), 1, 1), 0, stream, p);
 }
 
