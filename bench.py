@@ -471,6 +471,9 @@ PLAN_CHECK_SHAPES = [
     (64, 11008, 4096, 8, 0), (64, 8192, 8192, 8, 0), (96, 4096, 4096, 8, 0), (192, 4096, 4096, 8, 0), (128, 4096, 11008, 8, 0),
     (896, 4096, 4096, 8, 0), (64, 8192, 8192, 4, 128), (64, 28672, 8192, 4, 128), (96, 4096, 4096, 4, 128), (128, 4096, 4096, 4, 128),
     (192, 4096, 4096, 4, 128), (256, 4096, 4096, 4, 128),
+    # very wide matrices (output layers): the split factors of 256-column blocks by rounds, one row of small tiles
+    (1, 22016, 4096, 4, 128), (1, 128256, 4096, 8, 0), (1, 151936, 4096, 4, 128), (8, 36864, 8192, 8, 0), (64, 50304, 4096, 8, 0),
+    (96, 36864, 8192, 8, 0),
 ]
 
 
