@@ -1157,7 +1157,10 @@ static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
     const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits * (double)(uint64_t)((m + block_rows - 1.0) / block_rows);
     const double cus = (double)machine_cus();
     const double idle = wgs < cus ? pow(wgs / cus, 0.45) : 1.0;
-    return (pl.mb == 4u ? 0.84 : 0.76) * (0.65 + 0.35 * fill) * (5.0 + e.core * idle + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
+    // (a single block, since its kernels start each workgroup's walk over k at a step of its own: 0.92 of that — at 64 rows
+    // the family leads the tiles by 5 - 8 % on 11008 x 8192, 28672 x 8192, 32000 x 4096, 14336 x 8192, 12288 x 12288)
+    const double base = m <= block_rows ? 0.57 : 0.65;
+    return (pl.mb == 4u ? 0.84 : 0.76) * (base + 0.35 * fill) * (5.0 + e.core * idle + (pl.mb == 4u ? 0.7 : 0.35) * e.partial);
 }
 // Which kernel multiplies by packed weights: the decode kernels (the slab-streaming one while packed_uses_slab, the
 // row-blocked family without a split along k beyond) or the tiled kernel, by the estimates that choose for row-major weights.
