@@ -192,7 +192,15 @@ __device__ __forceinline__ void decode_packed_body(const GemmParams& p)
     const uint32_t lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t nl = lane & 15u, kg = lane >> 4;
-    const uint32_t nb = blockIdx.x, rb = blockIdx.z;
+    uint32_t nb = blockIdx.x;
+    const uint32_t rb = blockIdx.z;
+    if constexpr (GROUPED) {
+        // Four neighbouring slabs share a 128-byte line of every row of scales.  Workgroups that follow one another in
+        // dispatch order sit on different XCDs, each with an L2 of its own, and every one of the four fetched that line
+        // from memory.  Within whole runs of 32 workgroups, the four that share an XCD (ids 8 apart) take four neighbouring slabs.
+        const uint32_t run = nb & ~31u;
+        if (run + 32u <= gridDim.x) nb = run + 4u * (nb & 7u) + ((nb >> 3) & 3u);
+    }
     const uint32_t chunks = p.k / kChunkRows;
 
     const uint8_t* slab = p.b + ((size_t)nb * chunks) * 1024u + lane * 16u;
