@@ -132,6 +132,16 @@ def test_plan_corners_both_weight_orders(af, m, n, k, bits, group):
     assert_close_ulp(p, run_prepacked(af, p), f"packed {m}x{n}x{k} b{bits} g{group}")
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [(1, 640, 1024, 4, 128), (3, 1040, 512, 8, 64), (2, 496, 1024, 4, 256), (1, 1024, 2048, 8, 128)])
+def test_slab_kernel_hands_neighbouring_slabs_to_one_xcd_with_grouped_scales(af, m, n, k, bits, group):
+    """With grouped scales the slab kernel gives the four slabs that share a 128-byte line of scales to workgroups 8 apart
+    in dispatch order, within whole runs of 32 slabs; the slabs past the last whole run keep their place (40 slabs: one run
+    and 8; 65: two and one; 31: none; 64: two whole runs).  Every column must still come out of its own slab."""
+    assert af.plan(m, n, k, bits, group, packed=True).kernel == af.KERNEL_DECODE_SLAB
+    p = Problem(m, n, k, bits, group, seed=n + k + bits)
+    assert_close_ulp(p, run_prepacked(af, p), f"slab kernel {m}x{n}x{k} b{bits} g{group}")
+
+
 @pytest.mark.parametrize("m,n,k,bits,group", [
     (49, 128, 512, 8, 0), (64, 4096, 1024, 8, 0), (100, 272, 448, 8, 64), (130, 48, 1024, 8, 32), (200, 1040, 256, 8, 0), (300, 144, 2048, 8, 128),
     (64, 256, 512, 4, 0), (97, 528, 1024, 4, 128), (150, 80, 640, 4, 32), (260, 1296, 384, 4, 128),
