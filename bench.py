@@ -820,7 +820,7 @@ def main():
         del w
         torch.cuda.empty_cache()
 
-    # ---- BASELINE's decode sweep (N = 11008) and 4-bit group-128 shape (28672 x 8192): compact roofline rows
+    # ---- the headline benchmark's decode sweep (N = 11008) and 4-bit group-128 shape (28672 x 8192): compact roofline rows
     if args.only == "":
         rows = []
         w32 = config3_workload(32)

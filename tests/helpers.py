@@ -135,7 +135,7 @@ NEAR_ZERO = 0.125    # ... and only for outputs below this fraction of rms(C)
 
 
 def allowed_outside(outputs, rate=3e-5):
-    """How many outputs of a check may take the near-zero escape: the rate seen at the full-size BASELINE shapes is
+    """How many outputs of a check may take the near-zero escape: the rate seen at the full-size benchmark shapes is
     1.4e-5 to 2.1e-5 of the outputs (228 of 16.7 M at config 4, 98 of 4.6 M at config 5); allowed is 3e-5 of them plus
     four standard deviations of a count of that mean, and a handful for small problems — so that a kernel whose
     cancelling outputs are a few times worse than today's fails at the sizes where it can be told from chance
@@ -154,7 +154,7 @@ def assert_close_ulp(p, c_bits, what, rows=None, threads=8):
     ACCEPTANCE_LOG); each must be small (|ref| < rms(C) * NEAR_ZERO: an output of ordinary size has no such excuse)
     and must lie within 2 ULP + NOISE_FACTOR * 2^-24 * sum_k |a_k w_k| of the fp64-accumulated value.  The second
     term is a few times the rounding error an fp32 sum of those terms makes in any order (measured worst
-    over the BASELINE shapes: 1.3 of these units for the device, 4.4 for the sequential oracle); one
+    over the benchmark shapes: 1.3 of these units for the device, 4.4 for the sequential oracle); one
     dropped or doubled term of ordinary size is a thousand of them.
     Returns (worst error in ULP among the outputs inside the bound, number of outputs that took the escape)."""
     a = p.a_bf if rows is None else p.a_bf[rows]
