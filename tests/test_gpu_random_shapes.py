@@ -147,6 +147,20 @@ def test_ragged_shapes(af, m, n, k, bits, group, variant):
     assert_close_ulp(p, run_ragged(af, p, which, pad=8), f"ragged {m}x{n}x{k} int{bits} g{group} {variant}")
 
 
+@pytest.mark.parametrize("m,n,k,bits,group", [
+    (1, 33000, 512, 8, 0),       # n % 16 != 0: only 128-column blocks can read the last columns — 258 of them, two past a round
+    (5, 45072, 2048, 4, 128),    # 4-bit, 4 waves: 177 blocks of 256 columns, the last one 16 columns wide, k split four ways by rounds
+    (12, 36880, 4224, 4, 128),   # 8 waves, a half-filled round of 256-column blocks split three ways, a 16-column last block
+    (64, 36872, 192, 8, 0),      # one row of 289 small tiles in their 64-row form, the last tile 8 columns wide
+    (40, 50320, 256, 4, 64),     # the same for 4-bit codes: 394 tiles, 16 columns in the last
+    (70, 33032, 128, 8, 0),      # ... and with more than 64 rows: the whole-tile form, 259 tiles
+])
+def test_very_wide_ragged_shapes(af, m, n, k, bits, group):
+    """Column counts beyond 32768 that do not end on a block or tile, kernel left to the library; rows of B and C padded by 8 elements."""
+    p = Problem(m, n, k, bits, group, seed=m + n + k)
+    assert_close_ulp(p, run_ragged(af, p, af.AUTO, pad=8), f"very wide {m}x{n}x{k} bits={bits} g={group}")
+
+
 def draw_ragged(rng):
     bits = int(rng.choice([8, 8, 4]))
     m = int(rng.choice([rng.integers(1, 9), rng.integers(9, 49), rng.integers(49, 200), rng.integers(200, 500)]))
