@@ -371,6 +371,17 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
             if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
         }
     }
+    // 4-bit codes in rows, one block of 32 rows, one workgroup per column block and 40 % or more of the CUs idle: three splits,
+    // as for 16 rows (decode_plan) — the estimate's price of a split keeps it from them while k is short (m = 24 / 32,
+    // 36864 x 4096: 40.7 / 41.0 us unsplit, 36.6 / 37.6 split three ways; with k = 8192 the estimate picks the three itself)
+    if (bits == 4 && !packed && forced_splits == 0 && m <= 32u && best.mb == 2u && best.splits == 1u && best.cols == 256u) {
+        const uint32_t cus = machine_cus(), col_blocks = (n + 255u) / 256u;
+        if (col_blocks * 2u > cus && col_blocks * 5u <= cus * 3u) {
+            DecodePlan probe = best;
+            set_splits(probe, k, bits, 3u, packed);
+            if (probe.splits == 3u) best = probe;
+        }
+    }
     return best;
 }
 

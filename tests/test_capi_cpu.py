@@ -196,6 +196,8 @@ def test_plan_query_agrees_with_the_other_queries_and_follows_the_compute_units(
         assert [af.plan(mm, 36864, 8192, bb, gg).workgroups for (mm, bb, gg) in ((1, 8, 0), (16, 8, 0), (8, 4, 128), (16, 4, 128))] == [432] * 4
         # more than two rounds of 256-column blocks, fewer than 8 rows: the split that wastes the least of its last round
         assert [af.plan(1, n, 4096).splits for n in (128256, 131328, 151936)] == [1, 4, 3] and af.plan(8, 151936, 4096).splits == 1
+        # ... also for one 32-row block of 4-bit codes while k is short (the estimate alone would not split there)
+        assert [af.plan(mm, 36864, 4096, 4, 128).workgroups for mm in (17, 32)] == [432, 432]
         # one row of tiles is always 128 x 128 tiles, whatever their number; more rows go back to large tiles
         assert (af.prefill_tile(96, 36864), af.prefill_tile(128, 128256), af.prefill_tile(129, 36864)) == (128, 128, 256)
         for packed in (False, True):
