@@ -563,7 +563,7 @@ def roofline_entry(w, ms, bound, suffix=""):
     return out
 
 
-def cpu_baseline(w, c_gpu_f32, budget_s=8.0):
+def cpu_baseline(w, c_gpu_f32, budget_s=14.0):
     """host_ref.hpp's gemm_rrr timed on this machine's cores on the same inputs the GPU consumed:
     the reference's own compiled routine when the wrapper library is present, else the C port."""
     import ctypes as C
@@ -590,7 +590,7 @@ def cpu_baseline(w, c_gpu_f32, budget_s=8.0):
         call(0, n)
         reps += 1
         el = time.perf_counter() - t0
-        if el > budget_s * 0.6 or reps >= 50:
+        if el > budget_s * 0.6 or reps >= 100:
             break
     t1 = el / reps
     c_single = c.copy()
