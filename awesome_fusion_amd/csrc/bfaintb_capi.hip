@@ -163,7 +163,10 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
         if (m <= block_rows && pl.cols == 128u) {
             // (and CUs left idle slow the stream less than in proportion, as over packed weights: 86 column blocks x 2 splits)
             const double wgs = (double)((n + pl.cols - 1u) / pl.cols) * pl.splits, cus = (double)machine_cus();
-            const double idle = wgs < cus ? pow(wgs / cus, 0.45) : 1.0;
+            // (not below 0.65 of a round: 144 and 160 column blocks, unsplit, take all the estimate says and more — 18432 x 6144,
+            // m = 40 / 64: 44.6 / 52.8 us, where the tiles with k split three ways take 41.9 / 43.7; 20480 x 4096, m = 64: 39.0
+            // against the tiles' 34.8)
+            const double idle = wgs < cus && wgs * 20.0 >= cus * 13.0 ? pow(wgs / cus, 0.45) : 1.0;
             return 0.80 * (0.65 + 0.35 * m / block_rows) * (5.0 + e.core * idle + e.partial);
         }
         // (32-row blocks in more than a round and a half of workgroups take 0.82 - 0.86 of it: 48 / 64 x 128256 x 4096 161 / 163 us,
@@ -292,6 +295,17 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         // (at most 256 tiles' worth of sums in all, 14 MiB: within the 32-bit offsets of the kernel and within the scratch of
         // the entry point that brings its own)
         if (t.us < best.us) best = t;
+    }
+    // One row of tiles that leaves 40 % or more of the CUs idle (half to 0.6 of a round) and a long k: three splits, a round
+    // and two thirds of workgroups, as the decode family does on such widths — the estimate has the two forms level, the
+    // machine does not (us, unsplit / three splits, 8-bit and 4-bit codes: 48 x 18432 x 8192 56.0 / 47.2 and 50.3 / 42.9;
+    // 96 x 18432 x 8192 62.1 / 57.3 and 59.2 / 54.0; 48 x 19200 x 8192 55.5 / 47.8; with k = 4096 the split loses: 25.1 / 27.2).
+    // (While the partial sums stay within the 14 MiB of the note above.)
+    if (best.splits == 1u && m <= 128u && tiles * 2.0 > cus && tiles * 5.0 <= cus * 3.0 && k >= 6144u &&
+        2ull * m * n * sizeof(float) <= (14ull << 20)) {
+        TilePlan t = shape(3);
+        t.us *= 0.88;  // (measured against what shape() says of them: 0.85 - 0.92)
+        if (t.splits == 3u) best = t;
     }
     return best;
 }
