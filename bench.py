@@ -473,7 +473,7 @@ PLAN_CHECK_SHAPES = [
     (192, 4096, 4096, 4, 128), (256, 4096, 4096, 4, 128),
     # very wide matrices (output layers): the split factors of 256-column blocks by rounds, one row of small tiles
     (1, 22016, 4096, 4, 128), (1, 128256, 4096, 8, 0), (1, 151936, 4096, 4, 128), (8, 36864, 8192, 8, 0), (64, 50304, 4096, 8, 0),
-    (96, 36864, 8192, 8, 0),
+    (96, 36864, 8192, 8, 0), (48, 18432, 8192, 8, 0), (48, 18432, 8192, 4, 128),
 ]
 
 
