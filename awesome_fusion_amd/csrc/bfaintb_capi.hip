@@ -296,12 +296,15 @@ static TilePlan tile128_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint3
         // the entry point that brings its own)
         if (t.us < best.us) best = t;
     }
-    // One row of tiles that leaves 40 % or more of the CUs idle (half to 0.6 of a round) and a long k: three splits, a round
-    // and two thirds of workgroups, as the decode family does on such widths — the estimate has the two forms level, the
-    // machine does not (us, unsplit / three splits, 8-bit and 4-bit codes: 48 x 18432 x 8192 56.0 / 47.2 and 50.3 / 42.9;
-    // 96 x 18432 x 8192 62.1 / 57.3 and 59.2 / 54.0; 48 x 19200 x 8192 55.5 / 47.8; with k = 4096 the split loses: 25.1 / 27.2).
+    // One row of tiles that leaves a third or more of the CUs idle (half to five eighths of a round) and a long k: three
+    // splits, as the decode family does on such widths — the estimate has the two forms level, the machine does not (us,
+    // unsplit / three splits, 8-bit and 4-bit codes: 48 x 18432 x 8192, 144 tiles, 56.0 / 47.2 and 50.3 / 42.9; 96 x 18432 x
+    // 8192 62.1 / 57.3 and 59.2 / 54.0; 48 x 20480 x 8192, 160 tiles, 60.3 / 51.1 and 50.6 / 43.1).  The launch rounds a split's
+    // workgroups up to a multiple of 8, and three splits must stay clear of two rounds: 170 tiles make 528 and lose (57.9 /
+    // 69.7).  A shorter k gains little or loses (k = 6144: 35.3 / 33.4 at 48 rows, 42.5 / 43.4 at 96; k = 4096: 25.1 / 27.2).
     // (While the partial sums stay within the 14 MiB of the note above.)
-    if (best.splits == 1u && m <= 128u && tiles * 2.0 > cus && tiles * 5.0 <= cus * 3.0 && k >= 6144u &&
+    const double per_split = (double)(uint64_t)((tiles + 7.0) / 8.0) * 8.0;
+    if (best.splits == 1u && m <= 128u && tiles * 2.0 > cus && per_split * 3.0 * 16.0 <= cus * 31.0 && k >= 8192u &&
         2ull * m * n * sizeof(float) <= (14ull << 20)) {
         TilePlan t = shape(3);
         t.us *= 0.88;  // (measured against what shape() says of them: 0.85 - 0.92)
@@ -385,12 +388,12 @@ DecodePlan decode_plan_row_blocks(uint32_t m, uint32_t n, uint32_t k, int bits, 
             if (best_t == 0.0 || t < best_t) { best_t = t; best = c; }
         }
     }
-    // 4-bit codes in rows, one block of 32 rows, one workgroup per column block and 40 % or more of the CUs idle: three splits,
+    // 4-bit codes in rows, one block of 32 rows, one workgroup per column block and a third or more of the CUs idle: three splits,
     // as for 16 rows (decode_plan) — the estimate's price of a split keeps it from them while k is short (m = 24 / 32,
     // 36864 x 4096: 40.7 / 41.0 us unsplit, 36.6 / 37.6 split three ways; with k = 8192 the estimate picks the three itself)
     if (bits == 4 && !packed && forced_splits == 0 && m <= 32u && best.mb == 2u && best.splits == 1u && best.cols == 256u) {
         const uint32_t cus = machine_cus(), col_blocks = (n + 255u) / 256u;
-        if (col_blocks * 2u > cus && col_blocks * 5u <= cus * 3u) {
+        if (col_blocks * 2u > cus && col_blocks * 3u <= cus * 2u) {
             DecodePlan probe = best;
             set_splits(probe, k, bits, 3u, packed);
             if (probe.splits == 3u) best = probe;
@@ -535,11 +538,13 @@ DecodePlan decode_plan(uint32_t m, uint32_t n, uint32_t k, int bits, uint32_t fo
                 const bool one_round = pl.waves == 8u || bits == 8 || (bits == 4 && col_blocks <= cus / 4u);
                 splits = one_round ? decode_target_wgs_narrow() / col_blocks : (decode_target_wgs() + col_blocks / 2) / col_blocks;
                 if (splits > cap) splits = cap;
-                // One workgroup per column block that leaves 40 % or more of the CUs idle: three splits, one and a half rounds,
+                // One workgroup per column block that leaves a third or more of the CUs idle: three splits, one and a half to two rounds,
                 // once k is long enough to pay for them (m = 8 / 16, 1 split against 3: 4-bit 38400 x 8192 50.4 / 50.8 against
                 // 42.1 / 43.4 us, 34816 x 8192 51.2 / 53.9 against 43.4 / 46.3; 8-bit, m = 1 / 8 / 16, 36864 x 8192 59.2 / 62.5 / 66.4
                 // against 52.8 / 56.6 / 59.9; no difference at k = 4096: 4-bit 38400 x 4096 27.7 / 28.1 against 27.3 / 28.8)
-                if (one_round && splits == 1u && col_blocks * 5u <= cus * 3u && col_blocks * 2u > cus && k > 4096u && cap >= 3u) {
+                // (up to two thirds of a round, so that the three splits stay within two rounds: 40960 x 8192, 160 blocks, m = 1 / 8 / 16:
+                // 8-bit 61.4 / 64.9 / 68.6 against 55.3 / 59.1 / 62.7, 4-bit at m = 8 / 16 54.0 / 57.1 against 45.4 / 48.9; 170 blocks alike)
+                if (one_round && splits == 1u && col_blocks * 3u <= cus * 2u && col_blocks * 2u > cus && k > 4096u && cap >= 3u) {
                     DecodePlan probe = pl;
                     set_splits(probe, k, bits, 3u, packed);
                     if (probe.splits == 3u) splits = 3u;

@@ -198,10 +198,10 @@ def test_plan_query_agrees_with_the_other_queries_and_follows_the_compute_units(
         assert [af.plan(1, n, 4096).splits for n in (128256, 131328, 151936)] == [1, 4, 3] and af.plan(8, 151936, 4096).splits == 1
         # ... also for one 32-row block of 4-bit codes while k is short (the estimate alone would not split there)
         assert [af.plan(mm, 36864, 4096, 4, 128).workgroups for mm in (17, 32)] == [432, 432]
-        # one row of small tiles on half to 0.6 of a round, k of 6144 or more: three splits, while the sums stay within 14 MiB
+        # one row of small tiles on half to five eighths of a round, k of 8192 or more: three splits, while the sums stay within 14 MiB
         t = af.plan(48, 18432, 8192)
         assert (t.kernel, t.splits, t.workgroups) == (af.KERNEL_TILES_128, 3, 432) and t.workspace_bytes == 256 + 2 * 48 * 18432 * 4
-        assert af.plan(48, 18432, 4096).splits == 1 and af.plan(128, 18432, 8192).splits == 1
+        assert af.plan(48, 18432, 4096).splits == 1 and af.plan(128, 18432, 8192).splits == 1 and af.plan(48, 21760, 8192).splits == 1
         assert af.plan(96, 18432, 8192).workspace_bytes <= af.lib().bfaintb_gemm_static_scratch_bytes()
         # one row of tiles is always 128 x 128 tiles, whatever their number; more rows go back to large tiles
         assert (af.prefill_tile(96, 36864), af.prefill_tile(128, 128256), af.prefill_tile(129, 36864)) == (128, 128, 256)

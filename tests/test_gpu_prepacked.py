@@ -125,8 +125,8 @@ def test_decode_kernel_matches_oracle(af, m, n, k, bits, group):
     (16, 33024, 4224, 4, 128),   # the same for 4-bit codes with 8 waves
     (1, 131328, 512, 8, 0),      # 513 blocks of 256 columns, one past two rounds: k is split (two ways at this k)
     (24, 33024, 4096, 4, 128),   # one 32-row block of 4-bit codes over 129 blocks of 256 columns: three splits also at this k
-    (48, 18432, 6144, 8, 0),     # one row of 144 small tiles and a long k: k split three ways, 432 workgroups in two rounds
-    (40, 17408, 6144, 4, 128),   # the same with 4-bit codes and scale groups, 136 tiles
+    (40, 16512, 8192, 8, 0),     # one row of 129 small tiles and a long k: k split three ways, 387 workgroups in two rounds
+    (40, 17408, 8192, 4, 128),   # the same with 4-bit codes and scale groups, 136 tiles
 ])
 def test_plan_corners_both_weight_orders(af, m, n, k, bits, group):
     """Shapes on either side of the launch-plan rules for small, narrow and long matrices, kernel left to the library."""
