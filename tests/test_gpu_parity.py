@@ -497,6 +497,8 @@ def test_fused_bias(af, m, n, k, bits, group):
     (4200, 528, 256, 4, 128),   # tiled kernel (128x128 tiles), 4-bit
     (4200, 1040, 128, 8, 0),    # more than 256 small tiles: 256x256 tiles, ragged rows and columns
     (4200, 1296, 256, 4, 128),  # 256x256 tiles, 4-bit
+    (40, 33024, 256, 8, 0),     # one row of 258 small tiles in their 64-row form
+    (33, 16512, 8192, 8, 0),    # ... of 129 with k split three ways: the reducing workgroups add bias and residual
 ])
 def test_fused_residual(af, m, n, k, bits, group):
     """C = bf16(sum + bias + residual): against the oracle's fp32 sums plus the two fp32 additions, with and without the
@@ -539,6 +541,7 @@ GATED_SHAPES = [
     (4200, 544, 256, 4, 128),   # tiled kernel (128x128 tiles), 4-bit
     (4200, 1056, 128, 8, 0),    # more than 256 small tiles: 256x256 tiles
     (4200, 1312, 256, 4, 128),  # 256x256 tiles, 4-bit
+    (40, 33024, 256, 8, 0),     # one row of 258 small tiles in their 64-row form
 ]
 
 
