@@ -43,9 +43,10 @@ def _both(af, p):
 def test_static_scratch_matches_caller_workspace_on_calls_in_a_row(af):
     # the second input is smaller than the first (it finds the scratch as the first call left it), the third larger
     # again and 4-bit with group scales, the fourth runs without split-K (the tiled kernel: the scratch is not touched),
-    # the fifth is the tiled kernel with k split (its partial sums go through the scratch as well)
+    # the fifth is the tiled kernel with k split (its partial sums go through the scratch as well), the sixth one row of
+    # small tiles with k split three ways, two rounds of workgroups
     shapes = [(16, 4096, 4096, 8, 0), (1, 1024, 2048, 8, 0), (4, 4096, 8192, 4, 128), (300, 512, 256, 8, 0), (384, 2048, 8192, 8, 0),
-              (1, 4096, 4096, 8, 0)]
+              (33, 16512, 8192, 8, 0), (1, 4096, 4096, 8, 0)]
     used_split = 0
     for i, (m, n, k, bits, group) in enumerate(shapes):
         p = Problem(m, n, k, bits, group, seed=40 + i)
@@ -53,7 +54,7 @@ def test_static_scratch_matches_caller_workspace_on_calls_in_a_row(af):
         used_split += need > 0
         assert np.array_equal(c_static, c_plain), f"call {i}: {shapes[i]}"
         assert not np.isnan(c_plain.view(np.uint16).astype(np.uint32) << 16).any()
-    assert used_split >= 5  # the comparison did exercise the scratch
+    assert used_split >= 6  # the comparison did exercise the scratch
 
 
 def test_static_scratch_refuses_what_does_not_fit(af):
