@@ -117,6 +117,7 @@ static void set_splits(DecodePlan& pl, uint32_t k, int bits, uint32_t splits, bo
 // arithmetic and the stream slow down in proportion.  Fitted to measurements at N = 4096, 11008 and 28672.
 struct FamilyEstimate {
     double core, partial;  // the stream or the arithmetic, whichever is longer; the split's hand-over
+    double serial;         // what the ranking adds for the reducing workgroup's own fetches (not part of the time estimates)
 };
 static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl, FamilyEstimate* parts = nullptr)
 {
@@ -140,8 +141,12 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
     const double stream_busy = bits == 8 ? (wgs >= cus ? 1.0 : wgs / cus) : busy;
     const double stream = weights * bits / 8.0 * (1.0 + (bits == 8 ? 0.5 : 0.3) * (row_blocks - 1.0)) / 3.5e6 / stream_busy;
     const double partial = pl.splits > 1 ? 3.0 + 12.0 * (pl.splits - 1.0) * m * n / 1.5e6 : 0.0;
-    if (parts != nullptr) *parts = FamilyEstimate{compute > stream ? compute : stream, partial};
-    return 5.0 + (compute > stream ? compute : stream) + partial;
+    // (for the ranking only: the reducing workgroup fetches the other splits' sums of its block one after the other through
+    // its one CU — the larger the block and the more the splits, the longer.  48 x 2560 x 16384: 64-row blocks with k split
+    // 12 ways 27.0 us, 32-row blocks split 6 ways, the same number of workgroups, 20.6)
+    const double serial = pl.splits > 1 ? 0.0075 * (pl.splits - 1.0) * pl.mb * pl.mb * pl.mb : 0.0;
+    if (parts != nullptr) *parts = FamilyEstimate{compute > stream ? compute : stream, partial, serial};
+    return 5.0 + (compute > stream ? compute : stream) + partial + serial;
 }
 
 // The same estimate, corrected to what the family's own plan takes in absolute terms: the estimate above ranks the
@@ -154,7 +159,7 @@ static double decode_family_estimate_us(uint32_t m, uint32_t n, uint32_t k, int 
 static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
 {
     FamilyEstimate e;
-    const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
+    const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e) - e.serial;
     if (bits == 4) {
         // (one row block that is not full costs less, a full one a little more than the 0.76 says: 64-row blocks of the
         // 128-column form at m = 40 / 48 / 64 against the tiles, us: 11008 x 8192 32.4 / 36.3, 33.6 / 36.5, 36.5 / 36.8;
@@ -1176,7 +1181,7 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
 static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits, const DecodePlan& pl)
 {
     FamilyEstimate e;
-    const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e);
+    const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e) - e.serial;
     if (bits == 4) return (pl.cols == 128u ? 0.70 : 0.84) * ranked;  // (the 128-column form measures 0.52 - 0.79 of its estimate)
     // (a row block that is not full costs less: 64-row blocks at m = 40 / 48 / 64 measure 0.87 / 0.91 / 1.0 of the tiles' time
     // over 11 weight shapes where the estimate had them level — the rows past m are neither converted for nor multiplied)
