@@ -1114,7 +1114,11 @@ static double packed8_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
 {
     const double walks = packed_slab_walks(n);
     const double rows = m <= 6u ? 1.0 + 0.0136 * (m - 1.0) : m <= 16u ? 1.068 + 0.0578 * (m - 6.0) : 0.856 + 0.0608 * m;
-    const double walk_us = walks * k / 1544.0, stream_us = (double)n * k / 6.16e6;
+    // (from the third walk on a walk never takes less than 2.2 us: its start and its reduction weigh as much as 1300 rows —
+    // k = 2048, m = 8 / 12: 10496 columns 10.2 us, 16384 columns 15.3, where rows alone would say 7.2 and 10.6; one or two
+    // walks of a short k hide them behind the launch: 4096 x 2048 stays at 3.7 us)
+    const double per_walk = (k / 1544.0 > 2.2 || walks <= 2.0) ? k / 1544.0 : 2.2;
+    const double walk_us = walks * per_walk, stream_us = (double)n * k / 6.16e6;
     return 2.07 + 0.017 * m * walks + (walk_us > stream_us ? walk_us : stream_us) * rows;
 }
 static double packed8_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
