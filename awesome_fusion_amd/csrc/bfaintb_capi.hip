@@ -1096,7 +1096,7 @@ static DecodePlan packed_family_plan(uint32_t m, uint32_t n, uint32_t k, int bit
 // 5120 x 13824, m = 16: slab 31.0, family 17.2; 13824 x 5120: 26.0 / 15.5; 4096 x 2048, m = 32: 5.5 / 6.9; 1024 x 16384,
 // m = 1: 10.5 / 9.0.  8-bit codes, m = 8: 5120 x 13824 23.2 / 16.3; 13824 x 5120 20.2 / 15.0; 5120 x 5120 11.3 / 9.2;
 // 2048 x 4096, m = 12: 5.5 / 6.9).  Picks on the scan, weights cold: 4-bit 9 of 252 more than 5 % off the faster kernel
-// (worst 12 %), 8-bit 17 of 252 (worst 14 %); fixed row limits, as before: 22 of 196, up to 42 %.
+// (worst 12 %), 8-bit 12 of 252 (worst 14 %); fixed row limits, as before: 22 of 196, up to 42 %.
 static double packed_slab_walks(uint32_t n)
 {
     const double cus = (double)machine_cus();
@@ -1123,7 +1123,10 @@ static double packed8_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
 }
 static double packed8_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
 {
-    const double stream_us = (double)n * k / 1.0e6 / (5.63 * pow(packed_family_fill(m, n, pl), 0.638));
+    // (a long k streams faster, the workgroups' starts and hand-overs weighing less: 6 x 15104 x 11008 28.8 us, 6 x 7168 x 14336
+    // 20.6, where 5.63 TB/s would say 34.1 and 23.3)
+    const double long_k = k <= 4096u ? 0.0 : k >= 12288u ? 1.0 : (k - 4096.0) / 8192.0;
+    const double stream_us = (double)n * k / 1.0e6 / (5.63 * (1.0 + 0.12 * long_k) * pow(packed_family_fill(m, n, pl), 0.638));
     return 3.0 + 0.0885 * m + 0.118 * (pl.splits - 1.0) + stream_us * (1.0 - 0.0037 * m + (m > 16u ? 0.1076 : 0.0)) * (pl.cols == 256u ? 1.1 : 1.0);
 }
 static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
