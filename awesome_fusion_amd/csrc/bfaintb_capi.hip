@@ -1135,7 +1135,10 @@ static double packed4_slab_time_us(uint32_t m, uint32_t n, uint32_t k)
     // (more than seven slabs per CU: 5 % less than that — 32000 / 50304 / 128256 / 151936 x 4096, m = 1: 17.6 / 26.2 / 63.4 / 74.8 us;
     // 28672 x 8192, seven, is as the formula says: 31.1)
     const double many = n / 16.0 > 7.0 * (double)machine_cus() ? 0.95 : 1.0;
-    return 2.58 + many * packed_slab_walks(n) * k / 1975.0 * rows;
+    // (from the third walk on a walk never takes less than 1.45 us, as for 8-bit codes: k = 2048, 12 x 10240 9.6 us, 8 x 9984 8.3)
+    const double walks = packed_slab_walks(n);
+    const double per_walk = (k / 1975.0 > 1.45 || walks <= 2.0) ? k / 1975.0 : 1.45;
+    return 2.58 + many * walks * per_walk * rows;
 }
 static double packed4_family_time_us(uint32_t m, uint32_t n, uint32_t k, const DecodePlan& pl)
 {
