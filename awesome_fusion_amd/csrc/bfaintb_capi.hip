@@ -178,6 +178,14 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
         // 48 / 64 x 50304 x 4096 79 / 81, where the tiles take 138 / 146 and 66 / 67)
         const double wgs = (double)((m + 16u * pl.mb - 1u) / (16u * pl.mb)) * (double)((n + pl.cols - 1u) / pl.cols) * pl.splits;
         if (pl.mb == 2u && wgs * 2.0 > 3.0 * (double)machine_cus()) return 0.84 * ranked;
+        // (beyond 256 rows, unsplit: ten row blocks and more over few column blocks take all the estimate says and up to 1.4
+        // times it — 320 x 2816 x 6144: 39.9 us, the tiles 29.0; 512 x 1280 x 5120: 35.9 / 26.7; 320 x 12032 x 6144: 101.7 / 93.6)
+        // (... and their 8-wave workgroups count as a busy machine in the estimate from 128 of them on: CUs left without one
+        // are charged here)
+        if (m > 256u && pl.splits == 1u) {
+            const double cus = (double)machine_cus();
+            return 5.0 + e.core * (wgs < cus ? cus / wgs : 1.0);
+        }
         return 0.76 * ranked;
     }
     // (64-row blocks: the hand-over at 0.9 of its term — at 0.65 the family ran up to 13 % over the tiles' time at 48 - 64 rows
