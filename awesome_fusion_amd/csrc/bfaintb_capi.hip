@@ -201,7 +201,7 @@ static double decode_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 // large ones win (1536 x 4096: 81 / 72, 512 x 11008: 80 / 68).
 // (One gap: a few tall tiles more than CUs — 640 x 11008 makes 258 — would go to 129 large tiles on half the machine, 82 us;
 // the small tiles take it in two rounds, 430 of them, in 66 us.  So: also up to two rounds of small tiles where the tall
-// ones do not fit one round and the large ones fill at most 55 % of the CUs.)
+// ones do not fit one round and the large ones fill at most 60 % of the CUs.)
 static bool prefill_small_tiles(uint32_t m, uint32_t n, int bits)
 {
     const uint64_t cus = machine_cus();
@@ -219,7 +219,8 @@ static bool prefill_small_tiles(uint32_t m, uint32_t n, int bits)
     if (bits == 4 && small * 20u <= cus * 27u) return true;
     const uint64_t tall = (uint64_t)((m + 255u) / 256u) * ((n + 127u) / 128u);
     const uint64_t large = (uint64_t)((m + 255u) / 256u) * ((n + 255u) / 256u);
-    return small <= 2u * cus && tall > cus && large * 20u <= cus * 11u;
+    // (0.6 of the CUs at most: 640 x 12032 x 3584, 141 large tiles, 76.2 us; 470 small ones 67.6)
+    return small <= 2u * cus && tall > cus && large * 5u <= cus * 3u;
 }
 
 // Between the two: more small tiles than CUs, but at most one tile of 256 rows x 128 columns per CU.  The large tiles would

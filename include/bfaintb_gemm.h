@@ -367,7 +367,7 @@ BFAINTB_API int bfaintb_gemm_variant(uint32_t m, uint32_t n, uint32_t k, int wei
  * weights with: 128 x 128 while that makes at most 256 tiles (one per CU); else 256 rows x 128 columns while that
  * makes at most 256; else 256 x 256 (256 = the device's compute units: one tile per unit) — except that up to 512
  * tiles of 128 x 128 run in two rounds where the 256 x 128 ones just miss one round and the 256 x 256 ones would fill
- * at most 55 % of the units (640 x 11008), and that up to 128 rows always run 128 x 128 tiles, in as many rounds as it
+ * at most 60 % of the units (640 x 11008), and that up to 128 rows always run 128 x 128 tiles, in as many rounds as it
  * takes (taller tiles would be half empty).  The two functions answer for 8-bit codes; 4-bit codes keep the 128 x 128
  * tiles up to 345 of them (their 256 x 128 kernel is the weaker one); bfaintb_gemm_plan answers for either.  Pre-packed
  * weights run the same tiles.  (The reference arithmetic has no 256 x 128 form: 256 x 256 there.) */
