@@ -62,6 +62,11 @@ def test_variant_choice_and_split():
     # (the gap: 258 tall tiles just miss one round and the large ones would use half the machine: two rounds of small tiles)
     assert af.prefill_tile(640, 11008) == 128 and af.plan(640, 11008, 4096).workgroups == 430 and af.plan(640, 11008, 4096).splits == 1
     assert af.prefill_tile(704, 11008) == 256 and af.prefill_tile(512, 11008) == 256 and af.prefill_tile_cols(512, 11008) == 128
+    # (... while the large tiles would fill at most 60 % of the CUs: 141 of them at 640 x 12032, 500 small ones at 600 x 12800)
+    assert af.prefill_tile(640, 12032) == 128 and af.plan(600, 12800, 4096).workgroups == 500
+    # 4-bit codes beyond 256 rows: ten row blocks over few column blocks, unsplit, lose to the tiles (39.9 against 29.0 us)
+    assert af.variant(320, 2816, 6144, 4, 128) == af.PREFILL and af.variant(512, 1280, 5120, 4, 128) == af.PREFILL
+    assert af.variant(320, 1024, 14336, 4, 128) == af.DECODE     # (with k split the family stays ahead: 30.4 against 38.3)
     assert af.prefill_tile(128, 28672) == 128 and af.prefill_tile(4096, 4096) == 256 and af.prefill_tile(1, 16) == 128
     # the small tiles over row-major weights split k while tiles x splits fit one workgroup per CU: same workspace layout as
     # the decode family's; the large tiles, the both-operands-in-LDS form and an unsplit launch need none
