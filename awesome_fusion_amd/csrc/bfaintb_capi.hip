@@ -1201,6 +1201,13 @@ static double packed_family_time_us(uint32_t m, uint32_t n, uint32_t k, int bits
 {
     FamilyEstimate e;
     const double ranked = decode_family_estimate_us(m, n, k, bits, pl, &e) - e.serial;
+    // Beyond 256 rows, unsplit, more than two rounds of workgroups (five row blocks and more against very many columns):
+    // all the estimate says (us, family / tiles: 320 x 44032 x 2048 8-bit 132 / 87; 384 x 37120 x 2048 4-bit 132 / 76).  With
+    // fewer workgroups than that the factors below stand: 640 x 1024 x 2048 12.3 / 16.3.
+    if (m > 256u && pl.splits == 1u) {
+        const double wgs_ = (double)((n + pl.cols - 1u) / pl.cols) * (double)((m + 16u * pl.mb - 1u) / (16u * pl.mb));
+        if (wgs_ > 2.0 * (double)machine_cus()) return 5.0 + e.core;
+    }
     if (bits == 4) return (pl.cols == 128u ? 0.70 : 0.84) * ranked;  // (the 128-column form measures 0.52 - 0.79 of its estimate)
     // (a row block that is not full costs less: 64-row blocks at m = 40 / 48 / 64 measure 0.87 / 0.91 / 1.0 of the tiles' time
     // over 11 weight shapes where the estimate had them level — the rows past m are neither converted for nor multiplied)
